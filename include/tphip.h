@@ -1,0 +1,162 @@
+/*
+ * tphip.h -- C ABI of libtphip.so, the only library in this tree that includes
+ * HIP headers. The host-side channels (hip_xth, hip_ipc, hip_basic) reach the
+ * GPU exclusively through these entry points.
+ *
+ * Conventions: every function returns 0 on success or a positive hipError_t
+ * value (negative values are errors detected by this library itself, see
+ * tphip_strerror). No exceptions, no C++ types, no reliance on the caller's
+ * current device: every call that needs a device takes its index explicitly.
+ * Streams and events are passed as void* (hipStream_t / hipEvent_t values).
+ * All functions are thread-safe.
+ *
+ * Each declaration names the reference interface it replaces; paths are
+ * relative to the root of pytorch/tensorpipe.
+ */
+#ifndef TPHIP_H_
+#define TPHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPHIP_IPC_HANDLE_BYTES 64
+#define TPHIP_UUID_STRLEN 36 /* 8-4-4-4-12 hex digits, NUL not counted */
+
+/* Errors raised by the library itself (all negative). */
+#define TPHIP_ERR_INVALID_ARG (-1)
+#define TPHIP_ERR_TOO_LARGE (-2)
+#define TPHIP_ERR_OVERLAP (-3)
+#define TPHIP_ERR_NO_DEVICE (-4)
+
+/* One entry of the copy table: `bytes` bytes from `src` to `dst`. Any
+ * alignment, any length (including 0). Ranges of different entries must not
+ * overlap each other's destinations, and no src range may overlap a dst range.
+ * Replaces the (dst, src, length) triple handed to cudaMemcpyAsync at
+ * tensorpipe/channel/cuda_xth/channel_impl.cc:69-71,
+ * tensorpipe/channel/cuda_ipc/channel_impl.cc:244-249,456-461 and
+ * tensorpipe/channel/cuda_basic/channel_impl.cc:58-71. */
+typedef struct tphip_copy_desc {
+  const void* src;
+  void* dst;
+  uint64_t bytes;
+} tphip_copy_desc;
+
+/* Largest table accepted by one tphip_batched_copy call. */
+#define TPHIP_MAX_BATCH 4096u
+
+const char* tphip_strerror(int err);
+
+/* ---- devices and pointers ------------------------------------------------ */
+
+/* Number of visible GPUs. Replaces cudaGetDeviceCount as used at
+ * tensorpipe/channel/cuda_xth/context_impl.cc:52-56. */
+int tphip_device_count(int* count);
+
+/* Device UUID as a 36-character string plus NUL. Replaces
+ * getUuidOfDevice/getUuidsOfVisibleDevices, tensorpipe/common/cuda.h:293-321. */
+int tphip_device_uuid(int dev, char out[TPHIP_UUID_STRLEN + 1]);
+
+/* Device ordinal that owns `ptr`; *dev = -1 for host memory unknown to HIP.
+ * *is_host is set to 1 for (pinned) host allocations. Replaces
+ * cudaDeviceForPointer, tensorpipe/common/cuda.h:141-166. */
+int tphip_device_for_ptr(const void* ptr, int* dev, int* is_host);
+
+/* Base address and size of the allocation containing `ptr` (needed because an
+ * IPC handle always refers to the allocation base; cf. the offset test at
+ * tensorpipe/test/channel/channel_test_cuda.cc:96-139). */
+int tphip_mem_base(const void* ptr, void** base, size_t* size);
+
+/* ---- memory -------------------------------------------------------------- */
+
+/* Device slab. Replaces makeCudaDeviceBuffer, tensorpipe/common/cuda.h:213-218. */
+int tphip_malloc(int dev, size_t bytes, void** ptr);
+int tphip_free(int dev, void* ptr);
+
+/* Pinned host slab, mapped into the device address space and portable across
+ * devices. *dev_ptr (may be NULL) receives the address kernels use for it.
+ * Replaces makeCudaPinnedBuffer, tensorpipe/common/cuda.h:183-188. */
+int tphip_host_alloc(int dev, size_t bytes, void** host_ptr, void** dev_ptr);
+int tphip_host_free(void* host_ptr);
+
+/* ---- streams and events -------------------------------------------------- */
+
+int tphip_stream_create(int dev, void** stream);
+int tphip_stream_destroy(int dev, void* stream);
+int tphip_stream_sync(int dev, void* stream);
+
+/* interprocess != 0 creates an event exportable with tphip_ipc_event_export.
+ * Timing is always disabled. Replaces CudaEvent,
+ * tensorpipe/common/cuda.h:49-139. */
+int tphip_event_create(int dev, int interprocess, void** event);
+/* Timing-enabled event (bench and tests only). */
+int tphip_event_create_timed(int dev, void** event);
+int tphip_event_destroy(int dev, void* event);
+int tphip_event_record(int dev, void* event, void* stream);
+int tphip_stream_wait_event(int dev, void* stream, void* event);
+/* *done = 1 when all work captured by the last record has finished. */
+int tphip_event_query(int dev, void* event, int* done);
+int tphip_event_sync(int dev, void* event);
+int tphip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* Run fn(arg, status) on a runtime thread once all work enqueued on `stream`
+ * so far has completed. Replaces CudaLoop::addCallback,
+ * tensorpipe/common/cuda_loop.cc:86-124. */
+typedef void (*tphip_host_fn)(void* arg, int status);
+int tphip_stream_on_complete(int dev, void* stream, tphip_host_fn fn, void* arg);
+
+/* ---- inter-process handles ----------------------------------------------- */
+
+/* `base` must be the base of a device allocation (see tphip_mem_base).
+ * Replaces cudaIpcGetMemHandle / cudaIpcOpenMemHandle / cudaIpcCloseMemHandle,
+ * tensorpipe/common/cuda.h:226-268. */
+int tphip_ipc_mem_export(int dev, void* base, uint8_t out[TPHIP_IPC_HANDLE_BYTES]);
+int tphip_ipc_mem_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], void** ptr);
+int tphip_ipc_mem_close(int dev, void* ptr);
+
+/* Replaces cudaIpcGetEventHandle / cudaIpcOpenEventHandle,
+ * tensorpipe/common/cuda.h:88-93,119-124. */
+int tphip_ipc_event_export(int dev, void* event, uint8_t out[TPHIP_IPC_HANDLE_BYTES]);
+int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], void** event);
+
+/* ---- data movement ------------------------------------------------------- */
+
+/* The hot path. Enqueue on `stream` ONE kernel launch that performs every copy
+ * of `table[0..n)`; `table` is host memory and may be reused as soon as the
+ * call returns. Any mix of device, mapped-pinned-host and peer-mapped (IPC)
+ * addresses is accepted as long as the device can address them. n == 0 or an
+ * all-empty table enqueues nothing. n > TPHIP_MAX_BATCH returns
+ * TPHIP_ERR_TOO_LARGE. Replaces one cudaMemcpyAsync per tensor at the three
+ * call sites listed for tphip_copy_desc. */
+int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* stream);
+
+/* Single-copy convenience wrapper over the same kernel (n == 1, descriptor
+ * travels in the kernel arguments). */
+int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream);
+
+/* Same as tphip_batched_copy with explicit launch shape, for tuning sweeps:
+ * `unroll` in {1,2,4,8} 16-byte vectors per lane per slice, `blocks` workgroups
+ * of 256 threads (0 = default), `nontemporal` 0/1. */
+int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
+                             int unroll, uint32_t blocks, int nontemporal);
+
+/* Runtime copy engine path (hipMemcpyAsync), kept only as the A/B comparison
+ * for the kernel-driven copies; never used by the channels' data path. */
+int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream);
+
+/* Fill `bytes` bytes at `ptr` with `value` using a kernel (safe to capture in
+ * a HIP graph, unlike a memset node). */
+int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream);
+
+/* Keeps `stream` busy for a long time while repeatedly rewriting `ptr[0..n)`,
+ * leaving garbage behind; lets a test detect a missing event wait. HIP
+ * counterpart of slowKernel, tensorpipe/test/channel/kernel.cu:11-22. */
+int tphip_test_slow_kernel(int dev, void* ptr, uint64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPHIP_H_ */

@@ -1,0 +1,313 @@
+// Batched multi-tensor copy kernels for gfx950 (wave64).
+//
+// Work decomposition
+// ------------------
+// Every table entry {src, dst, bytes} is cut into
+//   head : the 0..15 bytes before the first 16-byte aligned destination address
+//   body : whole 16-byte vectors, destination aligned, source possibly not
+//   tail : the 0..15 bytes left after the last whole vector
+// The bodies of all entries are concatenated into one virtual sequence of
+// vectors (an exclusive prefix sum over per-entry vector counts, computed on
+// the host and shipped with the table). That sequence is cut into slices of
+// 64*U vectors; wavefront w of W takes slices w, w+W, w+2W, ... A slice that
+// lies inside one entry is copied with U independent 16-byte loads per lane
+// followed by U stores; a slice that straddles entries makes each lane look up
+// the entry of each of its vectors, so small tensors are packed lane-tight
+// into wavefronts instead of costing a launch (or a wavefront) each.
+// Heads and tails of 64 entries at a time are gathered by one wavefront: a
+// ballot skips the common all-aligned case, an inclusive wave scan of the
+// per-entry byte counts compacts the odd bytes over the 64 lanes.
+//
+// No LDS tiling is needed beyond the prefix array: the kernel is a pure HBM
+// stream (2 bytes of traffic per payload byte), never touches MFMA.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tphip.h"
+
+namespace tphip {
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+// Same vector, but the compiler may not assume any alignment: gfx950 global
+// loads accept unaligned addresses, so this still becomes one dwordx4 load.
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
+
+constexpr int kWave = 64;
+constexpr int kBlockThreads = 256;
+constexpr int kWavesPerBlock = kBlockThreads / kWave;
+
+template <bool NT>
+__device__ __forceinline__ u32x4 load16(const char* p) {
+  if (NT) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_unaligned*>(p));
+  }
+  return *reinterpret_cast<const u32x4_unaligned*>(p);
+}
+
+template <bool NT>
+__device__ __forceinline__ void store16(char* p, u32x4 v) {
+  if (NT) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+  } else {
+    *reinterpret_cast<u32x4*>(p) = v;
+  }
+}
+
+__device__ __forceinline__ uint32_t head_bytes(const void* dst, uint64_t bytes) {
+  uint64_t h = (0 - reinterpret_cast<uintptr_t>(dst)) & 15u;
+  return static_cast<uint32_t>(h < bytes ? h : bytes);
+}
+
+// Copy `nvec` (<= 64*U) vectors starting at s/d; d is 16-byte aligned.
+template <int U, bool NT>
+__device__ __forceinline__ void copy_span(const char* s, char* d, uint32_t nvec, uint32_t lane) {
+  u32x4 v[U];
+  if (nvec == kWave * U) {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      v[j] = load16<NT>(s + (static_cast<size_t>(j) * kWave + lane) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      store16<NT>(d + (static_cast<size_t>(j) * kWave + lane) * 16, v[j]);
+    }
+  } else {
+    // Partial slice (nvec >= 1): out-of-range lanes re-read the last vector so
+    // that all U loads are issued back to back without branches; only the
+    // stores are predicated.
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const uint32_t idx = j * kWave + lane;
+      const uint32_t ci = idx < nvec ? idx : nvec - 1;
+      v[j] = load16<NT>(s + static_cast<size_t>(ci) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const uint32_t idx = j * kWave + lane;
+      if (idx < nvec) {
+        store16<NT>(d + static_cast<size_t>(idx) * 16, v[j]);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ uint64_t shfl64(uint64_t v, int srcLane) {
+  uint32_t lo = __shfl(static_cast<uint32_t>(v), srcLane);
+  uint32_t hi = __shfl(static_cast<uint32_t>(v >> 32), srcLane);
+  return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+// One wavefront moves the heads and tails of entries [64*group, 64*group+64).
+__device__ __forceinline__ void copy_edges(
+    const tphip_copy_desc* __restrict__ descs, uint32_t n, uint32_t group, uint32_t lane) {
+  uint32_t t = group * kWave + lane;
+  uint64_t src = 0, dst = 0, bytes = 0;
+  if (t < n) {
+    src = reinterpret_cast<uint64_t>(descs[t].src);
+    dst = reinterpret_cast<uint64_t>(descs[t].dst);
+    bytes = descs[t].bytes;
+  }
+  uint32_t head = head_bytes(reinterpret_cast<const void*>(dst), bytes);
+  uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
+  uint64_t tailOff = bytes - tail;
+  uint32_t cnt = head + tail;
+  if (__ballot(cnt != 0) == 0) {
+    return; // every entry of this group is vector-aligned at both ends
+  }
+  uint32_t incl = cnt;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    uint32_t o = __shfl_up(incl, d);
+    if (lane >= static_cast<uint32_t>(d)) {
+      incl += o;
+    }
+  }
+  uint32_t excl = incl - cnt;
+  uint32_t total = __shfl(incl, kWave - 1);
+  for (uint32_t base = 0; base < total; base += kWave) {
+    uint32_t b = base + lane;
+    bool active = b < total;
+    uint32_t bb = active ? b : total - 1;
+    // Largest lane whose exclusive prefix is <= bb owns byte bb.
+    int lo = 0, hi = kWave;
+#pragma unroll
+    for (int it = 0; it < 6; ++it) {
+      int mid = (lo + hi) >> 1;
+      uint32_t e = __shfl(excl, mid);
+      if (e <= bb) {
+        lo = mid;
+      } else {
+        hi = mid;
+      }
+    }
+    uint32_t k = bb - __shfl(excl, lo);
+    uint32_t oh = __shfl(head, lo);
+    uint64_t osrc = shfl64(src, lo);
+    uint64_t odst = shfl64(dst, lo);
+    uint64_t otail = shfl64(tailOff, lo);
+    uint64_t off = k < oh ? k : otail + (k - oh);
+    if (active) {
+      reinterpret_cast<char*>(odst)[off] = reinterpret_cast<const char*>(osrc)[off];
+    }
+  }
+}
+
+// Table variant. prefix[0..n] is the exclusive prefix sum of body vector
+// counts (prefix[n] = total). Dynamic LDS: (n+1) * 4 bytes.
+template <int U, bool NT>
+__global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
+    const uint32_t* __restrict__ prefix,
+    const tphip_copy_desc* __restrict__ descs,
+    uint32_t n,
+    uint32_t nslices) {
+  extern __shared__ uint32_t sPrefix[];
+  for (uint32_t i = threadIdx.x; i <= n; i += kBlockThreads) {
+    sPrefix[i] = prefix[i];
+  }
+  __syncthreads();
+
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t wave = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const uint32_t nwaves = gridDim.x * kWavesPerBlock;
+  const uint32_t total = sPrefix[n];
+  constexpr uint32_t kSlice = kWave * U;
+
+  for (uint32_t g = wave; g * kWave < n; g += nwaves) {
+    copy_edges(descs, n, g, lane);
+  }
+
+  uint32_t t = 0;
+#pragma clang loop unroll(disable)
+  for (uint32_t s = wave; s < nslices; s += nwaves) {
+    const uint32_t v0 = s * kSlice;
+    const uint32_t left = total - v0;
+    const uint32_t cnt = left < kSlice ? left : kSlice;
+    // Largest entry index with prefix <= v0; slices only move forward.
+    uint32_t lo = t, hi = n;
+    while (hi - lo > 1) {
+      uint32_t mid = (lo + hi) >> 1;
+      if (sPrefix[mid] <= v0) {
+        lo = mid;
+      } else {
+        hi = mid;
+      }
+    }
+    t = __builtin_amdgcn_readfirstlane(lo);
+    const uint32_t tBegin = sPrefix[t];
+    const uint32_t tEnd = sPrefix[t + 1];
+    if (v0 + cnt <= tEnd) {
+      // Slice inside one entry: uniform addresses, U loads in flight per lane.
+      const char* src = static_cast<const char*>(descs[t].src);
+      char* dst = static_cast<char*>(descs[t].dst);
+      const uint64_t off =
+          static_cast<uint64_t>(v0 - tBegin) * 16 + head_bytes(dst, descs[t].bytes);
+      copy_span<U, NT>(src + off, dst + off, cnt, lane);
+    } else {
+      // Slice straddles entries: per-lane lookup packs small tensors tightly.
+      const char* sp[U];
+      char* dp[U];
+      u32x4 v[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const uint32_t idx = j * kWave + lane;
+        // Lanes past the end redo the slice's last vector (load only).
+        const uint32_t vv = v0 + (idx < cnt ? idx : cnt - 1);
+        uint32_t l = t, h = n;
+        while (h - l > 1) {
+          const uint32_t m = (l + h) >> 1;
+          if (sPrefix[m] <= vv) {
+            l = m;
+          } else {
+            h = m;
+          }
+        }
+        const char* src = static_cast<const char*>(descs[l].src);
+        char* dst = static_cast<char*>(descs[l].dst);
+        const uint64_t off =
+            static_cast<uint64_t>(vv - sPrefix[l]) * 16 + head_bytes(dst, descs[l].bytes);
+        sp[j] = src + off;
+        dp[j] = dst + off;
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        v[j] = load16<NT>(sp[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        if (j * kWave + lane < cnt) {
+          store16<NT>(dp[j], v[j]);
+        }
+      }
+    }
+  }
+}
+
+// Single-entry variant: the descriptor travels in the kernel arguments, no
+// table upload, no LDS, 64-bit vector counts (any size).
+template <int U, bool NT>
+__global__ __launch_bounds__(kBlockThreads) void single_copy_kernel(
+    const char* __restrict__ src, char* __restrict__ dst, uint64_t bytes) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+  const uint64_t nwaves = static_cast<uint64_t>(gridDim.x) * kWavesPerBlock;
+  const uint32_t head = head_bytes(dst, bytes);
+  const uint64_t nvec = (bytes - head) >> 4;
+  const uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
+  constexpr uint64_t kSlice = kWave * U;
+
+  if (wave == 0) {
+    if (lane < head) {
+      dst[lane] = src[lane];
+    } else if (lane >= 16 && lane - 16 < tail) {
+      const uint64_t o = bytes - tail + (lane - 16);
+      dst[o] = src[o];
+    }
+  }
+  const char* s = src + head;
+  char* d = dst + head;
+  const uint64_t nslices = (nvec + kSlice - 1) / kSlice;
+#pragma clang loop unroll(disable)
+  for (uint64_t sl = wave; sl < nslices; sl += nwaves) {
+    const uint64_t v0 = sl * kSlice;
+    const uint64_t left = nvec - v0;
+    const uint32_t cnt = static_cast<uint32_t>(left < kSlice ? left : kSlice);
+    copy_span<U, NT>(s + v0 * 16, d + v0 * 16, cnt, lane);
+  }
+}
+
+// Stages the host-written (pinned, device-mapped) plan into device memory so
+// that the copy kernel's table reads hit L2/HBM instead of the host link.
+__global__ __launch_bounds__(kBlockThreads) void stage_plan_kernel(
+    const u32x4* __restrict__ hostPlan, u32x4* __restrict__ devPlan, uint32_t nvec) {
+  for (uint32_t i = blockIdx.x * kBlockThreads + threadIdx.x; i < nvec;
+       i += gridDim.x * kBlockThreads) {
+    devPlan[i] = hostPlan[i];
+  }
+}
+
+__global__ __launch_bounds__(kBlockThreads) void fill_kernel(
+    unsigned char* __restrict__ p, unsigned char value, uint64_t n) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kBlockThreads;
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < n;
+       i += stride) {
+    p[i] = value;
+  }
+}
+
+// Long dependent chain of byte updates per element; bounded, always exits.
+__global__ __launch_bounds__(128) void slow_kernel(volatile unsigned char* p, uint64_t n) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    unsigned char x = p[i];
+    for (int k = 0; k < 100000; ++k) {
+      x = static_cast<unsigned char>(x * 5u + 1u);
+      p[i] = x;
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+}
+
+} // namespace tphip

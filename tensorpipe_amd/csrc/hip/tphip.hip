@@ -1,0 +1,656 @@
+// libtphip.so: the C ABI declared in include/tphip.h. Thin, exception-free
+// wrappers over the HIP runtime plus the launch logic of the batched copy
+// kernel. Nothing here knows about channels or pipes.
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "copy_kernels.hip.h"
+#include "tphip.h"
+
+namespace {
+
+using namespace tphip;
+
+#define TPHIP_TRY(expr)                     \
+  do {                                      \
+    hipError_t e_ = (expr);                 \
+    if (e_ != hipSuccess) {                 \
+      return static_cast<int>(e_);          \
+    }                                       \
+  } while (0)
+
+constexpr int kMaxDevices = 16;
+constexpr uint32_t kPlanSlots = 32;
+// One plan = prefix[n+1] (padded to 16 B) followed by n descriptors.
+constexpr size_t kPlanSlotBytes =
+    ((TPHIP_MAX_BATCH + 1) * sizeof(uint32_t) + 15) / 16 * 16 +
+    TPHIP_MAX_BATCH * sizeof(tphip_copy_desc);
+// Plans for small tables are packed into sub-slots so that a burst of
+// messages does not wait for a slot.
+constexpr uint64_t kMaxTableVectors = 0xFFFFFFFFull - 64ull * 8ull;
+
+struct DeviceState {
+  std::once_flag once;
+  int initError{0};
+  int numCus{0};
+  // Ring of plan slots: host side (pinned, device-mapped) and device side.
+  char* hostPlans{nullptr};
+  char* hostPlansDev{nullptr};
+  char* devPlans{nullptr};
+  hipEvent_t slotDone[kPlanSlots]{};
+  bool slotUsed[kPlanSlots]{};
+  uint32_t nextSlot{0};
+  std::mutex mutex;
+};
+
+DeviceState gDevices[kMaxDevices];
+
+int defaultUnroll() {
+  static int v = [] {
+    const char* e = getenv("TPHIP_COPY_UNROLL");
+    int u = e ? atoi(e) : 4;
+    return (u == 1 || u == 2 || u == 4 || u == 8) ? u : 4;
+  }();
+  return v;
+}
+
+int defaultBlocksPerCu() {
+  static int v = [] {
+    const char* e = getenv("TPHIP_COPY_BLOCKS_PER_CU");
+    int b = e ? atoi(e) : 8;
+    return b > 0 && b <= 64 ? b : 8;
+  }();
+  return v;
+}
+
+int defaultNontemporal() {
+  static int v = [] {
+    const char* e = getenv("TPHIP_COPY_NT");
+    return e ? (atoi(e) != 0) : 1;
+  }();
+  return v;
+}
+
+int planViaKernel() {
+  static int v = [] {
+    const char* e = getenv("TPHIP_PLAN_STAGE_KERNEL");
+    return e ? (atoi(e) != 0) : 1;
+  }();
+  return v;
+}
+
+int getDevice(int dev, DeviceState** out) {
+  if (dev < 0 || dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  DeviceState& st = gDevices[dev];
+  TPHIP_TRY(hipSetDevice(dev));
+  std::call_once(st.once, [&] {
+    hipError_t e = hipDeviceGetAttribute(&st.numCus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess) {
+      e = hipHostMalloc(
+          reinterpret_cast<void**>(&st.hostPlans),
+          kPlanSlots * kPlanSlotBytes,
+          hipHostMallocMapped | hipHostMallocPortable);
+    }
+    if (e == hipSuccess) {
+      e = hipHostGetDevicePointer(reinterpret_cast<void**>(&st.hostPlansDev), st.hostPlans, 0);
+    }
+    if (e == hipSuccess) {
+      e = hipMalloc(reinterpret_cast<void**>(&st.devPlans), kPlanSlots * kPlanSlotBytes);
+    }
+    for (uint32_t i = 0; e == hipSuccess && i < kPlanSlots; ++i) {
+      e = hipEventCreateWithFlags(&st.slotDone[i], hipEventDisableTiming);
+    }
+    st.initError = static_cast<int>(e);
+  });
+  if (st.initError != 0) {
+    return st.initError;
+  }
+  *out = &st;
+  return 0;
+}
+
+template <bool NT>
+int launchSingle(int unroll, uint32_t blocks, hipStream_t stream, const char* src, char* dst,
+                 uint64_t bytes) {
+  switch (unroll) {
+    case 1:
+      hipLaunchKernelGGL((single_copy_kernel<1, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
+                         src, dst, bytes);
+      break;
+    case 2:
+      hipLaunchKernelGGL((single_copy_kernel<2, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
+                         src, dst, bytes);
+      break;
+    case 8:
+      hipLaunchKernelGGL((single_copy_kernel<8, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
+                         src, dst, bytes);
+      break;
+    default:
+      hipLaunchKernelGGL((single_copy_kernel<4, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
+                         src, dst, bytes);
+      break;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+template <bool NT>
+int launchTable(int unroll, uint32_t blocks, size_t lds, hipStream_t stream,
+                const uint32_t* prefix, const tphip_copy_desc* descs, uint32_t n,
+                uint32_t nslices) {
+  switch (unroll) {
+    case 1:
+      hipLaunchKernelGGL((batched_copy_kernel<1, NT>), dim3(blocks), dim3(kBlockThreads), lds,
+                         stream, prefix, descs, n, nslices);
+      break;
+    case 2:
+      hipLaunchKernelGGL((batched_copy_kernel<2, NT>), dim3(blocks), dim3(kBlockThreads), lds,
+                         stream, prefix, descs, n, nslices);
+      break;
+    case 8:
+      hipLaunchKernelGGL((batched_copy_kernel<8, NT>), dim3(blocks), dim3(kBlockThreads), lds,
+                         stream, prefix, descs, n, nslices);
+      break;
+    default:
+      hipLaunchKernelGGL((batched_copy_kernel<4, NT>), dim3(blocks), dim3(kBlockThreads), lds,
+                         stream, prefix, descs, n, nslices);
+      break;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+uint32_t pickBlocks(const DeviceState& st, uint64_t nslices, uint32_t minWaves, uint32_t blocks) {
+  uint64_t wantWaves = nslices > minWaves ? nslices : minWaves;
+  uint64_t want = (wantWaves + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (want == 0) {
+    want = 1;
+  }
+  uint64_t cap = blocks != 0 ? blocks
+                             : static_cast<uint64_t>(st.numCus > 0 ? st.numCus : 256) *
+          defaultBlocksPerCu();
+  return static_cast<uint32_t>(want < cap ? want : cap);
+}
+
+int copySingle(DeviceState& st, const tphip_copy_desc& d, hipStream_t stream, int unroll,
+               uint32_t blocks, int nt) {
+  if (d.bytes == 0) {
+    return 0;
+  }
+  if (d.src == nullptr || d.dst == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  const uint64_t nvec = d.bytes >> 4;
+  const uint64_t nslices = (nvec + uint64_t(kWave) * unroll - 1) / (uint64_t(kWave) * unroll) + 1;
+  const uint32_t grid = pickBlocks(st, nslices, 1, blocks);
+  const char* src = static_cast<const char*>(d.src);
+  char* dst = static_cast<char*>(d.dst);
+  return nt ? launchSingle<true>(unroll, grid, stream, src, dst, d.bytes)
+            : launchSingle<false>(unroll, grid, stream, src, dst, d.bytes);
+}
+
+// Launch one table kernel over table[0..n) whose body vector total fits 32 bits.
+int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStream_t stream,
+              int unroll, uint32_t blocks, int nt) {
+  const size_t prefixBytes = ((size_t(n) + 1) * sizeof(uint32_t) + 15) / 16 * 16;
+  const size_t planBytes = prefixBytes + size_t(n) * sizeof(tphip_copy_desc);
+  const size_t planBytesPadded = (planBytes + 15) / 16 * 16;
+
+  uint32_t slot;
+  {
+    std::lock_guard<std::mutex> lock(st.mutex);
+    slot = st.nextSlot;
+    st.nextSlot = (st.nextSlot + 1) % kPlanSlots;
+    if (st.slotUsed[slot]) {
+      // The launch that last used this slot must have consumed its plan.
+      TPHIP_TRY(hipEventSynchronize(st.slotDone[slot]));
+    }
+    st.slotUsed[slot] = true;
+
+    char* host = st.hostPlans + size_t(slot) * kPlanSlotBytes;
+    char* hostDev = st.hostPlansDev + size_t(slot) * kPlanSlotBytes;
+    char* devp = st.devPlans + size_t(slot) * kPlanSlotBytes;
+    uint32_t* prefix = reinterpret_cast<uint32_t*>(host);
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+      prefix[i] = static_cast<uint32_t>(total);
+      const uint64_t bytes = table[i].bytes;
+      uint64_t head = (0 - reinterpret_cast<uintptr_t>(table[i].dst)) & 15u;
+      if (head > bytes) {
+        head = bytes;
+      }
+      total += (bytes - head) >> 4;
+    }
+    prefix[n] = static_cast<uint32_t>(total);
+    memcpy(host + prefixBytes, table, size_t(n) * sizeof(tphip_copy_desc));
+
+    if (planViaKernel()) {
+      const uint32_t nv = static_cast<uint32_t>(planBytesPadded / 16);
+      const uint32_t sb = (nv + kBlockThreads - 1) / kBlockThreads;
+      hipLaunchKernelGGL(stage_plan_kernel, dim3(sb < 8 ? sb : 8), dim3(kBlockThreads), 0, stream,
+                         reinterpret_cast<const u32x4*>(hostDev), reinterpret_cast<u32x4*>(devp),
+                         nv);
+      TPHIP_TRY(hipGetLastError());
+    } else {
+      TPHIP_TRY(hipMemcpyAsync(devp, host, planBytesPadded, hipMemcpyHostToDevice, stream));
+    }
+
+    const uint64_t slice = uint64_t(kWave) * unroll;
+    const uint32_t nslices = static_cast<uint32_t>((total + slice - 1) / slice);
+    const uint32_t edgeWaves = (n + kWave - 1) / kWave;
+    const uint32_t grid = pickBlocks(st, nslices, edgeWaves, blocks);
+    const size_t lds = (size_t(n) + 1) * sizeof(uint32_t);
+    const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
+    const tphip_copy_desc* dDescs = reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes);
+    int rc = nt ? launchTable<true>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices)
+                : launchTable<false>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices);
+    if (rc != 0) {
+      return rc;
+    }
+    TPHIP_TRY(hipEventRecord(st.slotDone[slot], stream));
+  }
+  return 0;
+}
+
+int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* streamPtr,
+                    int unroll, uint32_t blocks, int nt) {
+  if (n == 0) {
+    return 0;
+  }
+  if (table == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  if (n > TPHIP_MAX_BATCH) {
+    return TPHIP_ERR_TOO_LARGE;
+  }
+  if (!(unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8)) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  DeviceState* st = nullptr;
+  int rc = getDevice(dev, &st);
+  if (rc != 0) {
+    return rc;
+  }
+  hipStream_t stream = static_cast<hipStream_t>(streamPtr);
+
+  // Drop empty entries up front; reject null pointers on non-empty ones.
+  std::vector<tphip_copy_desc> live;
+  const tphip_copy_desc* cur = table;
+  uint32_t m = n;
+  bool anyEmpty = false;
+  for (uint32_t i = 0; i < n; ++i) {
+    if (table[i].bytes == 0) {
+      anyEmpty = true;
+    } else if (table[i].src == nullptr || table[i].dst == nullptr) {
+      return TPHIP_ERR_INVALID_ARG;
+    }
+  }
+  if (anyEmpty) {
+    live.reserve(n);
+    for (uint32_t i = 0; i < n; ++i) {
+      if (table[i].bytes != 0) {
+        live.push_back(table[i]);
+      }
+    }
+    cur = live.data();
+    m = static_cast<uint32_t>(live.size());
+    if (m == 0) {
+      return 0;
+    }
+  }
+
+  // Cut into launches whose body vector total fits the 32-bit prefix; entries
+  // too large for that go through the single-entry kernel (64-bit counts).
+  uint32_t begin = 0;
+  uint64_t acc = 0;
+  for (uint32_t i = 0; i <= m; ++i) {
+    const uint64_t vecs = i < m ? (cur[i].bytes >> 4) : 0;
+    const bool huge = i < m && vecs > kMaxTableVectors;
+    if (i == m || huge || acc + vecs > kMaxTableVectors) {
+      const uint32_t cnt = i - begin;
+      if (cnt == 1) {
+        rc = copySingle(*st, cur[begin], stream, unroll, blocks, nt);
+      } else if (cnt > 1) {
+        rc = copyTable(*st, cur + begin, cnt, stream, unroll, blocks, nt);
+      }
+      if (rc != 0) {
+        return rc;
+      }
+      begin = i;
+      acc = 0;
+      if (huge) {
+        rc = copySingle(*st, cur[i], stream, unroll, blocks, nt);
+        if (rc != 0) {
+          return rc;
+        }
+        begin = i + 1;
+        continue;
+      }
+    }
+    acc += vecs;
+  }
+  return 0;
+}
+
+struct HostFnThunk {
+  tphip_host_fn fn;
+  void* arg;
+};
+
+void hostFnTrampoline(hipStream_t, hipError_t status, void* userData) {
+  HostFnThunk* t = static_cast<HostFnThunk*>(userData);
+  t->fn(t->arg, static_cast<int>(status));
+  delete t;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* tphip_strerror(int err) {
+  switch (err) {
+    case 0:
+      return "success";
+    case TPHIP_ERR_INVALID_ARG:
+      return "tphip: invalid argument";
+    case TPHIP_ERR_TOO_LARGE:
+      return "tphip: table larger than TPHIP_MAX_BATCH";
+    case TPHIP_ERR_OVERLAP:
+      return "tphip: overlapping ranges in copy table";
+    case TPHIP_ERR_NO_DEVICE:
+      return "tphip: no usable GPU";
+    default:
+      return hipGetErrorString(static_cast<hipError_t>(err));
+  }
+}
+
+int tphip_device_count(int* count) {
+  if (count == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  *count = 0;
+  hipError_t e = hipGetDeviceCount(count);
+  if (e == hipErrorNoDevice) {
+    *count = 0;
+    (void)hipGetLastError();
+    return 0;
+  }
+  return static_cast<int>(e);
+}
+
+int tphip_device_uuid(int dev, char out[TPHIP_UUID_STRLEN + 1]) {
+  if (out == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  hipUUID uuid;
+  TPHIP_TRY(hipDeviceGetUuid(&uuid, dev));
+  static const char* hex = "0123456789abcdef";
+  int o = 0;
+  for (int i = 0; i < 16; ++i) {
+    if (i == 4 || i == 6 || i == 8 || i == 10) {
+      out[o++] = '-';
+    }
+    unsigned char b = static_cast<unsigned char>(uuid.bytes[i]);
+    out[o++] = hex[b >> 4];
+    out[o++] = hex[b & 15];
+  }
+  out[o] = '\0';
+  return 0;
+}
+
+int tphip_device_for_ptr(const void* ptr, int* dev, int* is_host) {
+  if (dev == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  hipPointerAttribute_t attr;
+  memset(&attr, 0, sizeof(attr));
+  hipError_t e = hipPointerGetAttributes(&attr, ptr);
+  if (e == hipErrorInvalidValue) {
+    // Plain host memory the runtime has never seen.
+    (void)hipGetLastError();
+    *dev = -1;
+    if (is_host) {
+      *is_host = 1;
+    }
+    return 0;
+  }
+  TPHIP_TRY(e);
+  const bool host = attr.type == hipMemoryTypeHost || attr.type == hipMemoryTypeUnregistered;
+  if (is_host) {
+    *is_host = host ? 1 : 0;
+  }
+  *dev = attr.type == hipMemoryTypeUnregistered ? -1 : attr.device;
+  return 0;
+}
+
+int tphip_mem_base(const void* ptr, void** base, size_t* size) {
+  hipDeviceptr_t b = nullptr;
+  size_t s = 0;
+  TPHIP_TRY(hipMemGetAddressRange(&b, &s, const_cast<void*>(ptr)));
+  if (base) {
+    *base = b;
+  }
+  if (size) {
+    *size = s;
+  }
+  return 0;
+}
+
+int tphip_malloc(int dev, size_t bytes, void** ptr) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipMalloc(ptr, bytes));
+  return 0;
+}
+
+int tphip_free(int dev, void* ptr) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipFree(ptr));
+  return 0;
+}
+
+int tphip_host_alloc(int dev, size_t bytes, void** host_ptr, void** dev_ptr) {
+  if (host_ptr == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipHostMalloc(host_ptr, bytes, hipHostMallocMapped | hipHostMallocPortable));
+  if (dev_ptr != nullptr) {
+    TPHIP_TRY(hipHostGetDevicePointer(dev_ptr, *host_ptr, 0));
+  }
+  return 0;
+}
+
+int tphip_host_free(void* host_ptr) {
+  TPHIP_TRY(hipHostFree(host_ptr));
+  return 0;
+}
+
+int tphip_stream_create(int dev, void** stream) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipStream_t s;
+  TPHIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = s;
+  return 0;
+}
+
+int tphip_stream_destroy(int dev, void* stream) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int tphip_stream_sync(int dev, void* stream) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int tphip_event_create(int dev, int interprocess, void** event) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipEvent_t e;
+  unsigned flags = hipEventDisableTiming;
+  if (interprocess) {
+    flags |= hipEventInterprocess;
+  }
+  TPHIP_TRY(hipEventCreateWithFlags(&e, flags));
+  *event = e;
+  return 0;
+}
+
+int tphip_event_create_timed(int dev, void** event) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipEvent_t e;
+  TPHIP_TRY(hipEventCreate(&e));
+  *event = e;
+  return 0;
+}
+
+int tphip_event_destroy(int dev, void* event) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return 0;
+}
+
+int tphip_event_record(int dev, void* event, void* stream) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int tphip_stream_wait_event(int dev, void* stream, void* event) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(
+      hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
+  return 0;
+}
+
+int tphip_event_query(int dev, void* event, int* done) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
+  if (e == hipErrorNotReady) {
+    (void)hipGetLastError();
+    *done = 0;
+    return 0;
+  }
+  TPHIP_TRY(e);
+  *done = 1;
+  return 0;
+}
+
+int tphip_event_sync(int dev, void* event) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+  return 0;
+}
+
+int tphip_event_elapsed_ms(void* start, void* stop, float* ms) {
+  TPHIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return 0;
+}
+
+int tphip_stream_on_complete(int dev, void* stream, tphip_host_fn fn, void* arg) {
+  if (fn == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_TRY(hipSetDevice(dev));
+  HostFnThunk* t = new HostFnThunk{fn, arg};
+  hipError_t e = hipStreamAddCallback(static_cast<hipStream_t>(stream), hostFnTrampoline, t, 0);
+  if (e != hipSuccess) {
+    delete t;
+    return static_cast<int>(e);
+  }
+  return 0;
+}
+
+int tphip_ipc_mem_export(int dev, void* base, uint8_t out[TPHIP_IPC_HANDLE_BYTES]) {
+  static_assert(sizeof(hipIpcMemHandle_t) == TPHIP_IPC_HANDLE_BYTES, "handle size");
+  TPHIP_TRY(hipSetDevice(dev));
+  hipIpcMemHandle_t h;
+  TPHIP_TRY(hipIpcGetMemHandle(&h, base));
+  memcpy(out, &h, sizeof(h));
+  return 0;
+}
+
+int tphip_ipc_mem_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], void** ptr) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipIpcMemHandle_t h;
+  memcpy(&h, handle, sizeof(h));
+  TPHIP_TRY(hipIpcOpenMemHandle(ptr, h, hipIpcMemLazyEnablePeerAccess));
+  return 0;
+}
+
+int tphip_ipc_mem_close(int dev, void* ptr) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipIpcCloseMemHandle(ptr));
+  return 0;
+}
+
+int tphip_ipc_event_export(int dev, void* event, uint8_t out[TPHIP_IPC_HANDLE_BYTES]) {
+  static_assert(sizeof(hipIpcEventHandle_t) == TPHIP_IPC_HANDLE_BYTES, "handle size");
+  TPHIP_TRY(hipSetDevice(dev));
+  hipIpcEventHandle_t h;
+  TPHIP_TRY(hipIpcGetEventHandle(&h, static_cast<hipEvent_t>(event)));
+  memcpy(out, &h, sizeof(h));
+  return 0;
+}
+
+int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], void** event) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipIpcEventHandle_t h;
+  memcpy(&h, handle, sizeof(h));
+  hipEvent_t e;
+  TPHIP_TRY(hipIpcOpenEventHandle(&e, h));
+  *event = e;
+  return 0;
+}
+
+int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* stream) {
+  return batchedCopyImpl(dev, table, n, stream, defaultUnroll(), 0, defaultNontemporal());
+}
+
+int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {
+  tphip_copy_desc d{src, dst, bytes};
+  return batchedCopyImpl(dev, &d, 1, stream, defaultUnroll(), 0, defaultNontemporal());
+}
+
+int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
+                             int unroll, uint32_t blocks, int nontemporal) {
+  return batchedCopyImpl(dev, table, n, stream, unroll, blocks, nontemporal);
+}
+
+int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {
+  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream) {
+  if (bytes == 0) {
+    return 0;
+  }
+  TPHIP_TRY(hipSetDevice(dev));
+  uint64_t blocks = (bytes + kBlockThreads - 1) / kBlockThreads;
+  if (blocks > 2048) {
+    blocks = 2048;
+  }
+  hipLaunchKernelGGL(fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlockThreads), 0,
+                     static_cast<hipStream_t>(stream), static_cast<unsigned char*>(ptr),
+                     static_cast<unsigned char>(value), bytes);
+  return static_cast<int>(hipGetLastError());
+}
+
+int tphip_test_slow_kernel(int dev, void* ptr, uint64_t n, void* stream) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipLaunchKernelGGL(slow_kernel, dim3(128), dim3(128), 0, static_cast<hipStream_t>(stream),
+                     static_cast<volatile unsigned char*>(ptr), n);
+  return static_cast<int>(hipGetLastError());
+}
+
+} // extern "C"
