@@ -70,6 +70,11 @@ int tphip_device_for_ptr(const void* ptr, int* dev, int* is_host);
  * tensorpipe/test/channel/channel_test_cuda.cc:96-139). */
 int tphip_mem_base(const void* ptr, void** base, size_t* size);
 
+/* Identifier of the allocation containing `ptr`, unique for the lifetime of
+ * the process; lets a cache keyed on the base address notice that the address
+ * was freed and handed out again. *id = 0 when the runtime cannot tell. */
+int tphip_mem_buffer_id(const void* ptr, uint64_t* id);
+
 /* ---- memory -------------------------------------------------------------- */
 
 /* Device slab. Replaces makeCudaDeviceBuffer, tensorpipe/common/cuda.h:213-218. */

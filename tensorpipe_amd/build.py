@@ -46,9 +46,45 @@ def build_datagen():
          os.path.join(CSRC, "datagen", "tp_datagen.c"), "-lm"])
 
 
+HOST_SOURCES = [
+    "tensorpipe/common/common.cc",
+    "tensorpipe/transport/shm/shm.cc",
+    "tensorpipe/channel/basic/basic.cc",
+    "tensorpipe/channel/xth/xth.cc",
+    "tensorpipe/channel/hip_common.cc",
+    "tensorpipe/channel/hip_xth/hip_xth.cc",
+    "tensorpipe/channel/hip_ipc/hip_ipc.cc",
+    "tensorpipe/channel/hip_basic/hip_basic.cc",
+    "tensorpipe/core/core.cc",
+    "capi/tensorpipe_c.cc",
+]
+HOST_FLAGS = ["-O2", "-g", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread"]
+
+
+def build_host(jobs=8):
+    """libtensorpipe_amd.so: channels, shm transport, core and the C harness API (g++)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+    os.makedirs(LIB, exist_ok=True)
+    sources = [s for s in HOST_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objs = [os.path.join(objdir, s.replace("/", "_") + ".o") for s in sources]
+
+    def compile_one(pair):
+        src, obj = pair
+        run(["g++", *HOST_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-c", os.path.join(CSRC, src), "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(compile_one, zip(sources, objs)))
+    run(["g++", "-shared", "-pthread", "-o", os.path.join(LIB, "libtensorpipe_amd.so"), *objs,
+         f"-L{LIB}", "-ltphip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"])
+
+
 def build_all():
     build_tphip()
     build_datagen()
+    build_host()
 
 
 if __name__ == "__main__":

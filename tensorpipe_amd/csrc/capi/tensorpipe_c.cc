@@ -1,0 +1,531 @@
+// C harness API (include/tensorpipe_c.h) over the C++ pipe/channel layer.
+
+#include <tensorpipe_c.h>
+
+#include <chrono>
+#include <condition_variable>
+#include <cstring>
+#include <future>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include <tensorpipe/tensorpipe.h>
+#include <tensorpipe/tensorpipe_hip.h>
+#include <tensorpipe/common/hip_api.h>
+
+using namespace tensorpipe;
+
+namespace {
+
+thread_local std::string gLastError;
+
+void setLastError(const std::string& what) {
+  gLastError = what;
+}
+
+// One-shot completion slot shared between a callback and a waiter.
+struct Completion {
+  std::mutex mutex;
+  std::condition_variable cv;
+  bool done{false};
+  Error error;
+
+  void set(const Error& e) {
+    {
+      std::lock_guard<std::mutex> lock(mutex);
+      error = e;
+      done = true;
+    }
+    cv.notify_all();
+  }
+
+  // 0 ok, TPC_ERR_FAILED, TPC_ERR_TIMEOUT
+  int wait(int timeoutMs) {
+    std::unique_lock<std::mutex> lock(mutex);
+    if (timeoutMs < 0) {
+      cv.wait(lock, [this] { return done; });
+    } else if (!cv.wait_for(lock, std::chrono::milliseconds(timeoutMs), [this] { return done; })) {
+      setLastError("timed out");
+      return TPC_ERR_TIMEOUT;
+    }
+    if (error) {
+      setLastError(error.what());
+      return TPC_ERR_FAILED;
+    }
+    return 0;
+  }
+};
+
+std::vector<std::pair<std::string, int64_t>> parseList(const char* spec) {
+  std::vector<std::pair<std::string, int64_t>> out;
+  if (spec == nullptr) {
+    return out;
+  }
+  std::stringstream ss(spec);
+  std::string item;
+  while (std::getline(ss, item, ',')) {
+    if (item.empty()) {
+      continue;
+    }
+    auto pos = item.find(':');
+    std::string name = item.substr(0, pos);
+    int64_t prio = pos == std::string::npos ? static_cast<int64_t>(out.size())
+                                            : std::stoll(item.substr(pos + 1));
+    out.emplace_back(name, prio);
+  }
+  return out;
+}
+
+Device deviceFromC(int32_t type, int32_t index) {
+  return Device{type == TPC_DEVICE_HIP ? kHipDeviceType : kCpuDeviceType, index};
+}
+
+Buffer bufferFromC(const tpc_tensor& t) {
+  if (t.device_type == TPC_DEVICE_HIP) {
+    return HipBuffer{t.ptr, t.stream};
+  }
+  return CpuBuffer{t.ptr};
+}
+
+Message makeMessage(
+    const char* metadata,
+    const tpc_payload* payloads,
+    uint32_t numPayloads,
+    const tpc_tensor* tensors,
+    uint32_t numTensors) {
+  Message m;
+  m.metadata = metadata != nullptr ? metadata : "";
+  for (uint32_t i = 0; i < numPayloads; ++i) {
+    Message::Payload p;
+    p.data = payloads[i].ptr;
+    p.length = payloads[i].length;
+    m.payloads.push_back(std::move(p));
+  }
+  for (uint32_t i = 0; i < numTensors; ++i) {
+    Message::Tensor t;
+    t.buffer = bufferFromC(tensors[i]);
+    t.length = tensors[i].length;
+    if (tensors[i].target_type != TPC_NO_TARGET) {
+      t.targetDevice = deviceFromC(tensors[i].target_type, tensors[i].target_index);
+    }
+    m.tensors.push_back(std::move(t));
+  }
+  return m;
+}
+
+Allocation makeAllocation(
+    void* const* payloadPtrs,
+    uint32_t numPayloads,
+    const tpc_tensor* tensors,
+    uint32_t numTensors) {
+  Allocation a;
+  a.payloads.resize(numPayloads);
+  for (uint32_t i = 0; i < numPayloads; ++i) {
+    a.payloads[i].data = payloadPtrs[i];
+  }
+  a.tensors.resize(numTensors);
+  for (uint32_t i = 0; i < numTensors; ++i) {
+    a.tensors[i].buffer = bufferFromC(tensors[i]);
+  }
+  return a;
+}
+
+void syncRecvStreams(const tpc_tensor* tensors, uint32_t n) {
+  std::vector<void*> seen;
+  for (uint32_t i = 0; i < n; ++i) {
+    if (tensors[i].device_type != TPC_DEVICE_HIP || tensors[i].length == 0) {
+      continue;
+    }
+    bool dup = false;
+    for (void* s : seen) {
+      dup |= s == tensors[i].stream;
+    }
+    if (dup) {
+      continue;
+    }
+    seen.push_back(tensors[i].stream);
+    int dev = hipDeviceForPointer(tensors[i].ptr);
+    TP_HIP_CHECK(tphip_stream_sync(dev < 0 ? 0 : dev, tensors[i].stream));
+  }
+}
+
+} // namespace
+
+struct tpc_context {
+  std::shared_ptr<Context> ctx;
+  std::vector<std::string> channels;
+};
+
+struct tpc_listener {
+  std::shared_ptr<Listener> listener;
+};
+
+struct tpc_pipe {
+  std::shared_ptr<Pipe> pipe;
+};
+
+struct tpc_op {
+  std::shared_ptr<Completion> completion;
+};
+
+#define TPC_GUARD_BEGIN try {
+#define TPC_GUARD_END(failure)            \
+  }                                       \
+  catch (const std::exception& e) {       \
+    setLastError(e.what());               \
+    return failure;                       \
+  }
+
+extern "C" {
+
+const char* tpc_last_error(void) {
+  return gLastError.c_str();
+}
+
+tpc_context* tpc_context_create(const char* name, const char* transports, const char* channels) {
+  TPC_GUARD_BEGIN
+  auto out = std::make_unique<tpc_context>();
+  out->ctx = std::make_shared<Context>(ContextOptions().name(name != nullptr ? name : ""));
+  for (auto& t : parseList(transports)) {
+    if (t.first == "shm") {
+      out->ctx->registerTransport(t.second, "shm", transport::shm::create());
+    } else {
+      setLastError("unknown transport " + t.first);
+      return nullptr;
+    }
+  }
+  for (auto& c : parseList(channels)) {
+    std::shared_ptr<channel::Context> cctx;
+    if (c.first == "basic") {
+      cctx = channel::basic::create();
+    } else if (c.first == "xth") {
+      cctx = channel::xth::create();
+    } else if (c.first == "hip_xth") {
+      cctx = channel::hip_xth::create();
+    } else if (c.first == "hip_ipc") {
+      cctx = channel::hip_ipc::create();
+    } else if (c.first == "hip_basic") {
+      cctx = channel::hip_basic::create(channel::basic::create());
+    } else {
+      setLastError("unknown channel " + c.first);
+      return nullptr;
+    }
+    if (cctx->isViable()) {
+      out->channels.push_back(c.first);
+    }
+    out->ctx->registerChannel(c.second, c.first, std::move(cctx));
+  }
+  return out.release();
+  TPC_GUARD_END(nullptr)
+}
+
+void tpc_context_close(tpc_context* ctx) {
+  if (ctx != nullptr) {
+    ctx->ctx->close();
+  }
+}
+
+void tpc_context_destroy(tpc_context* ctx) {
+  if (ctx != nullptr) {
+    ctx->ctx->join();
+    delete ctx;
+  }
+}
+
+int tpc_context_has_channel(tpc_context* ctx, const char* name) {
+  for (auto& c : ctx->channels) {
+    if (c == name) {
+      return 1;
+    }
+  }
+  return 0;
+}
+
+tpc_listener* tpc_listen(tpc_context* ctx, const char* url) {
+  TPC_GUARD_BEGIN
+  auto out = std::make_unique<tpc_listener>();
+  out->listener = ctx->ctx->listen({std::string(url)});
+  return out.release();
+  TPC_GUARD_END(nullptr)
+}
+
+int tpc_listener_url(tpc_listener* l, const char* transport, char* out, size_t outLen) {
+  TPC_GUARD_BEGIN
+  std::string url = l->listener->url(transport);
+  if (url.size() + 1 > outLen) {
+    setLastError("buffer too small");
+    return TPC_ERR_FAILED;
+  }
+  std::memcpy(out, url.c_str(), url.size() + 1);
+  return 0;
+  TPC_GUARD_END(TPC_ERR_FAILED)
+}
+
+tpc_pipe* tpc_accept(tpc_listener* l, int timeoutMs) {
+  TPC_GUARD_BEGIN
+  auto completion = std::make_shared<Completion>();
+  auto slot = std::make_shared<std::shared_ptr<Pipe>>();
+  l->listener->accept([completion, slot](const Error& error, std::shared_ptr<Pipe> pipe) {
+    *slot = std::move(pipe);
+    completion->set(error);
+  });
+  if (completion->wait(timeoutMs) != 0) {
+    return nullptr;
+  }
+  auto out = std::make_unique<tpc_pipe>();
+  out->pipe = std::move(*slot);
+  return out.release();
+  TPC_GUARD_END(nullptr)
+}
+
+void tpc_listener_destroy(tpc_listener* l) {
+  delete l;
+}
+
+tpc_pipe* tpc_connect(tpc_context* ctx, const char* url) {
+  TPC_GUARD_BEGIN
+  auto out = std::make_unique<tpc_pipe>();
+  out->pipe = ctx->ctx->connect(url);
+  return out.release();
+  TPC_GUARD_END(nullptr)
+}
+
+void tpc_pipe_close(tpc_pipe* p) {
+  if (p != nullptr) {
+    p->pipe->close();
+  }
+}
+
+void tpc_pipe_destroy(tpc_pipe* p) {
+  delete p;
+}
+
+int tpc_pipe_remote_name(tpc_pipe* p, char* out, size_t outLen) {
+  const std::string& n = p->pipe->getRemoteName();
+  if (n.size() + 1 > outLen) {
+    return TPC_ERR_FAILED;
+  }
+  std::memcpy(out, n.c_str(), n.size() + 1);
+  return 0;
+}
+
+tpc_op* tpc_write_async(
+    tpc_pipe* p,
+    const char* metadata,
+    const tpc_payload* payloads,
+    uint32_t numPayloads,
+    const tpc_tensor* tensors,
+    uint32_t numTensors) {
+  TPC_GUARD_BEGIN
+  auto op = std::make_unique<tpc_op>();
+  op->completion = std::make_shared<Completion>();
+  auto completion = op->completion;
+  p->pipe->write(
+      makeMessage(metadata, payloads, numPayloads, tensors, numTensors),
+      [completion](const Error& error) { completion->set(error); });
+  return op.release();
+  TPC_GUARD_END(nullptr)
+}
+
+int tpc_read_descriptor(tpc_pipe* p, tpc_descriptor* out, int timeoutMs) {
+  TPC_GUARD_BEGIN
+  auto completion = std::make_shared<Completion>();
+  auto slot = std::make_shared<Descriptor>();
+  p->pipe->readDescriptor([completion, slot](const Error& error, Descriptor d) {
+    *slot = std::move(d);
+    completion->set(error);
+  });
+  int rc = completion->wait(timeoutMs);
+  if (rc != 0) {
+    return rc;
+  }
+  const Descriptor& d = *slot;
+  if (d.payloads.size() > 64 || d.tensors.size() > TPC_MAX_DESC_ITEMS ||
+      d.metadata.size() >= sizeof(out->metadata)) {
+    setLastError("descriptor too large for tpc_descriptor");
+    return TPC_ERR_FAILED;
+  }
+  std::memset(out->metadata, 0, sizeof(out->metadata));
+  std::memcpy(out->metadata, d.metadata.data(), d.metadata.size());
+  out->num_payloads = static_cast<uint32_t>(d.payloads.size());
+  out->num_tensors = static_cast<uint32_t>(d.tensors.size());
+  for (size_t i = 0; i < d.payloads.size(); ++i) {
+    out->payload_lengths[i] = d.payloads[i].length;
+  }
+  for (size_t i = 0; i < d.tensors.size(); ++i) {
+    const auto& t = d.tensors[i];
+    out->tensor_lengths[i] = t.length;
+    out->tensor_source_type[i] = t.sourceDevice.type == kCpuDeviceType ? TPC_DEVICE_CPU : TPC_DEVICE_HIP;
+    out->tensor_source_index[i] = t.sourceDevice.index;
+    if (t.targetDevice.has_value()) {
+      out->tensor_target_type[i] =
+          t.targetDevice->type == kCpuDeviceType ? TPC_DEVICE_CPU : TPC_DEVICE_HIP;
+      out->tensor_target_index[i] = t.targetDevice->index;
+    } else {
+      out->tensor_target_type[i] = TPC_NO_TARGET;
+      out->tensor_target_index[i] = 0;
+    }
+  }
+  return 0;
+  TPC_GUARD_END(TPC_ERR_FAILED)
+}
+
+tpc_op* tpc_read_async(
+    tpc_pipe* p,
+    void* const* payloadPtrs,
+    uint32_t numPayloads,
+    const tpc_tensor* tensors,
+    uint32_t numTensors) {
+  TPC_GUARD_BEGIN
+  auto op = std::make_unique<tpc_op>();
+  op->completion = std::make_shared<Completion>();
+  auto completion = op->completion;
+  p->pipe->read(
+      makeAllocation(payloadPtrs, numPayloads, tensors, numTensors),
+      [completion](const Error& error) { completion->set(error); });
+  return op.release();
+  TPC_GUARD_END(nullptr)
+}
+
+int tpc_op_wait(tpc_op* op, int timeoutMs) {
+  if (op == nullptr) {
+    return TPC_ERR_FAILED;
+  }
+  int rc = op->completion->wait(timeoutMs);
+  if (rc != TPC_ERR_TIMEOUT) {
+    delete op;
+  }
+  return rc;
+}
+
+int tpc_bench_transfer(
+    tpc_pipe* sender,
+    tpc_pipe* receiver,
+    const tpc_payload* payloads,
+    uint32_t numPayloads,
+    void* const* recvPayloadPtrs,
+    const tpc_tensor* sendTensors,
+    const tpc_tensor* recvTensors,
+    uint32_t numTensors,
+    uint32_t warmup,
+    uint32_t iters,
+    double* perIterUs,
+    double* totalSeconds) {
+  TPC_GUARD_BEGIN
+  using Clock = std::chrono::steady_clock;
+  Clock::time_point begin;
+  const int kTimeoutMs = 60000;
+  for (uint32_t it = 0; it < warmup + iters; ++it) {
+    if (it == warmup) {
+      begin = Clock::now();
+    }
+    auto t0 = Clock::now();
+    auto wrote = std::make_shared<Completion>();
+    auto gotDescriptor = std::make_shared<Completion>();
+    auto readDone = std::make_shared<Completion>();
+    sender->pipe->write(
+        makeMessage("", payloads, numPayloads, sendTensors, numTensors),
+        [wrote](const Error& e) { wrote->set(e); });
+    receiver->pipe->readDescriptor(
+        [gotDescriptor](const Error& e, Descriptor) { gotDescriptor->set(e); });
+    int rc = gotDescriptor->wait(kTimeoutMs);
+    if (rc != 0) {
+      return rc;
+    }
+    receiver->pipe->read(
+        makeAllocation(recvPayloadPtrs, numPayloads, recvTensors, numTensors),
+        [readDone](const Error& e) { readDone->set(e); });
+    if ((rc = readDone->wait(kTimeoutMs)) != 0) {
+      return rc;
+    }
+    if ((rc = wrote->wait(kTimeoutMs)) != 0) {
+      return rc;
+    }
+    syncRecvStreams(recvTensors, numTensors);
+    if (it >= warmup && perIterUs != nullptr) {
+      perIterUs[it - warmup] =
+          std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+    }
+  }
+  if (totalSeconds != nullptr) {
+    *totalSeconds = std::chrono::duration<double>(Clock::now() - begin).count();
+  }
+  return 0;
+  TPC_GUARD_END(TPC_ERR_FAILED)
+}
+
+int tpc_bench_pingpong(
+    tpc_pipe* p,
+    int initiator,
+    const tpc_payload* payloads,
+    uint32_t numPayloads,
+    void* const* recvPayloadPtrs,
+    const tpc_tensor* sendTensors,
+    const tpc_tensor* recvTensors,
+    uint32_t numTensors,
+    uint32_t warmup,
+    uint32_t iters,
+    double* perIterUs,
+    double* totalSeconds) {
+  TPC_GUARD_BEGIN
+  using Clock = std::chrono::steady_clock;
+  Clock::time_point begin;
+  const int kTimeoutMs = 60000;
+  auto doWrite = [&](std::shared_ptr<Completion> c) {
+    p->pipe->write(
+        makeMessage("", payloads, numPayloads, sendTensors, numTensors),
+        [c](const Error& e) { c->set(e); });
+  };
+  auto doRead = [&]() -> int {
+    auto gotDescriptor = std::make_shared<Completion>();
+    auto readDone = std::make_shared<Completion>();
+    p->pipe->readDescriptor(
+        [gotDescriptor](const Error& e, Descriptor) { gotDescriptor->set(e); });
+    int rc = gotDescriptor->wait(kTimeoutMs);
+    if (rc != 0) {
+      return rc;
+    }
+    p->pipe->read(
+        makeAllocation(recvPayloadPtrs, numPayloads, recvTensors, numTensors),
+        [readDone](const Error& e) { readDone->set(e); });
+    return readDone->wait(kTimeoutMs);
+  };
+  for (uint32_t it = 0; it < warmup + iters; ++it) {
+    if (it == warmup) {
+      begin = Clock::now();
+    }
+    auto t0 = Clock::now();
+    auto wrote = std::make_shared<Completion>();
+    int rc;
+    if (initiator) {
+      doWrite(wrote);
+      if ((rc = doRead()) != 0) {
+        return rc;
+      }
+      syncRecvStreams(recvTensors, numTensors);
+    } else {
+      if ((rc = doRead()) != 0) {
+        return rc;
+      }
+      // The echo is ordered after the receive on the receive stream when the
+      // send buffers are the receive buffers on that same stream.
+      doWrite(wrote);
+    }
+    if ((rc = wrote->wait(kTimeoutMs)) != 0) {
+      return rc;
+    }
+    if (it >= warmup && perIterUs != nullptr) {
+      perIterUs[it - warmup] =
+          std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+    }
+  }
+  if (totalSeconds != nullptr) {
+    *totalSeconds = std::chrono::duration<double>(Clock::now() - begin).count();
+  }
+  return 0;
+  TPC_GUARD_END(TPC_ERR_FAILED)
+}
+
+} // extern "C"

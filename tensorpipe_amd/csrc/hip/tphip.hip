@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <tuple>
 #include <vector>
 
 #include "copy_kernels.hip.h"
@@ -22,6 +23,7 @@ using namespace tphip;
   do {                                      \
     hipError_t e_ = (expr);                 \
     if (e_ != hipSuccess) {                 \
+      (void)hipGetLastError();              \
       return static_cast<int>(e_);          \
     }                                       \
   } while (0)
@@ -118,28 +120,40 @@ int getDevice(int dev, DeviceState** out) {
   return 0;
 }
 
+// Launch through hipLaunchKernel so that the error code is this launch's own
+// (hipGetLastError would also report stale errors of unrelated earlier calls).
+template <typename... Params, typename... Args>
+int launchKernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                 Args... args) {
+  std::tuple<Params...> values{static_cast<Params>(args)...};
+  void* argv[sizeof...(Params)];
+  size_t i = 0;
+  std::apply([&](auto&... v) { ((argv[i++] = static_cast<void*>(&v)), ...); }, values);
+  hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds,
+                                 stream);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+  }
+  return static_cast<int>(e);
+}
+
 template <bool NT>
 int launchSingle(int unroll, uint32_t blocks, hipStream_t stream, const char* src, char* dst,
                  uint64_t bytes) {
   switch (unroll) {
     case 1:
-      hipLaunchKernelGGL((single_copy_kernel<1, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
-                         src, dst, bytes);
-      break;
+      return launchKernel(single_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
+                          dst, bytes);
     case 2:
-      hipLaunchKernelGGL((single_copy_kernel<2, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
-                         src, dst, bytes);
-      break;
+      return launchKernel(single_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
+                          dst, bytes);
     case 8:
-      hipLaunchKernelGGL((single_copy_kernel<8, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
-                         src, dst, bytes);
-      break;
+      return launchKernel(single_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
+                          dst, bytes);
     default:
-      hipLaunchKernelGGL((single_copy_kernel<4, NT>), dim3(blocks), dim3(kBlockThreads), 0, stream,
-                         src, dst, bytes);
-      break;
+      return launchKernel(single_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
+                          dst, bytes);
   }
-  return static_cast<int>(hipGetLastError());
 }
 
 template <bool NT>
@@ -148,23 +162,18 @@ int launchTable(int unroll, uint32_t blocks, size_t lds, hipStream_t stream,
                 uint32_t nslices) {
   switch (unroll) {
     case 1:
-      hipLaunchKernelGGL((batched_copy_kernel<1, NT>), dim3(blocks), dim3(kBlockThreads), lds,
-                         stream, prefix, descs, n, nslices);
-      break;
+      return launchKernel(batched_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
+                          prefix, descs, n, nslices);
     case 2:
-      hipLaunchKernelGGL((batched_copy_kernel<2, NT>), dim3(blocks), dim3(kBlockThreads), lds,
-                         stream, prefix, descs, n, nslices);
-      break;
+      return launchKernel(batched_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
+                          prefix, descs, n, nslices);
     case 8:
-      hipLaunchKernelGGL((batched_copy_kernel<8, NT>), dim3(blocks), dim3(kBlockThreads), lds,
-                         stream, prefix, descs, n, nslices);
-      break;
+      return launchKernel(batched_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
+                          prefix, descs, n, nslices);
     default:
-      hipLaunchKernelGGL((batched_copy_kernel<4, NT>), dim3(blocks), dim3(kBlockThreads), lds,
-                         stream, prefix, descs, n, nslices);
-      break;
+      return launchKernel(batched_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
+                          prefix, descs, n, nslices);
   }
-  return static_cast<int>(hipGetLastError());
 }
 
 uint32_t pickBlocks(const DeviceState& st, uint64_t nslices, uint32_t minWaves, uint32_t blocks) {
@@ -234,10 +243,12 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     if (planViaKernel()) {
       const uint32_t nv = static_cast<uint32_t>(planBytesPadded / 16);
       const uint32_t sb = (nv + kBlockThreads - 1) / kBlockThreads;
-      hipLaunchKernelGGL(stage_plan_kernel, dim3(sb < 8 ? sb : 8), dim3(kBlockThreads), 0, stream,
-                         reinterpret_cast<const u32x4*>(hostDev), reinterpret_cast<u32x4*>(devp),
-                         nv);
-      TPHIP_TRY(hipGetLastError());
+      int src = launchKernel(stage_plan_kernel, dim3(sb < 8 ? sb : 8), dim3(kBlockThreads), 0,
+                             stream, reinterpret_cast<const u32x4*>(hostDev),
+                             reinterpret_cast<u32x4*>(devp), nv);
+      if (src != 0) {
+        return src;
+      }
     } else {
       TPHIP_TRY(hipMemcpyAsync(devp, host, planBytesPadded, hipMemcpyHostToDevice, stream));
     }
@@ -443,6 +454,22 @@ int tphip_mem_base(const void* ptr, void** base, size_t* size) {
   return 0;
 }
 
+int tphip_mem_buffer_id(const void* ptr, uint64_t* id) {
+  if (id == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  unsigned long long v = 0;
+  hipError_t e = hipPointerGetAttribute(
+      &v, HIP_POINTER_ATTRIBUTE_BUFFER_ID, reinterpret_cast<hipDeviceptr_t>(const_cast<void*>(ptr)));
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *id = 0;
+    return 0;
+  }
+  *id = v;
+  return 0;
+}
+
 int tphip_malloc(int dev, size_t bytes, void** ptr) {
   TPHIP_TRY(hipSetDevice(dev));
   TPHIP_TRY(hipMalloc(ptr, bytes));
@@ -640,17 +667,15 @@ int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream) {
   if (blocks > 2048) {
     blocks = 2048;
   }
-  hipLaunchKernelGGL(fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlockThreads), 0,
-                     static_cast<hipStream_t>(stream), static_cast<unsigned char*>(ptr),
-                     static_cast<unsigned char>(value), bytes);
-  return static_cast<int>(hipGetLastError());
+  return launchKernel(fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlockThreads), 0,
+                      static_cast<hipStream_t>(stream), static_cast<unsigned char*>(ptr),
+                      static_cast<unsigned char>(value), bytes);
 }
 
 int tphip_test_slow_kernel(int dev, void* ptr, uint64_t n, void* stream) {
   TPHIP_TRY(hipSetDevice(dev));
-  hipLaunchKernelGGL(slow_kernel, dim3(128), dim3(128), 0, static_cast<hipStream_t>(stream),
-                     static_cast<volatile unsigned char*>(ptr), n);
-  return static_cast<int>(hipGetLastError());
+  return launchKernel(slow_kernel, dim3(128), dim3(128), 0, static_cast<hipStream_t>(stream),
+                      static_cast<volatile unsigned char*>(ptr), n);
 }
 
 } // extern "C"

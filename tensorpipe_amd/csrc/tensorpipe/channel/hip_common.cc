@@ -1,0 +1,117 @@
+#include <tensorpipe/channel/hip_common.h>
+
+#include <chrono>
+#include <fstream>
+#include <random>
+#include <sstream>
+
+#include <unistd.h>
+
+TP_AMD_NAMESPACE_BEGIN
+namespace channel {
+
+const std::string& bootIdentity() {
+  static const std::string id = [] {
+    std::ifstream f("/proc/sys/kernel/random/boot_id");
+    std::string s;
+    std::getline(f, s);
+    return s;
+  }();
+  return id;
+}
+
+const std::string& processIdentity() {
+  static const std::string id = [] {
+    std::random_device rd;
+    std::ostringstream ss;
+    ss << bootIdentity() << "_" << ::getpid() << "_" << std::hex << rd() << rd();
+    return ss.str();
+  }();
+  return id;
+}
+
+HipEventPoller::HipEventPoller() {
+  thread_ = std::thread([this] { run(); });
+}
+
+HipEventPoller::~HipEventPoller() {
+  join();
+}
+
+void HipEventPoller::watch(std::unique_ptr<HipEvent> event, HipEventPool* pool, TCallback fn) {
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    incoming_.push_back(Item{std::move(event), pool, std::move(fn)});
+  }
+  cv_.notify_one();
+}
+
+void HipEventPoller::join() {
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (stopping_) {
+      return;
+    }
+    stopping_ = true;
+  }
+  cv_.notify_one();
+  if (thread_.joinable()) {
+    thread_.join();
+  }
+}
+
+void HipEventPoller::run() {
+  std::deque<Item> active;
+  for (;;) {
+    {
+      std::unique_lock<std::mutex> lock(mutex_);
+      if (active.empty()) {
+        cv_.wait(lock, [this] { return stopping_ || !incoming_.empty(); });
+      }
+      while (!incoming_.empty()) {
+        active.push_back(std::move(incoming_.front()));
+        incoming_.pop_front();
+      }
+      if (stopping_ && active.empty()) {
+        return;
+      }
+    }
+    bool any = false;
+    for (auto it = active.begin(); it != active.end();) {
+      int done = 0;
+      int rc = tphip_event_query(it->event->device(), it->event->raw(), &done);
+      if (rc != 0 || done) {
+        Item item = std::move(*it);
+        it = active.erase(it);
+        any = true;
+        if (rc != 0) {
+          item.fn(TP_CREATE_ERROR(HipError, "tphip_event_query", rc));
+        } else {
+          item.fn(Error::kSuccess);
+        }
+        if (item.pool != nullptr) {
+          item.pool->put(std::move(item.event));
+        }
+      } else {
+        ++it;
+      }
+    }
+    if (!any) {
+#if defined(__x86_64__)
+      __builtin_ia32_pause();
+#endif
+    }
+  }
+}
+
+void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table) {
+  size_t off = 0;
+  while (off < table.size()) {
+    const size_t n = table.size() - off < TPHIP_MAX_BATCH ? table.size() - off : TPHIP_MAX_BATCH;
+    TP_HIP_CHECK(tphip_batched_copy(device, table.data() + off, static_cast<uint32_t>(n), stream));
+    off += n;
+  }
+}
+
+} // namespace channel
+TP_AMD_NAMESPACE_END

@@ -1,0 +1,66 @@
+// Pieces shared by the three HIP channels: the process identity used in
+// device descriptors, a completion poller for HIP events, and the helper that
+// turns a list of (src, dst, bytes) into ONE batched copy launch.
+#pragma once
+
+#include <condition_variable>
+#include <deque>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include <tensorpipe/common/error.h>
+#include <tensorpipe/common/hip_api.h>
+
+TP_AMD_NAMESPACE_BEGIN
+namespace channel {
+
+// "<boot id>_<pid>_<nonce>": equal in two contexts iff they live in the same
+// process (tensorpipe/channel/cuda_xth/context_impl.cc:28-73 builds the same
+// kind of string from boot id, pid namespace and pid).
+const std::string& processIdentity();
+// "<boot id>": equal iff same machine boot.
+const std::string& bootIdentity();
+
+// Thread that watches HIP events and runs a callback once an event's captured
+// work has finished. Replaces the stream-callback thread of the reference
+// (tensorpipe/common/cuda_loop.cc:62-124) with event polling, which completes
+// within a microsecond or two of the GPU instead of a runtime callback hop.
+// Callbacks run on the poller thread and must hop to their own loop.
+class HipEventPoller {
+ public:
+  using TCallback = std::function<void(const Error&)>;
+
+  HipEventPoller();
+  ~HipEventPoller();
+
+  // `event` must have been recorded already; ownership moves to the poller
+  // until the callback has run, then back to `pool` (if given).
+  void watch(std::unique_ptr<HipEvent> event, HipEventPool* pool, TCallback fn);
+
+  void join();
+
+ private:
+  struct Item {
+    std::unique_ptr<HipEvent> event;
+    HipEventPool* pool;
+    TCallback fn;
+  };
+
+  void run();
+
+  std::mutex mutex_;
+  std::condition_variable cv_;
+  std::deque<Item> incoming_;
+  bool stopping_{false};
+  std::thread thread_;
+};
+
+// Enqueue one batched copy on (device, stream); throws on a failed launch.
+void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table);
+
+} // namespace channel
+TP_AMD_NAMESPACE_END

@@ -1,0 +1,877 @@
+// hip_ipc: GPU-to-GPU channel between two processes of one machine.
+//
+// Two data paths, chosen per tensor by the sender:
+//
+//  direct  The sender exports the allocation that contains the tensor
+//          (hipIpcGetMemHandle on its base, cached per allocation) and sends
+//          {export id, handle the first time, offset, length}. The receiver
+//          maps the allocation (cached) and its batched copy kernel reads the
+//          sender's memory directly: one read and one write per payload byte,
+//          all tensors of a message in one launch.
+//  outbox  What the reference does for every transfer
+//          (tensorpipe/channel/cuda_ipc/channel_impl.cc:107-136,238-252,
+//          431-467, context_impl.cc:173-195,341-418): the tensor is cut into
+//          chunks of at most one slot, each chunk is copied into a slot of a
+//          per-device staging slab that was exported once, the receiver copies
+//          slot -> target and its reply frees the slot. Two reads and two
+//          writes per byte. Used when an allocation cannot be exported, or
+//          for everything when TP_HIP_IPC_MODE=outbox.
+//
+// Synchronisation between the two processes goes through the host: the sender
+// announces a tensor (or chunk) once a HIP event recorded behind the producing
+// work has completed, and the receiver replies once an event recorded behind
+// its copy has completed. Inter-process HIP events would let both sides skip
+// the host, as the reference does with CUDA IPC events, but exporting an event
+// fails on the deployment this was built for, so they are not used.
+//
+// The recv callback fires when the copy has been enqueued on the caller's
+// stream (as in the reference); the send callback fires when the source may be
+// reused: after the receiver's reply (direct) or after the last chunk has been
+// staged (outbox).
+
+#include <tensorpipe/channel/hip_ipc/factory.h>
+
+#include <array>
+#include <deque>
+#include <map>
+#include <mutex>
+#include <set>
+
+#include <tensorpipe/channel/channel_base.h>
+#include <tensorpipe/channel/hip_common.h>
+#include <tensorpipe/common/hip_buffer.h>
+#include <tensorpipe/common/slot_allocator.h>
+#include <tensorpipe/common/wire.h>
+
+TP_AMD_NAMESPACE_BEGIN
+namespace channel {
+namespace hip_ipc {
+
+namespace {
+
+// Staging geometry of the outbox path, as
+// tensorpipe/channel/cuda_ipc/constants.h:22-24.
+constexpr size_t kSlotSize = 8 * 1024 * 1024;
+constexpr size_t kNumSlots = 4;
+constexpr size_t kStagingAreaSize = kSlotSize * kNumSlots;
+
+using HandleBytes = std::array<uint8_t, TPHIP_IPC_HANDLE_BYTES>;
+
+// Read when a context is created, so that one process can host contexts of
+// both kinds.
+bool outboxForcedByEnv() {
+  const char* e = std::getenv("TP_HIP_IPC_MODE");
+  return e != nullptr && std::string(e) == "outbox";
+}
+
+// Allocations this process has exported, keyed by base address. Process-wide:
+// a handle describes an allocation, not a context.
+struct ExportedAllocation {
+  uint64_t id;
+  HandleBytes handle;
+  size_t size;
+  uint64_t bufferId;
+};
+
+class ExportRegistry {
+ public:
+  static ExportRegistry& get() {
+    static ExportRegistry* r = new ExportRegistry();
+    return *r;
+  }
+
+  // Returns false if the allocation containing ptr cannot be exported.
+  bool lookup(int device, const void* ptr, ExportedAllocation* out, uint64_t* offset) {
+    void* base = nullptr;
+    size_t size = 0;
+    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr) {
+      return false;
+    }
+    uint64_t bufferId = 0;
+    tphip_mem_buffer_id(base, &bufferId);
+    *offset = static_cast<uint64_t>(
+        static_cast<const uint8_t*>(ptr) - static_cast<const uint8_t*>(base));
+    std::lock_guard<std::mutex> lock(mutex_);
+    auto it = exports_.find(base);
+    if (it != exports_.end() && it->second.size == size && it->second.bufferId == bufferId) {
+      *out = it->second;
+      return true;
+    }
+    // New allocation, or the address was freed and handed out again.
+    ExportedAllocation e;
+    if (tphip_ipc_mem_export(device, base, e.handle.data()) != 0) {
+      return false;
+    }
+    e.id = nextId_++;
+    e.size = size;
+    e.bufferId = bufferId;
+    exports_[base] = e;
+    *out = e;
+    return true;
+  }
+
+ private:
+  std::mutex mutex_;
+  std::map<void*, ExportedAllocation> exports_;
+  uint64_t nextId_{1};
+};
+
+// Allocations of other processes mapped into this one, keyed by handle bytes.
+// Mappings stay open for the life of the process (opening is ~0.2 ms, and a
+// handle may be shared by several channels).
+class ImportRegistry {
+ public:
+  static ImportRegistry& get() {
+    static ImportRegistry* r = new ImportRegistry();
+    return *r;
+  }
+
+  int open(int device, const HandleBytes& handle, void** out) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    auto key = std::make_pair(device, handle);
+    auto it = opened_.find(key);
+    if (it != opened_.end()) {
+      *out = it->second;
+      return 0;
+    }
+    void* ptr = nullptr;
+    int rc = tphip_ipc_mem_open(device, handle.data(), &ptr);
+    if (rc != 0) {
+      return rc;
+    }
+    opened_[key] = ptr;
+    *out = ptr;
+    return 0;
+  }
+
+ private:
+  std::mutex mutex_;
+  std::map<std::pair<int, HandleBytes>, void*> opened_;
+};
+
+// Per-device staging slab of the outbox path, created on first use.
+struct Outbox {
+  explicit Outbox(int device)
+      : slab(device, kStagingAreaSize), allocator(slab.ptr(), kNumSlots, kSlotSize) {
+    TP_HIP_CHECK(tphip_ipc_mem_export(device, slab.ptr(), handle.data()));
+  }
+  HipDeviceSlab slab;
+  HandleBytes handle;
+  SlotAllocator allocator;
+};
+
+class IpcContextCore final : public ContextCore {
+ public:
+  HipEventPool events;
+  HipEventPoller poller;
+  const bool forceOutbox{outboxForcedByEnv()};
+
+  // Loop only.
+  Outbox& outbox(int device) {
+    if (device >= static_cast<int>(outboxes_.size())) {
+      outboxes_.resize(device + 1);
+    }
+    if (!outboxes_[device]) {
+      outboxes_[device] = std::make_unique<Outbox>(device);
+    }
+    return *outboxes_[device];
+  }
+
+  void closeAllocators() {
+    for (auto& o : outboxes_) {
+      if (o) {
+        o->allocator.close();
+      }
+    }
+  }
+
+  void joinImpl() override {
+    poller.join();
+  }
+
+ private:
+  std::vector<std::unique_ptr<Outbox>> outboxes_;
+};
+
+enum MsgKind : uint8_t { kDirect = 1, kChunk = 2 };
+
+class ChannelImpl final : public ChannelImplBase {
+ public:
+  ChannelImpl(
+      std::shared_ptr<IpcContextCore> ctx,
+      std::string id,
+      std::shared_ptr<transport::Connection> descriptorConnection,
+      std::shared_ptr<transport::Connection> replyConnection)
+      : ChannelImplBase(ctx, std::move(id)),
+        ictx_(std::move(ctx)),
+        descriptorConnection_(std::move(descriptorConnection)),
+        replyConnection_(std::move(replyConnection)) {}
+
+  void sendBatch(std::vector<BatchEntry> entries, TSendCallback callback) {
+    auto self = std::static_pointer_cast<ChannelImpl>(shared_from_this());
+    ctx_->defer([self, entries{std::move(entries)}, callback{std::move(callback)}]() mutable {
+      const uint64_t seq = self->nextSend_++;
+      if (self->error_) {
+        callback(self->error_);
+        return;
+      }
+      self->sendEntries(seq, std::move(entries), std::move(callback));
+    });
+  }
+
+  void recvBatch(std::vector<BatchEntry> entries, TRecvCallback callback) {
+    auto self = std::static_pointer_cast<ChannelImpl>(shared_from_this());
+    ctx_->defer([self, entries{std::move(entries)}, callback{std::move(callback)}]() mutable {
+      const uint64_t seq = self->nextRecv_++;
+      if (self->error_) {
+        callback(self->error_);
+        return;
+      }
+      self->recvEntries(seq, std::move(entries), std::move(callback));
+    });
+  }
+
+ protected:
+  void sendFromLoop(uint64_t seq, Buffer buffer, size_t length, TSendCallback cb) override {
+    std::vector<BatchEntry> entries;
+    entries.push_back({std::move(buffer), length});
+    sendEntries(seq, std::move(entries), std::move(cb));
+  }
+
+  void recvFromLoop(uint64_t seq, Buffer buffer, size_t length, TRecvCallback cb) override {
+    std::vector<BatchEntry> entries;
+    entries.push_back({std::move(buffer), length});
+    recvEntries(seq, std::move(entries), std::move(cb));
+  }
+
+  void handleError() override {
+    descriptorConnection_->close();
+    replyConnection_->close();
+    // Slot requests still queued fail with AllocatorClosedError, as in
+    // tensorpipe/channel/cuda_ipc/context_impl.cc:420-426; only when the whole
+    // context goes down, since the allocator is shared by its channels.
+    if (ctx_->closed()) {
+      ictx_->closeAllocators();
+    }
+    auto sends = std::move(sendOps_);
+    sendOps_.clear();
+    for (auto& op : sends) {
+      finishSend(op);
+    }
+    auto recvs = std::move(recvOps_);
+    recvOps_.clear();
+    for (auto& op : recvs) {
+      finishRecv(op);
+    }
+    wireQueue_.clear();
+    replyQueue_.clear();
+  }
+
+ private:
+  struct StreamRef {
+    void* stream;
+    int device;
+    bool operator==(const StreamRef& o) const {
+      return stream == o.stream && device == o.device;
+    }
+  };
+
+  // A unit that goes on the descriptor connection: a whole direct batch or one
+  // staged chunk. Units are written strictly in creation order.
+  struct WireUnit {
+    std::vector<uint8_t> bytes;
+    bool ready{false};
+    std::function<void()> onReply; // runs when the matching reply arrives
+  };
+
+  struct SendOp {
+    uint64_t seq;
+    TSendCallback cb;
+    size_t pending{0}; // things that must happen before the callback
+    bool done{false};
+  };
+
+  struct RecvOp {
+    uint64_t seq;
+    TRecvCallback cb;
+    std::vector<BatchEntry> entries;
+    size_t unitsExpected{0};
+    size_t unitsSeen{0};
+    bool done{false};
+  };
+
+  // A reply owed to the peer; replies are written in the order the units
+  // arrived, each once the copy it acknowledges has finished.
+  struct ReplyUnit {
+    bool ready{false};
+  };
+
+  static size_t numChunks(size_t length) {
+    return (length + kSlotSize - 1) / kSlotSize;
+  }
+
+  // ---- send -----------------------------------------------------------------
+
+  void sendEntries(uint64_t seq, std::vector<BatchEntry> entries, TSendCallback cb) {
+    std::vector<BatchEntry> live;
+    for (auto& e : entries) {
+      if (e.length > 0) {
+        live.push_back(std::move(e));
+      }
+    }
+    if (live.empty()) {
+      cb(error_); // zero length: tensorpipe/channel/cuda_ipc/channel_impl.cc:112-115
+      return;
+    }
+    auto op = std::make_shared<SendOp>();
+    op->seq = seq;
+    op->cb = std::move(cb);
+    sendOps_.push_back(op);
+    op->pending = 1; // guard until everything below has been issued
+
+    try {
+      // Split the batch: exportable tensors travel together in one direct unit,
+      // the others go through the outbox chunk by chunk. Both endpoints derive
+      // the unit sequence from the descriptors, so no negotiation is needed.
+      struct DirectItem {
+        ExportedAllocation alloc;
+        uint64_t offset;
+        uint64_t length;
+        uint32_t index;
+      };
+      std::vector<DirectItem> direct;
+      std::vector<uint32_t> staged;
+      std::vector<StreamRef> directStreams;
+      for (uint32_t i = 0; i < live.size(); ++i) {
+        const HipBuffer& hb = live[i].buffer.unwrap<HipBuffer>();
+        const int device = hipDeviceForPointer(hb.ptr);
+        TP_THROW_ASSERT_IF(device < 0);
+        DirectItem item;
+        if (!ictx_->forceOutbox && ExportRegistry::get().lookup(device, hb.ptr, &item.alloc, &item.offset)) {
+          item.length = live[i].length;
+          item.index = i;
+          direct.push_back(item);
+          StreamRef ref{hb.stream, device};
+          bool known = false;
+          for (auto& s : directStreams) {
+            known |= s == ref;
+          }
+          if (!known) {
+            directStreams.push_back(ref);
+          }
+        } else {
+          staged.push_back(i);
+        }
+      }
+
+      if (!direct.empty()) {
+        WireWriter w;
+        w.u8(kDirect);
+        w.u32(static_cast<uint32_t>(direct.size()));
+        for (auto& d : direct) {
+          w.u32(d.index);
+          w.u64(d.alloc.id);
+          const bool announce = announced_.insert(d.alloc.id).second;
+          w.u8(announce ? 1 : 0);
+          if (announce) {
+            w.raw(d.alloc.handle.data(), d.alloc.handle.size());
+          }
+          w.u64(d.offset);
+          w.u64(d.length);
+        }
+        auto unit = std::make_shared<WireUnit>();
+        unit->bytes = std::move(w.bytes());
+        // The source may be reused once the receiver has copied it.
+        ++op->pending;
+        unit->onReply = [this, op] { sendStepDone(op); };
+        wireQueue_.push_back(unit);
+        // Announce once the producing work on every source stream is done.
+        auto remaining = std::make_shared<size_t>(directStreams.size());
+        for (auto& s : directStreams) {
+          auto ev = ictx_->events.get(s.device);
+          ev->record(s.stream);
+          watch(std::move(ev), [this, unit, remaining] {
+            if (--*remaining == 0) {
+              unit->ready = true;
+              flushWire();
+            }
+          });
+        }
+      }
+
+      for (uint32_t i : staged) {
+        const HipBuffer& hb = live[i].buffer.unwrap<HipBuffer>();
+        const int device = hipDeviceForPointer(hb.ptr);
+        const size_t chunks = numChunks(live[i].length);
+        for (size_t k = 0; k < chunks; ++k) {
+          const size_t offset = k * kSlotSize;
+          const size_t len = std::min(live[i].length - offset, kSlotSize);
+          auto unit = std::make_shared<WireUnit>();
+          wireQueue_.push_back(unit);
+          ++op->pending; // staged copy of this chunk finished
+          stageChunk(op, unit, device, hb, i, offset, len);
+        }
+      }
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " send failed: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "hip_ipc send", TPHIP_ERR_INVALID_ARG));
+      return;
+    }
+    sendStepDone(op); // drop the guard
+  }
+
+  // Outbox path, one chunk: wait for a slot, copy source -> slot on the
+  // caller's stream, announce the slot when the copy is done, free the slot
+  // when the receiver has replied.
+  void stageChunk(
+      const std::shared_ptr<SendOp>& op,
+      const std::shared_ptr<WireUnit>& unit,
+      int device,
+      HipBuffer hb,
+      uint32_t index,
+      size_t offset,
+      size_t len) {
+    Outbox& outbox = ictx_->outbox(device);
+    auto self = shared_from_this();
+    outbox.allocator.alloc([this, self, op, unit, device, hb, index, offset, len, &outbox](
+                               const Error& error, SlotAllocator::TSlot slot) {
+      if (error) {
+        setError(error);
+        return;
+      }
+      if (error_) {
+        return;
+      }
+      const size_t slotIdx = outbox.allocator.slotIndex(slot.get());
+      int rc = tphip_copy(device, slot.get(), static_cast<const uint8_t*>(hb.ptr) + offset, len, hb.stream);
+      if (rc != 0) {
+        setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+        return;
+      }
+      WireWriter w;
+      w.u8(kChunk);
+      w.u32(index);
+      w.u32(static_cast<uint32_t>(device));
+      const bool announce = !outboxAnnounced_[device];
+      outboxAnnounced_[device] = true;
+      w.u8(announce ? 1 : 0);
+      if (announce) {
+        w.raw(outbox.handle.data(), outbox.handle.size());
+      }
+      w.u32(static_cast<uint32_t>(slotIdx));
+      w.u64(offset);
+      w.u64(len);
+      unit->bytes = std::move(w.bytes());
+      unit->onReply = [slot]() mutable { slot.reset(); }; // reply frees the slot
+      auto ev = ictx_->events.get(device);
+      ev->record(hb.stream);
+      watch(std::move(ev), [this, op, unit] {
+        unit->ready = true;
+        flushWire();
+        sendStepDone(op); // this chunk no longer needs the source
+      });
+    });
+  }
+
+  void sendStepDone(const std::shared_ptr<SendOp>& op) {
+    if (op->done || --op->pending > 0) {
+      return;
+    }
+    removeSend(op);
+    finishSend(op);
+  }
+
+  // Write every unit at the head of the queue whose data is ready, and post
+  // the read for its reply.
+  void flushWire() {
+    while (!wireQueue_.empty() && wireQueue_.front()->ready && !error_) {
+      auto unit = wireQueue_.front();
+      wireQueue_.pop_front();
+      writeMessage(*descriptorConnection_, std::move(unit->bytes));
+      replyConnection_->read(nullptr, 0, onRead([this, unit] {
+        if (!error_ && unit->onReply) {
+          unit->onReply();
+        }
+        unit->onReply = nullptr;
+      }));
+    }
+  }
+
+  // ---- recv -----------------------------------------------------------------
+
+  void recvEntries(uint64_t seq, std::vector<BatchEntry> entries, TRecvCallback cb) {
+    auto op = std::make_shared<RecvOp>();
+    op->seq = seq;
+    op->cb = std::move(cb);
+    for (auto& e : entries) {
+      if (e.length > 0) {
+        op->entries.push_back(std::move(e));
+      }
+    }
+    if (op->entries.empty()) {
+      op->cb(error_);
+      return;
+    }
+    recvOps_.push_back(op);
+    readNextUnit(op);
+  }
+
+  // The number of units of an op is only known once its first unit has been
+  // seen (a direct unit says how many tensors it covers), so units are read
+  // one at a time until every tensor of the op is accounted for.
+  void readNextUnit(const std::shared_ptr<RecvOp>& op) {
+    descriptorConnection_->read(onReadMessage([this, op](std::vector<uint8_t> bytes) {
+      if (error_) {
+        return;
+      }
+      onUnit(op, bytes);
+    }));
+  }
+
+  void onUnit(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
+    WireReader r(bytes.data(), bytes.size());
+    const uint8_t kind = r.u8();
+    auto reply = std::make_shared<ReplyUnit>();
+    replyQueue_.push_back(reply);
+    std::vector<StreamRef> touched;
+    try {
+      if (kind == kDirect) {
+        const uint32_t n = r.u32();
+        struct Group {
+          StreamRef dst;
+          std::vector<tphip_copy_desc> table;
+        };
+        std::vector<Group> groups;
+        for (uint32_t k = 0; k < n; ++k) {
+          const uint32_t index = r.u32();
+          const uint64_t exportId = r.u64();
+          const bool announce = r.u8() != 0;
+          if (!r.ok() || index >= op->entries.size()) {
+            failProtocol();
+            return;
+          }
+          const HipBuffer& hb = op->entries[index].buffer.unwrap<HipBuffer>();
+          const int device = hipDeviceForPointer(hb.ptr);
+          TP_THROW_ASSERT_IF(device < 0);
+          if (announce) {
+            HandleBytes h;
+            r.raw(h.data(), h.size());
+            void* mapped = nullptr;
+            int rc = ImportRegistry::get().open(device, h, &mapped);
+            if (rc != 0) {
+              setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
+              return;
+            }
+            remoteAllocations_[exportId] = mapped;
+          }
+          const uint64_t offset = r.u64();
+          const uint64_t length = r.u64();
+          auto it = remoteAllocations_.find(exportId);
+          if (!r.ok() || it == remoteAllocations_.end() || length != op->entries[index].length) {
+            failProtocol();
+            return;
+          }
+          StreamRef ref{hb.stream, device};
+          Group* g = nullptr;
+          for (auto& cand : groups) {
+            if (cand.dst == ref) {
+              g = &cand;
+            }
+          }
+          if (g == nullptr) {
+            groups.push_back(Group{ref, {}});
+            g = &groups.back();
+          }
+          g->table.push_back(
+              tphip_copy_desc{static_cast<const uint8_t*>(it->second) + offset, hb.ptr, length});
+          ++op->unitsSeen;
+        }
+        for (auto& g : groups) {
+          hipBatchedCopy(g.dst.device, g.dst.stream, g.table);
+          touched.push_back(g.dst);
+        }
+        op->unitsExpected += n;
+      } else if (kind == kChunk) {
+        const uint32_t index = r.u32();
+        const int srcDevice = static_cast<int>(r.u32());
+        const bool announce = r.u8() != 0;
+        if (!r.ok() || index >= op->entries.size()) {
+          failProtocol();
+          return;
+        }
+        const HipBuffer& hb = op->entries[index].buffer.unwrap<HipBuffer>();
+        const int device = hipDeviceForPointer(hb.ptr);
+        TP_THROW_ASSERT_IF(device < 0);
+        if (announce) {
+          HandleBytes h;
+          r.raw(h.data(), h.size());
+          void* mapped = nullptr;
+          int rc = ImportRegistry::get().open(device, h, &mapped);
+          if (rc != 0) {
+            setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
+            return;
+          }
+          remoteOutboxes_[srcDevice] = mapped;
+        }
+        const uint32_t slotIdx = r.u32();
+        const uint64_t offset = r.u64();
+        const uint64_t len = r.u64();
+        auto it = remoteOutboxes_.find(srcDevice);
+        if (!r.ok() || it == remoteOutboxes_.end() || slotIdx >= kNumSlots || len > kSlotSize ||
+            offset + len > op->entries[index].length) {
+          failProtocol();
+          return;
+        }
+        int rc = tphip_copy(
+            device,
+            static_cast<uint8_t*>(hb.ptr) + offset,
+            static_cast<const uint8_t*>(it->second) + slotIdx * kSlotSize,
+            len,
+            hb.stream);
+        if (rc != 0) {
+          setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+          return;
+        }
+        touched.push_back(StreamRef{hb.stream, device});
+        // A staged tensor counts as seen when its last chunk arrived.
+        if (offset + len == op->entries[index].length) {
+          ++op->unitsSeen;
+        }
+        if (offset == 0) {
+          ++op->unitsExpected;
+        }
+      } else {
+        failProtocol();
+        return;
+      }
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " recv failed: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "hip_ipc recv", TPHIP_ERR_INVALID_ARG));
+      return;
+    }
+
+    // Reply once the copies of this unit have finished.
+    auto remaining = std::make_shared<size_t>(touched.size());
+    for (auto& s : touched) {
+      auto ev = ictx_->events.get(s.device);
+      ev->record(s.stream);
+      watch(std::move(ev), [this, reply, remaining] {
+        if (--*remaining == 0) {
+          reply->ready = true;
+          flushReplies();
+        }
+      });
+    }
+
+    if (op->unitsSeen == op->entries.size()) {
+      // Every copy of the op is enqueued: that is what the recv callback means.
+      removeRecv(op);
+      finishRecv(op);
+    } else {
+      readNextUnit(op);
+    }
+  }
+
+  void flushReplies() {
+    while (!replyQueue_.empty() && replyQueue_.front()->ready && !error_) {
+      replyQueue_.pop_front();
+      replyConnection_->write(nullptr, 0, onWritten([] {}));
+    }
+  }
+
+  void failProtocol() {
+    setError(TP_CREATE_ERROR(ShortReadError, -1, -1));
+  }
+
+  // ---- helpers ----------------------------------------------------------------
+
+  // Run fn on the context loop once the event has completed.
+  template <typename F>
+  void watch(std::unique_ptr<HipEvent> ev, F fn) {
+    auto self = shared_from_this();
+    ictx_->poller.watch(
+        std::move(ev), &ictx_->events, [this, self, fn{std::move(fn)}](const Error& error) mutable {
+          ctx_->defer([this, self, fn{std::move(fn)}, error]() mutable {
+            setError(error);
+            if (!error_) {
+              fn();
+            }
+          });
+        });
+  }
+
+  void removeSend(const std::shared_ptr<SendOp>& op) {
+    for (auto it = sendOps_.begin(); it != sendOps_.end(); ++it) {
+      if (*it == op) {
+        sendOps_.erase(it);
+        return;
+      }
+    }
+  }
+
+  void removeRecv(const std::shared_ptr<RecvOp>& op) {
+    for (auto it = recvOps_.begin(); it != recvOps_.end(); ++it) {
+      if (*it == op) {
+        recvOps_.erase(it);
+        return;
+      }
+    }
+  }
+
+  void finishSend(const std::shared_ptr<SendOp>& op) {
+    if (op->done) {
+      return;
+    }
+    op->done = true;
+    auto cb = std::move(op->cb);
+    cb(error_);
+  }
+
+  void finishRecv(const std::shared_ptr<RecvOp>& op) {
+    if (op->done) {
+      return;
+    }
+    op->done = true;
+    auto cb = std::move(op->cb);
+    cb(error_);
+  }
+
+  std::shared_ptr<IpcContextCore> ictx_;
+  std::shared_ptr<transport::Connection> descriptorConnection_;
+  std::shared_ptr<transport::Connection> replyConnection_;
+  std::deque<std::shared_ptr<SendOp>> sendOps_;
+  std::deque<std::shared_ptr<RecvOp>> recvOps_;
+  std::deque<std::shared_ptr<WireUnit>> wireQueue_;
+  std::deque<std::shared_ptr<ReplyUnit>> replyQueue_;
+  std::set<uint64_t> announced_;
+  std::map<int, bool> outboxAnnounced_;
+  std::map<uint64_t, void*> remoteAllocations_;
+  std::map<int, void*> remoteOutboxes_;
+};
+
+class IpcChannel final : public ChannelHandle<ChannelImpl>, public BatchedChannel {
+ public:
+  using ChannelHandle<ChannelImpl>::ChannelHandle;
+  void sendBatch(std::vector<BatchEntry> entries, TSendCallback callback) override {
+    if (!impl_) {
+      callback(TP_CREATE_ERROR(ContextNotViableError));
+      return;
+    }
+    impl_->sendBatch(std::move(entries), std::move(callback));
+  }
+  void recvBatch(std::vector<BatchEntry> entries, TRecvCallback callback) override {
+    if (!impl_) {
+      callback(TP_CREATE_ERROR(ContextNotViableError));
+      return;
+    }
+    impl_->recvBatch(std::move(entries), std::move(callback));
+  }
+};
+
+// Device descriptor "<boot id>|<process identity>|<device uuid>"
+// (cf. DeviceDescriptor{bootId, pid, deviceUuid},
+// tensorpipe/channel/cuda_ipc/context_impl.cc:108-113).
+struct ParsedDescriptor {
+  std::string boot;
+  std::string process;
+  std::string uuid;
+};
+
+bool parseDescriptor(const std::string& s, ParsedDescriptor* out) {
+  auto a = s.find('|');
+  auto b = a == std::string::npos ? a : s.find('|', a + 1);
+  if (b == std::string::npos) {
+    return false;
+  }
+  out->boot = s.substr(0, a);
+  out->process = s.substr(a + 1, b - a - 1);
+  out->uuid = s.substr(b + 1);
+  return true;
+}
+
+class ContextImpl final : public Context {
+ public:
+  ContextImpl() {
+    const int n = hipDeviceCountNoThrow();
+    if (n <= 0) {
+      return;
+    }
+    for (int i = 0; i < n; ++i) {
+      char uuid[TPHIP_UUID_STRLEN + 1];
+      if (tphip_device_uuid(i, uuid) != 0) {
+        return;
+      }
+      descriptors_[Device{kHipDeviceType, i}] =
+          bootIdentity() + "|" + processIdentity() + "|" + uuid;
+    }
+    core_ = std::make_shared<IpcContextCore>();
+  }
+  ~ContextImpl() override {
+    join();
+  }
+  bool isViable() const override {
+    return core_ != nullptr;
+  }
+  size_t numConnectionsNeeded() const override {
+    return 2; // descriptors one way, replies the other
+  }
+  const std::unordered_map<Device, std::string>& deviceDescriptors() const override {
+    return descriptors_;
+  }
+  // Same machine boot, different process
+  // (tensorpipe/channel/cuda_ipc/context_impl.cc:310-335; the peer-to-peer
+  // matrix check of the reference has no counterpart on a one-GPU machine:
+  // a device can always reach itself).
+  bool canCommunicateWithRemote(const std::string& local, const std::string& remote)
+      const override {
+    ParsedDescriptor l, r;
+    if (!parseDescriptor(local, &l) || !parseDescriptor(remote, &r)) {
+      return false;
+    }
+    if (l.boot != r.boot || l.process == r.process) {
+      return false;
+    }
+    return l.uuid == r.uuid;
+  }
+  std::shared_ptr<Channel> createChannel(
+      std::vector<std::shared_ptr<transport::Connection>> connections,
+      Endpoint /*endpoint*/) override {
+    if (!core_) {
+      return std::make_shared<IpcChannel>(nullptr);
+    }
+    TP_THROW_ASSERT_IF(connections.size() != 2);
+    auto impl = std::make_shared<ChannelImpl>(
+        core_, core_->nextChannelId(), std::move(connections[0]), std::move(connections[1]));
+    impl->init();
+    return std::make_shared<IpcChannel>(std::move(impl));
+  }
+  void setId(std::string id) override {
+    if (core_) {
+      core_->setId(std::move(id));
+    }
+  }
+  void close() override {
+    if (core_) {
+      core_->close();
+    }
+  }
+  void join() override {
+    if (core_) {
+      core_->join();
+    }
+  }
+
+ private:
+  std::shared_ptr<IpcContextCore> core_;
+  std::unordered_map<Device, std::string> descriptors_;
+};
+
+} // namespace
+
+std::shared_ptr<Context> create() {
+  return std::make_shared<ContextImpl>();
+}
+
+} // namespace hip_ipc
+} // namespace channel
+TP_AMD_NAMESPACE_END

@@ -1,0 +1,16 @@
+#pragma once
+
+#include <tensorpipe/common/device.h>
+
+TP_AMD_NAMESPACE_BEGIN
+
+// tensorpipe/common/cpu_buffer.h:15-21
+struct CpuBuffer {
+  void* ptr{nullptr};
+
+  Device getDevice() const {
+    return Device{kCpuDeviceType, 0};
+  }
+};
+
+TP_AMD_NAMESPACE_END

@@ -1,0 +1,155 @@
+// C++ convenience over the HIP C ABI (include/tphip.h): error checking that
+// throws, RAII for events, streams, device and pinned slabs. The only way host
+// code in this library touches the GPU.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include <tphip.h>
+
+#include <tensorpipe/common/defs.h>
+#include <tensorpipe/common/error.h>
+
+#define TP_HIP_CHECK(call)                                                          \
+  do {                                                                              \
+    int tp_rc_ = (call);                                                            \
+    if (tp_rc_ != 0) {                                                              \
+      TP_THROW_MSG(#call << " failed: [" << tp_rc_ << "] " << tphip_strerror(tp_rc_)); \
+    }                                                                               \
+  } while (0)
+
+TP_AMD_NAMESPACE_BEGIN
+
+// Number of usable GPUs; 0 when the runtime reports none or fails to load.
+int hipDeviceCountNoThrow();
+
+// Device index owning ptr, -1 for host memory (tensorpipe/common/cuda.h:141-166).
+int hipDeviceForPointer(const void* ptr);
+
+class HipEvent {
+ public:
+  HipEvent(int device, bool interprocess = false) : device_(device) {
+    TP_HIP_CHECK(tphip_event_create(device, interprocess ? 1 : 0, &ev_));
+  }
+  HipEvent(const HipEvent&) = delete;
+  HipEvent& operator=(const HipEvent&) = delete;
+  ~HipEvent() {
+    if (ev_ != nullptr) {
+      tphip_event_destroy(device_, ev_);
+    }
+  }
+  void record(void* stream) {
+    TP_HIP_CHECK(tphip_event_record(device_, ev_, stream));
+  }
+  // Make `stream` (on `streamDevice`) wait for the work captured by the last record.
+  void wait(void* stream, int streamDevice) {
+    TP_HIP_CHECK(tphip_stream_wait_event(streamDevice, stream, ev_));
+  }
+  bool query() {
+    int done = 0;
+    TP_HIP_CHECK(tphip_event_query(device_, ev_, &done));
+    return done != 0;
+  }
+  void* raw() const {
+    return ev_;
+  }
+  int device() const {
+    return device_;
+  }
+
+ private:
+  int device_;
+  void* ev_{nullptr};
+};
+
+// Recycles events per device so the per-message path creates none.
+class HipEventPool {
+ public:
+  std::unique_ptr<HipEvent> get(int device) {
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      if (device < static_cast<int>(free_.size()) && !free_[device].empty()) {
+        auto ev = std::move(free_[device].back());
+        free_[device].pop_back();
+        return ev;
+      }
+    }
+    return std::make_unique<HipEvent>(device);
+  }
+  void put(std::unique_ptr<HipEvent> ev) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    const int device = ev->device();
+    if (device >= static_cast<int>(free_.size())) {
+      free_.resize(device + 1);
+    }
+    free_[device].push_back(std::move(ev));
+  }
+
+ private:
+  std::mutex mutex_;
+  std::vector<std::vector<std::unique_ptr<HipEvent>>> free_;
+};
+
+// Pinned, device-mapped host slab (tensorpipe/common/cuda.h:183-188).
+class HipPinnedSlab {
+ public:
+  HipPinnedSlab(int device, size_t bytes) : bytes_(bytes) {
+    TP_HIP_CHECK(tphip_host_alloc(device, bytes, &host_, &dev_));
+  }
+  HipPinnedSlab(const HipPinnedSlab&) = delete;
+  ~HipPinnedSlab() {
+    if (host_ != nullptr) {
+      tphip_host_free(host_);
+    }
+  }
+  uint8_t* host() const {
+    return static_cast<uint8_t*>(host_);
+  }
+  // Address of the same bytes as seen by kernels.
+  uint8_t* dev() const {
+    return static_cast<uint8_t*>(dev_);
+  }
+  size_t size() const {
+    return bytes_;
+  }
+
+ private:
+  size_t bytes_;
+  void* host_{nullptr};
+  void* dev_{nullptr};
+};
+
+// Device slab (tensorpipe/common/cuda.h:213-218).
+class HipDeviceSlab {
+ public:
+  HipDeviceSlab(int device, size_t bytes) : device_(device), bytes_(bytes) {
+    TP_HIP_CHECK(tphip_malloc(device, bytes, &ptr_));
+  }
+  HipDeviceSlab(const HipDeviceSlab&) = delete;
+  ~HipDeviceSlab() {
+    if (ptr_ != nullptr) {
+      tphip_free(device_, ptr_);
+    }
+  }
+  uint8_t* ptr() const {
+    return static_cast<uint8_t*>(ptr_);
+  }
+  size_t size() const {
+    return bytes_;
+  }
+  int device() const {
+    return device_;
+  }
+
+ private:
+  int device_;
+  size_t bytes_;
+  void* ptr_{nullptr};
+};
+
+TP_AMD_NAMESPACE_END

@@ -1,0 +1,1359 @@
+// Context, Listener and Pipe: the caller of the channels. A deliberately
+// small implementation of the reference's public API (tensorpipe/core/*) with
+// its own wire format: enough to drive channels through Pipe::write /
+// readDescriptor / read exactly the way user code drives the reference.
+//
+// Differences from the reference that a user can observe:
+//  * the pipe stays on the transport it was opened on (no transport upgrade);
+//  * control messages use common/wire.h instead of libnop, so this Pipe does
+//    not interoperate with a stock TensorPipe peer;
+//  * all tensors of a message that map to one channel are handed to that
+//    channel as ONE batch when it implements channel::BatchedChannel, so a
+//    message costs one control message and one kernel launch, not one per
+//    tensor (cf. the per-tensor loop at tensorpipe/core/pipe_impl.cc:884-915).
+
+#include <tensorpipe/core/context.h>
+#include <tensorpipe/core/listener.h>
+#include <tensorpipe/core/pipe.h>
+
+#include <atomic>
+#include <deque>
+#include <mutex>
+
+#include <unistd.h>
+
+#include <map>
+#include <unordered_map>
+#include <unordered_set>
+
+#include <tensorpipe/channel/channel.h>
+#include <tensorpipe/common/loop.h>
+#include <tensorpipe/common/wire.h>
+#include <tensorpipe/core/error.h>
+#include <tensorpipe/transport/connection.h>
+#include <tensorpipe/transport/listener.h>
+
+TP_AMD_NAMESPACE_BEGIN
+
+namespace {
+
+enum PacketType : uint8_t {
+  kHelloSpontaneous = 1,
+  kHelloRequested = 2,
+  kBrochureAnswer = 3,
+  kDescriptor = 4,
+  kDescriptorReply = 5,
+};
+
+void putDevice(WireWriter& w, const Device& d) {
+  w.str(d.type);
+  w.u32(static_cast<uint32_t>(d.index));
+}
+
+Device getDevice(WireReader& r) {
+  Device d;
+  d.type = r.str();
+  d.index = static_cast<int>(r.u32());
+  return d;
+}
+
+bool splitUrl(const std::string& url, std::string* transport, std::string* addr) {
+  const std::string sep = "://";
+  auto pos = url.find(sep);
+  if (pos == std::string::npos) {
+    return false;
+  }
+  *transport = url.substr(0, pos);
+  *addr = url.substr(pos + sep.size());
+  return true;
+}
+
+using DevicePairMap = std::unordered_map<std::pair<Device, Device>, std::string>;
+
+} // namespace
+
+class PipeImpl;
+
+class ContextImpl final : public std::enable_shared_from_this<ContextImpl> {
+ public:
+  explicit ContextImpl(ContextOptions opts) : name_(std::move(opts.name_)) {
+    static std::atomic<uint64_t> counter{0};
+    id_ = std::to_string(::getpid()) + ":c" + std::to_string(counter.fetch_add(1));
+  }
+
+  struct ChannelEntry {
+    int64_t priority;
+    std::string name;
+    std::shared_ptr<channel::Context> context;
+  };
+
+  void registerTransport(
+      int64_t priority,
+      std::string name,
+      std::shared_ptr<transport::Context> context) {
+    TP_THROW_ASSERT_IF(name.empty());
+    std::lock_guard<std::mutex> lock(mutex_);
+    TP_THROW_ASSERT_IF(transports_.count(name) != 0);
+    for (auto& t : transports_) {
+      TP_THROW_ASSERT_IF(t.second.first == priority);
+    }
+    if (!context->isViable()) {
+      TP_VLOG(1) << "Context " << id_ << " is not registering transport " << name
+                 << " because it is not viable";
+      return;
+    }
+    context->setId(id_ + ".tr_" + name);
+    transports_.emplace(std::move(name), std::make_pair(priority, std::move(context)));
+  }
+
+  // Rejects duplicate names and priorities, skips non-viable contexts, keeps
+  // channels sorted by descending priority (tensorpipe/core/context_impl.cc:89-110).
+  void registerChannel(
+      int64_t priority,
+      std::string name,
+      std::shared_ptr<channel::Context> context) {
+    TP_THROW_ASSERT_IF(name.empty());
+    std::lock_guard<std::mutex> lock(mutex_);
+    for (auto& c : channels_) {
+      TP_THROW_ASSERT_IF(c.name == name);
+      TP_THROW_ASSERT_IF(c.priority == priority);
+    }
+    if (!context->isViable()) {
+      TP_VLOG(1) << "Context " << id_ << " is not registering channel " << name
+                 << " because it is not viable";
+      return;
+    }
+    context->setId(id_ + ".ch_" + name);
+    ChannelEntry e{priority, std::move(name), std::move(context)};
+    auto it = channels_.begin();
+    while (it != channels_.end() && it->priority > priority) {
+      ++it;
+    }
+    channels_.insert(it, std::move(e));
+  }
+
+  std::shared_ptr<transport::Context> transport(const std::string& name) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    auto it = transports_.find(name);
+    return it == transports_.end() ? nullptr : it->second.second;
+  }
+
+  std::vector<ChannelEntry> channels() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return channels_;
+  }
+
+  std::shared_ptr<channel::Context> channel(const std::string& name) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    for (auto& c : channels_) {
+      if (c.name == name) {
+        return c.context;
+      }
+    }
+    return nullptr;
+  }
+
+  std::unordered_map<std::string, std::string> transportDescriptors() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    std::unordered_map<std::string, std::string> out;
+    for (auto& t : transports_) {
+      out[t.first] = t.second.second->domainDescriptor();
+    }
+    return out;
+  }
+
+  std::shared_ptr<Listener> listen(const std::vector<std::string>& urls);
+  std::shared_ptr<Pipe> connect(const std::string& url, PipeOptions opts);
+
+  void defer(TTask fn) {
+    loop_.defer(std::move(fn));
+  }
+  bool closed() const {
+    return closed_.load();
+  }
+  const std::string& name() const {
+    return name_;
+  }
+  const std::string& id() const {
+    return id_;
+  }
+  std::string nextPipeId() {
+    return id_ + ".p" + std::to_string(pipeCounter_.fetch_add(1));
+  }
+
+  // Children register a closer so that Context::close() reaches them.
+  uint64_t enroll(std::function<void()> closer) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    uint64_t k = nextChild_++;
+    children_[k] = std::move(closer);
+    return k;
+  }
+  void unenroll(uint64_t k) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    children_.erase(k);
+  }
+
+  void close() {
+    if (closed_.exchange(true)) {
+      return;
+    }
+    std::map<uint64_t, std::function<void()>> children;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      children = children_;
+    }
+    for (auto& c : children) {
+      c.second();
+    }
+    std::lock_guard<std::mutex> lock(mutex_);
+    for (auto& c : channels_) {
+      c.context->close();
+    }
+    for (auto& t : transports_) {
+      t.second.second->close();
+    }
+  }
+
+  void join() {
+    close();
+    if (joined_.exchange(true)) {
+      return;
+    }
+    std::vector<ChannelEntry> channels;
+    std::map<std::string, std::pair<int64_t, std::shared_ptr<transport::Context>>> transports;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      channels = channels_;
+      transports = transports_;
+    }
+    for (auto& c : channels) {
+      c.context->join();
+    }
+    for (auto& t : transports) {
+      t.second.second->join();
+    }
+  }
+
+ private:
+  const std::string name_;
+  std::string id_;
+  OnDemandLoop loop_;
+  std::mutex mutex_;
+  std::map<std::string, std::pair<int64_t, std::shared_ptr<transport::Context>>> transports_;
+  std::vector<ChannelEntry> channels_;
+  std::map<uint64_t, std::function<void()>> children_;
+  uint64_t nextChild_{0};
+  std::atomic<uint64_t> pipeCounter_{0};
+  std::atomic<bool> closed_{false};
+  std::atomic<bool> joined_{false};
+};
+
+// ---------------------------------------------------------------------------
+
+class ListenerImpl final : public std::enable_shared_from_this<ListenerImpl> {
+ public:
+  using accept_callback_fn = Listener::accept_callback_fn;
+  using connection_request_fn =
+      std::function<void(const Error&, std::shared_ptr<transport::Connection>)>;
+
+  ListenerImpl(std::shared_ptr<ContextImpl> ctx, const std::vector<std::string>& urls)
+      : ctx_(std::move(ctx)) {
+    for (const auto& url : urls) {
+      std::string transport, addr;
+      TP_THROW_ASSERT_IF(!splitUrl(url, &transport, &addr));
+      auto tctx = ctx_->transport(transport);
+      TP_THROW_ASSERT_IF(tctx == nullptr);
+      auto l = tctx->listen(addr);
+      addresses_[transport] = l->addr();
+      listeners_[transport] = std::move(l);
+    }
+  }
+
+  void init() {
+    auto self = shared_from_this();
+    childKey_ = ctx_->enroll([self] { self->close(); });
+    ctx_->defer([self] {
+      if (self->ctx_->closed()) {
+        self->fail(TP_CREATE_ERROR(ContextClosedError));
+        return;
+      }
+      for (auto& l : self->listeners_) {
+        self->armAccept(l.first);
+      }
+    });
+  }
+
+  void accept(accept_callback_fn fn) {
+    auto self = shared_from_this();
+    ctx_->defer([self, fn{std::move(fn)}]() mutable {
+      if (self->error_) {
+        fn(self->error_, nullptr);
+        return;
+      }
+      self->acceptors_.push_back(std::move(fn));
+      self->matchPipes();
+    });
+  }
+
+  const std::map<std::string, std::string>& addresses() const {
+    return addresses_;
+  }
+
+  // Loop only. The returned token is sent to the peer, which presents it as
+  // the first packet of a new connection (tensorpipe/core/listener_impl.h:52-56).
+  uint64_t registerConnectionRequest(connection_request_fn fn) {
+    uint64_t token = nextToken_++;
+    requests_[token] = std::move(fn);
+    return token;
+  }
+
+  void unregisterConnectionRequest(uint64_t token) {
+    requests_.erase(token);
+  }
+
+  void close() {
+    auto self = shared_from_this();
+    ctx_->defer([self] { self->fail(TP_CREATE_ERROR(ListenerClosedError)); });
+  }
+
+  void onPipeReady(std::shared_ptr<Pipe> pipe) {
+    readyPipes_.push_back(std::move(pipe));
+    matchPipes();
+  }
+
+  std::shared_ptr<ContextImpl> context() {
+    return ctx_;
+  }
+
+ private:
+  void armAccept(const std::string& transport) {
+    auto self = shared_from_this();
+    listeners_[transport]->accept(
+        [self, transport](const Error& error, std::shared_ptr<transport::Connection> conn) {
+          self->ctx_->defer([self, transport, error, conn]() mutable {
+            if (self->error_) {
+              return;
+            }
+            if (error) {
+              self->fail(error);
+              return;
+            }
+            self->armAccept(transport);
+            self->onConnection(std::move(conn));
+          });
+        });
+  }
+
+  void onConnection(std::shared_ptr<transport::Connection> conn);
+
+  void matchPipes() {
+    while (!acceptors_.empty() && !readyPipes_.empty()) {
+      auto fn = std::move(acceptors_.front());
+      acceptors_.pop_front();
+      auto pipe = std::move(readyPipes_.front());
+      readyPipes_.pop_front();
+      fn(Error::kSuccess, std::move(pipe));
+    }
+  }
+
+  void fail(Error error) {
+    if (error_) {
+      return;
+    }
+    error_ = std::move(error);
+    for (auto& l : listeners_) {
+      l.second->close();
+    }
+    auto acceptors = std::move(acceptors_);
+    acceptors_.clear();
+    for (auto& fn : acceptors) {
+      fn(error_, nullptr);
+    }
+    auto requests = std::move(requests_);
+    requests_.clear();
+    for (auto& r : requests) {
+      r.second(error_, nullptr);
+    }
+    readyPipes_.clear();
+    ctx_->unenroll(childKey_);
+  }
+
+  std::shared_ptr<ContextImpl> ctx_;
+  std::map<std::string, std::shared_ptr<transport::Listener>> listeners_;
+  std::map<std::string, std::string> addresses_;
+  Error error_;
+  uint64_t childKey_{0};
+  std::deque<accept_callback_fn> acceptors_;
+  std::deque<std::shared_ptr<Pipe>> readyPipes_;
+  std::unordered_map<uint64_t, connection_request_fn> requests_;
+  uint64_t nextToken_{1};
+};
+
+// ---------------------------------------------------------------------------
+
+class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
+ public:
+  // Client side.
+  PipeImpl(
+      std::shared_ptr<ContextImpl> ctx,
+      std::string id,
+      std::string remoteName,
+      std::string transport,
+      std::string addr)
+      : ctx_(std::move(ctx)),
+        id_(std::move(id)),
+        remoteName_(std::move(remoteName)),
+        transport_(std::move(transport)),
+        addr_(std::move(addr)),
+        isClient_(true) {}
+
+  // Server side: `hello` is the spontaneous-connection packet already read.
+  PipeImpl(
+      std::shared_ptr<ContextImpl> ctx,
+      std::shared_ptr<ListenerImpl> listener,
+      std::string id,
+      std::shared_ptr<transport::Connection> conn,
+      std::vector<uint8_t> hello)
+      : ctx_(std::move(ctx)),
+        listener_(std::move(listener)),
+        id_(std::move(id)),
+        connection_(std::move(conn)),
+        hello_(std::move(hello)),
+        isClient_(false) {}
+
+  void init() {
+    auto self = shared_from_this();
+    childKey_ = ctx_->enroll([self] { self->close(); });
+    ctx_->defer([self] {
+      if (self->ctx_->closed()) {
+        self->setError(TP_CREATE_ERROR(ContextClosedError));
+        return;
+      }
+      if (self->isClient_) {
+        self->initClient();
+      } else {
+        self->initServer();
+      }
+    });
+  }
+
+  void readDescriptor(Pipe::read_descriptor_callback_fn fn) {
+    auto self = shared_from_this();
+    ctx_->defer([self, fn{std::move(fn)}]() mutable {
+      if (self->error_) {
+        fn(self->error_, Descriptor());
+        return;
+      }
+      self->descriptorWaiters_.push_back(std::move(fn));
+      self->deliverDescriptors();
+    });
+  }
+
+  void read(Allocation allocation, Pipe::read_callback_fn fn) {
+    auto self = shared_from_this();
+    ctx_->defer([self, allocation{std::move(allocation)}, fn{std::move(fn)}]() mutable {
+      self->readFromLoop(std::move(allocation), std::move(fn));
+    });
+  }
+
+  void write(Message message, Pipe::write_callback_fn fn) {
+    auto self = shared_from_this();
+    ctx_->defer([self, message{std::move(message)}, fn{std::move(fn)}]() mutable {
+      self->writeFromLoop(std::move(message), std::move(fn));
+    });
+  }
+
+  const std::string& remoteName() {
+    return remoteName_;
+  }
+
+  void close() {
+    auto self = shared_from_this();
+    ctx_->defer([self] { self->setError(TP_CREATE_ERROR(PipeClosedError)); });
+  }
+
+ private:
+  struct WriteOp {
+    uint64_t seq;
+    Message message;
+    Pipe::write_callback_fn fn;
+    bool needsReply{false};
+    bool haveReply{false};
+    bool tensorsIssued{false};
+    std::vector<Device> targetDevices;
+    size_t pendingWrites{0};
+    size_t pendingSends{0};
+    bool finished{false};
+  };
+
+  struct ReadOp {
+    uint64_t seq;
+    Descriptor descriptor;
+    bool delivered{false};
+    bool readCalled{false};
+    Allocation allocation;
+    Pipe::read_callback_fn fn;
+    size_t pendingPayloads{0};
+    size_t pendingRecvs{0};
+    bool finished{false};
+  };
+
+  // ---- set-up -------------------------------------------------------------
+
+  void initClient() {
+    auto tctx = ctx_->transport(transport_);
+    if (tctx == nullptr) {
+      setError(TP_CREATE_ERROR(LogicError, "unknown transport " + transport_));
+      return;
+    }
+    connection_ = tctx->connect(addr_);
+    connection_->setId(id_ + ".tr_" + transport_);
+    WireWriter w;
+    w.u8(kHelloSpontaneous);
+    w.str(ctx_->name());
+    auto tds = ctx_->transportDescriptors();
+    w.u32(static_cast<uint32_t>(tds.size()));
+    for (auto& t : tds) {
+      w.str(t.first);
+      w.str(t.second);
+    }
+    auto channels = ctx_->channels();
+    w.u32(static_cast<uint32_t>(channels.size()));
+    for (auto& c : channels) {
+      w.str(c.name);
+      const auto& dd = c.context->deviceDescriptors();
+      w.u32(static_cast<uint32_t>(dd.size()));
+      for (auto& d : dd) {
+        putDevice(w, d.first);
+        w.str(d.second);
+      }
+    }
+    writeControl(std::move(w.bytes()));
+    readControl([this](std::vector<uint8_t> bytes) { onBrochureAnswer(std::move(bytes)); });
+  }
+
+  void onBrochureAnswer(std::vector<uint8_t> bytes) {
+    if (error_) {
+      return;
+    }
+    WireReader r(bytes.data(), bytes.size());
+    if (r.u8() != kBrochureAnswer) {
+      setError(TP_CREATE_ERROR(LogicError, "unexpected packet during handshake"));
+      return;
+    }
+    if (remoteName_.empty()) {
+      remoteName_ = r.str();
+    } else {
+      (void)r.str();
+    }
+    auto tctx = ctx_->transport(transport_);
+    const uint32_t nChannels = r.u32();
+    for (uint32_t i = 0; i < nChannels && r.ok(); ++i) {
+      std::string name = r.str();
+      const uint32_t nTokens = r.u32();
+      std::vector<std::shared_ptr<transport::Connection>> conns;
+      for (uint32_t k = 0; k < nTokens && r.ok(); ++k) {
+        const uint64_t token = r.u64();
+        auto conn = tctx->connect(addr_);
+        conn->setId(id_ + ".ch_" + name + "_" + std::to_string(k));
+        WireWriter w;
+        w.u8(kHelloRequested);
+        w.u64(token);
+        auto holder = std::make_shared<std::vector<uint8_t>>(std::move(w.bytes()));
+        conn->write(holder->data(), holder->size(), [holder](const Error&) {});
+        conns.push_back(std::move(conn));
+      }
+      auto cctx = ctx_->channel(name);
+      if (cctx == nullptr) {
+        setError(TP_CREATE_ERROR(LogicError, "peer selected unknown channel " + name));
+        return;
+      }
+      auto ch = cctx->createChannel(std::move(conns), channel::Endpoint::kConnect);
+      ch->setId(id_ + ".ch_" + name);
+      channels_[name] = std::move(ch);
+    }
+    const uint32_t nPairs = r.u32();
+    for (uint32_t i = 0; i < nPairs && r.ok(); ++i) {
+      Device serverDev = getDevice(r);
+      Device clientDev = getDevice(r);
+      std::string name = r.str();
+      // The server lists (its device, our device); we key on (ours, theirs).
+      channelForDevicePair_[{clientDev, serverDev}] = std::move(name);
+    }
+    if (!r.ok()) {
+      setError(TP_CREATE_ERROR(LogicError, "malformed brochure answer"));
+      return;
+    }
+    establish();
+  }
+
+  void initServer() {
+    WireReader r(hello_.data(), hello_.size());
+    (void)r.u8();
+    remoteName_ = r.str();
+    std::unordered_map<std::string, std::string> remoteTransports;
+    const uint32_t nT = r.u32();
+    for (uint32_t i = 0; i < nT && r.ok(); ++i) {
+      std::string n = r.str();
+      remoteTransports[n] = r.str();
+    }
+    std::unordered_map<std::string, std::unordered_map<Device, std::string>> remoteChannels;
+    const uint32_t nC = r.u32();
+    for (uint32_t i = 0; i < nC && r.ok(); ++i) {
+      std::string n = r.str();
+      const uint32_t nD = r.u32();
+      for (uint32_t k = 0; k < nD && r.ok(); ++k) {
+        Device d = getDevice(r);
+        remoteChannels[n][d] = r.str();
+      }
+    }
+    if (!r.ok()) {
+      setError(TP_CREATE_ERROR(LogicError, "malformed brochure"));
+      return;
+    }
+    hello_.clear();
+
+    // For every (local device, remote device) pair the first channel in
+    // priority order that accepts the two descriptors wins
+    // (tensorpipe/core/pipe_impl.cc:166-219).
+    std::vector<std::string> selected;
+    for (auto& c : ctx_->channels()) {
+      auto it = remoteChannels.find(c.name);
+      if (it == remoteChannels.end()) {
+        continue;
+      }
+      bool used = false;
+      for (auto& local : c.context->deviceDescriptors()) {
+        for (auto& remote : it->second) {
+          auto key = std::make_pair(local.first, remote.first);
+          if (channelForDevicePair_.count(key) != 0) {
+            continue;
+          }
+          if (!c.context->canCommunicateWithRemote(local.second, remote.second)) {
+            continue;
+          }
+          channelForDevicePair_[key] = c.name;
+          used = true;
+        }
+      }
+      if (used) {
+        selected.push_back(c.name);
+      }
+    }
+
+    WireWriter w;
+    w.u8(kBrochureAnswer);
+    w.str(ctx_->name());
+    w.u32(static_cast<uint32_t>(selected.size()));
+    auto self = shared_from_this();
+    for (auto& name : selected) {
+      auto cctx = ctx_->channel(name);
+      const size_t n = cctx->numConnectionsNeeded();
+      w.str(name);
+      w.u32(static_cast<uint32_t>(n));
+      auto& slots = pendingChannelConns_[name];
+      slots.resize(n);
+      for (size_t k = 0; k < n; ++k) {
+        ++connectionsAwaited_;
+        uint64_t token = listener_->registerConnectionRequest(
+            [self, name, k](const Error& error, std::shared_ptr<transport::Connection> conn) {
+              self->onRequestedConnection(name, k, error, std::move(conn));
+            });
+        tokens_.push_back(token);
+        w.u64(token);
+      }
+    }
+    w.u32(static_cast<uint32_t>(channelForDevicePair_.size()));
+    for (auto& p : channelForDevicePair_) {
+      putDevice(w, p.first.first);
+      putDevice(w, p.first.second);
+      w.str(p.second);
+    }
+    writeControl(std::move(w.bytes()));
+    if (connectionsAwaited_ == 0) {
+      createServerChannels();
+    }
+  }
+
+  void onRequestedConnection(
+      const std::string& name,
+      size_t k,
+      const Error& error,
+      std::shared_ptr<transport::Connection> conn) {
+    if (error_) {
+      return;
+    }
+    if (error) {
+      setError(error);
+      return;
+    }
+    conn->setId(id_ + ".ch_" + name + "_" + std::to_string(k));
+    pendingChannelConns_[name][k] = std::move(conn);
+    if (--connectionsAwaited_ == 0) {
+      createServerChannels();
+    }
+  }
+
+  void createServerChannels() {
+    tokens_.clear();
+    for (auto& p : pendingChannelConns_) {
+      auto cctx = ctx_->channel(p.first);
+      auto ch = cctx->createChannel(std::move(p.second), channel::Endpoint::kListen);
+      ch->setId(id_ + ".ch_" + p.first);
+      channels_[p.first] = std::move(ch);
+    }
+    pendingChannelConns_.clear();
+    establish();
+  }
+
+  void establish() {
+    established_ = true;
+    TP_VLOG(2) << "Pipe " << id_ << " is established with " << channels_.size() << " channel(s)";
+    pumpPackets();
+    advanceWrites();
+  }
+
+  // ---- control-connection plumbing ---------------------------------------
+
+  template <typename F>
+  void readControl(F fn) {
+    auto self = shared_from_this();
+    connection_->read(
+        [self, fn{std::move(fn)}](const Error& error, const void* ptr, size_t len) mutable {
+          std::vector<uint8_t> bytes;
+          if (!error) {
+            bytes.assign(
+                static_cast<const uint8_t*>(ptr), static_cast<const uint8_t*>(ptr) + len);
+          }
+          self->ctx_->defer([self, fn{std::move(fn)}, error, bytes{std::move(bytes)}]() mutable {
+            self->setError(error);
+            fn(std::move(bytes));
+          });
+        });
+  }
+
+  void writeControl(std::vector<uint8_t> bytes) {
+    auto self = shared_from_this();
+    auto holder = std::make_shared<std::vector<uint8_t>>(std::move(bytes));
+    connection_->write(holder->data(), holder->size(), [self, holder](const Error& error) {
+      if (error) {
+        self->ctx_->defer([self, error] { self->setError(error); });
+      }
+    });
+  }
+
+  // One packet read is outstanding at any time, except while the payloads of
+  // the most recent descriptor have not been claimed by a read() call: those
+  // are the next messages on the connection and go straight to user memory.
+  void pumpPackets() {
+    if (!established_ || error_ || packetReadOutstanding_ || payloadsUnclaimed_) {
+      return;
+    }
+    packetReadOutstanding_ = true;
+    readControl([this](std::vector<uint8_t> bytes) {
+      packetReadOutstanding_ = false;
+      if (error_) {
+        return;
+      }
+      onPacket(std::move(bytes));
+      pumpPackets();
+    });
+  }
+
+  void onPacket(std::vector<uint8_t> bytes) {
+    WireReader r(bytes.data(), bytes.size());
+    const uint8_t type = r.u8();
+    if (type == kDescriptor) {
+      auto op = std::make_shared<ReadOp>();
+      op->seq = nextReadSeq_++;
+      Descriptor& d = op->descriptor;
+      d.metadata = r.str();
+      const uint32_t nP = r.u32();
+      for (uint32_t i = 0; i < nP && r.ok(); ++i) {
+        Descriptor::Payload p;
+        p.length = r.u64();
+        p.metadata = r.str();
+        d.payloads.push_back(std::move(p));
+      }
+      const uint32_t nT = r.u32();
+      for (uint32_t i = 0; i < nT && r.ok(); ++i) {
+        Descriptor::Tensor t;
+        t.length = r.u64();
+        t.sourceDevice = getDevice(r);
+        if (r.u8() != 0) {
+          t.targetDevice = getDevice(r);
+        }
+        t.metadata = r.str();
+        d.tensors.push_back(std::move(t));
+      }
+      if (!r.ok()) {
+        setError(TP_CREATE_ERROR(LogicError, "malformed descriptor"));
+        return;
+      }
+      bool hasPayloadBytes = false;
+      for (auto& p : d.payloads) {
+        hasPayloadBytes |= p.length > 0;
+      }
+      if (hasPayloadBytes) {
+        payloadsUnclaimed_ = true;
+      }
+      readOps_.push_back(std::move(op));
+      deliverDescriptors();
+    } else if (type == kDescriptorReply) {
+      const uint32_t n = r.u32();
+      std::vector<Device> devices;
+      for (uint32_t i = 0; i < n && r.ok(); ++i) {
+        devices.push_back(getDevice(r));
+      }
+      for (auto& op : writeOps_) {
+        if (op->needsReply && !op->haveReply) {
+          if (!r.ok() || devices.size() != op->message.tensors.size()) {
+            setError(TP_CREATE_ERROR(LogicError, "malformed descriptor reply"));
+            return;
+          }
+          op->haveReply = true;
+          op->targetDevices = std::move(devices);
+          break;
+        }
+      }
+      advanceWrites();
+    } else {
+      setError(TP_CREATE_ERROR(LogicError, "unexpected packet type"));
+    }
+  }
+
+  // ---- read side ----------------------------------------------------------
+
+  void deliverDescriptors() {
+    while (!descriptorWaiters_.empty()) {
+      std::shared_ptr<ReadOp> next;
+      for (auto& op : readOps_) {
+        if (!op->delivered) {
+          next = op;
+          break;
+        }
+      }
+      if (!next) {
+        break;
+      }
+      next->delivered = true;
+      auto fn = std::move(descriptorWaiters_.front());
+      descriptorWaiters_.pop_front();
+      TP_VLOG(3) << "Pipe " << id_ << " is calling a readDescriptor callback (#" << next->seq
+                 << ")";
+      fn(Error::kSuccess, next->descriptor);
+    }
+  }
+
+  void readFromLoop(Allocation allocation, Pipe::read_callback_fn fn) {
+    if (error_) {
+      fn(error_);
+      return;
+    }
+    std::shared_ptr<ReadOp> op;
+    for (auto& o : readOps_) {
+      if (o->delivered && !o->readCalled) {
+        op = o;
+        break;
+      }
+    }
+    if (!op) {
+      fn(TP_CREATE_ERROR(LogicError, "read() without a preceding readDescriptor()"));
+      return;
+    }
+    op->readCalled = true;
+    op->fn = std::move(fn);
+    op->allocation = std::move(allocation);
+    const Descriptor& d = op->descriptor;
+    // checkAllocationCompatibility, tensorpipe/core/pipe_impl.cc:49-65
+    TP_THROW_ASSERT_IF(op->allocation.payloads.size() != d.payloads.size());
+    TP_THROW_ASSERT_IF(op->allocation.tensors.size() != d.tensors.size());
+    for (size_t i = 0; i < d.tensors.size(); ++i) {
+      if (d.tensors[i].targetDevice.has_value() && d.tensors[i].length > 0) {
+        TP_THROW_ASSERT_IF(
+            !(op->allocation.tensors[i].buffer.device() == *d.tensors[i].targetDevice));
+      }
+    }
+
+    // Payloads: the next messages on the connection.
+    auto self = shared_from_this();
+    bool claimed = false;
+    for (size_t i = 0; i < d.payloads.size(); ++i) {
+      if (d.payloads[i].length == 0) {
+        continue;
+      }
+      claimed = true;
+      ++op->pendingPayloads;
+      connection_->read(
+          op->allocation.payloads[i].data,
+          d.payloads[i].length,
+          [self, op](const Error& error, const void*, size_t) {
+            self->ctx_->defer([self, op, error] {
+              self->setError(error);
+              --op->pendingPayloads;
+              self->maybeFinishRead(op);
+            });
+          });
+    }
+    if (claimed) {
+      payloadsUnclaimed_ = false;
+      pumpPackets();
+    }
+
+    // Tell the sender where tensors without a target device ended up.
+    bool needsReply = false;
+    for (auto& t : d.tensors) {
+      needsReply |= !t.targetDevice.has_value();
+    }
+    std::vector<Device> targets;
+    for (size_t i = 0; i < d.tensors.size(); ++i) {
+      targets.push_back(op->allocation.tensors[i].buffer.device());
+    }
+    if (needsReply) {
+      WireWriter w;
+      w.u8(kDescriptorReply);
+      w.u32(static_cast<uint32_t>(targets.size()));
+      for (auto& dev : targets) {
+        putDevice(w, dev);
+      }
+      writeControl(std::move(w.bytes()));
+    }
+
+    // Tensors, grouped per channel in message order.
+    std::vector<std::pair<std::string, std::vector<size_t>>> groups;
+    for (size_t i = 0; i < d.tensors.size(); ++i) {
+      auto it = channelForDevicePair_.find({targets[i], d.tensors[i].sourceDevice});
+      if (it == channelForDevicePair_.end()) {
+        setError(TP_CREATE_ERROR(
+            LogicError,
+            "no channel between " + targets[i].toString() + " and " +
+                d.tensors[i].sourceDevice.toString()));
+        return;
+      }
+      addToGroup(groups, it->second, i);
+    }
+    for (auto& g : groups) {
+      auto& ch = channels_.at(g.first);
+      auto done = [self, op](const Error& error) {
+        self->ctx_->defer([self, op, error] {
+          self->setError(error);
+          --op->pendingRecvs;
+          self->maybeFinishRead(op);
+        });
+      };
+      auto* batched = dynamic_cast<channel::BatchedChannel*>(ch.get());
+      if (batched != nullptr && g.second.size() > 1) {
+        std::vector<channel::BatchEntry> entries;
+        for (size_t i : g.second) {
+          entries.push_back({op->allocation.tensors[i].buffer, d.tensors[i].length});
+        }
+        ++op->pendingRecvs;
+        batched->recvBatch(std::move(entries), done);
+      } else {
+        for (size_t i : g.second) {
+          ++op->pendingRecvs;
+          ch->recv(op->allocation.tensors[i].buffer, d.tensors[i].length, done);
+        }
+      }
+    }
+    maybeFinishRead(op);
+  }
+
+  void maybeFinishRead(const std::shared_ptr<ReadOp>& /*op*/) {
+    flushReads();
+  }
+
+  // Read callbacks fire in descriptor order, each once nothing of the op is in
+  // flight any more (successfully or not).
+  void flushReads() {
+    while (!readOps_.empty()) {
+      auto& front = readOps_.front();
+      if (!front->readCalled) {
+        if (error_) {
+          readOps_.pop_front(); // never claimed: a later read() fails on entry
+          continue;
+        }
+        break;
+      }
+      if (front->pendingPayloads != 0 || front->pendingRecvs != 0) {
+        break;
+      }
+      auto op = front;
+      readOps_.pop_front();
+      if (op->fn) {
+        TP_VLOG(3) << "Pipe " << id_ << " is calling a read callback (#" << op->seq << ")";
+        auto fn = std::move(op->fn);
+        fn(error_);
+      }
+    }
+  }
+
+  // ---- write side ---------------------------------------------------------
+
+  void writeFromLoop(Message message, Pipe::write_callback_fn fn) {
+    if (error_) {
+      fn(error_);
+      return;
+    }
+    auto op = std::make_shared<WriteOp>();
+    op->seq = nextWriteSeq_++;
+    op->message = std::move(message);
+    op->fn = std::move(fn);
+    for (auto& t : op->message.tensors) {
+      op->needsReply |= !t.targetDevice.has_value();
+    }
+    writeOps_.push_back(op);
+    advanceWrites();
+  }
+
+  void advanceWrites() {
+    if (!established_ || error_) {
+      return;
+    }
+    // Stage 1: descriptor + payloads, in order, as soon as the op exists.
+    for (auto& op : writeOps_) {
+      if (op->seq < nextDescriptorToWrite_) {
+        continue;
+      }
+      writeDescriptorAndPayloads(op);
+      nextDescriptorToWrite_ = op->seq + 1;
+    }
+    // Stage 2: tensors, strictly in op order (channels pair sends and recvs by
+    // position), each op as soon as its target devices are known.
+    for (auto& op : writeOps_) {
+      if (op->tensorsIssued) {
+        continue;
+      }
+      if (op->needsReply && !op->haveReply) {
+        break;
+      }
+      op->tensorsIssued = true;
+      issueTensors(op);
+      if (error_) {
+        return;
+      }
+    }
+    flushWrites();
+  }
+
+  void writeDescriptorAndPayloads(const std::shared_ptr<WriteOp>& op) {
+    const Message& m = op->message;
+    WireWriter w;
+    w.u8(kDescriptor);
+    w.str(m.metadata);
+    w.u32(static_cast<uint32_t>(m.payloads.size()));
+    for (auto& p : m.payloads) {
+      w.u64(p.length);
+      w.str(p.metadata);
+    }
+    w.u32(static_cast<uint32_t>(m.tensors.size()));
+    for (auto& t : m.tensors) {
+      w.u64(t.length);
+      putDevice(w, t.buffer.device());
+      w.u8(t.targetDevice.has_value() ? 1 : 0);
+      if (t.targetDevice.has_value()) {
+        putDevice(w, *t.targetDevice);
+      }
+      w.str(t.metadata);
+    }
+    auto self = shared_from_this();
+    auto done = [self, op](const Error& error) {
+      self->ctx_->defer([self, op, error] {
+        self->setError(error);
+        --op->pendingWrites;
+        self->flushWrites();
+      });
+    };
+    auto holder = std::make_shared<std::vector<uint8_t>>(std::move(w.bytes()));
+    ++op->pendingWrites;
+    connection_->write(holder->data(), holder->size(), [holder, done](const Error& e) { done(e); });
+    for (auto& p : m.payloads) {
+      if (p.length == 0) {
+        continue;
+      }
+      ++op->pendingWrites;
+      connection_->write(p.data, p.length, done);
+    }
+  }
+
+  void issueTensors(const std::shared_ptr<WriteOp>& op) {
+    const Message& m = op->message;
+    std::vector<std::pair<std::string, std::vector<size_t>>> groups;
+    for (size_t i = 0; i < m.tensors.size(); ++i) {
+      const Device src = m.tensors[i].buffer.device();
+      const Device dst =
+          m.tensors[i].targetDevice.has_value() ? *m.tensors[i].targetDevice : op->targetDevices[i];
+      auto it = channelForDevicePair_.find({src, dst});
+      if (it == channelForDevicePair_.end()) {
+        setError(TP_CREATE_ERROR(
+            LogicError, "no channel between " + src.toString() + " and " + dst.toString()));
+        return;
+      }
+      addToGroup(groups, it->second, i);
+    }
+    auto self = shared_from_this();
+    for (auto& g : groups) {
+      auto& ch = channels_.at(g.first);
+      auto done = [self, op](const Error& error) {
+        self->ctx_->defer([self, op, error] {
+          self->setError(error);
+          --op->pendingSends;
+          self->flushWrites();
+        });
+      };
+      auto* batched = dynamic_cast<channel::BatchedChannel*>(ch.get());
+      if (batched != nullptr && g.second.size() > 1) {
+        std::vector<channel::BatchEntry> entries;
+        for (size_t i : g.second) {
+          entries.push_back({m.tensors[i].buffer, m.tensors[i].length});
+        }
+        ++op->pendingSends;
+        batched->sendBatch(std::move(entries), done);
+      } else {
+        for (size_t i : g.second) {
+          ++op->pendingSends;
+          ch->send(m.tensors[i].buffer, m.tensors[i].length, done);
+        }
+      }
+    }
+  }
+
+  static void addToGroup(
+      std::vector<std::pair<std::string, std::vector<size_t>>>& groups,
+      const std::string& name,
+      size_t idx) {
+    for (auto& g : groups) {
+      if (g.first == name) {
+        g.second.push_back(idx);
+        return;
+      }
+    }
+    groups.emplace_back(name, std::vector<size_t>{idx});
+  }
+
+  // Write callbacks fire in the order the writes were issued.
+  void flushWrites() {
+    while (!writeOps_.empty()) {
+      auto& op = writeOps_.front();
+      const bool idle = op->pendingWrites == 0 && op->pendingSends == 0;
+      const bool complete = idle && op->tensorsIssued && op->seq < nextDescriptorToWrite_;
+      if (!(complete || (error_ && idle))) {
+        break;
+      }
+      auto done = writeOps_.front();
+      writeOps_.pop_front();
+      TP_VLOG(3) << "Pipe " << id_ << " is calling a write callback (#" << done->seq << ")";
+      auto fn = std::move(done->fn);
+      fn(error_);
+    }
+  }
+
+  // ---- errors ---------------------------------------------------------------
+
+  void setError(Error error) {
+    if (error_ || !error) {
+      return;
+    }
+    error_ = std::move(error);
+    TP_VLOG(2) << "Pipe " << id_ << " is handling error " << error_.what();
+    if (connection_) {
+      connection_->close();
+    }
+    for (auto& ch : channels_) {
+      ch.second->close();
+    }
+    if (listener_) {
+      for (uint64_t t : tokens_) {
+        listener_->unregisterConnectionRequest(t);
+      }
+    }
+    auto waiters = std::move(descriptorWaiters_);
+    descriptorWaiters_.clear();
+    for (auto& fn : waiters) {
+      fn(error_, Descriptor());
+    }
+    // Ops with transport/channel callbacks still in flight are flushed when
+    // those callbacks arrive (closing the connection and channels makes them
+    // arrive); ops that never started are flushed now.
+    flushReads();
+    flushWrites();
+    ctx_->unenroll(childKey_);
+  }
+
+  std::shared_ptr<ContextImpl> ctx_;
+  std::shared_ptr<ListenerImpl> listener_;
+  const std::string id_;
+  std::string remoteName_;
+  std::string transport_;
+  std::string addr_;
+  std::shared_ptr<transport::Connection> connection_;
+  std::vector<uint8_t> hello_;
+  const bool isClient_;
+  uint64_t childKey_{0};
+  Error error_;
+  bool established_{false};
+
+  std::unordered_map<std::string, std::shared_ptr<channel::Channel>> channels_;
+  DevicePairMap channelForDevicePair_;
+  std::map<std::string, std::vector<std::shared_ptr<transport::Connection>>> pendingChannelConns_;
+  size_t connectionsAwaited_{0};
+  std::vector<uint64_t> tokens_;
+
+  bool packetReadOutstanding_{false};
+  bool payloadsUnclaimed_{false};
+  uint64_t nextReadSeq_{0};
+  uint64_t nextWriteSeq_{0};
+  uint64_t nextDescriptorToWrite_{0};
+  std::deque<std::shared_ptr<ReadOp>> readOps_;
+  std::deque<std::shared_ptr<WriteOp>> writeOps_;
+  std::deque<Pipe::read_descriptor_callback_fn> descriptorWaiters_;
+};
+
+// ---------------------------------------------------------------------------
+
+void ListenerImpl::onConnection(std::shared_ptr<transport::Connection> conn) {
+  auto self = shared_from_this();
+  // The first packet says whether this is a new pipe or a connection a pipe
+  // asked for (tensorpipe/core/listener_impl.cc, "hello" handling).
+  auto* raw = conn.get();
+  raw->read([self, conn](const Error& error, const void* ptr, size_t len) mutable {
+    std::vector<uint8_t> bytes;
+    if (!error) {
+      bytes.assign(static_cast<const uint8_t*>(ptr), static_cast<const uint8_t*>(ptr) + len);
+    }
+    self->ctx_->defer([self, conn, error, bytes{std::move(bytes)}]() mutable {
+      if (self->error_ || error || bytes.empty()) {
+        return;
+      }
+      WireReader r(bytes.data(), bytes.size());
+      const uint8_t type = r.u8();
+      if (type == kHelloSpontaneous) {
+        auto impl = std::make_shared<PipeImpl>(
+            self->ctx_, self, self->ctx_->nextPipeId(), std::move(conn), std::move(bytes));
+        impl->init();
+        self->onPipeReady(std::make_shared<Pipe>(Pipe::ConstructorToken(), std::move(impl)));
+      } else if (type == kHelloRequested) {
+        const uint64_t token = r.u64();
+        auto it = self->requests_.find(token);
+        if (it == self->requests_.end()) {
+          TP_VLOG(1) << "Listener got a connection for unknown token " << token;
+          return;
+        }
+        auto fn = std::move(it->second);
+        self->requests_.erase(it);
+        fn(Error::kSuccess, std::move(conn));
+      }
+    });
+  });
+}
+
+std::shared_ptr<Listener> ContextImpl::listen(const std::vector<std::string>& urls) {
+  auto impl = std::make_shared<ListenerImpl>(shared_from_this(), urls);
+  impl->init();
+  return std::make_shared<Listener>(Listener::ConstructorToken(), std::move(impl));
+}
+
+std::shared_ptr<Pipe> ContextImpl::connect(const std::string& url, PipeOptions opts) {
+  std::string transport, addr;
+  TP_THROW_ASSERT_IF(!splitUrl(url, &transport, &addr));
+  auto impl = std::make_shared<PipeImpl>(
+      shared_from_this(), nextPipeId(), std::move(opts.remoteName_), transport, addr);
+  impl->init();
+  return std::make_shared<Pipe>(Pipe::ConstructorToken(), std::move(impl));
+}
+
+// ---- public wrappers --------------------------------------------------------
+
+Context::Context(ContextOptions opts) : impl_(std::make_shared<ContextImpl>(std::move(opts))) {}
+
+void Context::registerTransport(
+    int64_t priority,
+    std::string transport,
+    std::shared_ptr<transport::Context> context) {
+  impl_->registerTransport(priority, std::move(transport), std::move(context));
+}
+
+void Context::registerChannel(
+    int64_t priority,
+    std::string channel,
+    std::shared_ptr<channel::Context> context) {
+  impl_->registerChannel(priority, std::move(channel), std::move(context));
+}
+
+std::shared_ptr<Listener> Context::listen(const std::vector<std::string>& urls) {
+  return impl_->listen(urls);
+}
+
+std::shared_ptr<Pipe> Context::connect(const std::string& url, PipeOptions opts) {
+  return impl_->connect(url, std::move(opts));
+}
+
+void Context::close() {
+  impl_->close();
+}
+
+void Context::join() {
+  impl_->join();
+}
+
+Context::~Context() {
+  impl_->join();
+}
+
+Listener::Listener(ConstructorToken /*token*/, std::shared_ptr<ListenerImpl> impl)
+    : impl_(std::move(impl)) {}
+
+void Listener::accept(accept_callback_fn fn) {
+  impl_->accept(std::move(fn));
+}
+
+const std::map<std::string, std::string>& Listener::addresses() const {
+  return impl_->addresses();
+}
+
+const std::string& Listener::address(const std::string& transport) const {
+  const auto& a = impl_->addresses();
+  auto it = a.find(transport);
+  TP_THROW_ASSERT_IF(it == a.end());
+  return it->second;
+}
+
+std::string Listener::url(const std::string& transport) const {
+  return transport + "://" + address(transport);
+}
+
+void Listener::close() {
+  impl_->close();
+}
+
+Listener::~Listener() {
+  impl_->close();
+}
+
+Pipe::Pipe(ConstructorToken /*token*/, std::shared_ptr<PipeImpl> impl) : impl_(std::move(impl)) {}
+
+void Pipe::readDescriptor(read_descriptor_callback_fn fn) {
+  impl_->readDescriptor(std::move(fn));
+}
+
+void Pipe::read(Allocation allocation, read_callback_fn fn) {
+  impl_->read(std::move(allocation), std::move(fn));
+}
+
+void Pipe::write(Message message, write_callback_fn fn) {
+  impl_->write(std::move(message), std::move(fn));
+}
+
+const std::string& Pipe::getRemoteName() {
+  return impl_->remoteName();
+}
+
+void Pipe::close() {
+  impl_->close();
+}
+
+Pipe::~Pipe() {
+  impl_->close();
+}
+
+TP_AMD_NAMESPACE_END

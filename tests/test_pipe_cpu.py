@@ -1,0 +1,157 @@
+"""CPU-only tests of the pipe layer (shm transport, basic and xth channels):
+the reference's generic channel cases (tensorpipe/test/channel/channel_test.cc)
+driven through Pipe::write/read, plus close/error behaviour."""
+import numpy as np
+import pytest
+
+from tensorpipe_amd import pipe as tp
+
+
+@pytest.fixture
+def pair():
+    made = []
+
+    def make(channels="basic:0"):
+        server = tp.Context("server", channels=channels)
+        client = tp.Context("client", channels=channels)
+        listener = server.listen()
+        cpipe = client.connect(listener.url())
+        spipe = listener.accept()
+        made.append((cpipe, spipe, listener, client, server))
+        return cpipe, spipe
+
+    yield make
+    for cpipe, spipe, listener, client, server in made:
+        cpipe.destroy()
+        spipe.destroy()
+        listener.destroy()
+        client.destroy()
+        server.destroy()
+
+
+def _roundtrip(sender, receiver, arrays, payloads=(), targets=False):
+    tensors = [tp.make_tensor(a, target=(tp.CPU, 0) if targets else None) for a in arrays]
+    w = sender.write(tensors, payloads=payloads, metadata="meta")
+    d = receiver.read_descriptor()
+    assert d.metadata.decode() == "meta"
+    assert d.num_tensors == len(arrays) and d.num_payloads == len(payloads)
+    outs = [np.full(d.tensor_lengths[i], 0xEE, np.uint8) for i in range(d.num_tensors)]
+    pouts = [np.zeros(d.payload_lengths[i], np.uint8) for i in range(d.num_payloads)]
+    r = receiver.read([tp.make_tensor(o) for o in outs], pouts)
+    r.wait()
+    w.wait()
+    return outs, pouts
+
+
+@pytest.mark.parametrize("channels", ["basic:0", "xth:5,basic:0"])
+def test_client_to_server_and_back(pair, channels):
+    cpipe, spipe = pair(channels)
+    assert spipe.remote_name() == "client"
+    data = np.arange(256, dtype=np.uint8)
+    outs, _ = _roundtrip(cpipe, spipe, [data])
+    assert (outs[0] == data).all()
+    outs, _ = _roundtrip(spipe, cpipe, [data[::-1].copy()])
+    assert (outs[0] == data[::-1]).all()
+
+
+@pytest.mark.parametrize("channels", ["basic:0", "xth:5,basic:0"])
+@pytest.mark.parametrize("targets", [False, True])
+def test_send_multiple_tensors(pair, channels, targets):
+    cpipe, spipe = pair(channels)
+    n = 256 * 1024
+    src = (np.arange(n) % 256).astype(np.uint8)
+    outs, _ = _roundtrip(cpipe, spipe, [src] * 20, targets=targets)
+    for o in outs:
+        assert (o == src).all()
+
+
+def test_payloads_and_empty_tensors(pair):
+    cpipe, spipe = pair()
+    a, z, b = np.array([7], np.uint8), np.zeros(0, np.uint8), np.array([9], np.uint8)
+    outs, pouts = _roundtrip(cpipe, spipe, [a, z, b], payloads=[b"payload #0", b"", b"payload #2"])
+    assert outs[0][0] == 7 and outs[1].size == 0 and outs[2][0] == 9
+    assert bytes(pouts[0]) == b"payload #0" and bytes(pouts[2]) == b"payload #2"
+    outs, _ = _roundtrip(cpipe, spipe, [z])
+    assert outs[0].size == 0
+    outs, pouts = _roundtrip(cpipe, spipe, [], payloads=[b"only payload"])
+    assert bytes(pouts[0]) == b"only payload"
+
+
+def test_large_message_exceeds_ring(pair):
+    cpipe, spipe = pair()
+    rng = np.random.default_rng(0)
+    big = rng.integers(0, 256, 9 * 1024 * 1024 + 13, dtype=np.uint8)
+    outs, _ = _roundtrip(cpipe, spipe, [big])
+    assert (outs[0] == big).all()
+
+
+def test_both_ways_interleaved(pair):
+    cpipe, spipe = pair()
+    a = np.full(100000, 1, np.uint8)
+    b = np.full(50000, 2, np.uint8)
+    w1 = cpipe.write([tp.make_tensor(a)])
+    w2 = spipe.write([tp.make_tensor(b)])
+    d1 = spipe.read_descriptor()
+    d2 = cpipe.read_descriptor()
+    o1 = np.zeros(d1.tensor_lengths[0], np.uint8)
+    o2 = np.zeros(d2.tensor_lengths[0], np.uint8)
+    r1 = spipe.read([tp.make_tensor(o1)])
+    r2 = cpipe.read([tp.make_tensor(o2)])
+    for op in (r1, r2, w1, w2):
+        op.wait()
+    assert (o1 == 1).all() and (o2 == 2).all()
+
+
+def test_many_messages_in_order(pair):
+    cpipe, spipe = pair()
+    sources = [np.full(1000, i, np.uint8) for i in range(50)]  # must outlive the writes
+    writes = [cpipe.write([tp.make_tensor(sources[i])], metadata=str(i)) for i in range(50)]
+    for i in range(50):
+        d = spipe.read_descriptor()
+        assert d.metadata.decode() == str(i)
+        o = np.zeros(1000, np.uint8)
+        spipe.read([tp.make_tensor(o)]).wait()
+        assert (o == i).all()
+    for w in writes:
+        w.wait()
+
+
+def test_close_fails_pending_and_future_ops(pair):
+    cpipe, spipe = pair()
+    # make sure the pipe is established first
+    _roundtrip(cpipe, spipe, [np.arange(10, dtype=np.uint8)])
+    cpipe.close()
+    with pytest.raises(tp.PipeError):
+        cpipe.write([tp.make_tensor(np.zeros(10, np.uint8))]).wait()
+    # the peer notices the closed connection
+    with pytest.raises(tp.PipeError):
+        spipe.read_descriptor(timeout_ms=5000)
+
+
+def test_context_close_fails_pipes(pair):
+    cpipe, spipe = pair()
+    _roundtrip(cpipe, spipe, [np.arange(10, dtype=np.uint8)])
+    # last tuple created by the fixture holds the contexts
+    with pytest.raises(tp.PipeError):
+        # closing the remote context makes our reads fail
+        import threading
+
+        t = threading.Timer(0.2, lambda: spipe.close())
+        t.start()
+        cpipe.read_descriptor(timeout_ms=5000)
+
+
+def test_unknown_channel_and_missing_gpu():
+    with pytest.raises(tp.PipeError):
+        tp.Context("x", channels="nope:0")
+    # Without a GPU the HIP channels are not viable and are skipped, like a
+    # reference context skips a non-viable channel (core/context_impl.cc:89-110).
+    import torch
+
+    ctx = tp.Context("y", channels="basic:0,hip_xth:10,hip_ipc:11,hip_basic:12")
+    assert ctx.has_channel("basic")
+    if not torch.cuda.is_available():
+        assert not ctx.has_channel("hip_xth")
+        assert not ctx.has_channel("hip_ipc")
+        assert not ctx.has_channel("hip_basic")
+    ctx.destroy()
