@@ -1,0 +1,421 @@
+#!/usr/bin/env python3
+"""Benchmark of the HIP device channels on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+The headline line is BASELINE.json's configs[1]: same-process device-to-device
+(hip_xth channel), one 64 MiB uint8 tensor, two connected pipes in one process,
+K write/read steps after W warm-up steps, received bytes compared with the sent
+ones. One step = Pipe::write + Pipe::readDescriptor + Pipe::read of one message
+and a synchronisation of the receive stream. `value` is payload bytes delivered
+per second with the tensors already resident in HBM.
+
+The other configurations (cross-process IPC size sweep and 4 KiB round trip,
+host-staged 256 MiB, 256-tensor RPC-style message) and the CPU baseline are
+reported under "extra" / "cpu_baseline" of the same JSON line.
+"""
+import argparse
+import json
+import os
+import subprocess
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+PCIE_PEAK_GBPS = 63.0
+MIB = 1 << 20
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def profiled(fn, max_launches):
+    """Run fn() with per-launch device timing of the copy kernels switched on."""
+    import ctypes
+
+    from tensorpipe_amd import _native
+
+    lib = _native.tphip()
+    _native.check(lib.tphip_profile_start(0, max_launches), "profile_start")
+    out = fn()
+    n, ms, nbytes = ctypes.c_uint32(), ctypes.c_double(), ctypes.c_uint64()
+    _native.check(lib.tphip_profile_stop(0, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(nbytes)),
+                  "profile_stop")
+    return out, n.value, ms.value, nbytes.value
+
+
+def make_pair(channels):
+    from tensorpipe_amd import pipe as tp
+
+    server = tp.Context("bench_server", channels=channels)
+    client = tp.Context("bench_client", channels=channels)
+    listener = server.listen()
+    cpipe = client.connect(listener.url())
+    spipe = listener.accept()
+    return cpipe, spipe, listener, client, server
+
+
+def destroy(objs):
+    for o in objs:
+        o.destroy()
+
+
+def bench_d2d(steps, warmup):
+    """configs[1]: hip_xth, 1 x 64 MiB uint8, same process."""
+    import torch
+
+    from tensorpipe_amd import datagen, hip
+    from tensorpipe_amd import pipe as tp
+
+    nbytes = 64 * MIB
+    host = datagen.uniform_u8(datagen.SEED_BASE + 2, nbytes)
+    src = torch.from_numpy(host).cuda()
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    objs = make_pair("basic:0,hip_xth:10")
+    cpipe, spipe = objs[0], objs[1]
+    send_stream, recv_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    st = [tp.make_tensor(src, stream=send_stream, target=(tp.HIP, 0))]
+    rt = [tp.make_tensor(dst, stream=recv_stream)]
+    torch.cuda.synchronize()
+
+    # warm-up steps, then a full compare of the first transfer
+    tp.bench_transfer(cpipe, spipe, st, rt, warmup=0, iters=max(warmup, 1))
+    assert torch.equal(src, dst), "received bytes differ from sent bytes"
+    dst.zero_()
+    torch.cuda.synchronize()
+
+    (per_us, total_s), launches, kernel_ms, kernel_bytes = profiled(
+        lambda: tp.bench_transfer(cpipe, spipe, st, rt, warmup=0, iters=steps), steps + 8)
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst), "received bytes differ from sent bytes after the timed loop"
+    assert launches == steps and kernel_bytes == steps * nbytes, (launches, kernel_bytes)
+
+    # practical ceiling: the runtime's own D2D copy of the same size, same timing method
+    e0, e1 = hip.TimedEvent(), hip.TimedEvent()
+    for _ in range(5):
+        hip.memcpy_async(dst, src, nbytes, stream=recv_stream)
+    e0.record(recv_stream)
+    for _ in range(50):
+        hip.memcpy_async(dst, src, nbytes, stream=recv_stream)
+    e1.record(recv_stream)
+    e1.synchronize()
+    memcpy_us = e0.elapsed_ms(e1) / 50 * 1e3
+    destroy(objs)
+
+    kernel_us = kernel_ms / launches * 1e3
+    achieved = 2.0 * nbytes / (kernel_us * 1e-6) / 1e9
+    per_us.sort()
+    return {
+        "value": nbytes * steps / total_s / 1e9,
+        "ms_per_step": total_s / steps * 1e3,
+        "step_p50_us": float(per_us[int(0.5 * len(per_us))]),
+        "roofline": {
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "kernel": "tphip::single_copy_kernel<4, true>", "kernel_avg_us": kernel_us,
+            "algorithmic_bytes_per_launch": 2 * nbytes,
+        },
+        "hipMemcpyAsync_d2d_us": memcpy_us,
+        "hipMemcpyAsync_d2d_hbm_GBps": 2.0 * nbytes / (memcpy_us * 1e-6) / 1e9,
+    }
+
+
+def bench_rpc_message(messages=100, warmup=5):
+    """configs[4]: 256 fp16 tensors, log-uniform sizes, 4 KiB payload, one launch per message."""
+    import numpy as np
+    import torch
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    sizes = [int(s) for s in datagen.loguniform_sizes(datagen.SEED_BASE + 5, 256, 4 * MIB, 256)]
+    total = sum(sizes)
+    arena_src = torch.empty(total + 16 * len(sizes), dtype=torch.uint8, device="cuda")
+    arena_dst = torch.zeros_like(arena_src)
+    st, rt, off = [], [], 0
+    for i, n in enumerate(sizes):
+        h = datagen.normal(1000 + i, n // 2, "f16", sigma=0.02).view(np.uint8)
+        arena_src[off:off + n] = torch.from_numpy(h).cuda()
+        st.append(tp.make_tensor(arena_src.data_ptr() + off, nbytes=n, device=tp.HIP,
+                                 target=(tp.HIP, 0)))
+        rt.append(tp.make_tensor(arena_dst.data_ptr() + off, nbytes=n, device=tp.HIP))
+        off += (n + 15) // 16 * 16
+    payload = datagen.bench_pattern(4096)
+    pout = np.zeros(4096, np.uint8)
+    objs = make_pair("basic:0,hip_xth:10")
+    torch.cuda.synchronize()
+    tp.bench_transfer(objs[0], objs[1], st, rt, payloads=[payload], recv_payloads=[pout],
+                      warmup=0, iters=warmup)
+    (per_us, total_s), launches, kernel_ms, _ = profiled(
+        lambda: tp.bench_transfer(objs[0], objs[1], st, rt, payloads=[payload],
+                                  recv_payloads=[pout], warmup=0, iters=messages), messages + 8)
+    torch.cuda.synchronize()
+    ok = bool(torch.equal(arena_src[:off], arena_dst[:off])) and bytes(pout) == bytes(payload)
+    destroy(objs)
+    per_us.sort()
+    kernel_us = kernel_ms / max(launches, 1) * 1e3
+    return {
+        "tensors": len(sizes), "total_bytes": total, "messages": messages,
+        "launches_per_message": launches / messages,
+        "payload_GBps": total * messages / total_s / 1e9,
+        "message_p50_us": float(per_us[int(0.5 * len(per_us))]),
+        "kernel_avg_us": kernel_us,
+        "kernel_hbm_GBps": 2.0 * total / (kernel_us * 1e-6) / 1e9,
+        "kernel_hbm_frac": 2.0 * total / (kernel_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+        "byte_exact": ok,
+    }
+
+
+class PeerRun:
+    """A bench_peer child process connected through one pipe."""
+
+    def __init__(self, channels, env=None):
+        from tensorpipe_amd import pipe as tp
+
+        self.tp = tp
+        saved = {k: os.environ.get(k) for k in (env or {})}
+        os.environ.update(env or {})
+        try:
+            self.ctx = tp.Context("bench_main", channels=channels)
+        finally:
+            for k, v in saved.items():
+                if v is None:
+                    os.environ.pop(k, None)
+                else:
+                    os.environ[k] = v
+        self.listener = self.ctx.listen()
+        child_env = dict(os.environ)
+        child_env.update(env or {})
+        child_env["PYTHONPATH"] = ROOT + os.pathsep + child_env.get("PYTHONPATH", "")
+        self.proc = subprocess.Popen(
+            [sys.executable, "-m", "tensorpipe_amd.bench_peer", self.listener.url(), channels],
+            env=child_env, cwd=ROOT)
+        self.pipe = self.listener.accept(180000)
+
+    def pingpong(self, send, recv, sizes, device, warmup, iters, payloads=(), recv_payloads=()):
+        cmd = {"op": "pingpong", "sizes": sizes, "device": device, "warmup": warmup,
+               "iters": iters, "payload": payloads[0].nbytes if payloads else 0}
+        self.pipe.write([], metadata=json.dumps(cmd)).wait()
+        d = self.pipe.read_descriptor(120000)
+        self.pipe.read([], []).wait()
+        assert d.metadata.decode() == "ready"
+        return self.tp.bench_pingpong(self.pipe, True, send, recv, payloads=payloads,
+                                      recv_payloads=recv_payloads, warmup=warmup, iters=iters)
+
+    def close(self):
+        try:
+            self.pipe.write([], metadata=json.dumps({"op": "quit"})).wait(10000)
+            self.proc.wait(30)
+        finally:
+            if self.proc.poll() is None:
+                self.proc.kill()
+            destroy([self.pipe, self.listener, self.ctx])
+
+
+def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
+    """configs[2]: hip_ipc, one fp32 tensor, 4 KiB * 4^k up to 1 GiB, ping-pong with a peer process."""
+    import numpy as np
+    import torch
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    peer = PeerRun("basic:0,hip_ipc:11")
+    out = {"sizes": {}}
+    try:
+        size = 4096
+        while size <= max_bytes:
+            sample = min(size, 16 * MIB)  # seeded values in the first 16 MiB, repeated beyond
+            host = datagen.normal(datagen.SEED_BASE + 3, sample // 4, "f32").view(np.uint8)
+            src = torch.from_numpy(host).cuda().repeat(size // sample)
+            dst = torch.zeros(size, dtype=torch.uint8, device="cuda")
+            st = [tp.make_tensor(src, target=(tp.HIP, 0))]
+            rt = [tp.make_tensor(dst)]
+            torch.cuda.synchronize()
+            n_it = iters if size <= 256 * MIB else max(iters // 4, 10)
+            per_us, total_s = peer.pingpong(st, rt, [size], "gpu", warmup, n_it)
+            torch.cuda.synchronize()
+            ok = bool(torch.equal(src, dst))
+            per_us.sort()
+            p50 = float(per_us[int(0.5 * len(per_us))])
+            # one round trip carries the tensor once in each direction
+            gbps = 2.0 * size / (p50 * 1e-6) / 1e9
+            out["sizes"][str(size)] = {
+                "rtt_p50_us": p50, "payload_GBps": gbps, "hbm_GBps": 2 * gbps,
+                "hbm_frac": 2 * gbps / HBM_PEAK_GBPS, "byte_exact": ok, "iters": n_it}
+            log(f"  ipc {size:>11d} B  rtt p50 {p50:10.1f} us  payload {gbps:8.1f} GB/s  exact={ok}")
+            del src, dst
+            size *= 4
+        out["rtt_4KiB_p50_us"] = out["sizes"]["4096"]["rtt_p50_us"]
+    finally:
+        peer.close()
+    return out
+
+
+def bench_staged(iters=50, warmup=3, nbytes=256 * MIB):
+    """configs[3]: hip_basic, 256 MiB bf16, GPU -> pinned -> shm -> pinned -> GPU, 4-deep ring."""
+    import numpy as np
+    import torch
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    out = {}
+    sample = 16 * MIB
+    host = datagen.normal(datagen.SEED_BASE + 4, sample // 2, "bf16").view(np.uint8)
+    src = torch.from_numpy(host).cuda().repeat(nbytes // sample)
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    for chunk in (1 * MIB, 4 * MIB):
+        env = {"TP_HIP_BASIC_SLOT_BYTES": str(chunk), "TP_HIP_BASIC_NUM_SLOTS": "4"}
+        peer = PeerRun("basic:0,hip_basic:10", env=env)
+        try:
+            dst.zero_()
+            st = [tp.make_tensor(src, target=(tp.HIP, 0))]
+            rt = [tp.make_tensor(dst)]
+            torch.cuda.synchronize()
+            per_us, total_s = peer.pingpong(st, rt, [nbytes], "gpu", warmup, iters)
+            torch.cuda.synchronize()
+            ok = bool(torch.equal(src, dst))
+            per_us.sort()
+            p50 = float(per_us[int(0.5 * len(per_us))])
+            # a round trip is two staged transfers back to back
+            gbps = 2.0 * nbytes / (p50 * 1e-6) / 1e9
+            out[f"chunk_{chunk // MIB}MiB"] = {
+                "rtt_p50_ms": p50 / 1e3, "payload_GBps": gbps, "pcie_frac": gbps / PCIE_PEAK_GBPS,
+                "byte_exact": ok, "iters": iters}
+            log(f"  staged chunk {chunk // MIB} MiB: {gbps:.2f} GB/s ({gbps / PCIE_PEAK_GBPS:.1%} of PCIe) exact={ok}")
+        finally:
+            peer.close()
+    return out
+
+
+def bench_link_ceiling(nbytes=256 * MIB):
+    """Pinned D2H / H2D: the copy kernel against the runtime's copy engine path."""
+    import torch
+
+    from tensorpipe_amd import hip
+
+    dev = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_()
+    pinned = torch.empty(nbytes, dtype=torch.uint8).pin_memory()
+    out = {}
+    for name, fn in (
+        ("d2h_kernel", lambda: hip.copy(pinned, dev, nbytes)),
+        ("d2h_hipMemcpyAsync", lambda: hip.memcpy_async(pinned, dev, nbytes)),
+        ("h2d_kernel", lambda: hip.copy(dev, pinned, nbytes)),
+        ("h2d_hipMemcpyAsync", lambda: hip.memcpy_async(dev, pinned, nbytes)),
+    ):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = hip.TimedEvent(), hip.TimedEvent()
+        e0.record()
+        for _ in range(5):
+            fn()
+        e1.record()
+        e1.synchronize()
+        out[name + "_GBps"] = nbytes / (e0.elapsed_ms(e1) / 5 * 1e-3) / 1e9
+    return out
+
+
+def cpu_baseline():
+    """The CPU port of the reference's shm + basic path (oracle/), on this box's host cores."""
+    exe = os.path.join(ROOT, "oracle", "cpu_shm_basic")
+    if not os.path.exists(exe):
+        return {"error": "oracle/cpu_shm_basic not built"}
+
+    def run(tensor, payload, warmup, iters):
+        r = subprocess.run([exe, str(tensor), str(payload), str(warmup), str(iters)],
+                           stdout=subprocess.PIPE, text=True, timeout=300)
+        return json.loads(r.stdout.strip().splitlines()[-1])
+
+    same = run(64 * MIB, 0, 2, 40)        # the headline workload's tensor, bounded sample
+    cfg1 = run(1 * MIB, 64, 5, 1000)      # configs[0]
+    rtt = run(4096, 64, 5, 2000)          # 4 KiB round trip
+    ref = None
+    ref_exe = os.path.join(ROOT, "oracle", "_ref", "ref_pipe_bench")
+    if os.path.exists(ref_exe):
+        try:
+            r = subprocess.run([ref_exe], stdout=subprocess.PIPE, text=True, timeout=300)
+            ref = json.loads(r.stdout.strip().splitlines()[-1])
+        except Exception as e:  # the prebuilt reference is optional
+            ref = {"error": repr(e)}
+    return {
+        "value": same["payload_GBps"], "unit": "GB/s", "cores": 2, "kind": "port",
+        "sample": "40 round trips of one 64 MiB CPU tensor through the shm ring + basic channel "
+                  "port (80 transfers), 2 processes x 1 busy-polling thread",
+        "config1_1MiB_rtt_p50_us": cfg1["rtt_p50_us"], "config1_payload_GBps": cfg1["payload_GBps"],
+        "rtt_4KiB_p50_us": rtt["rtt_p50_us"],
+        "host_cpus": os.cpu_count(),
+        "reference_prebuilt": ref,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-extras", action="store_true",
+                    help="only the headline configuration and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; every configuration of the device "
+                 "channels is single-GPU (run with --gpus 1)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    from tensorpipe_amd import _native
+
+    _native.tphip()  # fails loudly if the HIP library is not built
+
+    t_start = time.time()
+    log("[bench] same-process D2D, 64 MiB (headline)")
+    d2d = bench_d2d(args.steps, args.warmup)
+    extra = {
+        "d2d_step_p50_us": d2d["step_p50_us"],
+        "hipMemcpyAsync_d2d_us": d2d["hipMemcpyAsync_d2d_us"],
+        "hipMemcpyAsync_d2d_hbm_GBps": d2d["hipMemcpyAsync_d2d_hbm_GBps"],
+    }
+    if not args.skip_extras:
+        log("[bench] many-tensor message (256 tensors, one launch per message)")
+        extra["rpc_message"] = bench_rpc_message()
+        log("[bench] cross-process IPC sweep")
+        extra["ipc"] = bench_ipc()
+        log("[bench] host-staged 256 MiB")
+        extra["staged"] = bench_staged()
+        extra["host_link"] = bench_link_ceiling()
+    log("[bench] CPU baseline (port of shm + basic)")
+    cpu = cpu_baseline()
+    extra["bench_wall_s"] = time.time() - t_start
+
+    line = {
+        "metric": "payload GB/s, same-process D2D channel (fraction of HBM roofline under roofline.frac; "
+                  "p50 RTT at 4 KiB under extra.ipc)",
+        "value": d2d["value"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": d2d["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic (seeded uniform bytes)",
+        "config": {"workload": "configs[1]: hip_xth same-process D2D, 1 x 64 MiB uint8 tensor, "
+                               "two connected pipes in one process, write/read per step, byte-exact"},
+        "roofline": d2d["roofline"],
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

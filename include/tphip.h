@@ -148,6 +148,16 @@ int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream
 int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                              int unroll, uint32_t blocks, int nontemporal);
 
+/* Device-time measurement of the copy launches themselves. After
+ * tphip_profile_start every tphip_batched_copy / tphip_copy launch on `dev` is
+ * bracketed by two timing events on its own stream (up to `max_launches`, the
+ * rest are counted but not timed); tphip_profile_stop waits for them and
+ * reports how many launches were timed, their summed device time and the
+ * payload bytes they moved. Profiling serialises nothing and is off by
+ * default. The reference has no counterpart (it has no kernels). */
+int tphip_profile_start(int dev, uint32_t max_launches);
+int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* total_bytes);
+
 /* Runtime copy engine path (hipMemcpyAsync), kept only as the A/B comparison
  * for the kernel-driven copies; never used by the channels' data path. */
 int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream);

@@ -74,6 +74,9 @@ def tphip():
         lib.tphip_batched_copy.argtypes = [i32, P(CopyDesc), u32, vp]
         lib.tphip_copy.argtypes = [i32, vp, vp, u64, vp]
         lib.tphip_batched_copy_tuned.argtypes = [i32, P(CopyDesc), u32, vp, i32, u32, i32]
+        lib.tphip_profile_start.argtypes = [i32, u32]
+        lib.tphip_profile_stop.argtypes = [i32, P(u32), P(ctypes.c_double), P(u64)]
+        lib.tphip_mem_buffer_id.argtypes = [vp, P(u64)]
         lib.tphip_memcpy_async.argtypes = [i32, vp, vp, u64, vp]
         lib.tphip_fill.argtypes = [i32, vp, i32, u64, vp]
         lib.tphip_test_slow_kernel.argtypes = [i32, vp, u64, vp]

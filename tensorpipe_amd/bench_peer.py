@@ -1,0 +1,49 @@
+"""Echo side of the two-process benchmark configurations.
+
+    python -m tensorpipe_amd.bench_peer URL CHANNELS
+
+Connects to URL, then serves commands that arrive as the metadata (JSON) of
+tensor-less messages: {"op": "pingpong", "sizes": [...], "device": "gpu"|"cpu",
+"warmup": W, "iters": K} allocates buffers, answers "ready" and runs the native
+echo loop; {"op": "quit"} ends the process."""
+import json
+import sys
+
+
+def main(url, channels):
+    import numpy as np
+    import torch
+
+    from tensorpipe_amd import pipe as tp
+
+    ctx = tp.Context("bench_peer", channels=channels)
+    p = ctx.connect(url)
+    while True:
+        d = p.read_descriptor(timeout_ms=600000)
+        p.read([], []).wait()
+        cmd = json.loads(d.metadata.decode())
+        if cmd["op"] == "quit":
+            break
+        if cmd["op"] == "pingpong":
+            bufs, tensors = [], []
+            for n in cmd["sizes"]:
+                if cmd["device"] == "gpu":
+                    b = torch.zeros(max(n, 1), dtype=torch.uint8, device="cuda")
+                    tensors.append(tp.make_tensor(b, nbytes=n, target=(tp.HIP, 0)))
+                else:
+                    b = np.zeros(max(n, 1), np.uint8)
+                    tensors.append(tp.make_tensor(b, nbytes=n, target=(tp.CPU, 0)))
+                bufs.append(b)
+            payload = np.zeros(cmd.get("payload", 0), np.uint8)
+            payloads = [payload] if payload.size else []
+            if cmd["device"] == "gpu":
+                torch.cuda.synchronize()
+            p.write([], metadata="ready").wait()
+            tp.bench_pingpong(p, False, tensors, tensors, payloads=payloads,
+                              recv_payloads=payloads, warmup=cmd["warmup"], iters=cmd["iters"])
+    p.destroy()
+    ctx.destroy()
+
+
+if __name__ == "__main__":
+    main(sys.argv[1], sys.argv[2])

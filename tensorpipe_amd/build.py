@@ -58,7 +58,7 @@ HOST_SOURCES = [
     "tensorpipe/core/core.cc",
     "capi/tensorpipe_c.cc",
 ]
-HOST_FLAGS = ["-O2", "-g", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread"]
 
 
 def build_host(jobs=8):

@@ -50,6 +50,41 @@ struct DeviceState {
   bool slotUsed[kPlanSlots]{};
   uint32_t nextSlot{0};
   std::mutex mutex;
+  // Launch profiling (tphip_profile_start/stop).
+  std::mutex profMutex;
+  bool profiling{false};
+  uint32_t profMax{0};
+  uint64_t profBytes{0};
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> profEvents;
+};
+
+// Brackets one launch with timing events while profiling is on.
+class ProfileScope {
+ public:
+  ProfileScope(DeviceState& st, hipStream_t stream, uint64_t bytes) : stream_(stream) {
+    std::lock_guard<std::mutex> lock(st.profMutex);
+    if (!st.profiling || st.profEvents.size() >= st.profMax) {
+      return;
+    }
+    if (hipEventCreate(&begin_) != hipSuccess || hipEventCreate(&end_) != hipSuccess) {
+      (void)hipGetLastError();
+      begin_ = end_ = nullptr;
+      return;
+    }
+    st.profEvents.emplace_back(begin_, end_);
+    st.profBytes += bytes;
+    (void)hipEventRecord(begin_, stream_);
+  }
+  ~ProfileScope() {
+    if (end_ != nullptr) {
+      (void)hipEventRecord(end_, stream_);
+    }
+  }
+
+ private:
+  hipStream_t stream_;
+  hipEvent_t begin_{nullptr};
+  hipEvent_t end_{nullptr};
 };
 
 DeviceState gDevices[kMaxDevices];
@@ -201,6 +236,7 @@ int copySingle(DeviceState& st, const tphip_copy_desc& d, hipStream_t stream, in
   const uint32_t grid = pickBlocks(st, nslices, 1, blocks);
   const char* src = static_cast<const char*>(d.src);
   char* dst = static_cast<char*>(d.dst);
+  ProfileScope prof(st, stream, d.bytes);
   return nt ? launchSingle<true>(unroll, grid, stream, src, dst, d.bytes)
             : launchSingle<false>(unroll, grid, stream, src, dst, d.bytes);
 }
@@ -260,8 +296,16 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     const size_t lds = (size_t(n) + 1) * sizeof(uint32_t);
     const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
     const tphip_copy_desc* dDescs = reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes);
-    int rc = nt ? launchTable<true>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices)
-                : launchTable<false>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices);
+    int rc;
+    {
+      uint64_t payload = 0;
+      for (uint32_t i = 0; i < n; ++i) {
+        payload += table[i].bytes;
+      }
+      ProfileScope prof(st, stream, payload);
+      rc = nt ? launchTable<true>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices)
+              : launchTable<false>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices);
+    }
     if (rc != 0) {
       return rc;
     }
@@ -650,6 +694,65 @@ int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream
 int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                              int unroll, uint32_t blocks, int nontemporal) {
   return batchedCopyImpl(dev, table, n, stream, unroll, blocks, nontemporal);
+}
+
+int tphip_profile_start(int dev, uint32_t max_launches) {
+  DeviceState* st = nullptr;
+  int rc = getDevice(dev, &st);
+  if (rc != 0) {
+    return rc;
+  }
+  std::lock_guard<std::mutex> lock(st->profMutex);
+  for (auto& p : st->profEvents) {
+    (void)hipEventDestroy(p.first);
+    (void)hipEventDestroy(p.second);
+  }
+  st->profEvents.clear();
+  st->profEvents.reserve(max_launches);
+  st->profBytes = 0;
+  st->profMax = max_launches;
+  st->profiling = true;
+  return 0;
+}
+
+int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* total_bytes) {
+  DeviceState* st = nullptr;
+  int rc = getDevice(dev, &st);
+  if (rc != 0) {
+    return rc;
+  }
+  std::lock_guard<std::mutex> lock(st->profMutex);
+  st->profiling = false;
+  double sum = 0;
+  uint32_t count = 0;
+  int err = 0;
+  for (auto& p : st->profEvents) {
+    hipError_t e = hipEventSynchronize(p.second);
+    float ms = 0;
+    if (e == hipSuccess) {
+      e = hipEventElapsedTime(&ms, p.first, p.second);
+    }
+    if (e == hipSuccess) {
+      sum += ms;
+      ++count;
+    } else {
+      (void)hipGetLastError();
+      err = static_cast<int>(e);
+    }
+    (void)hipEventDestroy(p.first);
+    (void)hipEventDestroy(p.second);
+  }
+  st->profEvents.clear();
+  if (launches) {
+    *launches = count;
+  }
+  if (total_ms) {
+    *total_ms = sum;
+  }
+  if (total_bytes) {
+    *total_bytes = st->profBytes;
+  }
+  return count > 0 ? 0 : err;
 }
 
 int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {

@@ -324,7 +324,7 @@ def test_ipc_refuses_same_process():
 
 def test_basic_staged_sizes(oracle, basic_peer):
     for k, n in enumerate([1024, 1 << 20, (1 << 20) + 1, (5 << 20) + 3, 40 << 20, 1, 0]):
-        host = datagen.normal(datagen.SEED_BASE + 4 + k, max(n // 2, 1), "bf16").view(np.uint8)
+        host = datagen.normal(datagen.SEED_BASE + 4 + k, max((n + 1) // 2, 1), "bf16").view(np.uint8)
         src = _gpu(host)
         outs, _ = basic_peer.echo([tp.make_tensor(src, nbytes=n, target=(tp.HIP, 0))], "gpu")
         ref = np.full(n, FILL, np.uint8)
