@@ -117,7 +117,7 @@ def bench_d2d(steps, warmup):
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-            "kernel": "tphip::single_copy_kernel<4, true>", "kernel_avg_us": kernel_us,
+            "kernel": "tphip::single_copy_kernel<4, 2>", "kernel_avg_us": kernel_us,
             "algorithmic_bytes_per_launch": 2 * nbytes,
         },
         "hipMemcpyAsync_d2d_us": memcpy_us,

@@ -92,6 +92,8 @@ int tphip_host_free(void* host_ptr);
 int tphip_stream_create(int dev, void** stream);
 int tphip_stream_destroy(int dev, void* stream);
 int tphip_stream_sync(int dev, void* stream);
+/* *done = 1 when everything enqueued on `stream` so far has finished. */
+int tphip_stream_query(int dev, void* stream, int* done);
 
 /* interprocess != 0 creates an event exportable with tphip_ipc_event_export.
  * Timing is always disabled. Replaces CudaEvent,
@@ -143,8 +145,9 @@ int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* 
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream);
 
 /* Same as tphip_batched_copy with explicit launch shape, for tuning sweeps:
- * `unroll` in {1,2,4,8} 16-byte vectors per lane per slice, `blocks` workgroups
- * of 256 threads (0 = default), `nontemporal` 0/1. */
+ * `unroll` in {1,2,4,8} 16-byte vectors in flight per lane, `blocks` workgroups
+ * of 256 threads (0 = default: one per CU), `nontemporal` a mask (bit 0 =
+ * nontemporal loads, bit 1 = nontemporal stores; the default is 3). */
 int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                              int unroll, uint32_t blocks, int nontemporal);
 

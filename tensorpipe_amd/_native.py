@@ -58,6 +58,7 @@ def tphip():
         lib.tphip_stream_create.argtypes = [i32, P(vp)]
         lib.tphip_stream_destroy.argtypes = [i32, vp]
         lib.tphip_stream_sync.argtypes = [i32, vp]
+        lib.tphip_stream_query.argtypes = [i32, vp, P(i32)]
         lib.tphip_event_create.argtypes = [i32, i32, P(vp)]
         lib.tphip_event_create_timed.argtypes = [i32, P(vp)]
         lib.tphip_event_destroy.argtypes = [i32, vp]

@@ -2,6 +2,7 @@
 
 #include <tensorpipe_c.h>
 
+#include <atomic>
 #include <chrono>
 #include <condition_variable>
 #include <cstring>
@@ -30,6 +31,7 @@ struct Completion {
   std::mutex mutex;
   std::condition_variable cv;
   bool done{false};
+  std::atomic<bool> flag{false};
   Error error;
 
   void set(const Error& e) {
@@ -37,12 +39,21 @@ struct Completion {
       std::lock_guard<std::mutex> lock(mutex);
       error = e;
       done = true;
+      flag.store(true, std::memory_order_release);
     }
     cv.notify_all();
   }
 
-  // 0 ok, TPC_ERR_FAILED, TPC_ERR_TIMEOUT
+  // 0 ok, TPC_ERR_FAILED, TPC_ERR_TIMEOUT. Spins briefly before blocking: the
+  // callbacks of a transfer in flight arrive within microseconds.
   int wait(int timeoutMs) {
+    const auto spinUntil = std::chrono::steady_clock::now() + std::chrono::microseconds(200);
+    while (!flag.load(std::memory_order_acquire) &&
+           std::chrono::steady_clock::now() < spinUntil) {
+#if defined(__x86_64__)
+      __builtin_ia32_pause();
+#endif
+    }
     std::unique_lock<std::mutex> lock(mutex);
     if (timeoutMs < 0) {
       cv.wait(lock, [this] { return done; });
@@ -147,7 +158,17 @@ void syncRecvStreams(const tpc_tensor* tensors, uint32_t n) {
     }
     seen.push_back(tensors[i].stream);
     int dev = hipDeviceForPointer(tensors[i].ptr);
-    TP_HIP_CHECK(tphip_stream_sync(dev < 0 ? 0 : dev, tensors[i].stream));
+    dev = dev < 0 ? 0 : dev;
+    // Poll rather than block: the blocking wait of the runtime adds several
+    // microseconds of wake-up latency to every step.
+    int done = 0;
+    const auto spinUntil = std::chrono::steady_clock::now() + std::chrono::milliseconds(2);
+    while (!done && std::chrono::steady_clock::now() < spinUntil) {
+      TP_HIP_CHECK(tphip_stream_query(dev, tensors[i].stream, &done));
+    }
+    if (!done) {
+      TP_HIP_CHECK(tphip_stream_sync(dev, tensors[i].stream));
+    }
   }
 }
 

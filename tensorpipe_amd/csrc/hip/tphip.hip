@@ -3,6 +3,7 @@
 // kernel. Nothing here knows about channels or pipes.
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <atomic>
 #include <cstdio>
@@ -58,61 +59,84 @@ struct DeviceState {
   std::vector<std::pair<hipEvent_t, hipEvent_t>> profEvents;
 };
 
-// Brackets one launch with timing events while profiling is on.
+// While profiling is on, hands a pair of timing events to the next kernel
+// launch of this thread; the runtime stamps them with the kernel's own start
+// and end, so their distance is the kernel's execution time.
+thread_local hipEvent_t tlsProfStart = nullptr;
+thread_local hipEvent_t tlsProfStop = nullptr;
+
 class ProfileScope {
  public:
-  ProfileScope(DeviceState& st, hipStream_t stream, uint64_t bytes) : stream_(stream) {
+  ProfileScope(DeviceState& st, hipStream_t /*stream*/, uint64_t bytes) {
     std::lock_guard<std::mutex> lock(st.profMutex);
     if (!st.profiling || st.profEvents.size() >= st.profMax) {
       return;
     }
-    if (hipEventCreate(&begin_) != hipSuccess || hipEventCreate(&end_) != hipSuccess) {
+    hipEvent_t begin = nullptr, end = nullptr;
+    if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
       (void)hipGetLastError();
-      begin_ = end_ = nullptr;
       return;
     }
-    st.profEvents.emplace_back(begin_, end_);
+    st.profEvents.emplace_back(begin, end);
     st.profBytes += bytes;
-    (void)hipEventRecord(begin_, stream_);
+    tlsProfStart = begin;
+    tlsProfStop = end;
   }
   ~ProfileScope() {
-    if (end_ != nullptr) {
-      (void)hipEventRecord(end_, stream_);
-    }
+    tlsProfStart = nullptr;
+    tlsProfStop = nullptr;
   }
-
- private:
-  hipStream_t stream_;
-  hipEvent_t begin_{nullptr};
-  hipEvent_t end_{nullptr};
 };
 
 DeviceState gDevices[kMaxDevices];
 
-int defaultUnroll() {
-  static int v = [] {
-    const char* e = getenv("TPHIP_COPY_UNROLL");
-    int u = e ? atoi(e) : 4;
+// Launch shape defaults, from sweeps on MI355X (256 CUs, 256 MiB Infinity
+// Cache). Each can be overridden through the environment for experiments.
+int envInt(const char* name, int fallback) {
+  const char* e = getenv(name);
+  return e != nullptr ? atoi(e) : fallback;
+}
+
+// 16-byte vectors in flight per lane.
+int defaultUnroll(bool table) {
+  static const int single = [] {
+    int u = envInt("TPHIP_COPY_UNROLL", 4);
     return (u == 1 || u == 2 || u == 4 || u == 8) ? u : 4;
   }();
-  return v;
+  static const int multi = [] {
+    int u = envInt("TPHIP_TABLE_UNROLL", 2);
+    return (u == 1 || u == 2 || u == 4 || u == 8) ? u : 2;
+  }();
+  return table ? multi : single;
 }
 
-int defaultBlocksPerCu() {
-  static int v = [] {
-    const char* e = getenv("TPHIP_COPY_BLOCKS_PER_CU");
-    int b = e ? atoi(e) : 8;
-    return b > 0 && b <= 64 ? b : 8;
+// Workgroups per CU: one for the single-entry kernel (the grid then sweeps one
+// compact window of memory at a time), four for the table kernel (its lookups
+// need more wavefronts to hide behind).
+int defaultBlocksPerCu(bool table) {
+  static const int single = [] {
+    int b = envInt("TPHIP_COPY_BLOCKS_PER_CU", 1);
+    return b > 0 && b <= 64 ? b : 1;
   }();
-  return v;
+  static const int multi = [] {
+    int b = envInt("TPHIP_TABLE_BLOCKS_PER_CU", 4);
+    return b > 0 && b <= 64 ? b : 4;
+  }();
+  return table ? multi : single;
 }
 
-int defaultNontemporal() {
-  static int v = [] {
-    const char* e = getenv("TPHIP_COPY_NT");
-    return e ? (atoi(e) != 0) : 1;
-  }();
-  return v;
+// Cache policy mask (bit 0 = nontemporal loads, bit 1 = nontemporal stores).
+// Stores always stream: the consumer runs later. Loads stream only for copies
+// too large for any of the source to still sit in the Infinity Cache; below
+// that, a source that was produced just before the copy is partly resident
+// and cached loads pick it up (7.2 vs 6.5 TB/s at 256 MiB, and the reverse,
+// 5.9 vs 6.3 TB/s, at 1 GiB).
+int defaultNontemporal(uint64_t totalBytes) {
+  static const int forced = envInt("TPHIP_COPY_NT", -1);
+  if (forced >= 0) {
+    return forced & 3;
+  }
+  return totalBytes <= (512ull << 20) ? 2 : 3;
 }
 
 int planViaKernel() {
@@ -164,15 +188,22 @@ int launchKernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, h
   void* argv[sizeof...(Params)];
   size_t i = 0;
   std::apply([&](auto&... v) { ((argv[i++] = static_cast<void*>(&v)), ...); }, values);
-  hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds,
-                                 stream);
+  hipError_t e;
+  if (tlsProfStart != nullptr) {
+    e = hipExtLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream,
+                           tlsProfStart, tlsProfStop, 0);
+    tlsProfStart = nullptr;
+    tlsProfStop = nullptr;
+  } else {
+    e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream);
+  }
   if (e != hipSuccess) {
     (void)hipGetLastError();
   }
   return static_cast<int>(e);
 }
 
-template <bool NT>
+template <int NT>
 int launchSingle(int unroll, uint32_t blocks, hipStream_t stream, const char* src, char* dst,
                  uint64_t bytes) {
   switch (unroll) {
@@ -191,35 +222,37 @@ int launchSingle(int unroll, uint32_t blocks, hipStream_t stream, const char* sr
   }
 }
 
-template <bool NT>
+template <int NT>
 int launchTable(int unroll, uint32_t blocks, size_t lds, hipStream_t stream,
                 const uint32_t* prefix, const tphip_copy_desc* descs, uint32_t n,
-                uint32_t nslices) {
+                uint32_t nchunks) {
   switch (unroll) {
     case 1:
       return launchKernel(batched_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nslices);
+                          prefix, descs, n, nchunks);
     case 2:
       return launchKernel(batched_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nslices);
+                          prefix, descs, n, nchunks);
     case 8:
       return launchKernel(batched_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nslices);
+                          prefix, descs, n, nchunks);
     default:
       return launchKernel(batched_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nslices);
+                          prefix, descs, n, nchunks);
   }
 }
 
-uint32_t pickBlocks(const DeviceState& st, uint64_t nslices, uint32_t minWaves, uint32_t blocks) {
-  uint64_t wantWaves = nslices > minWaves ? nslices : minWaves;
-  uint64_t want = (wantWaves + kWavesPerBlock - 1) / kWavesPerBlock;
+// Workgroups for `units` work units of one workgroup-iteration each: enough to
+// give every unit a workgroup, capped at blocksPerCu * CUs (or `blocks`).
+uint32_t pickBlocks(const DeviceState& st, uint64_t units, uint32_t minBlocks, uint32_t blocks,
+                    bool table) {
+  uint64_t want = units > minBlocks ? units : minBlocks;
   if (want == 0) {
     want = 1;
   }
-  uint64_t cap = blocks != 0 ? blocks
-                             : static_cast<uint64_t>(st.numCus > 0 ? st.numCus : 256) *
-          defaultBlocksPerCu();
+  const uint64_t cap = blocks != 0
+      ? blocks
+      : static_cast<uint64_t>(st.numCus > 0 ? st.numCus : 256) * defaultBlocksPerCu(table);
   return static_cast<uint32_t>(want < cap ? want : cap);
 }
 
@@ -231,19 +264,43 @@ int copySingle(DeviceState& st, const tphip_copy_desc& d, hipStream_t stream, in
   if (d.src == nullptr || d.dst == nullptr) {
     return TPHIP_ERR_INVALID_ARG;
   }
+  if (unroll == 0) {
+    unroll = defaultUnroll(false);
+  }
+  if (nt < 0) {
+    nt = defaultNontemporal(d.bytes);
+  }
   const uint64_t nvec = d.bytes >> 4;
-  const uint64_t nslices = (nvec + uint64_t(kWave) * unroll - 1) / (uint64_t(kWave) * unroll) + 1;
-  const uint32_t grid = pickBlocks(st, nslices, 1, blocks);
+  const uint64_t perBlock = uint64_t(kBlockThreads) * unroll;
+  const uint32_t grid = pickBlocks(st, (nvec + perBlock - 1) / perBlock, 1, blocks, false);
   const char* src = static_cast<const char*>(d.src);
   char* dst = static_cast<char*>(d.dst);
   ProfileScope prof(st, stream, d.bytes);
-  return nt ? launchSingle<true>(unroll, grid, stream, src, dst, d.bytes)
-            : launchSingle<false>(unroll, grid, stream, src, dst, d.bytes);
+  switch (nt & 3) {
+    case 0:
+      return launchSingle<0>(unroll, grid, stream, src, dst, d.bytes);
+    case 1:
+      return launchSingle<1>(unroll, grid, stream, src, dst, d.bytes);
+    case 2:
+      return launchSingle<2>(unroll, grid, stream, src, dst, d.bytes);
+    default:
+      return launchSingle<3>(unroll, grid, stream, src, dst, d.bytes);
+  }
 }
 
 // Launch one table kernel over table[0..n) whose body vector total fits 32 bits.
 int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStream_t stream,
               int unroll, uint32_t blocks, int nt) {
+  if (unroll == 0) {
+    unroll = defaultUnroll(true);
+  }
+  if (nt < 0) {
+    uint64_t payload = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+      payload += table[i].bytes;
+    }
+    nt = defaultNontemporal(payload);
+  }
   const size_t prefixBytes = ((size_t(n) + 1) * sizeof(uint32_t) + 15) / 16 * 16;
   const size_t planBytes = prefixBytes + size_t(n) * sizeof(tphip_copy_desc);
   const size_t planBytesPadded = (planBytes + 15) / 16 * 16;
@@ -289,10 +346,10 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
       TPHIP_TRY(hipMemcpyAsync(devp, host, planBytesPadded, hipMemcpyHostToDevice, stream));
     }
 
-    const uint64_t slice = uint64_t(kWave) * unroll;
-    const uint32_t nslices = static_cast<uint32_t>((total + slice - 1) / slice);
-    const uint32_t edgeWaves = (n + kWave - 1) / kWave;
-    const uint32_t grid = pickBlocks(st, nslices, edgeWaves, blocks);
+    const uint64_t chunk = uint64_t(kBlockThreads) * unroll;
+    const uint32_t nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
+    const uint32_t edgeBlocks = (n + kBlockThreads - 1) / kBlockThreads;
+    const uint32_t grid = pickBlocks(st, nchunks, edgeBlocks, blocks, true);
     const size_t lds = (size_t(n) + 1) * sizeof(uint32_t);
     const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
     const tphip_copy_desc* dDescs = reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes);
@@ -303,8 +360,20 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
         payload += table[i].bytes;
       }
       ProfileScope prof(st, stream, payload);
-      rc = nt ? launchTable<true>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices)
-              : launchTable<false>(unroll, grid, lds, stream, dPrefix, dDescs, n, nslices);
+      switch (nt & 3) {
+        case 0:
+          rc = launchTable<0>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          break;
+        case 1:
+          rc = launchTable<1>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          break;
+        case 2:
+          rc = launchTable<2>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          break;
+        default:
+          rc = launchTable<3>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          break;
+      }
     }
     if (rc != 0) {
       return rc;
@@ -325,7 +394,8 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
   if (n > TPHIP_MAX_BATCH) {
     return TPHIP_ERR_TOO_LARGE;
   }
-  if (!(unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8)) {
+  // unroll 0 and nt < 0 select the defaults, resolved per launch.
+  if (!(unroll == 0 || unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8)) {
     return TPHIP_ERR_INVALID_ARG;
   }
   DeviceState* st = nullptr;
@@ -563,6 +633,19 @@ int tphip_stream_sync(int dev, void* stream) {
   return 0;
 }
 
+int tphip_stream_query(int dev, void* stream, int* done) {
+  TPHIP_TRY(hipSetDevice(dev));
+  hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
+  if (e == hipErrorNotReady) {
+    (void)hipGetLastError();
+    *done = 0;
+    return 0;
+  }
+  TPHIP_TRY(e);
+  *done = 1;
+  return 0;
+}
+
 int tphip_event_create(int dev, int interprocess, void** event) {
   TPHIP_TRY(hipSetDevice(dev));
   hipEvent_t e;
@@ -683,17 +766,17 @@ int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], 
 }
 
 int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* stream) {
-  return batchedCopyImpl(dev, table, n, stream, defaultUnroll(), 0, defaultNontemporal());
+  return batchedCopyImpl(dev, table, n, stream, 0, 0, -1);
 }
 
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {
   tphip_copy_desc d{src, dst, bytes};
-  return batchedCopyImpl(dev, &d, 1, stream, defaultUnroll(), 0, defaultNontemporal());
+  return batchedCopyImpl(dev, &d, 1, stream, 0, 0, -1);
 }
 
 int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                              int unroll, uint32_t blocks, int nontemporal) {
-  return batchedCopyImpl(dev, table, n, stream, unroll, blocks, nontemporal);
+  return batchedCopyImpl(dev, table, n, stream, unroll, blocks, nontemporal & 3);
 }
 
 int tphip_profile_start(int dev, uint32_t max_launches) {

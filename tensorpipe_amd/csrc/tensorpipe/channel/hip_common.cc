@@ -61,11 +61,23 @@ void HipEventPoller::join() {
 }
 
 void HipEventPoller::run() {
+  using Clock = std::chrono::steady_clock;
   std::deque<Item> active;
+  auto lastBusy = Clock::now();
   for (;;) {
     {
       std::unique_lock<std::mutex> lock(mutex_);
-      if (active.empty()) {
+      if (active.empty() && incoming_.empty() && !stopping_) {
+        // Stay hot for a short while after the last event: in a ping-pong the
+        // next one arrives within microseconds and a sleeping thread would add
+        // its wake-up time to every transfer.
+        if (Clock::now() - lastBusy < std::chrono::microseconds(300)) {
+          lock.unlock();
+#if defined(__x86_64__)
+          __builtin_ia32_pause();
+#endif
+          continue;
+        }
         cv_.wait(lock, [this] { return stopping_ || !incoming_.empty(); });
       }
       while (!incoming_.empty()) {
@@ -95,6 +107,9 @@ void HipEventPoller::run() {
       } else {
         ++it;
       }
+    }
+    if (any || !active.empty()) {
+      lastBusy = Clock::now();
     }
     if (!any) {
 #if defined(__x86_64__)

@@ -386,8 +386,20 @@ class ChannelImpl final : public ChannelImplBase {
         unit->onReply = [this, op] { sendStepDone(op); };
         wireQueue_.push_back(unit);
         // Announce once the producing work on every source stream is done.
-        auto remaining = std::make_shared<size_t>(directStreams.size());
+        // Streams with nothing pending need no event at all.
+        std::vector<StreamRef> busy;
         for (auto& s : directStreams) {
+          int idle = 0;
+          if (tphip_stream_query(s.device, s.stream, &idle) != 0 || !idle) {
+            busy.push_back(s);
+          }
+        }
+        if (busy.empty()) {
+          unit->ready = true;
+          flushWire();
+        }
+        auto remaining = std::make_shared<size_t>(busy.size());
+        for (auto& s : busy) {
           auto ev = ictx_->events.get(s.device);
           ev->record(s.stream);
           watch(std::move(ev), [this, unit, remaining] {

@@ -1,19 +1,26 @@
 // hip_xth: GPU-to-GPU channel between two pipe endpoints of ONE process.
 //
-// Sender: records a start event on the stream(s) of the source buffers and
-// ships raw {event, stream, device, src pointer, length} words over the
+// Sender: ships raw {stream, device, src pointer, length} words over the
 // descriptor connection -- they are valid in the receiver because it is the
-// same address space. Receiver: makes its stream wait for the start event(s),
-// enqueues ONE batched copy kernel for all tensors of the message, records a
-// stop event, makes the sender's stream(s) wait for it, fires the recv
-// callback (copy enqueued, not finished: consumers order on their stream) and
-// acknowledges with an empty message, upon which the send callback fires.
+// same address space -- and waits for an empty completion message.
+// Receiver: enqueues ONE batched copy kernel for all tensors of the message
+// ON THE SENDER'S STREAM, which orders the copy after the work that produced
+// the source and before anything the sender enqueues later (it may overwrite
+// the source as soon as its send callback has fired), without a single
+// cross-stream dependency. A destination stream that still has work pending is
+// made a dependency of the copy (event + stream wait); an idle one costs one
+// query. A poller thread watches an event recorded behind the copy; when it
+// has completed the recv callback fires and the completion message goes out.
 //
-// Same protocol and stream semantics as
-// tensorpipe/channel/cuda_xth/channel_impl.cc:40-77,96-315; what differs is
-// that a whole message travels in one descriptor and one kernel launch
-// instead of one cudaMemcpyAsync and three event operations per tensor, and
-// that events come from a pool instead of being created per operation.
+// Same wire protocol as tensorpipe/channel/cuda_xth/channel_impl.cc:30-36,
+// 96-315 (descriptor one way, empty completion back). Differences, all for
+// latency: a whole message travels in one descriptor and one kernel launch
+// instead of one cudaMemcpyAsync per tensor; there are no start/stop events
+// and no stream waits on the common path (a stream wait costs 12-19 us of host
+// time on MI355X with ROCm 7, an event query about one); and the recv
+// callback fires when the copy has FINISHED rather than when it was enqueued
+// (cuda_xth/channel_impl.cc:66-77), which is the stronger guarantee and is
+// required because the copy does not run on the receiver's stream.
 
 #include <tensorpipe/channel/hip_xth/factory.h>
 
@@ -33,6 +40,10 @@ namespace {
 class XthContextCore final : public ContextCore {
  public:
   HipEventPool events;
+  HipEventPoller poller;
+  void joinImpl() override {
+    poller.join();
+  }
 };
 
 struct StreamRef {
@@ -112,7 +123,6 @@ class ChannelImpl final : public ChannelImplBase {
   struct SendOp {
     uint64_t seq;
     TSendCallback cb;
-    std::vector<std::unique_ptr<HipEvent>> startEvents;
     bool done{false};
   };
 
@@ -120,6 +130,8 @@ class ChannelImpl final : public ChannelImplBase {
     uint64_t seq;
     TRecvCallback cb;
     std::vector<BatchEntry> entries; // non-empty ones only
+    size_t copiesInFlight{0};
+    bool copied{false}; // every copy of the op has completed
     bool done{false};
   };
 
@@ -140,27 +152,18 @@ class ChannelImpl final : public ChannelImplBase {
     op->seq = seq;
     op->cb = std::move(cb);
 
-    std::vector<StreamRef> streams;
-    WireWriter body;
+    // Wire format: n, then per tensor {src stream, src device, src pointer, length}.
+    WireWriter w;
+    w.u32(static_cast<uint32_t>(live.size()));
     try {
       for (auto& e : live) {
         const HipBuffer& hb = e.buffer.unwrap<HipBuffer>();
-        StreamRef ref{hb.stream, hipDeviceForPointer(hb.ptr)};
-        TP_THROW_ASSERT_IF(ref.device < 0);
-        bool known = false;
-        for (auto& s : streams) {
-          known |= s == ref;
-        }
-        if (!known) {
-          streams.push_back(ref);
-        }
-        body.u64(reinterpret_cast<uint64_t>(hb.ptr));
-        body.u64(e.length);
-      }
-      for (auto& s : streams) {
-        auto ev = xctx_->events.get(s.device);
-        ev->record(s.stream);
-        op->startEvents.push_back(std::move(ev));
+        const int device = hipDeviceForPointer(hb.ptr);
+        TP_THROW_ASSERT_IF(device < 0);
+        w.u64(reinterpret_cast<uint64_t>(hb.stream));
+        w.u32(static_cast<uint32_t>(device));
+        w.u64(reinterpret_cast<uint64_t>(hb.ptr));
+        w.u64(e.length);
       }
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " send failed: " << ex.what();
@@ -168,16 +171,6 @@ class ChannelImpl final : public ChannelImplBase {
       setError(TP_CREATE_ERROR(HipError, "hip_xth send", TPHIP_ERR_INVALID_ARG));
       return;
     }
-
-    WireWriter w;
-    w.u32(static_cast<uint32_t>(live.size()));
-    w.u32(static_cast<uint32_t>(streams.size()));
-    for (size_t i = 0; i < streams.size(); ++i) {
-      w.u64(reinterpret_cast<uint64_t>(op->startEvents[i]->raw()));
-      w.u64(reinterpret_cast<uint64_t>(streams[i].stream));
-      w.u32(static_cast<uint32_t>(streams[i].device));
-    }
-    w.raw(body.bytes().data(), body.bytes().size());
 
     sendOps_.push_back(op);
     TP_VLOG(6) << "Channel " << id_ << " is writing descriptor (#" << seq << ")";
@@ -210,46 +203,28 @@ class ChannelImpl final : public ChannelImplBase {
       if (!error_) {
         copyFromDescriptor(op, bytes);
       }
-      removeRecv(op);
-      finishRecv(op);
-      if (!error_) {
-        TP_VLOG(6) << "Channel " << id_ << " is writing completion (#" << op->seq << ")";
-        completionConnection_->write(nullptr, 0, onWritten([] {}));
-      }
     }));
   }
 
-  // Wait for the sender's start events, copy everything with one launch per
-  // (device, stream) of the destination buffers (normally one in total), and
-  // make the sender's streams wait for the copy.
+  // One launch per source stream (normally one in total), on that stream.
   void copyFromDescriptor(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
     WireReader r(bytes.data(), bytes.size());
     const uint32_t n = r.u32();
-    const uint32_t nStreams = r.u32();
-    struct SrcStream {
-      void* event;
-      void* stream;
-      int device;
-    };
-    std::vector<SrcStream> srcStreams;
-    for (uint32_t i = 0; i < nStreams && r.ok(); ++i) {
-      SrcStream s;
-      s.event = reinterpret_cast<void*>(r.u64());
-      s.stream = reinterpret_cast<void*>(r.u64());
-      s.device = static_cast<int>(r.u32());
-      srcStreams.push_back(s);
-    }
     if (!r.ok() || n != op->entries.size()) {
       setError(TP_CREATE_ERROR(ShortReadError, static_cast<ssize_t>(op->entries.size()), n));
       return;
     }
     struct Group {
-      StreamRef dst;
+      StreamRef src;
+      std::vector<StreamRef> dstStreams;
       std::vector<tphip_copy_desc> table;
     };
     std::vector<Group> groups;
     try {
       for (uint32_t i = 0; i < n; ++i) {
+        StreamRef srcRef;
+        srcRef.stream = reinterpret_cast<void*>(r.u64());
+        srcRef.device = static_cast<int>(r.u32());
         const void* src = reinterpret_cast<const void*>(r.u64());
         const uint64_t len = r.u64();
         if (!r.ok() || len != op->entries[i].length) {
@@ -258,37 +233,73 @@ class ChannelImpl final : public ChannelImplBase {
           return;
         }
         const HipBuffer& hb = op->entries[i].buffer.unwrap<HipBuffer>();
-        StreamRef ref{hb.stream, hipDeviceForPointer(hb.ptr)};
-        TP_THROW_ASSERT_IF(ref.device < 0);
+        StreamRef dstRef{hb.stream, hipDeviceForPointer(hb.ptr)};
+        TP_THROW_ASSERT_IF(dstRef.device < 0);
         Group* g = nullptr;
         for (auto& cand : groups) {
-          if (cand.dst == ref) {
+          if (cand.src == srcRef) {
             g = &cand;
           }
         }
         if (g == nullptr) {
-          groups.push_back(Group{ref, {}});
+          groups.push_back(Group{srcRef, {}, {}});
           g = &groups.back();
+        }
+        bool known = false;
+        for (auto& d : g->dstStreams) {
+          known |= d == dstRef;
+        }
+        if (!known && !(dstRef == srcRef)) {
+          g->dstStreams.push_back(dstRef);
         }
         g->table.push_back(tphip_copy_desc{src, hb.ptr, len});
       }
+      op->copiesInFlight = groups.size();
       for (auto& g : groups) {
-        for (auto& s : srcStreams) {
-          TP_HIP_CHECK(tphip_stream_wait_event(g.dst.device, g.dst.stream, s.event));
+        // The copy may only touch a destination once everything the receiver
+        // enqueued before recv() on that buffer's stream is done.
+        for (auto& d : g.dstStreams) {
+          int idle = 0;
+          TP_HIP_CHECK(tphip_stream_query(d.device, d.stream, &idle));
+          if (!idle) {
+            auto ev = xctx_->events.get(d.device);
+            ev->record(d.stream);
+            ev->wait(g.src.stream, g.src.device);
+            xctx_->events.put(std::move(ev)); // the wait captured the record
+          }
         }
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
-        hipBatchedCopy(g.dst.device, g.dst.stream, g.table);
-        auto stop = xctx_->events.get(g.dst.device);
-        stop->record(g.dst.stream);
-        for (auto& s : srcStreams) {
-          stop->wait(s.stream, s.device);
-        }
-        // The waits above captured the record; the event can be reused.
-        xctx_->events.put(std::move(stop));
+        hipBatchedCopy(g.src.device, g.src.stream, g.table);
+        auto done = xctx_->events.get(g.src.device);
+        done->record(g.src.stream);
+        auto self = shared_from_this();
+        xctx_->poller.watch(std::move(done), &xctx_->events, [this, self, op](const Error& error) {
+          ctx_->defer([this, self, op, error] {
+            setError(error);
+            if (error_ || --op->copiesInFlight > 0) {
+              return;
+            }
+            TP_VLOG(6) << "Channel " << id_ << " done copying payload (#" << op->seq << ")";
+            op->copied = true;
+            flushRecvs();
+          });
+        });
       }
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " copy failed: " << ex.what();
       setError(TP_CREATE_ERROR(HipError, "hip_xth copy", TPHIP_ERR_INVALID_ARG));
+    }
+  }
+
+  // Completions go out in the order the descriptors came in (the sender pairs
+  // them by position), each once its copies have finished.
+  void flushRecvs() {
+    while (!recvOps_.empty() && recvOps_.front()->copied && !error_) {
+      auto op = recvOps_.front();
+      recvOps_.pop_front();
+      finishRecv(op);
+      TP_VLOG(6) << "Channel " << id_ << " is writing completion (#" << op->seq << ")";
+      completionConnection_->write(nullptr, 0, onWritten([] {}));
     }
   }
 
@@ -315,10 +326,6 @@ class ChannelImpl final : public ChannelImplBase {
       return;
     }
     op->done = true;
-    for (auto& ev : op->startEvents) {
-      xctx_->events.put(std::move(ev));
-    }
-    op->startEvents.clear();
     auto cb = std::move(op->cb);
     cb(error_);
   }

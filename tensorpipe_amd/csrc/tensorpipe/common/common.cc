@@ -57,6 +57,12 @@ int hipDeviceCountNoThrow() {
 }
 
 int hipDeviceForPointer(const void* ptr) {
+  // With a single visible GPU every device pointer belongs to device 0: skip
+  // the driver query, which would otherwise run several times per tensor.
+  static const int count = hipDeviceCountNoThrow();
+  if (count == 1 && ptr != nullptr) {
+    return 0;
+  }
   int dev = -1;
   int isHost = 0;
   TP_HIP_CHECK(tphip_device_for_ptr(ptr, &dev, &isHost));

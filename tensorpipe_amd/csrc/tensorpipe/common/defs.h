@@ -6,8 +6,10 @@
 // same process (PyTorch's libtorch_cpu.so carries one).
 #pragma once
 
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <iostream>
 #include <sstream>
 #include <stdexcept>
@@ -40,7 +42,13 @@ inline int tpVerbosity() {
 class LogLine {
  public:
   LogLine(const char* file, int line, char severity) {
-    ss_ << severity << " " << tpTrimFilename(file) << ":" << line << "] ";
+    // Monotonic microseconds, so that lines of several processes on one
+    // machine can be put on one time axis.
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    char stamp[32];
+    snprintf(stamp, sizeof(stamp), "%lld.%03ld", static_cast<long long>(ts.tv_sec) * 1000000 + ts.tv_nsec / 1000, ts.tv_nsec % 1000);
+    ss_ << severity << stamp << " " << tpTrimFilename(file) << ":" << line << "] ";
   }
   ~LogLine() {
     ss_ << "\n";

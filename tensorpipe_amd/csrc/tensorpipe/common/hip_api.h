@@ -28,7 +28,9 @@ TP_AMD_NAMESPACE_BEGIN
 // Number of usable GPUs; 0 when the runtime reports none or fails to load.
 int hipDeviceCountNoThrow();
 
-// Device index owning ptr, -1 for host memory (tensorpipe/common/cuda.h:141-166).
+// Device index owning the device pointer ptr (tensorpipe/common/cuda.h:141-166).
+// Callers pass pointers taken from a HipBuffer, i.e. device memory; on a
+// multi-GPU machine a host pointer yields -1.
 int hipDeviceForPointer(const void* ptr);
 
 class HipEvent {

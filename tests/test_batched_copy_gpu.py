@@ -111,7 +111,7 @@ def test_single_tensor(oracle, nbytes, soff, doff):
 
 
 @pytest.mark.parametrize("unroll", [1, 2, 4, 8])
-@pytest.mark.parametrize("nt", [0, 1])
+@pytest.mark.parametrize("nt", [0, 1, 2, 3])
 def test_launch_shapes(oracle, unroll, nt):
     sizes = list(datagen.loguniform_sizes(77, 16, 1 << 20, 96)) + [0, 1, 5, 100000, 3 << 20]
     layout = _pack(sizes, lambda i: i % 16, lambda i: (i * 3) % 16)
