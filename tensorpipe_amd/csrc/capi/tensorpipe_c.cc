@@ -6,6 +6,7 @@
 #include <chrono>
 #include <condition_variable>
 #include <cstring>
+#include <functional>
 #include <future>
 #include <mutex>
 #include <sstream>
@@ -477,6 +478,106 @@ int tpc_bench_transfer(
   TPC_GUARD_END(TPC_ERR_FAILED)
 }
 
+// Callback-chained ping-pong, the shape of the reference's own benchmark
+// (tensorpipe/benchmark/benchmark_pipe.cc:463-468,571-577): every step is
+// issued from the callback of the previous one on the library's threads, so
+// no thread hand-off is on the clock. The caller only waits for the end.
+struct PingPong : std::enable_shared_from_this<PingPong> {
+  using Clock = std::chrono::steady_clock;
+  std::shared_ptr<Pipe> pipe;
+  bool initiator{false};
+  std::vector<tpc_payload> payloads;
+  std::vector<void*> recvPayloadPtrs;
+  std::vector<tpc_tensor> sendTensors, recvTensors;
+  uint32_t warmup{0}, iters{0}, round{0};
+  double* perIterUs{nullptr};
+  Clock::time_point begin, end, t0;
+  Completion finished;
+  std::atomic<bool> failed{false};
+
+  void fail(const Error& e) {
+    if (!failed.exchange(true)) {
+      finished.set(e);
+    }
+  }
+
+  void doWrite(std::function<void()> next) {
+    auto self = shared_from_this();
+    pipe->write(
+        makeMessage(
+            "", payloads.data(), static_cast<uint32_t>(payloads.size()), sendTensors.data(),
+            static_cast<uint32_t>(sendTensors.size())),
+        [self, next{std::move(next)}](const Error& e) {
+          if (e) {
+            self->fail(e);
+          } else if (next) {
+            next();
+          }
+        });
+  }
+
+  void doRead(std::function<void()> next) {
+    auto self = shared_from_this();
+    pipe->readDescriptor([self, next{std::move(next)}](const Error& e, Descriptor) {
+      if (e) {
+        self->fail(e);
+        return;
+      }
+      self->pipe->read(
+          makeAllocation(
+              self->recvPayloadPtrs.data(), static_cast<uint32_t>(self->recvPayloadPtrs.size()),
+              self->recvTensors.data(), static_cast<uint32_t>(self->recvTensors.size())),
+          [self, next](const Error& e2) {
+            if (e2) {
+              self->fail(e2);
+            } else {
+              next();
+            }
+          });
+    });
+  }
+
+  void step() {
+    if (round == warmup + iters) {
+      end = Clock::now();
+      finished.set(Error::kSuccess);
+      return;
+    }
+    if (round == warmup) {
+      begin = Clock::now();
+    }
+    auto self = shared_from_this();
+    if (initiator) {
+      t0 = Clock::now();
+      doWrite(nullptr);
+      doRead([self] {
+        try {
+          syncRecvStreams(self->recvTensors.data(), static_cast<uint32_t>(self->recvTensors.size()));
+        } catch (const std::exception&) {
+          self->fail(TP_CREATE_ERROR(HipError, "stream sync", TPHIP_ERR_INVALID_ARG));
+          return;
+        }
+        if (self->round >= self->warmup && self->perIterUs != nullptr) {
+          self->perIterUs[self->round - self->warmup] =
+              std::chrono::duration<double, std::micro>(Clock::now() - self->t0).count();
+        }
+        ++self->round;
+        self->step();
+      });
+    } else {
+      // The echo leaves from the buffers the message arrived in; a channel
+      // whose recv callback means "enqueued" keeps the two ordered on the
+      // buffers' stream.
+      doRead([self] {
+        self->doWrite([self] {
+          ++self->round;
+          self->step();
+        });
+      });
+    }
+  }
+};
+
 int tpc_bench_pingpong(
     tpc_pipe* p,
     int initiator,
@@ -491,59 +592,23 @@ int tpc_bench_pingpong(
     double* perIterUs,
     double* totalSeconds) {
   TPC_GUARD_BEGIN
-  using Clock = std::chrono::steady_clock;
-  Clock::time_point begin;
-  const int kTimeoutMs = 60000;
-  auto doWrite = [&](std::shared_ptr<Completion> c) {
-    p->pipe->write(
-        makeMessage("", payloads, numPayloads, sendTensors, numTensors),
-        [c](const Error& e) { c->set(e); });
-  };
-  auto doRead = [&]() -> int {
-    auto gotDescriptor = std::make_shared<Completion>();
-    auto readDone = std::make_shared<Completion>();
-    p->pipe->readDescriptor(
-        [gotDescriptor](const Error& e, Descriptor) { gotDescriptor->set(e); });
-    int rc = gotDescriptor->wait(kTimeoutMs);
-    if (rc != 0) {
-      return rc;
-    }
-    p->pipe->read(
-        makeAllocation(recvPayloadPtrs, numPayloads, recvTensors, numTensors),
-        [readDone](const Error& e) { readDone->set(e); });
-    return readDone->wait(kTimeoutMs);
-  };
-  for (uint32_t it = 0; it < warmup + iters; ++it) {
-    if (it == warmup) {
-      begin = Clock::now();
-    }
-    auto t0 = Clock::now();
-    auto wrote = std::make_shared<Completion>();
-    int rc;
-    if (initiator) {
-      doWrite(wrote);
-      if ((rc = doRead()) != 0) {
-        return rc;
-      }
-      syncRecvStreams(recvTensors, numTensors);
-    } else {
-      if ((rc = doRead()) != 0) {
-        return rc;
-      }
-      // The echo is ordered after the receive on the receive stream when the
-      // send buffers are the receive buffers on that same stream.
-      doWrite(wrote);
-    }
-    if ((rc = wrote->wait(kTimeoutMs)) != 0) {
-      return rc;
-    }
-    if (it >= warmup && perIterUs != nullptr) {
-      perIterUs[it - warmup] =
-          std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
-    }
+  auto pp = std::make_shared<PingPong>();
+  pp->pipe = p->pipe;
+  pp->initiator = initiator != 0;
+  pp->payloads.assign(payloads, payloads + numPayloads);
+  pp->recvPayloadPtrs.assign(recvPayloadPtrs, recvPayloadPtrs + numPayloads);
+  pp->sendTensors.assign(sendTensors, sendTensors + numTensors);
+  pp->recvTensors.assign(recvTensors, recvTensors + numTensors);
+  pp->warmup = warmup;
+  pp->iters = iters;
+  pp->perIterUs = perIterUs;
+  pp->step();
+  int rc = pp->finished.wait(600000);
+  if (rc != 0) {
+    return rc;
   }
   if (totalSeconds != nullptr) {
-    *totalSeconds = std::chrono::duration<double>(Clock::now() - begin).count();
+    *totalSeconds = std::chrono::duration<double>(pp->end - pp->begin).count();
   }
   return 0;
   TPC_GUARD_END(TPC_ERR_FAILED)

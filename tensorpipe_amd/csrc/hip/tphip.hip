@@ -54,7 +54,7 @@ struct DeviceState {
   // Launch profiling (tphip_profile_start/stop).
   std::mutex profMutex;
   bool profiling{false};
-  uint32_t profMax{0};
+  uint32_t profUsed{0};
   uint64_t profBytes{0};
   std::vector<std::pair<hipEvent_t, hipEvent_t>> profEvents;
 };
@@ -69,18 +69,16 @@ class ProfileScope {
  public:
   ProfileScope(DeviceState& st, hipStream_t /*stream*/, uint64_t bytes) {
     std::lock_guard<std::mutex> lock(st.profMutex);
-    if (!st.profiling || st.profEvents.size() >= st.profMax) {
+    if (!st.profiling) {
       return;
     }
-    hipEvent_t begin = nullptr, end = nullptr;
-    if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
-      (void)hipGetLastError();
+    if (st.profUsed >= st.profEvents.size()) {
       return;
     }
-    st.profEvents.emplace_back(begin, end);
+    auto& pair = st.profEvents[st.profUsed++];
     st.profBytes += bytes;
-    tlsProfStart = begin;
-    tlsProfStop = end;
+    tlsProfStart = pair.first;
+    tlsProfStop = pair.second;
   }
   ~ProfileScope() {
     tlsProfStart = nullptr;
@@ -792,8 +790,17 @@ int tphip_profile_start(int dev, uint32_t max_launches) {
   }
   st->profEvents.clear();
   st->profEvents.reserve(max_launches);
+  // Events are created up front so that the measured region creates none.
+  for (uint32_t i = 0; i < max_launches; ++i) {
+    hipEvent_t begin = nullptr, end = nullptr;
+    if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) {
+      (void)hipGetLastError();
+      break;
+    }
+    st->profEvents.emplace_back(begin, end);
+  }
+  st->profUsed = 0;
   st->profBytes = 0;
-  st->profMax = max_launches;
   st->profiling = true;
   return 0;
 }
@@ -809,22 +816,26 @@ int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* 
   double sum = 0;
   uint32_t count = 0;
   int err = 0;
-  for (auto& p : st->profEvents) {
-    hipError_t e = hipEventSynchronize(p.second);
-    float ms = 0;
-    if (e == hipSuccess) {
-      e = hipEventElapsedTime(&ms, p.first, p.second);
-    }
-    if (e == hipSuccess) {
-      sum += ms;
-      ++count;
-    } else {
-      (void)hipGetLastError();
-      err = static_cast<int>(e);
+  for (uint32_t i = 0; i < st->profEvents.size(); ++i) {
+    auto& p = st->profEvents[i];
+    if (i < st->profUsed) {
+      hipError_t e = hipEventSynchronize(p.second);
+      float ms = 0;
+      if (e == hipSuccess) {
+        e = hipEventElapsedTime(&ms, p.first, p.second);
+      }
+      if (e == hipSuccess) {
+        sum += ms;
+        ++count;
+      } else {
+        (void)hipGetLastError();
+        err = static_cast<int>(e);
+      }
     }
     (void)hipEventDestroy(p.first);
     (void)hipEventDestroy(p.second);
   }
+  st->profUsed = 0;
   st->profEvents.clear();
   if (launches) {
     *launches = count;

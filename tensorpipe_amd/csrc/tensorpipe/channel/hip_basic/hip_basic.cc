@@ -1,29 +1,43 @@
 // hip_basic: host-staged GPU channel that wraps a CPU channel.
 //
-// A tensor is cut into chunks of at most one staging slot. Sender, per chunk:
-// take a slot of the pinned send ring, copy GPU -> slot with the batched copy
-// kernel on the caller's stream (the kernel stores straight into host-mapped
-// pinned memory), and when that copy has completed hand the slot to the inner
-// CPU channel. Receiver, per chunk: take a slot of the pinned receive ring,
-// let the inner CPU channel fill it, copy slot -> GPU on the caller's stream,
-// free the slot when that copy has completed. CPU-resident buffers skip the
-// staging hop on their side, so the channel also carries CPU<->GPU transfers.
+// A tensor is cut into chunks of at most one staging slot and every chunk
+// bounces through pinned host memory. Two routes, chosen per tensor by the
+// sender and announced on the channel's control connection:
 //
-// Follows tensorpipe/channel/cuda_basic/channel_impl.cc:84-229 (send) and
-// :335-506 (recv), context_impl.cc:27-154, constants.h:22-24, with these
-// differences: copies are kernel launches instead of cudaMemcpyAsync,
-// completion is detected by polling an event instead of a stream callback,
-// and the "ready to send" notification is replaced by a one-time exchange of
-// the chunk size (both sides know every tensor's length, so the receiver can
-// post its inner recvs without being told).
+//  ring   (GPU source, both endpoints on one machine) The sender's pinned send
+//         ring is exported once with a HIP IPC memory handle and mapped by the
+//         receiver's GPU. Per chunk the sender's copy kernel stores GPU -> ring
+//         slot and, once that has completed, a {slot, length} notification
+//         goes over the control connection; the receiver's copy kernel then
+//         loads ring slot -> GPU straight from the sender's pinned memory and
+//         acknowledges the slot. The bytes cross the host link twice and are
+//         never touched by a CPU; the two directions overlap, which is what
+//         lets the path approach the PCIe rate.
+//  inner  (CPU source, or the ring could not be shared) What the reference
+//         does for every chunk (tensorpipe/channel/cuda_basic/channel_impl.cc
+//         :84-229 send, :335-506 recv): GPU -> pinned slot, the wrapped CPU
+//         channel moves the slot to a pinned slot of the receiver, pinned
+//         slot -> GPU. CPU-resident buffers skip the staging on their side,
+//         so the channel also carries CPU<->GPU transfers.
+//
+// Geometry defaults follow tensorpipe/channel/cuda_basic/constants.h:22-24
+// (16 slots of 1 MiB per ring); TP_HIP_BASIC_SLOT_BYTES and
+// TP_HIP_BASIC_NUM_SLOTS override them per context. Copies are launches of the
+// batched copy kernel instead of cudaMemcpyAsync, completion is detected by
+// polling an event instead of a stream callback, and the reference's
+// per-chunk "ready to send" message is replaced by a hello exchange (chunk
+// size, ring handle) plus one route message per tensor.
 //
 // Callbacks: send fires once the last chunk has left the GPU (source
-// reusable); recv fires once the last host-to-device copy has been enqueued.
+// reusable); recv fires once the last host-to-device copy has been enqueued
+// (GPU target) or the last byte has landed (CPU target).
 
 #include <tensorpipe/channel/hip_basic/factory.h>
 
 #include <algorithm>
+#include <cstring>
 #include <deque>
+#include <map>
 
 #include <tensorpipe/channel/channel_base.h>
 #include <tensorpipe/channel/hip_common.h>
@@ -38,8 +52,6 @@ namespace hip_basic {
 
 namespace {
 
-// Defaults as tensorpipe/channel/cuda_basic/constants.h:22-24 (16 x 1 MiB per
-// ring); TP_HIP_BASIC_SLOT_BYTES and TP_HIP_BASIC_NUM_SLOTS override them.
 // Both are read when a context is created.
 size_t slotBytesFromEnv() {
   const char* e = std::getenv("TP_HIP_BASIC_SLOT_BYTES");
@@ -50,7 +62,12 @@ size_t slotBytesFromEnv() {
 size_t numSlotsFromEnv() {
   const char* e = std::getenv("TP_HIP_BASIC_NUM_SLOTS");
   size_t n = e != nullptr ? std::strtoull(e, nullptr, 10) : 16;
-  return n < 1 ? size_t(1) : n;
+  return n < 1 ? size_t(1) : (n > 4096 ? size_t(4096) : n);
+}
+
+bool ringSharingDisabled() {
+  const char* e = std::getenv("TP_HIP_BASIC_NO_SHARED_RING");
+  return e != nullptr && e[0] == '1';
 }
 
 struct PinnedRing {
@@ -70,20 +87,42 @@ class BasicContextCore final : public ContextCore {
   HipEventPoller poller;
   const size_t slotBytes{slotBytesFromEnv()};
   const size_t numSlots{numSlotsFromEnv()};
+  const bool shareRing{!ringSharingDisabled()};
 
-  // Rings are created on first use (loop only), as the reference allocates its
-  // pinned buffers lazily (tensorpipe/channel/cuda_basic/context_impl.cc:134-154).
+  // Loop only. The send ring exists from the first channel on (its handle is
+  // part of the hello); the receive ring is created on first use, as the
+  // reference allocates its pinned buffers lazily
+  // (tensorpipe/channel/cuda_basic/context_impl.cc:134-154).
   PinnedRing& sendRing() {
     if (!sendRing_) {
       sendRing_ = std::make_unique<PinnedRing>(0, numSlots, slotBytes);
+      if (shareRing &&
+          tphip_ipc_mem_export(0, sendRing_->slab.host(), sendRingHandle_.data()) == 0) {
+        sendRingExported_ = true;
+      }
     }
     return *sendRing_;
+  }
+  bool sendRingExported() {
+    sendRing();
+    return sendRingExported_;
+  }
+  const HandleBytes& sendRingHandle() const {
+    return sendRingHandle_;
   }
   PinnedRing& recvRing() {
     if (!recvRing_) {
       recvRing_ = std::make_unique<PinnedRing>(0, numSlots, slotBytes);
     }
     return *recvRing_;
+  }
+  // Stream for copies that belong to no caller stream (ring -> local pinned
+  // slot on behalf of a CPU target).
+  void* internalStream() {
+    if (internalStream_ == nullptr) {
+      TP_HIP_CHECK(tphip_stream_create(0, &internalStream_));
+    }
+    return internalStream_;
   }
   void closeRings() {
     if (sendRing_) {
@@ -100,7 +139,20 @@ class BasicContextCore final : public ContextCore {
  private:
   std::unique_ptr<PinnedRing> sendRing_;
   std::unique_ptr<PinnedRing> recvRing_;
+  HandleBytes sendRingHandle_{};
+  bool sendRingExported_{false};
+  void* internalStream_{nullptr};
 };
+
+enum MsgKind : uint8_t {
+  kHello = 1,    // chunk size, slots, identities, ring handle
+  kHelloAck = 2, // whether the peer's ring could be mapped
+  kRoute = 3,    // start of a tensor: route and length
+  kNotify = 4,   // ring route: chunk staged in {slot}
+  kAck = 5,      // ring route: slot consumed
+};
+
+enum Route : uint8_t { kRouteInner = 0, kRouteRing = 1 };
 
 class ChannelImpl final : public ChannelImplBase {
  public:
@@ -116,27 +168,26 @@ class ChannelImpl final : public ChannelImplBase {
 
  protected:
   void initFromLoop() override {
-    // Agree on the chunk size: both sides announce theirs, the smaller wins.
     WireWriter w;
+    w.u8(kHello);
     w.u64(bctx_->slotBytes);
+    w.u64(bctx_->numSlots);
+    w.str(bootIdentity());
+    w.str(processIdentity());
+    bool exported = false;
+    try {
+      exported = bctx_->sendRingExported();
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " cannot create its send ring: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "tphip_host_alloc", TPHIP_ERR_INVALID_ARG));
+      return;
+    }
+    w.u8(exported ? 1 : 0);
+    if (exported) {
+      w.raw(bctx_->sendRingHandle().data(), TPHIP_IPC_HANDLE_BYTES);
+    }
     writeMessage(*controlConnection_, std::move(w.bytes()));
-    controlConnection_->read(onReadMessage([this](std::vector<uint8_t> bytes) {
-      if (error_) {
-        return;
-      }
-      WireReader r(bytes.data(), bytes.size());
-      const uint64_t remote = r.u64();
-      if (!r.ok() || remote == 0) {
-        setError(TP_CREATE_ERROR(ShortReadError, 8, static_cast<ssize_t>(bytes.size())));
-        return;
-      }
-      chunkBytes_ = std::min<uint64_t>(remote, bctx_->slotBytes);
-      auto deferred = std::move(deferred_);
-      deferred_.clear();
-      for (auto& fn : deferred) {
-        fn();
-      }
-    }));
+    readControl();
   }
 
   void sendFromLoop(uint64_t seq, Buffer buffer, size_t length, TSendCallback cb) override {
@@ -164,7 +215,8 @@ class ChannelImpl final : public ChannelImplBase {
     op->buffer = std::move(buffer);
     op->length = length;
     ops_.push_back(op);
-    whenReady([this, op] { startRecv(op); });
+    recvOps_.push_back(op);
+    whenReady([this] { advanceRecvs(); });
   }
 
   void handleError() override {
@@ -175,7 +227,10 @@ class ChannelImpl final : public ChannelImplBase {
     }
     deferred_.clear();
     sendQueue_.clear();
-    recvQueue_.clear();
+    recvPostQueue_.clear();
+    recvOps_.clear();
+    inbox_.clear();
+    slotsInFlight_.clear();
     auto ops = std::move(ops_);
     ops_.clear();
     for (auto& op : ops) {
@@ -190,16 +245,22 @@ class ChannelImpl final : public ChannelImplBase {
     Buffer buffer;
     size_t length{0};
     size_t pending{0};
+    // recv side
+    bool routed{false};
+    uint8_t route{kRouteInner};
+    size_t received{0}; // bytes of this tensor already handled (ring route)
     bool done{false};
   };
 
-  // One chunk waiting for its turn on the inner channel: inner sends must be
-  // issued in chunk order even if device-to-host copies finish out of order.
+  // A chunk waiting for its turn: inner sends / control notifications must go
+  // out in chunk order even if device-to-host copies finish out of order.
   struct SendChunk {
     void* hostPtr{nullptr};
     size_t length{0};
     SlotAllocator::TSlot slot;
     bool ready{false};
+    bool ring{false};
+    bool isRoute{false}; // not a chunk: the tensor's route message
     std::shared_ptr<Op> op;
   };
 
@@ -212,8 +273,16 @@ class ChannelImpl final : public ChannelImplBase {
     std::shared_ptr<Op> op;
   };
 
+  // A control message for the receive side, kept until a recv op consumes it.
+  struct Incoming {
+    uint8_t kind;
+    uint8_t route;
+    uint32_t slot;
+    uint64_t length;
+  };
+
   void whenReady(std::function<void()> fn) {
-    if (chunkBytes_ != 0) {
+    if (ready_) {
       fn();
     } else {
       deferred_.push_back(std::move(fn));
@@ -224,11 +293,120 @@ class ChannelImpl final : public ChannelImplBase {
     return b.device().type == kCpuDeviceType;
   }
 
-  // ---- send -----------------------------------------------------------------
+  // ---- control connection -----------------------------------------------------
+
+  void readControl() {
+    controlConnection_->read(onReadMessage([this](std::vector<uint8_t> bytes) {
+      if (error_) {
+        return;
+      }
+      onControl(bytes);
+      if (!error_) {
+        readControl();
+      }
+    }));
+  }
+
+  void onControl(const std::vector<uint8_t>& bytes) {
+    WireReader r(bytes.data(), bytes.size());
+    const uint8_t kind = r.u8();
+    if (kind == kHello) {
+      const uint64_t remoteSlot = r.u64();
+      const uint64_t remoteSlots = r.u64();
+      const std::string boot = r.str();
+      const std::string process = r.str();
+      const bool hasHandle = r.u8() != 0;
+      if (!r.ok() || remoteSlot == 0) {
+        failProtocol();
+        return;
+      }
+      chunkBytes_ = std::min<uint64_t>(remoteSlot, bctx_->slotBytes);
+      remoteSlotBytes_ = remoteSlot;
+      remoteNumSlots_ = remoteSlots;
+      bool mapped = false;
+      if (hasHandle) {
+        HandleBytes h;
+        r.raw(h.data(), h.size());
+        // Map the peer's send ring if it lives on this machine in another
+        // process; otherwise its chunks come through the inner channel.
+        if (r.ok() && bctx_->shareRing && boot == bootIdentity() && process != processIdentity()) {
+          void* ptr = nullptr;
+          if (HipIpcImports::get().open(0, h, &ptr) == 0) {
+            remoteRing_ = static_cast<uint8_t*>(ptr);
+            mapped = true;
+          }
+        }
+      }
+      WireWriter w;
+      w.u8(kHelloAck);
+      w.u8(mapped ? 1 : 0);
+      writeMessage(*controlConnection_, std::move(w.bytes()));
+      gotHello_ = true;
+    } else if (kind == kHelloAck) {
+      peerMappedOurRing_ = r.u8() != 0;
+      gotHelloAck_ = true;
+    } else if (kind == kAck) {
+      const uint32_t slot = r.u32();
+      auto it = slotsInFlight_.find(slot);
+      if (!r.ok() || it == slotsInFlight_.end()) {
+        failProtocol();
+        return;
+      }
+      TP_VLOG(7) << "Channel " << id_ << " got ack for slot " << slot;
+      slotsInFlight_.erase(it); // drops the slot back into the ring
+    } else if (kind == kRoute || kind == kNotify) {
+      Incoming in{};
+      in.kind = kind;
+      if (kind == kRoute) {
+        in.route = r.u8();
+      } else {
+        in.slot = r.u32();
+      }
+      in.length = r.u64();
+      if (!r.ok()) {
+        failProtocol();
+        return;
+      }
+      inbox_.push_back(in);
+      advanceRecvs();
+    } else {
+      failProtocol();
+      return;
+    }
+    if (!ready_ && gotHello_ && gotHelloAck_) {
+      ready_ = true;
+      TP_VLOG(5) << "Channel " << id_ << " ready: chunk " << chunkBytes_ << " B, ring route "
+                 << (peerMappedOurRing_ ? "on" : "off") << " for sends, "
+                 << (remoteRing_ != nullptr ? "on" : "off") << " for recvs";
+      auto deferred = std::move(deferred_);
+      deferred_.clear();
+      for (auto& fn : deferred) {
+        fn();
+      }
+    }
+  }
+
+  void failProtocol() {
+    setError(TP_CREATE_ERROR(ShortReadError, -1, -1));
+  }
+
+  // ---- send -------------------------------------------------------------------
 
   void startSend(const std::shared_ptr<Op>& op) {
     if (error_) {
       return;
+    }
+    const bool cpuSource = isCpu(op->buffer);
+    const bool ring = !cpuSource && peerMappedOurRing_;
+    {
+      // The route message takes its place in the queue: it must reach the peer
+      // after the last notification of the previous tensor.
+      auto marker = std::make_shared<SendChunk>();
+      marker->isRoute = true;
+      marker->ring = ring;
+      marker->length = op->length;
+      marker->ready = true;
+      sendQueue_.push_back(marker);
     }
     const size_t chunks = (op->length + chunkBytes_ - 1) / chunkBytes_;
     op->pending = chunks; // chunks whose source bytes are still needed
@@ -238,8 +416,9 @@ class ChannelImpl final : public ChannelImplBase {
       auto chunk = std::make_shared<SendChunk>();
       chunk->length = len;
       chunk->op = op;
+      chunk->ring = ring;
       sendQueue_.push_back(chunk);
-      if (isCpu(op->buffer)) {
+      if (cpuSource) {
         // Host source: no staging (tensorpipe/channel/cuda_basic/channel_impl.cc:138-145).
         chunk->hostPtr = static_cast<uint8_t*>(op->buffer.unwrap<CpuBuffer>().ptr) + offset;
         chunk->ready = true;
@@ -247,9 +426,9 @@ class ChannelImpl final : public ChannelImplBase {
       }
       const HipBuffer hb = op->buffer.unwrap<HipBuffer>();
       auto self = shared_from_this();
-      PinnedRing& ring = bctx_->sendRing();
-      ring.allocator.alloc([this, self, chunk, hb, offset, len, &ring](
-                               const Error& error, SlotAllocator::TSlot slot) {
+      PinnedRing& sring = bctx_->sendRing();
+      sring.allocator.alloc([this, self, chunk, hb, offset, len, &sring](
+                                const Error& error, SlotAllocator::TSlot slot) {
         if (error) {
           setError(error);
           return;
@@ -260,9 +439,10 @@ class ChannelImpl final : public ChannelImplBase {
         chunk->slot = std::move(slot);
         chunk->hostPtr = chunk->slot.get();
         const int device = hipDeviceForPointer(hb.ptr);
+        TP_VLOG(7) << "Channel " << id_ << " stages " << len << " B at offset " << offset;
         int rc = tphip_copy(
             device,
-            ring.devAddress(chunk->slot.get()),
+            sring.devAddress(chunk->slot.get()),
             static_cast<const uint8_t*>(hb.ptr) + offset,
             len,
             hb.stream);
@@ -285,11 +465,34 @@ class ChannelImpl final : public ChannelImplBase {
     while (!sendQueue_.empty() && sendQueue_.front()->ready && !error_) {
       auto chunk = sendQueue_.front();
       sendQueue_.pop_front();
+      if (chunk->isRoute) {
+        WireWriter w;
+        w.u8(kRoute);
+        w.u8(chunk->ring ? kRouteRing : kRouteInner);
+        w.u64(chunk->length);
+        writeMessage(*controlConnection_, std::move(w.bytes()));
+        continue;
+      }
+      if (chunk->ring) {
+        // The bytes sit in our pinned ring, which the peer's GPU has mapped:
+        // tell it where; the slot comes back with the ack.
+        const uint32_t slotIdx =
+            static_cast<uint32_t>(bctx_->sendRing().allocator.slotIndex(chunk->slot.get()));
+        slotsInFlight_[slotIdx] = std::move(chunk->slot);
+        TP_VLOG(7) << "Channel " << id_ << " notifies slot " << slotIdx << " (" << chunk->length
+                   << " B)";
+        WireWriter w;
+        w.u8(kNotify);
+        w.u32(slotIdx);
+        w.u64(chunk->length);
+        writeMessage(*controlConnection_, std::move(w.bytes()));
+        sourceDone(chunk->op);
+        continue;
+      }
       auto self = shared_from_this();
       const bool staged = static_cast<bool>(chunk->slot);
       if (staged) {
-        // The bytes now live in the pinned slot: the source is free.
-        sourceDone(chunk->op);
+        sourceDone(chunk->op); // the bytes now live in the pinned slot
       }
       cpuChannel_->send(
           CpuBuffer{chunk->hostPtr}, chunk->length, [this, self, chunk, staged](const Error& error) {
@@ -312,14 +515,122 @@ class ChannelImpl final : public ChannelImplBase {
     finish(op);
   }
 
-  // ---- recv -----------------------------------------------------------------
+  // ---- recv -------------------------------------------------------------------
 
-  void startRecv(const std::shared_ptr<Op>& op) {
+  // Feed control messages to the recv ops, strictly in order.
+  void advanceRecvs() {
+    while (ready_ && !error_ && !recvOps_.empty() && !inbox_.empty()) {
+      auto op = recvOps_.front();
+      const Incoming in = inbox_.front();
+      if (!op->routed) {
+        if (in.kind != kRoute || in.length != op->length) {
+          failProtocol();
+          return;
+        }
+        inbox_.pop_front();
+        op->routed = true;
+        op->route = in.route;
+        const size_t chunks = (op->length + chunkBytes_ - 1) / chunkBytes_;
+        op->pending = chunks; // chunks not yet landed (CPU) / enqueued (GPU)
+        if (op->route == kRouteInner) {
+          recvOps_.pop_front();
+          startInnerRecv(op);
+        } else if (remoteRing_ == nullptr) {
+          failProtocol();
+          return;
+        }
+        continue;
+      }
+      // Ring route: one notification per chunk.
+      if (in.kind != kNotify) {
+        failProtocol();
+        return;
+      }
+      inbox_.pop_front();
+      const size_t offset = op->received;
+      const size_t expect = std::min<size_t>(op->length - offset, chunkBytes_);
+      if (in.length != expect || in.slot >= remoteNumSlots_) {
+        failProtocol();
+        return;
+      }
+      op->received += in.length;
+      if (op->received == op->length) {
+        recvOps_.pop_front();
+      }
+      ringChunkArrived(op, in.slot, offset, in.length);
+    }
+  }
+
+  void ringChunkArrived(const std::shared_ptr<Op>& op, uint32_t slot, size_t offset, size_t len) {
+    const uint8_t* remote = remoteRing_ + static_cast<size_t>(slot) * remoteSlotBytes_;
+    TP_VLOG(7) << "Channel " << id_ << " got notification for slot " << slot << " (" << len
+               << " B)";
+    if (!isCpu(op->buffer)) {
+      const HipBuffer hb = op->buffer.unwrap<HipBuffer>();
+      const int device = hipDeviceForPointer(hb.ptr);
+      int rc = tphip_copy(device, static_cast<uint8_t*>(hb.ptr) + offset, remote, len, hb.stream);
+      if (rc != 0) {
+        setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+        return;
+      }
+      auto ev = bctx_->events.get(device);
+      ev->record(hb.stream);
+      watch(std::move(ev), [this, slot] { ackSlot(slot); });
+      chunkLanded(op);
+      return;
+    }
+    // CPU target: the mapping of the peer's ring is only addressable by the
+    // GPU, so the GPU moves the chunk into a local pinned slot first.
+    auto self = shared_from_this();
+    PinnedRing& rring = bctx_->recvRing();
+    rring.allocator.alloc([this, self, op, remote, slot, offset, len, &rring](
+                              const Error& error, SlotAllocator::TSlot local) {
+      if (error) {
+        setError(error);
+        return;
+      }
+      if (error_) {
+        return;
+      }
+      void* stream = nullptr;
+      try {
+        stream = bctx_->internalStream();
+      } catch (const std::exception&) {
+        setError(TP_CREATE_ERROR(HipError, "tphip_stream_create", TPHIP_ERR_INVALID_ARG));
+        return;
+      }
+      int rc = tphip_copy(0, rring.devAddress(local.get()), remote, len, stream);
+      if (rc != 0) {
+        setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+        return;
+      }
+      auto ev = bctx_->events.get(0);
+      ev->record(stream);
+      watch(std::move(ev), [this, op, slot, offset, len, local] {
+        if (error_) {
+          return;
+        }
+        ackSlot(slot);
+        std::memcpy(
+            static_cast<uint8_t*>(op->buffer.unwrap<CpuBuffer>().ptr) + offset, local.get(), len);
+        chunkLanded(op);
+      });
+    });
+  }
+
+  void ackSlot(uint32_t slot) {
     if (error_) {
       return;
     }
+    TP_VLOG(7) << "Channel " << id_ << " acks slot " << slot;
+    WireWriter w;
+    w.u8(kAck);
+    w.u32(slot);
+    writeMessage(*controlConnection_, std::move(w.bytes()));
+  }
+
+  void startInnerRecv(const std::shared_ptr<Op>& op) {
     const size_t chunks = (op->length + chunkBytes_ - 1) / chunkBytes_;
-    op->pending = chunks; // chunks not yet landed (CPU) / not yet enqueued (GPU)
     for (size_t k = 0; k < chunks; ++k) {
       const size_t offset = k * chunkBytes_;
       const size_t len = std::min<size_t>(op->length - offset, chunkBytes_);
@@ -327,7 +638,7 @@ class ChannelImpl final : public ChannelImplBase {
       chunk->length = len;
       chunk->offset = offset;
       chunk->op = op;
-      recvQueue_.push_back(chunk);
+      recvPostQueue_.push_back(chunk);
       if (isCpu(op->buffer)) {
         chunk->hostPtr = static_cast<uint8_t*>(op->buffer.unwrap<CpuBuffer>().ptr) + offset;
         chunk->ready = true;
@@ -355,47 +666,45 @@ class ChannelImpl final : public ChannelImplBase {
   // Inner recvs are posted strictly in chunk order (the inner channel pairs
   // sends and recvs by position), each as soon as its landing area exists.
   void flushRecvPosts() {
-    while (!recvQueue_.empty() && recvQueue_.front()->ready && !error_) {
-      auto chunk = recvQueue_.front();
-      recvQueue_.pop_front();
-      postInnerRecv(chunk->hostPtr, chunk->length, [this, chunk] {
-        if (!chunk->slot) {
-          chunkLanded(chunk->op); // host target: the bytes are where they belong
-          return;
-        }
-        const HipBuffer hb = chunk->op->buffer.unwrap<HipBuffer>();
-        PinnedRing& ring = bctx_->recvRing();
-        const int device = hipDeviceForPointer(hb.ptr);
-        int rc = tphip_copy(
-            device,
-            static_cast<uint8_t*>(hb.ptr) + chunk->offset,
-            ring.devAddress(chunk->slot.get()),
-            chunk->length,
-            hb.stream);
-        if (rc != 0) {
-          setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
-          return;
-        }
-        auto ev = bctx_->events.get(device);
-        ev->record(hb.stream);
-        // The slot goes back to the ring when the copy has read it.
-        watch(std::move(ev), [chunk] { chunk->slot.reset(); });
-        chunkLanded(chunk->op);
-      });
+    while (!recvPostQueue_.empty() && recvPostQueue_.front()->ready && !error_) {
+      auto chunk = recvPostQueue_.front();
+      recvPostQueue_.pop_front();
+      auto self = shared_from_this();
+      cpuChannel_->recv(
+          CpuBuffer{chunk->hostPtr}, chunk->length, [this, self, chunk](const Error& error) {
+            ctx_->defer([this, self, chunk, error] {
+              setError(error);
+              if (!error_) {
+                innerChunkArrived(chunk);
+              }
+            });
+          });
     }
   }
 
-  template <typename F>
-  void postInnerRecv(void* host, size_t len, F fn) {
-    auto self = shared_from_this();
-    cpuChannel_->recv(CpuBuffer{host}, len, [this, self, fn{std::move(fn)}](const Error& error) mutable {
-      ctx_->defer([this, self, fn{std::move(fn)}, error]() mutable {
-        setError(error);
-        if (!error_) {
-          fn();
-        }
-      });
-    });
+  void innerChunkArrived(const std::shared_ptr<RecvChunk>& chunk) {
+    if (!chunk->slot) {
+      chunkLanded(chunk->op); // host target: the bytes are where they belong
+      return;
+    }
+    const HipBuffer hb = chunk->op->buffer.unwrap<HipBuffer>();
+    PinnedRing& rring = bctx_->recvRing();
+    const int device = hipDeviceForPointer(hb.ptr);
+    int rc = tphip_copy(
+        device,
+        static_cast<uint8_t*>(hb.ptr) + chunk->offset,
+        rring.devAddress(chunk->slot.get()),
+        chunk->length,
+        hb.stream);
+    if (rc != 0) {
+      setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+      return;
+    }
+    auto ev = bctx_->events.get(device);
+    ev->record(hb.stream);
+    // The slot goes back to the ring when the copy has read it.
+    watch(std::move(ev), [chunk] { chunk->slot.reset(); });
+    chunkLanded(chunk->op);
   }
 
   void chunkLanded(const std::shared_ptr<Op>& op) {
@@ -406,7 +715,7 @@ class ChannelImpl final : public ChannelImplBase {
     finish(op);
   }
 
-  // ---- helpers ----------------------------------------------------------------
+  // ---- helpers ------------------------------------------------------------------
 
   template <typename F>
   void watch(std::unique_ptr<HipEvent> ev, F fn) {
@@ -441,11 +750,21 @@ class ChannelImpl final : public ChannelImplBase {
   std::shared_ptr<BasicContextCore> bctx_;
   std::shared_ptr<transport::Connection> controlConnection_;
   std::shared_ptr<Channel> cpuChannel_;
+  bool gotHello_{false};
+  bool gotHelloAck_{false};
+  bool ready_{false};
   uint64_t chunkBytes_{0};
+  uint64_t remoteSlotBytes_{0};
+  uint64_t remoteNumSlots_{0};
+  uint8_t* remoteRing_{nullptr};  // peer's send ring as mapped by our GPU
+  bool peerMappedOurRing_{false}; // peer can read our send ring
   std::vector<std::function<void()>> deferred_;
   std::deque<std::shared_ptr<Op>> ops_;
+  std::deque<std::shared_ptr<Op>> recvOps_; // not yet fully routed / notified
+  std::deque<Incoming> inbox_;
   std::deque<std::shared_ptr<SendChunk>> sendQueue_;
-  std::deque<std::shared_ptr<RecvChunk>> recvQueue_;
+  std::deque<std::shared_ptr<RecvChunk>> recvPostQueue_;
+  std::map<uint32_t, SlotAllocator::TSlot> slotsInFlight_;
 };
 
 class ContextImpl final : public Context {

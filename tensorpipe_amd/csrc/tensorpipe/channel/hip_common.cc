@@ -119,6 +119,29 @@ void HipEventPoller::run() {
   }
 }
 
+HipIpcImports& HipIpcImports::get() {
+  static HipIpcImports* r = new HipIpcImports();
+  return *r;
+}
+
+int HipIpcImports::open(int device, const HandleBytes& handle, void** out) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  auto key = std::make_pair(device, handle);
+  auto it = opened_.find(key);
+  if (it != opened_.end()) {
+    *out = it->second;
+    return 0;
+  }
+  void* ptr = nullptr;
+  int rc = tphip_ipc_mem_open(device, handle.data(), &ptr);
+  if (rc != 0) {
+    return rc;
+  }
+  opened_[key] = ptr;
+  *out = ptr;
+  return 0;
+}
+
 void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table) {
   size_t off = 0;
   while (off < table.size()) {

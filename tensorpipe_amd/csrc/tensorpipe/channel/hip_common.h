@@ -3,9 +3,11 @@
 // turns a list of (src, dst, bytes) into ONE batched copy launch.
 #pragma once
 
+#include <array>
 #include <condition_variable>
 #include <deque>
 #include <functional>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -57,6 +59,24 @@ class HipEventPoller {
   std::deque<Item> incoming_;
   bool stopping_{false};
   std::thread thread_;
+};
+
+using HandleBytes = std::array<uint8_t, TPHIP_IPC_HANDLE_BYTES>;
+
+// Allocations of other processes mapped into this one, keyed by device and
+// handle bytes. Mappings stay open for the life of the process: opening takes
+// about 0.2 ms, a handle may be shared by several channels, and the reference
+// keeps its opened handles until the context closes for the same reasons
+// (tensorpipe/channel/cuda_ipc/context_impl.cc:388-418).
+class HipIpcImports {
+ public:
+  static HipIpcImports& get();
+  // Returns a tphip error code.
+  int open(int device, const HandleBytes& handle, void** out);
+
+ private:
+  std::mutex mutex_;
+  std::map<std::pair<int, HandleBytes>, void*> opened_;
 };
 
 // Enqueue one batched copy on (device, stream); throws on a failed launch.

@@ -55,8 +55,6 @@ constexpr size_t kSlotSize = 8 * 1024 * 1024;
 constexpr size_t kNumSlots = 4;
 constexpr size_t kStagingAreaSize = kSlotSize * kNumSlots;
 
-using HandleBytes = std::array<uint8_t, TPHIP_IPC_HANDLE_BYTES>;
-
 // Read when a context is created, so that one process can host contexts of
 // both kinds.
 bool outboxForcedByEnv() {
@@ -114,39 +112,6 @@ class ExportRegistry {
   std::mutex mutex_;
   std::map<void*, ExportedAllocation> exports_;
   uint64_t nextId_{1};
-};
-
-// Allocations of other processes mapped into this one, keyed by handle bytes.
-// Mappings stay open for the life of the process (opening is ~0.2 ms, and a
-// handle may be shared by several channels).
-class ImportRegistry {
- public:
-  static ImportRegistry& get() {
-    static ImportRegistry* r = new ImportRegistry();
-    return *r;
-  }
-
-  int open(int device, const HandleBytes& handle, void** out) {
-    std::lock_guard<std::mutex> lock(mutex_);
-    auto key = std::make_pair(device, handle);
-    auto it = opened_.find(key);
-    if (it != opened_.end()) {
-      *out = it->second;
-      return 0;
-    }
-    void* ptr = nullptr;
-    int rc = tphip_ipc_mem_open(device, handle.data(), &ptr);
-    if (rc != 0) {
-      return rc;
-    }
-    opened_[key] = ptr;
-    *out = ptr;
-    return 0;
-  }
-
- private:
-  std::mutex mutex_;
-  std::map<std::pair<int, HandleBytes>, void*> opened_;
 };
 
 // Per-device staging slab of the outbox path, created on first use.
@@ -569,7 +534,7 @@ class ChannelImpl final : public ChannelImplBase {
             HandleBytes h;
             r.raw(h.data(), h.size());
             void* mapped = nullptr;
-            int rc = ImportRegistry::get().open(device, h, &mapped);
+            int rc = HipIpcImports::get().open(device, h, &mapped);
             if (rc != 0) {
               setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
               return;
@@ -618,7 +583,7 @@ class ChannelImpl final : public ChannelImplBase {
           HandleBytes h;
           r.raw(h.data(), h.size());
           void* mapped = nullptr;
-          int rc = ImportRegistry::get().open(device, h, &mapped);
+          int rc = HipIpcImports::get().open(device, h, &mapped);
           if (rc != 0) {
             setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
             return;

@@ -263,6 +263,32 @@ def basic_peer():
     peer.close()
 
 
+@pytest.fixture(scope="module")
+def basic_inner_peer():
+    # the reference's route for every chunk: through the wrapped CPU channel
+    os.environ["TP_HIP_BASIC_NO_SHARED_RING"] = "1"
+    try:
+        peer = Peer("basic:0,hip_basic:10", env={"TP_HIP_BASIC_NO_SHARED_RING": "1"})
+    finally:
+        del os.environ["TP_HIP_BASIC_NO_SHARED_RING"]
+    yield peer
+    peer.close()
+
+
+@pytest.fixture(scope="module")
+def basic_small_ring_peer():
+    # 4-deep ring of 64 KiB slots: many chunks per tensor, constant slot reuse
+    env = {"TP_HIP_BASIC_SLOT_BYTES": str(64 << 10), "TP_HIP_BASIC_NUM_SLOTS": "4"}
+    os.environ.update(env)
+    try:
+        peer = Peer("basic:0,hip_basic:10", env=env)
+    finally:
+        for k in env:
+            del os.environ[k]
+    yield peer
+    peer.close()
+
+
 def _ipc_cases(oracle, peer, slot, sizes):
     for k, n in enumerate(sizes):
         host = datagen.normal(datagen.SEED_BASE + 3 + k, max(n // 4, 1), "f32").view(np.uint8)
@@ -322,14 +348,33 @@ def test_ipc_refuses_same_process():
         o.destroy()
 
 
-def test_basic_staged_sizes(oracle, basic_peer):
-    for k, n in enumerate([1024, 1 << 20, (1 << 20) + 1, (5 << 20) + 3, 40 << 20, 1, 0]):
+def _staged_cases(oracle, peer, sizes, slot=1 << 20, num_slots=16):
+    for k, n in enumerate(sizes):
         host = datagen.normal(datagen.SEED_BASE + 4 + k, max((n + 1) // 2, 1), "bf16").view(np.uint8)
         src = _gpu(host)
-        outs, _ = basic_peer.echo([tp.make_tensor(src, nbytes=n, target=(tp.HIP, 0))], "gpu")
+        outs, _ = peer.echo([tp.make_tensor(src, nbytes=n, target=(tp.HIP, 0))], "gpu")
         ref = np.full(n, FILL, np.uint8)
-        oracle.staged_tensor(host, ref, n)
+        oracle.staged_tensor(host, ref, n, slot=slot, num_slots=num_slots)
         _check_echo(outs[0], ref, n)
+
+
+def test_basic_staged_sizes(oracle, basic_peer):
+    _staged_cases(oracle, basic_peer, [1024, 1 << 20, (1 << 20) + 1, (5 << 20) + 3, 40 << 20, 1, 0])
+
+
+def test_basic_staged_inner_route(oracle, basic_inner_peer):
+    _staged_cases(oracle, basic_inner_peer, [1024, (1 << 20) + 1, (20 << 20) + 3, 1, 0])
+
+
+def test_basic_staged_small_ring(oracle, basic_small_ring_peer):
+    _staged_cases(oracle, basic_small_ring_peer, [1024, (64 << 10) + 1, (3 << 20) + 5, 17],
+                  slot=64 << 10, num_slots=4)
+    # several tensors in one message share the 4 slots
+    hosts = [datagen.uniform_u8(200 + i, (300 << 10) + i) for i in range(5)]
+    outs, _ = basic_small_ring_peer.echo(
+        [tp.make_tensor(_gpu(h), target=(tp.HIP, 0)) for h in hosts], "gpu")
+    for o, h in zip(outs, hosts):
+        _check_echo(o, h, h.size)
 
 
 def test_basic_cross_device_types(oracle, basic_peer):
