@@ -231,6 +231,8 @@ class ChannelImpl final : public ChannelImplBase {
     recvOps_.clear();
     inbox_.clear();
     slotsInFlight_.clear();
+    stagePending_.clear();
+    ringPending_.clear();
     auto ops = std::move(ops_);
     ops_.clear();
     for (auto& op : ops) {
@@ -271,6 +273,23 @@ class ChannelImpl final : public ChannelImplBase {
     SlotAllocator::TSlot slot;
     bool ready{false};
     std::shared_ptr<Op> op;
+  };
+
+  // A staging copy (GPU -> ring slot) waiting to be launched.
+  struct StageItem {
+    std::shared_ptr<SendChunk> chunk;
+    tphip_copy_desc desc;
+    void* stream;
+    int device;
+  };
+
+  // A ring-route copy (peer's ring slot -> GPU) waiting to be launched.
+  struct RingItem {
+    std::shared_ptr<Op> op;
+    uint32_t slot;
+    tphip_copy_desc desc;
+    void* stream;
+    int device;
   };
 
   // A control message for the receive side, kept until a recv op consumes it.
@@ -346,28 +365,41 @@ class ChannelImpl final : public ChannelImplBase {
       peerMappedOurRing_ = r.u8() != 0;
       gotHelloAck_ = true;
     } else if (kind == kAck) {
-      const uint32_t slot = r.u32();
-      auto it = slotsInFlight_.find(slot);
-      if (!r.ok() || it == slotsInFlight_.end()) {
-        failProtocol();
-        return;
+      const uint32_t count = r.u32();
+      for (uint32_t i = 0; i < count; ++i) {
+        const uint32_t slot = r.u32();
+        auto it = slotsInFlight_.find(slot);
+        if (!r.ok() || it == slotsInFlight_.end()) {
+          failProtocol();
+          return;
+        }
+        TP_VLOG(7) << "Channel " << id_ << " got ack for slot " << slot;
+        slotsInFlight_.erase(it); // drops the slot back into the ring
       }
-      TP_VLOG(7) << "Channel " << id_ << " got ack for slot " << slot;
-      slotsInFlight_.erase(it); // drops the slot back into the ring
-    } else if (kind == kRoute || kind == kNotify) {
+    } else if (kind == kRoute) {
       Incoming in{};
       in.kind = kind;
-      if (kind == kRoute) {
-        in.route = r.u8();
-      } else {
-        in.slot = r.u32();
-      }
+      in.route = r.u8();
       in.length = r.u64();
       if (!r.ok()) {
         failProtocol();
         return;
       }
       inbox_.push_back(in);
+      advanceRecvs();
+    } else if (kind == kNotify) {
+      const uint32_t count = r.u32();
+      for (uint32_t i = 0; i < count; ++i) {
+        Incoming in{};
+        in.kind = kind;
+        in.slot = r.u32();
+        in.length = r.u64();
+        if (!r.ok()) {
+          failProtocol();
+          return;
+        }
+        inbox_.push_back(in);
+      }
       advanceRecvs();
     } else {
       failProtocol();
@@ -438,34 +470,122 @@ class ChannelImpl final : public ChannelImplBase {
         }
         chunk->slot = std::move(slot);
         chunk->hostPtr = chunk->slot.get();
-        const int device = hipDeviceForPointer(hb.ptr);
         TP_VLOG(7) << "Channel " << id_ << " stages " << len << " B at offset " << offset;
-        int rc = tphip_copy(
-            device,
-            sring.devAddress(chunk->slot.get()),
-            static_cast<const uint8_t*>(hb.ptr) + offset,
-            len,
-            hb.stream);
-        if (rc != 0) {
-          setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
-          return;
-        }
-        auto ev = bctx_->events.get(device);
-        ev->record(hb.stream);
-        watch(std::move(ev), [this, chunk] {
-          chunk->ready = true;
-          flushSends();
-        });
+        // Launched together with every other chunk that gets its slot in this
+        // turn of the loop: one kernel and one event for all of them.
+        stagePending_.push_back(StageItem{
+            chunk,
+            tphip_copy_desc{
+                static_cast<const uint8_t*>(hb.ptr) + offset,
+                sring.devAddress(chunk->slot.get()),
+                len},
+            hb.stream,
+            hipDeviceForPointer(hb.ptr)});
+        scheduleLaunches();
       });
     }
     flushSends();
   }
 
+  // Copies queued during one turn of the loop are launched together at its
+  // end: a burst of freed slots or of notifications costs one kernel launch
+  // and one event per stream instead of one per chunk.
+  void scheduleLaunches() {
+    if (launchScheduled_) {
+      return;
+    }
+    launchScheduled_ = true;
+    auto self = shared_from_this();
+    ctx_->defer([this, self] {
+      launchScheduled_ = false;
+      if (error_) {
+        stagePending_.clear();
+        ringPending_.clear();
+        return;
+      }
+      launchStaging();
+      launchRingCopies();
+    });
+  }
+
+  void launchStaging() {
+    while (!stagePending_.empty()) {
+      // One launch per (device, stream); normally there is only one.
+      void* stream = stagePending_.front().stream;
+      const int device = stagePending_.front().device;
+      std::vector<tphip_copy_desc> table;
+      std::vector<std::shared_ptr<SendChunk>> chunks;
+      const size_t cap = batchCap(bctx_->numSlots);
+      for (auto it = stagePending_.begin(); it != stagePending_.end() && table.size() < cap;) {
+        if (it->stream == stream && it->device == device) {
+          table.push_back(it->desc);
+          chunks.push_back(std::move(it->chunk));
+          it = stagePending_.erase(it);
+        } else {
+          ++it;
+        }
+      }
+      if (!launchHostLinkCopy(device, stream, table)) {
+        return;
+      }
+      auto ev = bctx_->events.get(device);
+      ev->record(stream);
+      watch(std::move(ev), [this, chunks{std::move(chunks)}] {
+        for (auto& c : chunks) {
+          c->ready = true;
+        }
+        flushSends();
+      });
+    }
+  }
+
+  // Chunks per launch. One launch for the whole ring would put the two ends in
+  // lock step (the sender stages all slots, then idles while the receiver
+  // drains all of them); half the ring (a quarter for deep rings) lets one end
+  // fill slots while the other drains the rest.
+  static size_t batchCap(size_t numSlots) {
+    const size_t quarter = std::max<size_t>(numSlots / 4, 2);
+    return std::max<size_t>(1, std::min(numSlots / 2, quarter));
+  }
+
+  // A copy with one end in pinned host memory: the host link saturates with
+  // about 32 workgroups, more only add contention (50 vs 42 GB/s reading).
+  bool launchHostLinkCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table) {
+    size_t off = 0;
+    while (off < table.size()) {
+      const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
+      int rc = tphip_batched_copy_tuned(
+          device, table.data() + off, static_cast<uint32_t>(n), stream, 4, 32, 3);
+      if (rc != 0) {
+        setError(TP_CREATE_ERROR(HipError, "tphip_batched_copy", rc));
+        return false;
+      }
+      off += n;
+    }
+    return true;
+  }
+
   void flushSends() {
+    std::vector<std::pair<uint32_t, uint64_t>> notifies;
+    auto flushNotifies = [&] {
+      if (notifies.empty()) {
+        return;
+      }
+      WireWriter w;
+      w.u8(kNotify);
+      w.u32(static_cast<uint32_t>(notifies.size()));
+      for (auto& n : notifies) {
+        w.u32(n.first);
+        w.u64(n.second);
+      }
+      writeMessage(*controlConnection_, std::move(w.bytes()));
+      notifies.clear();
+    };
     while (!sendQueue_.empty() && sendQueue_.front()->ready && !error_) {
       auto chunk = sendQueue_.front();
       sendQueue_.pop_front();
       if (chunk->isRoute) {
+        flushNotifies();
         WireWriter w;
         w.u8(kRoute);
         w.u8(chunk->ring ? kRouteRing : kRouteInner);
@@ -481,14 +601,11 @@ class ChannelImpl final : public ChannelImplBase {
         slotsInFlight_[slotIdx] = std::move(chunk->slot);
         TP_VLOG(7) << "Channel " << id_ << " notifies slot " << slotIdx << " (" << chunk->length
                    << " B)";
-        WireWriter w;
-        w.u8(kNotify);
-        w.u32(slotIdx);
-        w.u64(chunk->length);
-        writeMessage(*controlConnection_, std::move(w.bytes()));
+        notifies.emplace_back(slotIdx, chunk->length);
         sourceDone(chunk->op);
         continue;
       }
+      flushNotifies();
       auto self = shared_from_this();
       const bool staged = static_cast<bool>(chunk->slot);
       if (staged) {
@@ -505,6 +622,7 @@ class ChannelImpl final : public ChannelImplBase {
             });
           });
     }
+    flushNotifies();
   }
 
   void sourceDone(const std::shared_ptr<Op>& op) {
@@ -567,16 +685,13 @@ class ChannelImpl final : public ChannelImplBase {
                << " B)";
     if (!isCpu(op->buffer)) {
       const HipBuffer hb = op->buffer.unwrap<HipBuffer>();
-      const int device = hipDeviceForPointer(hb.ptr);
-      int rc = tphip_copy(device, static_cast<uint8_t*>(hb.ptr) + offset, remote, len, hb.stream);
-      if (rc != 0) {
-        setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
-        return;
-      }
-      auto ev = bctx_->events.get(device);
-      ev->record(hb.stream);
-      watch(std::move(ev), [this, slot] { ackSlot(slot); });
-      chunkLanded(op);
+      ringPending_.push_back(RingItem{
+          op,
+          slot,
+          tphip_copy_desc{remote, static_cast<uint8_t*>(hb.ptr) + offset, len},
+          hb.stream,
+          hipDeviceForPointer(hb.ptr)});
+      scheduleLaunches();
       return;
     }
     // CPU target: the mapping of the peer's ring is only addressable by the
@@ -618,14 +733,52 @@ class ChannelImpl final : public ChannelImplBase {
     });
   }
 
+  void launchRingCopies() {
+    while (!ringPending_.empty()) {
+      void* stream = ringPending_.front().stream;
+      const int device = ringPending_.front().device;
+      std::vector<tphip_copy_desc> table;
+      std::vector<uint32_t> slots;
+      std::vector<std::shared_ptr<Op>> ops;
+      const size_t cap = batchCap(remoteNumSlots_);
+      for (auto it = ringPending_.begin(); it != ringPending_.end() && table.size() < cap;) {
+        if (it->stream == stream && it->device == device) {
+          table.push_back(it->desc);
+          slots.push_back(it->slot);
+          ops.push_back(std::move(it->op));
+          it = ringPending_.erase(it);
+        } else {
+          ++it;
+        }
+      }
+      if (!launchHostLinkCopy(device, stream, table)) {
+        return;
+      }
+      auto ev = bctx_->events.get(device);
+      ev->record(stream);
+      // The slots go back to the sender when the copy has read them.
+      watch(std::move(ev), [this, slots{std::move(slots)}] { ackSlots(slots); });
+      for (auto& op : ops) {
+        chunkLanded(op); // enqueued on the caller's stream
+      }
+    }
+  }
+
   void ackSlot(uint32_t slot) {
+    ackSlots(std::vector<uint32_t>{slot});
+  }
+
+  void ackSlots(const std::vector<uint32_t>& slots) {
     if (error_) {
       return;
     }
-    TP_VLOG(7) << "Channel " << id_ << " acks slot " << slot;
     WireWriter w;
     w.u8(kAck);
-    w.u32(slot);
+    w.u32(static_cast<uint32_t>(slots.size()));
+    for (uint32_t slot : slots) {
+      TP_VLOG(7) << "Channel " << id_ << " acks slot " << slot;
+      w.u32(slot);
+    }
     writeMessage(*controlConnection_, std::move(w.bytes()));
   }
 
@@ -690,14 +843,13 @@ class ChannelImpl final : public ChannelImplBase {
     const HipBuffer hb = chunk->op->buffer.unwrap<HipBuffer>();
     PinnedRing& rring = bctx_->recvRing();
     const int device = hipDeviceForPointer(hb.ptr);
-    int rc = tphip_copy(
-        device,
-        static_cast<uint8_t*>(hb.ptr) + chunk->offset,
-        rring.devAddress(chunk->slot.get()),
-        chunk->length,
-        hb.stream);
-    if (rc != 0) {
-      setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+    if (!launchHostLinkCopy(
+            device,
+            hb.stream,
+            {tphip_copy_desc{
+                rring.devAddress(chunk->slot.get()),
+                static_cast<uint8_t*>(hb.ptr) + chunk->offset,
+                chunk->length}})) {
       return;
     }
     auto ev = bctx_->events.get(device);
@@ -765,6 +917,9 @@ class ChannelImpl final : public ChannelImplBase {
   std::deque<std::shared_ptr<SendChunk>> sendQueue_;
   std::deque<std::shared_ptr<RecvChunk>> recvPostQueue_;
   std::map<uint32_t, SlotAllocator::TSlot> slotsInFlight_;
+  std::vector<StageItem> stagePending_;
+  std::vector<RingItem> ringPending_;
+  bool launchScheduled_{false};
 };
 
 class ContextImpl final : public Context {

@@ -464,6 +464,7 @@ class ChannelImpl final : public ChannelImplBase {
     while (!wireQueue_.empty() && wireQueue_.front()->ready && !error_) {
       auto unit = wireQueue_.front();
       wireQueue_.pop_front();
+      TP_VLOG(6) << "Channel " << id_ << " is writing a descriptor";
       writeMessage(*descriptorConnection_, std::move(unit->bytes));
       replyConnection_->read(nullptr, 0, onRead([this, unit] {
         if (!error_ && unit->onReply) {
@@ -508,6 +509,8 @@ class ChannelImpl final : public ChannelImplBase {
   void onUnit(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
     WireReader r(bytes.data(), bytes.size());
     const uint8_t kind = r.u8();
+    TP_VLOG(6) << "Channel " << id_ << " got a descriptor of kind " << int(kind) << " (#"
+               << op->seq << ")";
     auto reply = std::make_shared<ReplyUnit>();
     replyQueue_.push_back(reply);
     std::vector<StreamRef> touched;
@@ -627,6 +630,7 @@ class ChannelImpl final : public ChannelImplBase {
       return;
     }
 
+    TP_VLOG(6) << "Channel " << id_ << " enqueued the copies (#" << op->seq << ")";
     // Reply once the copies of this unit have finished.
     auto remaining = std::make_shared<size_t>(touched.size());
     for (auto& s : touched) {
@@ -652,6 +656,7 @@ class ChannelImpl final : public ChannelImplBase {
   void flushReplies() {
     while (!replyQueue_.empty() && replyQueue_.front()->ready && !error_) {
       replyQueue_.pop_front();
+      TP_VLOG(6) << "Channel " << id_ << " is writing a reply";
       replyConnection_->write(nullptr, 0, onWritten([] {}));
     }
   }

@@ -763,6 +763,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   void onPacket(std::vector<uint8_t> bytes) {
     WireReader r(bytes.data(), bytes.size());
     const uint8_t type = r.u8();
+    TP_VLOG(9) << "Pipe " << id_ << " got a packet of type " << int(type);
     if (type == kDescriptor) {
       auto op = std::make_shared<ReadOp>();
       op->seq = nextReadSeq_++;
@@ -850,6 +851,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       fn(error_);
       return;
     }
+    TP_VLOG(9) << "Pipe " << id_ << " received a read request";
     std::shared_ptr<ReadOp> op;
     for (auto& o : readOps_) {
       if (o->delivered && !o->readCalled) {
@@ -997,6 +999,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
     auto op = std::make_shared<WriteOp>();
     op->seq = nextWriteSeq_++;
+    TP_VLOG(9) << "Pipe " << id_ << " received a write request (#" << op->seq << ")";
     op->message = std::move(message);
     op->fn = std::move(fn);
     for (auto& t : op->message.tensors) {
@@ -1077,6 +1080,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   }
 
   void issueTensors(const std::shared_ptr<WriteOp>& op) {
+    TP_VLOG(9) << "Pipe " << id_ << " is sending tensors (#" << op->seq << ")";
     const Message& m = op->message;
     std::vector<std::pair<std::string, std::vector<size_t>>> groups;
     for (size_t i = 0; i < m.tensors.size(); ++i) {

@@ -371,8 +371,9 @@ def test_basic_staged_small_ring(oracle, basic_small_ring_peer):
                   slot=64 << 10, num_slots=4)
     # several tensors in one message share the 4 slots
     hosts = [datagen.uniform_u8(200 + i, (300 << 10) + i) for i in range(5)]
+    srcs = [_gpu(h) for h in hosts]  # must stay alive until the echo is back
     outs, _ = basic_small_ring_peer.echo(
-        [tp.make_tensor(_gpu(h), target=(tp.HIP, 0)) for h in hosts], "gpu")
+        [tp.make_tensor(s, target=(tp.HIP, 0)) for s in srcs], "gpu")
     for o, h in zip(outs, hosts):
         _check_echo(o, h, h.size)
 
@@ -386,7 +387,8 @@ def test_basic_cross_device_types(oracle, basic_peer):
     outs, _ = basic_peer.echo([tp.make_tensor(src, target=(tp.CPU, 0))], "cpu")
     _check_echo(outs[0], host, 1024)  # GPU -> CPU there, CPU -> GPU back
     big = datagen.uniform_u8(77, (3 << 20) + 5)
-    outs, _ = basic_peer.echo([tp.make_tensor(_gpu(big), target=(tp.CPU, 0)),
+    big_gpu = _gpu(big)
+    outs, _ = basic_peer.echo([tp.make_tensor(big_gpu, target=(tp.CPU, 0)),
                                tp.make_tensor(big, target=(tp.HIP, 0))], "cpu,gpu")
     _check_echo(outs[0], big, big.size)
     _check_echo(outs[1], big, big.size)
