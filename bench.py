@@ -89,10 +89,20 @@ def bench_d2d(steps, warmup):
     dst.zero_()
     torch.cuda.synchronize()
 
-    (per_us, total_s), launches, kernel_ms, kernel_bytes = profiled(
-        lambda: tp.bench_transfer(cpipe, spipe, st, rt, warmup=0, iters=steps), steps + 8)
+    # Timed region: K steps, nothing instrumented.
+    per_us, total_s = tp.bench_transfer(cpipe, spipe, st, rt, warmup=0, iters=steps)
     torch.cuda.synchronize()
     assert torch.equal(src, dst), "received bytes differ from sent bytes after the timed loop"
+
+    # The same K steps once more with every copy launch bracketed by the kernel's own
+    # start/stop events (the instrumented launch path costs host time, so it is kept out
+    # of the timed region above; the kernel and its arguments are identical).
+    dst.zero_()
+    torch.cuda.synchronize()
+    (prof_per_us, prof_total_s), launches, kernel_ms, kernel_bytes = profiled(
+        lambda: tp.bench_transfer(cpipe, spipe, st, rt, warmup=0, iters=steps), steps + 8)
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst), "received bytes differ from sent bytes after the profiled loop"
     assert launches == steps and kernel_bytes == steps * nbytes, (launches, kernel_bytes)
 
     # practical ceiling: the runtime's own D2D copy of the same size, same timing method
@@ -114,6 +124,7 @@ def bench_d2d(steps, warmup):
         "value": nbytes * steps / total_s / 1e9,
         "ms_per_step": total_s / steps * 1e3,
         "step_p50_us": float(per_us[int(0.5 * len(per_us))]),
+        "profiled_pass_ms_per_step": prof_total_s / steps * 1e3,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
@@ -151,7 +162,9 @@ def bench_rpc_message(messages=100, warmup=5):
     torch.cuda.synchronize()
     tp.bench_transfer(objs[0], objs[1], st, rt, payloads=[payload], recv_payloads=[pout],
                       warmup=0, iters=warmup)
-    (per_us, total_s), launches, kernel_ms, _ = profiled(
+    per_us, total_s = tp.bench_transfer(objs[0], objs[1], st, rt, payloads=[payload],
+                                        recv_payloads=[pout], warmup=0, iters=messages)
+    _, launches, kernel_ms, _ = profiled(
         lambda: tp.bench_transfer(objs[0], objs[1], st, rt, payloads=[payload],
                                   recv_payloads=[pout], warmup=0, iters=messages), messages + 8)
     torch.cuda.synchronize()
@@ -396,6 +409,7 @@ def main():
     d2d = bench_d2d(args.steps, args.warmup)
     extra = {
         "d2d_step_p50_us": d2d["step_p50_us"],
+        "d2d_profiled_pass_ms_per_step": d2d["profiled_pass_ms_per_step"],
         "hipMemcpyAsync_d2d_us": d2d["hipMemcpyAsync_d2d_us"],
         "hipMemcpyAsync_d2d_hbm_GBps": d2d["hipMemcpyAsync_d2d_hbm_GBps"],
     }

@@ -126,19 +126,42 @@ __device__ __forceinline__ void copy_edges(
   }
 }
 
+// Where the 16-byte aligned body of an entry starts (src + head, dst + head),
+// precomputed on the host.
+struct CopyBody {
+  const char* src;
+  char* dst;
+};
+
+// Entries whose bodies are also kept in LDS (16 B each) next to the prefix;
+// larger tables read them from global memory.
+constexpr uint32_t kLdsBodies = 1024;
+
 // Table variant. prefix[0..n] is the exclusive prefix sum of body vector
-// counts (prefix[n] = total). Dynamic LDS: (n+1) * 4 bytes.
+// counts (prefix[n] = total). Dynamic LDS: prefix padded to 16 B, then the
+// bodies if n <= kLdsBodies. A chunk's lookup then costs LDS reads only; a
+// dependent global load per chunk used to stall every workgroup for the best
+// part of a microsecond.
 template <int U, int NT>
 __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
     const uint32_t* __restrict__ prefix,
+    const CopyBody* __restrict__ bodies,
     const tphip_copy_desc* __restrict__ descs,
     uint32_t n,
     uint32_t nchunks) {
-  extern __shared__ uint32_t sPrefix[];
+  extern __shared__ __align__(16) uint32_t sPrefix[];
+  const bool cached = n <= kLdsBodies;
+  CopyBody* sBodies = reinterpret_cast<CopyBody*>(sPrefix + ((n + 1 + 3) & ~3u));
   for (uint32_t i = threadIdx.x; i <= n; i += kBlockThreads) {
     sPrefix[i] = prefix[i];
   }
+  if (cached) {
+    for (uint32_t i = threadIdx.x; i < n; i += kBlockThreads) {
+      sBodies[i] = bodies[i];
+    }
+  }
   __syncthreads();
+  const CopyBody* body = cached ? sBodies : bodies;
 
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t waveInBlock = threadIdx.x >> 6;
@@ -172,12 +195,9 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
     u32x4 v[U];
     if (cEnd <= tEnd) {
       // Whole chunk inside one entry: uniform base, contiguous addresses.
-      const char* src = static_cast<const char*>(descs[t].src);
-      char* dst = static_cast<char*>(descs[t].dst);
-      const uint64_t off =
-          static_cast<uint64_t>(c0 - tBegin) * 16 + head_bytes(dst, descs[t].bytes);
-      const char* s = src + off;
-      char* d = dst + off;
+      const uint64_t off = static_cast<uint64_t>(c0 - tBegin) * 16;
+      const char* s = body[t].src + off;
+      char* d = body[t].dst + off;
       const uint32_t cnt = cEnd - c0;
       if (cnt == kChunk) {
 #pragma unroll
@@ -221,12 +241,9 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
             h = m;
           }
         }
-        const char* src = static_cast<const char*>(descs[l].src);
-        char* dst = static_cast<char*>(descs[l].dst);
-        const uint64_t off =
-            static_cast<uint64_t>(vv - sPrefix[l]) * 16 + head_bytes(dst, descs[l].bytes);
-        v[j] = load16<NT>(src + off);
-        dp[j] = dst + off;
+        const uint64_t off = static_cast<uint64_t>(vv - sPrefix[l]) * 16;
+        v[j] = load16<NT>(body[l].src + off);
+        dp[j] = body[l].dst + off;
       }
 #pragma unroll
       for (int j = 0; j < U; ++j) {

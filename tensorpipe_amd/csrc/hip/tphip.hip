@@ -31,10 +31,10 @@ using namespace tphip;
 
 constexpr int kMaxDevices = 16;
 constexpr uint32_t kPlanSlots = 32;
-// One plan = prefix[n+1] (padded to 16 B) followed by n descriptors.
+// One plan = prefix[n+1] (padded to 16 B), n body pointer pairs, n descriptors.
 constexpr size_t kPlanSlotBytes =
     ((TPHIP_MAX_BATCH + 1) * sizeof(uint32_t) + 15) / 16 * 16 +
-    TPHIP_MAX_BATCH * sizeof(tphip_copy_desc);
+    TPHIP_MAX_BATCH * (sizeof(CopyBody) + sizeof(tphip_copy_desc));
 // Plans for small tables are packed into sub-slots so that a burst of
 // messages does not wait for a slot.
 constexpr uint64_t kMaxTableVectors = 0xFFFFFFFFull - 64ull * 8ull;
@@ -222,21 +222,21 @@ int launchSingle(int unroll, uint32_t blocks, hipStream_t stream, const char* sr
 
 template <int NT>
 int launchTable(int unroll, uint32_t blocks, size_t lds, hipStream_t stream,
-                const uint32_t* prefix, const tphip_copy_desc* descs, uint32_t n,
-                uint32_t nchunks) {
+                const uint32_t* prefix, const CopyBody* bodies, const tphip_copy_desc* descs,
+                uint32_t n, uint32_t nchunks) {
   switch (unroll) {
     case 1:
       return launchKernel(batched_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks);
     case 2:
       return launchKernel(batched_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks);
     case 8:
       return launchKernel(batched_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks);
     default:
       return launchKernel(batched_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks);
   }
 }
 
@@ -300,7 +300,8 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     nt = defaultNontemporal(payload);
   }
   const size_t prefixBytes = ((size_t(n) + 1) * sizeof(uint32_t) + 15) / 16 * 16;
-  const size_t planBytes = prefixBytes + size_t(n) * sizeof(tphip_copy_desc);
+  const size_t bodyBytes = size_t(n) * sizeof(CopyBody);
+  const size_t planBytes = prefixBytes + bodyBytes + size_t(n) * sizeof(tphip_copy_desc);
   const size_t planBytesPadded = (planBytes + 15) / 16 * 16;
 
   uint32_t slot;
@@ -318,6 +319,7 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     char* hostDev = st.hostPlansDev + size_t(slot) * kPlanSlotBytes;
     char* devp = st.devPlans + size_t(slot) * kPlanSlotBytes;
     uint32_t* prefix = reinterpret_cast<uint32_t*>(host);
+    CopyBody* hostBodies = reinterpret_cast<CopyBody*>(host + prefixBytes);
     uint64_t total = 0;
     for (uint32_t i = 0; i < n; ++i) {
       prefix[i] = static_cast<uint32_t>(total);
@@ -326,10 +328,12 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
       if (head > bytes) {
         head = bytes;
       }
+      hostBodies[i].src = static_cast<const char*>(table[i].src) + head;
+      hostBodies[i].dst = static_cast<char*>(table[i].dst) + head;
       total += (bytes - head) >> 4;
     }
     prefix[n] = static_cast<uint32_t>(total);
-    memcpy(host + prefixBytes, table, size_t(n) * sizeof(tphip_copy_desc));
+    memcpy(host + prefixBytes + bodyBytes, table, size_t(n) * sizeof(tphip_copy_desc));
 
     if (planViaKernel()) {
       const uint32_t nv = static_cast<uint32_t>(planBytesPadded / 16);
@@ -348,9 +352,11 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     const uint32_t nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
     const uint32_t edgeBlocks = (n + kBlockThreads - 1) / kBlockThreads;
     const uint32_t grid = pickBlocks(st, nchunks, edgeBlocks, blocks, true);
-    const size_t lds = (size_t(n) + 1) * sizeof(uint32_t);
+    const size_t lds = prefixBytes + (n <= kLdsBodies ? bodyBytes : 0);
     const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
-    const tphip_copy_desc* dDescs = reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes);
+    const CopyBody* dBodies = reinterpret_cast<const CopyBody*>(devp + prefixBytes);
+    const tphip_copy_desc* dDescs =
+        reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes + bodyBytes);
     int rc;
     {
       uint64_t payload = 0;
@@ -360,16 +366,16 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
       ProfileScope prof(st, stream, payload);
       switch (nt & 3) {
         case 0:
-          rc = launchTable<0>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          rc = launchTable<0>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, n, nchunks);
           break;
         case 1:
-          rc = launchTable<1>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          rc = launchTable<1>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, n, nchunks);
           break;
         case 2:
-          rc = launchTable<2>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          rc = launchTable<2>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, n, nchunks);
           break;
         default:
-          rc = launchTable<3>(unroll, grid, lds, stream, dPrefix, dDescs, n, nchunks);
+          rc = launchTable<3>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, n, nchunks);
           break;
       }
     }
