@@ -250,8 +250,10 @@ def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
             st = [tp.make_tensor(src, target=(tp.HIP, 0))]
             rt = [tp.make_tensor(dst)]
             torch.cuda.synchronize()
-            n_it = iters if size <= 256 * MIB else max(iters // 4, 10)
-            per_us, total_s = peer.pingpong(st, rt, [size], "gpu", warmup, n_it)
+            # latency-sized transfers get more round trips (clocks and the
+            # polling threads settle within the first few milliseconds)
+            n_it = iters * 10 if size <= MIB else iters if size <= 256 * MIB else max(iters // 4, 10)
+            per_us, total_s = peer.pingpong(st, rt, [size], "gpu", warmup * 10 if size <= MIB else warmup, n_it)
             torch.cuda.synchronize()
             ok = bool(torch.equal(src, dst))
             per_us.sort()

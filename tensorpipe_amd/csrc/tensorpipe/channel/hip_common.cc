@@ -1,6 +1,7 @@
 #include <tensorpipe/channel/hip_common.h>
 
 #include <chrono>
+#include <cstdlib>
 #include <fstream>
 #include <random>
 #include <sstream>
@@ -60,6 +61,16 @@ void HipEventPoller::join() {
   }
 }
 
+namespace {
+int pollGapNanos() {
+  static const int v = [] {
+    const char* e = std::getenv("TP_HIP_POLL_GAP_NS");
+    return e != nullptr ? std::atoi(e) : 0;
+  }();
+  return v;
+}
+} // namespace
+
 void HipEventPoller::run() {
   using Clock = std::chrono::steady_clock;
   std::deque<Item> active;
@@ -112,9 +123,14 @@ void HipEventPoller::run() {
       lastBusy = Clock::now();
     }
     if (!any) {
+      // Leave the runtime's locks alone for a moment between rounds: the
+      // threads that launch the next copies need them too.
+      const auto until = Clock::now() + std::chrono::nanoseconds(pollGapNanos());
+      do {
 #if defined(__x86_64__)
-      __builtin_ia32_pause();
+        __builtin_ia32_pause();
 #endif
+      } while (Clock::now() < until);
     }
   }
 }

@@ -80,6 +80,25 @@ class ExportRegistry {
 
   // Returns false if the allocation containing ptr cannot be exported.
   bool lookup(int device, const void* ptr, ExportedAllocation* out, uint64_t* offset) {
+    // Common case first: ptr falls inside an allocation exported before. One
+    // runtime query (the allocation's identifier) confirms that the address
+    // range still belongs to that allocation.
+    {
+      uint64_t bufferId = 0;
+      const bool haveId = tphip_mem_buffer_id(ptr, &bufferId) == 0 && bufferId != 0;
+      std::lock_guard<std::mutex> lock(mutex_);
+      auto it = exports_.upper_bound(const_cast<void*>(ptr));
+      if (haveId && it != exports_.begin()) {
+        --it;
+        const uint8_t* base = static_cast<const uint8_t*>(it->first);
+        const uint8_t* p = static_cast<const uint8_t*>(ptr);
+        if (p < base + it->second.size && it->second.bufferId == bufferId) {
+          *out = it->second;
+          *offset = static_cast<uint64_t>(p - base);
+          return true;
+        }
+      }
+    }
     void* base = nullptr;
     size_t size = 0;
     if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr) {

@@ -463,19 +463,39 @@ class ConnectionImpl final : public FdHandler,
   void read(read_callback_fn fn) {
     auto self = shared_from_this();
     ctx_->defer([self, fn{std::move(fn)}]() mutable {
-      self->enqueueRead(ReadOp{nullptr, 0, false, std::move(fn)});
+      self->enqueueRead(ReadOp{nullptr, 0, false, std::move(fn), false, 0, 0, nullptr});
     });
   }
 
   void read(void* ptr, size_t length, read_callback_fn fn) {
     auto self = shared_from_this();
     ctx_->defer([self, ptr, length, fn{std::move(fn)}]() mutable {
-      self->enqueueRead(ReadOp{static_cast<uint8_t*>(ptr), length, true, std::move(fn)});
+      self->enqueueRead(ReadOp{static_cast<uint8_t*>(ptr), length, true, std::move(fn), false, 0, 0, nullptr});
     });
   }
 
   void write(const void* ptr, size_t length, write_callback_fn fn) {
     auto self = shared_from_this();
+    // Fast path: when nothing is queued ahead and the whole message fits, the
+    // calling thread publishes it itself and only the callback goes through
+    // the reactor; this takes one thread hop off every small control message.
+    bool published = false;
+    {
+      std::lock_guard<std::mutex> lock(producerMutex_);
+      if (inlineWritable_ && queuedWrites_ == 0 && outbox_.space() >= kLenPrefix + length) {
+        uint64_t len = length;
+        outbox_.push(reinterpret_cast<const uint8_t*>(&len), kLenPrefix);
+        outbox_.push(static_cast<const uint8_t*>(ptr), length);
+        published = true;
+      } else {
+        ++queuedWrites_;
+      }
+    }
+    if (published) {
+      notifyPeerConsumer();
+      ctx_->defer([self, fn{std::move(fn)}]() mutable { fn(Error::kSuccess); });
+      return;
+    }
     ctx_->defer([self, ptr, length, fn{std::move(fn)}]() mutable {
       self->enqueueWrite(WriteOp{static_cast<const uint8_t*>(ptr), length, std::move(fn)});
     });
@@ -534,6 +554,10 @@ class ConnectionImpl final : public FdHandler,
         }
         peerWakeFd_ = fds[1];
         established_ = true;
+        {
+          std::lock_guard<std::mutex> lock(producerMutex_);
+          inlineWritable_ = true;
+        }
         TP_VLOG(8) << "Connection " << id_ << " established";
         poll();
         return;
@@ -564,6 +588,10 @@ class ConnectionImpl final : public FdHandler,
       return;
     }
     error_ = std::move(error);
+    {
+      std::lock_guard<std::mutex> lock(producerMutex_);
+      inlineWritable_ = false;
+    }
     TP_VLOG(8) << "Connection " << id_ << " is failing: " << error_.what();
     if (sock_ >= 0) {
       ctx_->unwatch(sock_);
@@ -581,6 +609,7 @@ class ConnectionImpl final : public FdHandler,
       r.fn(error_, nullptr, 0);
     }
     for (auto& w : writes) {
+      retireQueuedWrite();
       w.fn(error_);
     }
     ctx_->unenroll(this);
@@ -649,8 +678,14 @@ class ConnectionImpl final : public FdHandler,
     }
   }
 
+  void retireQueuedWrite() {
+    std::lock_guard<std::mutex> lock(producerMutex_);
+    --queuedWrites_;
+  }
+
   void enqueueWrite(WriteOp op) {
     if (error_) {
+      retireQueuedWrite();
       op.fn(error_);
       return;
     }
@@ -664,24 +699,28 @@ class ConnectionImpl final : public FdHandler,
     bool progress = false;
     while (!writes_.empty() && !error_) {
       WriteOp& op = writes_.front();
-      if (!op.lenSent) {
-        if (outbox_.space() < kLenPrefix) {
-          break;
-        }
-        uint64_t len = op.length;
-        outbox_.push(reinterpret_cast<const uint8_t*>(&len), kLenPrefix);
-        op.lenSent = true;
-        progress = true;
-      }
-      if (op.done < op.length) {
-        size_t n = outbox_.push(op.ptr + op.done, op.length - op.done);
-        op.done += n;
-        if (n > 0) {
+      {
+        std::lock_guard<std::mutex> lock(producerMutex_);
+        if (!op.lenSent) {
+          if (outbox_.space() < kLenPrefix) {
+            break;
+          }
+          uint64_t len = op.length;
+          outbox_.push(reinterpret_cast<const uint8_t*>(&len), kLenPrefix);
+          op.lenSent = true;
           progress = true;
         }
-      }
-      if (op.done < op.length) {
-        break; // ring full
+        if (op.done < op.length) {
+          size_t n = outbox_.push(op.ptr + op.done, op.length - op.done);
+          op.done += n;
+          if (n > 0) {
+            progress = true;
+          }
+        }
+        if (op.done < op.length) {
+          break; // ring full
+        }
+        --queuedWrites_;
       }
       write_callback_fn fn = std::move(op.fn);
       writes_.pop_front();
@@ -763,6 +802,11 @@ class ConnectionImpl final : public FdHandler,
   Error error_;
   Ring inbox_;
   Ring outbox_;
+  // Guards the producer side of outbox_, which the reactor and the threads
+  // calling write() share.
+  std::mutex producerMutex_;
+  bool inlineWritable_{false};
+  int queuedWrites_{0};
   std::deque<ReadOp> reads_;
   std::deque<WriteOp> writes_;
 };
