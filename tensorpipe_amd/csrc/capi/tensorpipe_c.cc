@@ -13,6 +13,7 @@
 #include <string>
 #include <vector>
 
+#include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/tensorpipe.h>
 #include <tensorpipe/tensorpipe_hip.h>
 #include <tensorpipe/common/hip_api.h>
@@ -90,10 +91,6 @@ std::vector<std::pair<std::string, int64_t>> parseList(const char* spec) {
   return out;
 }
 
-Device deviceFromC(int32_t type, int32_t index) {
-  return Device{type == TPC_DEVICE_HIP ? kHipDeviceType : kCpuDeviceType, index};
-}
-
 Buffer bufferFromC(const tpc_tensor& t) {
   if (t.device_type == TPC_DEVICE_HIP) {
     return HipBuffer{t.ptr, t.stream};
@@ -115,14 +112,16 @@ Message makeMessage(
     p.length = payloads[i].length;
     m.payloads.push_back(std::move(p));
   }
+  m.tensors.resize(numTensors);
   for (uint32_t i = 0; i < numTensors; ++i) {
-    Message::Tensor t;
+    Message::Tensor& t = m.tensors[i];
     t.buffer = bufferFromC(tensors[i]);
     t.length = tensors[i].length;
     if (tensors[i].target_type != TPC_NO_TARGET) {
-      t.targetDevice = deviceFromC(tensors[i].target_type, tensors[i].target_index);
+      t.targetDevice.emplace(
+          tensors[i].target_type == TPC_DEVICE_HIP ? kHipDeviceType : kCpuDeviceType,
+          tensors[i].target_index);
     }
-    m.tensors.push_back(std::move(t));
   }
   return m;
 }
@@ -422,6 +421,85 @@ int tpc_op_wait(tpc_op* op, int timeoutMs) {
   return rc;
 }
 
+// One-way transfers between two pipe endpoints of this process, chained through
+// callbacks like the reference's own benchmark
+// (tensorpipe/benchmark/benchmark_pipe.cc:463-468,571-577): the write of step
+// k+1 is issued from whichever callback of step k (write done, read done) fires
+// last, on the library's threads. The caller only waits for the end.
+struct TransferChain : std::enable_shared_from_this<TransferChain> {
+  using Clock = std::chrono::steady_clock;
+  std::shared_ptr<Pipe> sender, receiver;
+  std::vector<tpc_payload> payloads;
+  std::vector<void*> recvPayloadPtrs;
+  std::vector<tpc_tensor> sendTensors, recvTensors;
+  uint32_t warmup{0}, iters{0}, round{0};
+  double* perIterUs{nullptr};
+  Clock::time_point begin, end, t0;
+  std::atomic<int> pending{0};
+  Completion finished;
+  std::atomic<bool> failed{false};
+
+  void fail(const Error& e) {
+    if (!failed.exchange(true)) {
+      finished.set(e);
+    }
+  }
+
+  void halfDone(const Error& e) {
+    if (e) {
+      fail(e);
+      return;
+    }
+    if (pending.fetch_sub(1, std::memory_order_acq_rel) != 1) {
+      return;
+    }
+    try {
+      StageScope syncTimer(Stage::kHarnessSync);
+      syncRecvStreams(recvTensors.data(), static_cast<uint32_t>(recvTensors.size()));
+    } catch (const std::exception&) {
+      fail(TP_CREATE_ERROR(HipError, "stream sync", TPHIP_ERR_INVALID_ARG));
+      return;
+    }
+    if (round >= warmup && perIterUs != nullptr) {
+      perIterUs[round - warmup] = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+    }
+    ++round;
+    step();
+  }
+
+  void step() {
+    if (round == warmup + iters) {
+      end = Clock::now();
+      finished.set(Error::kSuccess);
+      return;
+    }
+    if (round == warmup) {
+      begin = Clock::now();
+    }
+    auto self = shared_from_this();
+    t0 = Clock::now();
+    pending.store(2, std::memory_order_release);
+    optional<StageScope> makeTimer;
+    makeTimer.emplace(Stage::kHarnessMakeMessage);
+    Message message = makeMessage(
+        "", payloads.data(), static_cast<uint32_t>(payloads.size()), sendTensors.data(),
+        static_cast<uint32_t>(sendTensors.size()));
+    makeTimer.reset();
+    receiver->readDescriptor([self](const Error& e, Descriptor) {
+      if (e) {
+        self->fail(e);
+        return;
+      }
+      self->receiver->read(
+          makeAllocation(
+              self->recvPayloadPtrs.data(), static_cast<uint32_t>(self->recvPayloadPtrs.size()),
+              self->recvTensors.data(), static_cast<uint32_t>(self->recvTensors.size())),
+          [self](const Error& e2) { self->halfDone(e2); });
+    });
+    sender->write(std::move(message), [self](const Error& e) { self->halfDone(e); });
+  }
+};
+
 int tpc_bench_transfer(
     tpc_pipe* sender,
     tpc_pipe* receiver,
@@ -436,43 +514,23 @@ int tpc_bench_transfer(
     double* perIterUs,
     double* totalSeconds) {
   TPC_GUARD_BEGIN
-  using Clock = std::chrono::steady_clock;
-  Clock::time_point begin;
-  const int kTimeoutMs = 60000;
-  for (uint32_t it = 0; it < warmup + iters; ++it) {
-    if (it == warmup) {
-      begin = Clock::now();
-    }
-    auto t0 = Clock::now();
-    auto wrote = std::make_shared<Completion>();
-    auto gotDescriptor = std::make_shared<Completion>();
-    auto readDone = std::make_shared<Completion>();
-    sender->pipe->write(
-        makeMessage("", payloads, numPayloads, sendTensors, numTensors),
-        [wrote](const Error& e) { wrote->set(e); });
-    receiver->pipe->readDescriptor(
-        [gotDescriptor](const Error& e, Descriptor) { gotDescriptor->set(e); });
-    int rc = gotDescriptor->wait(kTimeoutMs);
-    if (rc != 0) {
-      return rc;
-    }
-    receiver->pipe->read(
-        makeAllocation(recvPayloadPtrs, numPayloads, recvTensors, numTensors),
-        [readDone](const Error& e) { readDone->set(e); });
-    if ((rc = readDone->wait(kTimeoutMs)) != 0) {
-      return rc;
-    }
-    if ((rc = wrote->wait(kTimeoutMs)) != 0) {
-      return rc;
-    }
-    syncRecvStreams(recvTensors, numTensors);
-    if (it >= warmup && perIterUs != nullptr) {
-      perIterUs[it - warmup] =
-          std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
-    }
+  auto chain = std::make_shared<TransferChain>();
+  chain->sender = sender->pipe;
+  chain->receiver = receiver->pipe;
+  chain->payloads.assign(payloads, payloads + numPayloads);
+  chain->recvPayloadPtrs.assign(recvPayloadPtrs, recvPayloadPtrs + numPayloads);
+  chain->sendTensors.assign(sendTensors, sendTensors + numTensors);
+  chain->recvTensors.assign(recvTensors, recvTensors + numTensors);
+  chain->warmup = warmup;
+  chain->iters = iters;
+  chain->perIterUs = perIterUs;
+  chain->step();
+  int rc = chain->finished.wait(600000);
+  if (rc != 0) {
+    return rc;
   }
   if (totalSeconds != nullptr) {
-    *totalSeconds = std::chrono::duration<double>(Clock::now() - begin).count();
+    *totalSeconds = std::chrono::duration<double>(chain->end - chain->begin).count();
   }
   return 0;
   TPC_GUARD_END(TPC_ERR_FAILED)

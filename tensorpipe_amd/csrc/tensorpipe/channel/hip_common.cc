@@ -43,6 +43,7 @@ void HipEventPoller::watch(std::unique_ptr<HipEvent> event, HipEventPool* pool, 
   {
     std::lock_guard<std::mutex> lock(mutex_);
     incoming_.push_back(Item{std::move(event), pool, std::move(fn)});
+    incomingPending_.store(true, std::memory_order_release);
   }
   cv_.notify_one();
 }
@@ -54,6 +55,7 @@ void HipEventPoller::join() {
       return;
     }
     stopping_ = true;
+    incomingPending_.store(true, std::memory_order_release);
   }
   cv_.notify_one();
   if (thread_.joinable()) {
@@ -76,6 +78,14 @@ void HipEventPoller::run() {
   std::deque<Item> active;
   auto lastBusy = Clock::now();
   for (;;) {
+    // Idle and hot: watch one flag, leave the mutex to the threads that post.
+    if (active.empty() && !incomingPending_.load(std::memory_order_acquire) &&
+        Clock::now() - lastBusy < std::chrono::microseconds(300)) {
+#if defined(__x86_64__)
+      __builtin_ia32_pause();
+#endif
+      continue;
+    }
     {
       std::unique_lock<std::mutex> lock(mutex_);
       if (active.empty() && incoming_.empty() && !stopping_) {
@@ -95,6 +105,7 @@ void HipEventPoller::run() {
         active.push_back(std::move(incoming_.front()));
         incoming_.pop_front();
       }
+      incomingPending_.store(false, std::memory_order_relaxed);
       if (stopping_ && active.empty()) {
         return;
       }

@@ -5,6 +5,7 @@
 
 #include <array>
 #include <condition_variable>
+#include <atomic>
 #include <deque>
 #include <functional>
 #include <map>
@@ -57,6 +58,8 @@ class HipEventPoller {
   std::mutex mutex_;
   std::condition_variable cv_;
   std::deque<Item> incoming_;
+  // Set whenever incoming_ may be non-empty or the thread must look at stopping_.
+  std::atomic<bool> incomingPending_{false};
   bool stopping_{false};
   std::thread thread_;
 };

@@ -29,6 +29,8 @@
 #include <tensorpipe/channel/channel_base.h>
 #include <tensorpipe/channel/hip_common.h>
 #include <tensorpipe/common/hip_buffer.h>
+#include <tensorpipe/common/optional.h>
+#include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
 
 TP_AMD_NAMESPACE_BEGIN
@@ -151,9 +153,12 @@ class ChannelImpl final : public ChannelImplBase {
     auto op = std::make_shared<SendOp>();
     op->seq = seq;
     op->cb = std::move(cb);
+    TP_VLOG(9) << "Channel " << id_ << " is encoding descriptor (#" << seq << ")";
 
     // Wire format: n, then per tensor {src stream, src device, src pointer, length}.
+    StageScope timer(Stage::kXthEncode);
     WireWriter w;
+    w.reserve(8 + 28 * live.size());
     w.u32(static_cast<uint32_t>(live.size()));
     try {
       for (auto& e : live) {
@@ -220,6 +225,8 @@ class ChannelImpl final : public ChannelImplBase {
       std::vector<tphip_copy_desc> table;
     };
     std::vector<Group> groups;
+    optional<StageScope> decodeTimer;
+    decodeTimer.emplace(Stage::kXthDecode);
     try {
       for (uint32_t i = 0; i < n; ++i) {
         StreamRef srcRef;
@@ -255,7 +262,9 @@ class ChannelImpl final : public ChannelImplBase {
         g->table.push_back(tphip_copy_desc{src, hb.ptr, len});
       }
       op->copiesInFlight = groups.size();
+      decodeTimer.reset();
       for (auto& g : groups) {
+        StageScope launchTimer(Stage::kXthLaunch);
         // The copy may only touch a destination once everything the receiver
         // enqueued before recv() on that buffer's stream is done.
         for (auto& d : g.dstStreams) {
@@ -270,6 +279,7 @@ class ChannelImpl final : public ChannelImplBase {
         }
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
         hipBatchedCopy(g.src.device, g.src.stream, g.table);
+        TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
         auto done = xctx_->events.get(g.src.device);
         done->record(g.src.stream);
         auto self = shared_from_this();

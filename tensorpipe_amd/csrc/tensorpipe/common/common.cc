@@ -76,3 +76,65 @@ Device HipBuffer::getDevice() const {
 }
 
 TP_AMD_NAMESPACE_END
+
+#include <tensorpipe/common/stage_timer.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+TP_AMD_NAMESPACE_BEGIN
+
+namespace {
+
+struct StageTable {
+  std::atomic<uint64_t> nanos[static_cast<int>(Stage::kCount)];
+  std::atomic<uint64_t> calls[static_cast<int>(Stage::kCount)];
+  bool enabled{false};
+  StageTable() {
+    for (auto& v : nanos) {
+      v.store(0);
+    }
+    for (auto& v : calls) {
+      v.store(0);
+    }
+    const char* e = std::getenv("TP_STAGE_STATS");
+    enabled = e != nullptr && e[0] == '1';
+  }
+  ~StageTable() {
+    if (!enabled) {
+      return;
+    }
+    static const char* const kNames[] = {
+        "pipe: encode descriptor", "pipe: write descriptor+payloads", "pipe: issue tensors",
+        "pipe: parse descriptor",  "pipe: read request",               "hip_xth: encode descriptor",
+        "hip_xth: decode+group",   "hip_xth: launch",                  "hip_xth: copy in flight",
+        "harness: make message",   "harness: stream sync"};
+    for (int i = 0; i < static_cast<int>(Stage::kCount); ++i) {
+      const uint64_t c = calls[i].load();
+      if (c != 0) {
+        std::fprintf(
+            stderr, "[stage] %-34s %9llu calls  %9.2f us avg\n", kNames[i],
+            static_cast<unsigned long long>(c), nanos[i].load() / 1e3 / static_cast<double>(c));
+      }
+    }
+  }
+};
+
+StageTable& stageTable() {
+  static StageTable t;
+  return t;
+}
+
+} // namespace
+
+bool stageStatsEnabled() {
+  return stageTable().enabled;
+}
+
+void stageAdd(Stage s, uint64_t nanos) {
+  StageTable& t = stageTable();
+  t.nanos[static_cast<int>(s)].fetch_add(nanos, std::memory_order_relaxed);
+  t.calls[static_cast<int>(s)].fetch_add(1, std::memory_order_relaxed);
+}
+
+TP_AMD_NAMESPACE_END

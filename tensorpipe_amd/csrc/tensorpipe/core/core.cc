@@ -28,6 +28,7 @@
 
 #include <tensorpipe/channel/channel.h>
 #include <tensorpipe/common/loop.h>
+#include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
 #include <tensorpipe/core/error.h>
 #include <tensorpipe/transport/connection.h>
@@ -45,15 +46,45 @@ enum PacketType : uint8_t {
   kDescriptorReply = 5,
 };
 
+// A device travels as one code byte (the two well-known types) plus its index;
+// any other type follows the code as a string.
+// Flag byte of a tensor inside a descriptor packet.
+constexpr uint8_t kTensorHasTarget = 1;
+constexpr uint8_t kTensorSameSource = 2; // source device = previous tensor's
+constexpr uint8_t kTensorSameTarget = 4; // target device = previous targeted tensor's
+constexpr uint8_t kTensorHasMetadata = 8;
+
+constexpr uint8_t kDevCpu = 0;
+constexpr uint8_t kDevGpu = 1;
+constexpr uint8_t kDevOther = 255;
+
 void putDevice(WireWriter& w, const Device& d) {
-  w.str(d.type);
+  if (d.type == kCpuDeviceType) {
+    w.u8(kDevCpu);
+  } else if (d.type == kHipDeviceType) {
+    w.u8(kDevGpu);
+  } else {
+    w.u8(kDevOther);
+    w.str(d.type);
+  }
   w.u32(static_cast<uint32_t>(d.index));
+}
+
+void getDevice(WireReader& r, Device* d) {
+  const uint8_t code = r.u8();
+  if (code == kDevCpu) {
+    d->type = kCpuDeviceType;
+  } else if (code == kDevGpu) {
+    d->type = kHipDeviceType;
+  } else {
+    d->type = r.str();
+  }
+  d->index = static_cast<int>(r.u32());
 }
 
 Device getDevice(WireReader& r) {
   Device d;
-  d.type = r.str();
-  d.index = static_cast<int>(r.u32());
+  getDevice(r, &d);
   return d;
 }
 
@@ -765,6 +796,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     const uint8_t type = r.u8();
     TP_VLOG(9) << "Pipe " << id_ << " got a packet of type " << int(type);
     if (type == kDescriptor) {
+      StageScope timer(Stage::kPipeParseDescriptor);
       auto op = std::make_shared<ReadOp>();
       op->seq = nextReadSeq_++;
       Descriptor& d = op->descriptor;
@@ -777,17 +809,42 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         d.payloads.push_back(std::move(p));
       }
       const uint32_t nT = r.u32();
-      for (uint32_t i = 0; i < nT && r.ok(); ++i) {
-        Descriptor::Tensor t;
+      // every tensor takes at least 9 bytes on the wire
+      bool wellFormed = nT <= r.remaining() / 9;
+      d.tensors.reserve(wellFormed ? nT : 0); // no reallocation below: prevTarget points inside
+      const Device* prevTarget = nullptr;
+      for (uint32_t i = 0; wellFormed && i < nT && r.ok(); ++i) {
+        d.tensors.emplace_back();
+        Descriptor::Tensor& t = d.tensors.back();
         t.length = r.u64();
-        t.sourceDevice = getDevice(r);
-        if (r.u8() != 0) {
-          t.targetDevice = getDevice(r);
+        const uint8_t flags = r.u8();
+        if (flags & kTensorSameSource) {
+          if (i == 0) {
+            wellFormed = false;
+            break;
+          }
+          t.sourceDevice = d.tensors[i - 1].sourceDevice;
+        } else {
+          getDevice(r, &t.sourceDevice);
         }
-        t.metadata = r.str();
-        d.tensors.push_back(std::move(t));
+        if (flags & kTensorHasTarget) {
+          if (flags & kTensorSameTarget) {
+            if (prevTarget == nullptr) {
+              wellFormed = false;
+              break;
+            }
+            t.targetDevice.emplace(*prevTarget);
+          } else {
+            t.targetDevice.emplace();
+            getDevice(r, &*t.targetDevice);
+          }
+          prevTarget = &*t.targetDevice;
+        }
+        if (flags & kTensorHasMetadata) {
+          r.str(&t.metadata);
+        }
       }
-      if (!r.ok()) {
+      if (!r.ok() || !wellFormed) {
         setError(TP_CREATE_ERROR(LogicError, "malformed descriptor"));
         return;
       }
@@ -798,6 +855,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       if (hasPayloadBytes) {
         payloadsUnclaimed_ = true;
       }
+      TP_VLOG(9) << "Pipe " << id_ << " parsed descriptor (#" << op->seq << ")";
       readOps_.push_back(std::move(op));
       deliverDescriptors();
     } else if (type == kDescriptorReply) {
@@ -852,6 +910,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       return;
     }
     TP_VLOG(9) << "Pipe " << id_ << " received a read request";
+    StageScope timer(Stage::kPipeReadRequest);
     std::shared_ptr<ReadOp> op;
     for (auto& o : readOps_) {
       if (o->delivered && !o->readCalled) {
@@ -870,10 +929,16 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     // checkAllocationCompatibility, tensorpipe/core/pipe_impl.cc:49-65
     TP_THROW_ASSERT_IF(op->allocation.payloads.size() != d.payloads.size());
     TP_THROW_ASSERT_IF(op->allocation.tensors.size() != d.tensors.size());
-    for (size_t i = 0; i < d.tensors.size(); ++i) {
-      if (d.tensors[i].targetDevice.has_value() && d.tensors[i].length > 0) {
-        TP_THROW_ASSERT_IF(
-            !(op->allocation.tensors[i].buffer.device() == *d.tensors[i].targetDevice));
+    const size_t nT = d.tensors.size();
+    bool needsReply = false;
+    std::vector<Device> targets;
+    targets.reserve(nT);
+    for (size_t i = 0; i < nT; ++i) {
+      targets.push_back(op->allocation.tensors[i].buffer.device());
+      if (d.tensors[i].targetDevice.has_value()) {
+        TP_THROW_ASSERT_IF(d.tensors[i].length > 0 && !(targets[i] == *d.tensors[i].targetDevice));
+      } else {
+        needsReply = true;
       }
     }
 
@@ -903,14 +968,6 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
 
     // Tell the sender where tensors without a target device ended up.
-    bool needsReply = false;
-    for (auto& t : d.tensors) {
-      needsReply |= !t.targetDevice.has_value();
-    }
-    std::vector<Device> targets;
-    for (size_t i = 0; i < d.tensors.size(); ++i) {
-      targets.push_back(op->allocation.tensors[i].buffer.device());
-    }
     if (needsReply) {
       WireWriter w;
       w.u8(kDescriptorReply);
@@ -922,20 +979,21 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
 
     // Tensors, grouped per channel in message order.
-    std::vector<std::pair<std::string, std::vector<size_t>>> groups;
-    for (size_t i = 0; i < d.tensors.size(); ++i) {
-      auto it = channelForDevicePair_.find({targets[i], d.tensors[i].sourceDevice});
-      if (it == channelForDevicePair_.end()) {
+    std::vector<ChannelGroup> groups;
+    ChannelLookup lookup(channelForDevicePair_);
+    for (size_t i = 0; i < nT; ++i) {
+      const std::string* name = lookup.find(targets[i], d.tensors[i].sourceDevice);
+      if (name == nullptr) {
         setError(TP_CREATE_ERROR(
             LogicError,
             "no channel between " + targets[i].toString() + " and " +
                 d.tensors[i].sourceDevice.toString()));
         return;
       }
-      addToGroup(groups, it->second, i);
+      addToGroup(groups, name, i, nT);
     }
     for (auto& g : groups) {
-      auto& ch = channels_.at(g.first);
+      auto& ch = channels_.at(*g.first);
       auto done = [self, op](const Error& error) {
         self->ctx_->defer([self, op, error] {
           self->setError(error);
@@ -946,10 +1004,13 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       auto* batched = dynamic_cast<channel::BatchedChannel*>(ch.get());
       if (batched != nullptr && g.second.size() > 1) {
         std::vector<channel::BatchEntry> entries;
+        entries.reserve(g.second.size());
         for (size_t i : g.second) {
           entries.push_back({op->allocation.tensors[i].buffer, d.tensors[i].length});
         }
         ++op->pendingRecvs;
+        TP_VLOG(9) << "Pipe " << id_ << " expects " << entries.size() << " tensors from channel "
+                   << *g.first << " (#" << op->seq << ")";
         batched->recvBatch(std::move(entries), done);
       } else {
         for (size_t i : g.second) {
@@ -1041,7 +1102,11 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
 
   void writeDescriptorAndPayloads(const std::shared_ptr<WriteOp>& op) {
     const Message& m = op->message;
+    StageScope writeTimer(Stage::kPipeWriteDescriptor);
+    optional<StageScope> encodeTimer;
+    encodeTimer.emplace(Stage::kPipeEncodeDescriptor);
     WireWriter w;
+    w.reserve(64 + m.metadata.size() + 32 * m.payloads.size() + 32 * m.tensors.size());
     w.u8(kDescriptor);
     w.str(m.metadata);
     w.u32(static_cast<uint32_t>(m.payloads.size()));
@@ -1049,15 +1114,39 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       w.u64(p.length);
       w.str(p.metadata);
     }
+    // Per tensor: length and a flag byte; a device or a metadata string
+    // follows only where the flags say so. The tensors of a message mostly
+    // share their devices, so a device is spelled out when it differs from the
+    // previous tensor's only.
     w.u32(static_cast<uint32_t>(m.tensors.size()));
-    for (auto& t : m.tensors) {
+    Device prevSource;
+    const Device* prevTarget = nullptr;
+    for (size_t i = 0; i < m.tensors.size(); ++i) {
+      const Message::Tensor& t = m.tensors[i];
+      Device source = t.buffer.device();
+      uint8_t flags = 0;
+      const bool sameSource = i > 0 && source == prevSource;
+      const bool hasTarget = t.targetDevice.has_value();
+      const bool sameTarget = hasTarget && prevTarget != nullptr && *t.targetDevice == *prevTarget;
+      flags |= hasTarget ? kTensorHasTarget : 0;
+      flags |= sameSource ? kTensorSameSource : 0;
+      flags |= sameTarget ? kTensorSameTarget : 0;
+      flags |= t.metadata.empty() ? 0 : kTensorHasMetadata;
       w.u64(t.length);
-      putDevice(w, t.buffer.device());
-      w.u8(t.targetDevice.has_value() ? 1 : 0);
-      if (t.targetDevice.has_value()) {
-        putDevice(w, *t.targetDevice);
+      w.u8(flags);
+      if (!sameSource) {
+        putDevice(w, source);
+        prevSource = std::move(source);
       }
-      w.str(t.metadata);
+      if (hasTarget) {
+        if (!sameTarget) {
+          putDevice(w, *t.targetDevice);
+        }
+        prevTarget = &*t.targetDevice;
+      }
+      if (!t.metadata.empty()) {
+        w.str(t.metadata);
+      }
     }
     auto self = shared_from_this();
     auto done = [self, op](const Error& error) {
@@ -1069,7 +1158,11 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     };
     auto holder = std::make_shared<std::vector<uint8_t>>(std::move(w.bytes()));
     ++op->pendingWrites;
+    encodeTimer.reset();
+    TP_VLOG(9) << "Pipe " << id_ << " encoded descriptor (#" << op->seq << "), " << holder->size()
+               << " bytes";
     connection_->write(holder->data(), holder->size(), [holder, done](const Error& e) { done(e); });
+    TP_VLOG(9) << "Pipe " << id_ << " wrote descriptor (#" << op->seq << ")";
     for (auto& p : m.payloads) {
       if (p.length == 0) {
         continue;
@@ -1081,23 +1174,26 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
 
   void issueTensors(const std::shared_ptr<WriteOp>& op) {
     TP_VLOG(9) << "Pipe " << id_ << " is sending tensors (#" << op->seq << ")";
+    StageScope timer(Stage::kPipeIssueTensors);
     const Message& m = op->message;
-    std::vector<std::pair<std::string, std::vector<size_t>>> groups;
-    for (size_t i = 0; i < m.tensors.size(); ++i) {
+    const size_t nT = m.tensors.size();
+    std::vector<ChannelGroup> groups;
+    ChannelLookup lookup(channelForDevicePair_);
+    for (size_t i = 0; i < nT; ++i) {
       const Device src = m.tensors[i].buffer.device();
-      const Device dst =
+      const Device& dst =
           m.tensors[i].targetDevice.has_value() ? *m.tensors[i].targetDevice : op->targetDevices[i];
-      auto it = channelForDevicePair_.find({src, dst});
-      if (it == channelForDevicePair_.end()) {
+      const std::string* name = lookup.find(src, dst);
+      if (name == nullptr) {
         setError(TP_CREATE_ERROR(
             LogicError, "no channel between " + src.toString() + " and " + dst.toString()));
         return;
       }
-      addToGroup(groups, it->second, i);
+      addToGroup(groups, name, i, nT);
     }
     auto self = shared_from_this();
     for (auto& g : groups) {
-      auto& ch = channels_.at(g.first);
+      auto& ch = channels_.at(*g.first);
       auto done = [self, op](const Error& error) {
         self->ctx_->defer([self, op, error] {
           self->setError(error);
@@ -1108,10 +1204,13 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       auto* batched = dynamic_cast<channel::BatchedChannel*>(ch.get());
       if (batched != nullptr && g.second.size() > 1) {
         std::vector<channel::BatchEntry> entries;
+        entries.reserve(g.second.size());
         for (size_t i : g.second) {
           entries.push_back({m.tensors[i].buffer, m.tensors[i].length});
         }
         ++op->pendingSends;
+        TP_VLOG(9) << "Pipe " << id_ << " hands " << entries.size() << " tensors to channel "
+                   << *g.first << " (#" << op->seq << ")";
         batched->sendBatch(std::move(entries), done);
       } else {
         for (size_t i : g.second) {
@@ -1122,17 +1221,50 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
   }
 
+  // Channel name per tensor; remembers the previous answer because the
+  // tensors of a message nearly always share one device pair.
+  class ChannelLookup {
+   public:
+    explicit ChannelLookup(const DevicePairMap& map) : map_(map) {}
+    // (local device, remote device) -> channel name, nullptr when none serves it.
+    const std::string* find(const Device& local, const Device& remote) {
+      if (last_ != nullptr && local == lastLocal_ && remote == lastRemote_) {
+        return last_;
+      }
+      auto it = map_.find({local, remote});
+      if (it == map_.end()) {
+        return nullptr;
+      }
+      lastLocal_ = local;
+      lastRemote_ = remote;
+      last_ = &it->second;
+      return last_;
+    }
+
+   private:
+    const DevicePairMap& map_;
+    Device lastLocal_;
+    Device lastRemote_;
+    const std::string* last_{nullptr};
+  };
+
+  // Tensor indices per channel (named by a pointer into channelForDevicePair_).
+  using ChannelGroup = std::pair<const std::string*, std::vector<size_t>>;
+
   static void addToGroup(
-      std::vector<std::pair<std::string, std::vector<size_t>>>& groups,
-      const std::string& name,
-      size_t idx) {
+      std::vector<ChannelGroup>& groups,
+      const std::string* name,
+      size_t idx,
+      size_t expected) {
     for (auto& g : groups) {
-      if (g.first == name) {
+      if (g.first == name || *g.first == *name) {
         g.second.push_back(idx);
         return;
       }
     }
-    groups.emplace_back(name, std::vector<size_t>{idx});
+    groups.emplace_back(name, std::vector<size_t>());
+    groups.back().second.reserve(expected);
+    groups.back().second.push_back(idx);
   }
 
   // Write callbacks fire in the order the writes were issued.
