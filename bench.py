@@ -136,7 +136,7 @@ def bench_d2d(steps, warmup):
     }
 
 
-def bench_rpc_message(messages=100, warmup=5):
+def bench_rpc_message(messages=500, warmup=20):
     """configs[4]: 256 fp16 tensors, log-uniform sizes, 4 KiB payload, one launch per message."""
     import numpy as np
     import torch
@@ -386,6 +386,25 @@ def cpu_baseline():
     }
 
 
+# The configurations besides the headline. Each runs in a process of its own so that
+# none inherits runtime state from another (streams a process has used change what the
+# runtime does on later launches, which shifts small-transfer latencies by microseconds).
+LEGS = {
+    "rpc_message": bench_rpc_message,
+    "ipc": bench_ipc,
+    "staged": bench_staged,
+    "host_link": bench_link_ceiling,
+}
+
+
+def run_leg(name, timeout_s=600):
+    proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--leg", name],
+                          stdout=subprocess.PIPE, timeout=timeout_s)
+    if proc.returncode != 0:
+        raise RuntimeError(f"bench leg {name} failed with exit code {proc.returncode}")
+    return json.loads(proc.stdout.decode().strip().splitlines()[-1])
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -393,6 +412,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the headline configuration and the CPU baseline")
+    ap.add_argument("--leg", choices=sorted(LEGS), default=None,
+                    help="run one of the other configurations alone and print its JSON (internal)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; every configuration of the device "
@@ -406,6 +427,10 @@ def main():
 
     _native.tphip()  # fails loudly if the HIP library is not built
 
+    if args.leg is not None:
+        print(json.dumps(LEGS[args.leg]()), flush=True)
+        return
+
     t_start = time.time()
     log("[bench] same-process D2D, 64 MiB (headline)")
     d2d = bench_d2d(args.steps, args.warmup)
@@ -417,12 +442,12 @@ def main():
     }
     if not args.skip_extras:
         log("[bench] many-tensor message (256 tensors, one launch per message)")
-        extra["rpc_message"] = bench_rpc_message()
+        extra["rpc_message"] = run_leg("rpc_message")
         log("[bench] cross-process IPC sweep")
-        extra["ipc"] = bench_ipc()
+        extra["ipc"] = run_leg("ipc")
         log("[bench] host-staged 256 MiB")
-        extra["staged"] = bench_staged()
-        extra["host_link"] = bench_link_ceiling()
+        extra["staged"] = run_leg("staged")
+        extra["host_link"] = run_leg("host_link")
     log("[bench] CPU baseline (port of shm + basic)")
     cpu = cpu_baseline()
     extra["bench_wall_s"] = time.time() - t_start
