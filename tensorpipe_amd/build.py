@@ -81,10 +81,26 @@ def build_host(jobs=8):
          f"-L{LIB}", "-ltphip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"])
 
 
+CPP_TESTS = ["channel_tests", "pipe_tests"]
+
+
+def build_cpp_tests():
+    """The C++ test programs under tests/cpp (plain executables driving the C++ API)."""
+    src_dir = os.path.join(ROOT, "tests", "cpp")
+    bin_dir = os.path.join(src_dir, "bin")
+    os.makedirs(bin_dir, exist_ok=True)
+    for name in CPP_TESTS:
+        run(["g++", "-O1", "-g", "-std=c++17", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
+             f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(src_dir, name + ".cc"),
+             "-o", os.path.join(bin_dir, name), f"-L{LIB}", "-ltensorpipe_amd", "-ltphip",
+             "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib"])
+
+
 def build_all():
     build_tphip()
     build_datagen()
     build_host()
+    build_cpp_tests()
 
 
 if __name__ == "__main__":

@@ -140,6 +140,12 @@ class BasicContextCore final : public ContextCore {
   std::unique_ptr<PinnedRing> sendRing_;
   std::unique_ptr<PinnedRing> recvRing_;
   HandleBytes sendRingHandle_{};
+
+ public:
+  // Names the send ring towards peers that map it.
+  const uint64_t sendRingId{nextExportId()};
+
+ private:
   bool sendRingExported_{false};
   void* internalStream_{nullptr};
 };
@@ -166,6 +172,14 @@ class ChannelImpl final : public ChannelImplBase {
         controlConnection_(std::move(controlConnection)),
         cpuChannel_(std::move(cpuChannel)) {}
 
+  // Every copy out of the peer's ring is followed by an event whose watcher
+  // keeps this object alive, so nothing reads the mapping any more.
+  ~ChannelImpl() override {
+    if (remoteRing_ != nullptr) {
+      HipIpcImports::get().release(0, remoteRingPeer_, remoteRingId_);
+    }
+  }
+
  protected:
   void initFromLoop() override {
     WireWriter w;
@@ -184,6 +198,7 @@ class ChannelImpl final : public ChannelImplBase {
     }
     w.u8(exported ? 1 : 0);
     if (exported) {
+      w.u64(bctx_->sendRingId);
       w.raw(bctx_->sendRingHandle().data(), TPHIP_IPC_HANDLE_BYTES);
     }
     writeMessage(*controlConnection_, std::move(w.bytes()));
@@ -344,13 +359,16 @@ class ChannelImpl final : public ChannelImplBase {
       remoteNumSlots_ = remoteSlots;
       bool mapped = false;
       if (hasHandle) {
+        const uint64_t ringId = r.u64();
         HandleBytes h;
         r.raw(h.data(), h.size());
         // Map the peer's send ring if it lives on this machine in another
         // process; otherwise its chunks come through the inner channel.
         if (r.ok() && bctx_->shareRing && boot == bootIdentity() && process != processIdentity()) {
           void* ptr = nullptr;
-          if (HipIpcImports::get().open(0, h, &ptr) == 0) {
+          if (HipIpcImports::get().acquire(0, process, ringId, h, &ptr) == 0) {
+            remoteRingPeer_ = process;
+            remoteRingId_ = ringId;
             remoteRing_ = static_cast<uint8_t*>(ptr);
             mapped = true;
           }
@@ -909,6 +927,8 @@ class ChannelImpl final : public ChannelImplBase {
   uint64_t remoteSlotBytes_{0};
   uint64_t remoteNumSlots_{0};
   uint8_t* remoteRing_{nullptr};  // peer's send ring as mapped by our GPU
+  std::string remoteRingPeer_;    // who exported it, and under which identifier
+  uint64_t remoteRingId_{0};
   bool peerMappedOurRing_{false}; // peer can read our send ring
   std::vector<std::function<void()>> deferred_;
   std::deque<std::shared_ptr<Op>> ops_;

@@ -146,27 +146,67 @@ void HipEventPoller::run() {
   }
 }
 
+uint64_t nextExportId() {
+  static std::atomic<uint64_t> next{1};
+  return next.fetch_add(1, std::memory_order_relaxed);
+}
+
 HipIpcImports& HipIpcImports::get() {
   static HipIpcImports* r = new HipIpcImports();
   return *r;
 }
 
-int HipIpcImports::open(int device, const HandleBytes& handle, void** out) {
+int HipIpcImports::acquire(
+    int device,
+    const std::string& peer,
+    uint64_t id,
+    const HandleBytes& handle,
+    void** out) {
   std::lock_guard<std::mutex> lock(mutex_);
-  auto key = std::make_pair(device, handle);
-  auto it = opened_.find(key);
-  if (it != opened_.end()) {
-    *out = it->second;
+  const Key key{device, peer, id};
+  auto it = entries_.find(key);
+  if (it != entries_.end() && it->second.mapped) {
+    ++it->second.refs;
+    *out = it->second.ptr;
     return 0;
+  }
+  // Same handle bytes under another identifier: stale, unmap before mapping anew.
+  for (auto& kv : entries_) {
+    if (std::get<0>(kv.first) == device && kv.second.mapped && kv.second.handle == handle) {
+      tphip_ipc_mem_close(device, kv.second.ptr);
+      kv.second.mapped = false;
+      kv.second.ptr = nullptr;
+    }
   }
   void* ptr = nullptr;
   int rc = tphip_ipc_mem_open(device, handle.data(), &ptr);
   if (rc != 0) {
     return rc;
   }
-  opened_[key] = ptr;
+  Entry& e = entries_[key];
+  e.ptr = ptr;
+  e.handle = handle;
+  e.mapped = true;
+  ++e.refs;
   *out = ptr;
   return 0;
+}
+
+void HipIpcImports::release(int device, const std::string& peer, uint64_t id) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  auto it = entries_.find(Key{device, peer, id});
+  if (it == entries_.end()) {
+    return;
+  }
+  if (it->second.refs > 0) {
+    --it->second.refs;
+  }
+  if (it->second.refs == 0) {
+    if (it->second.mapped) {
+      tphip_ipc_mem_close(device, it->second.ptr);
+    }
+    entries_.erase(it);
+  }
 }
 
 void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table) {

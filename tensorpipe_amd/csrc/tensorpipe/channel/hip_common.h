@@ -13,6 +13,7 @@
 #include <mutex>
 #include <string>
 #include <thread>
+#include <tuple>
 #include <vector>
 
 #include <tensorpipe/common/error.h>
@@ -71,15 +72,37 @@ using HandleBytes = std::array<uint8_t, TPHIP_IPC_HANDLE_BYTES>;
 // about 0.2 ms, a handle may be shared by several channels, and the reference
 // keeps its opened handles until the context closes for the same reasons
 // (tensorpipe/channel/cuda_ipc/context_impl.cc:388-418).
+// Process-wide identifiers for things this process exports to peers (tensor
+// allocations, staging slabs, pinned rings). A peer keys its mapping on
+// (exporting process, identifier), never on the handle bytes: an address that
+// is freed and handed out again may come with the very same handle.
+uint64_t nextExportId();
+
+// Mappings of peer memory, shared by the channels of this process and counted:
+// every acquire() is paired with a release(), the last one unmaps. Mapping a
+// handle costs a few hundred microseconds, so a mapping lives as long as any
+// channel uses it.
 class HipIpcImports {
  public:
   static HipIpcImports& get();
-  // Returns a tphip error code.
-  int open(int device, const HandleBytes& handle, void** out);
+  // `peer` is the exporter's processIdentity(), `id` its nextExportId() value
+  // for the allocation, `handle` what tphip_ipc_mem_export gave it. Returns a
+  // tphip error code. An older mapping with the same handle bytes belongs to
+  // memory the exporter has freed since (two live allocations never share a
+  // handle) and is unmapped first.
+  int acquire(int device, const std::string& peer, uint64_t id, const HandleBytes& handle, void** out);
+  void release(int device, const std::string& peer, uint64_t id);
 
  private:
+  struct Entry {
+    void* ptr{nullptr};
+    HandleBytes handle;
+    size_t refs{0};
+    bool mapped{false};
+  };
+  using Key = std::tuple<int, std::string, uint64_t>;
   std::mutex mutex_;
-  std::map<std::pair<int, HandleBytes>, void*> opened_;
+  std::map<Key, Entry> entries_;
 };
 
 // Enqueue one batched copy on (device, stream); throws on a failed launch.

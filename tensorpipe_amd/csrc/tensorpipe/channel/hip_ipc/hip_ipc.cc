@@ -119,7 +119,7 @@ class ExportRegistry {
     if (tphip_ipc_mem_export(device, base, e.handle.data()) != 0) {
       return false;
     }
-    e.id = nextId_++;
+    e.id = nextExportId();
     e.size = size;
     e.bufferId = bufferId;
     exports_[base] = e;
@@ -130,7 +130,6 @@ class ExportRegistry {
  private:
   std::mutex mutex_;
   std::map<void*, ExportedAllocation> exports_;
-  uint64_t nextId_{1};
 };
 
 // Per-device staging slab of the outbox path, created on first use.
@@ -142,6 +141,7 @@ struct Outbox {
   HipDeviceSlab slab;
   HandleBytes handle;
   SlotAllocator allocator;
+  const uint64_t id{nextExportId()};
 };
 
 class IpcContextCore final : public ContextCore {
@@ -190,6 +190,14 @@ class ChannelImpl final : public ChannelImplBase {
         ictx_(std::move(ctx)),
         descriptorConnection_(std::move(descriptorConnection)),
         replyConnection_(std::move(replyConnection)) {}
+
+  // Every copy out of a mapped peer allocation is followed by an event whose
+  // watcher keeps this object alive, so nothing reads the mappings any more.
+  ~ChannelImpl() override {
+    for (auto& i : imports_) {
+      HipIpcImports::get().release(i.device, i.peer, i.id);
+    }
+  }
 
   void sendBatch(std::vector<BatchEntry> entries, TSendCallback callback) {
     auto self = std::static_pointer_cast<ChannelImpl>(shared_from_this());
@@ -358,6 +366,7 @@ class ChannelImpl final : public ChannelImplBase {
           const bool announce = announced_.insert(d.alloc.id).second;
           w.u8(announce ? 1 : 0);
           if (announce) {
+            w.str(processIdentity());
             w.raw(d.alloc.handle.data(), d.alloc.handle.size());
           }
           w.u64(d.offset);
@@ -452,6 +461,8 @@ class ChannelImpl final : public ChannelImplBase {
       outboxAnnounced_[device] = true;
       w.u8(announce ? 1 : 0);
       if (announce) {
+        w.str(processIdentity());
+        w.u64(outbox.id);
         w.raw(outbox.handle.data(), outbox.handle.size());
       }
       w.u32(static_cast<uint32_t>(slotIdx));
@@ -553,15 +564,21 @@ class ChannelImpl final : public ChannelImplBase {
           const int device = hipDeviceForPointer(hb.ptr);
           TP_THROW_ASSERT_IF(device < 0);
           if (announce) {
+            const std::string peer = r.str();
             HandleBytes h;
             r.raw(h.data(), h.size());
+            if (!r.ok() || remoteAllocations_.count(exportId) != 0) {
+              failProtocol();
+              return;
+            }
             void* mapped = nullptr;
-            int rc = HipIpcImports::get().open(device, h, &mapped);
+            int rc = HipIpcImports::get().acquire(device, peer, exportId, h, &mapped);
             if (rc != 0) {
               setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
               return;
             }
             remoteAllocations_[exportId] = mapped;
+            imports_.push_back(Import{device, peer, exportId});
           }
           const uint64_t offset = r.u64();
           const uint64_t length = r.u64();
@@ -602,15 +619,22 @@ class ChannelImpl final : public ChannelImplBase {
         const int device = hipDeviceForPointer(hb.ptr);
         TP_THROW_ASSERT_IF(device < 0);
         if (announce) {
+          const std::string peer = r.str();
+          const uint64_t outboxId = r.u64();
           HandleBytes h;
           r.raw(h.data(), h.size());
+          if (!r.ok() || remoteOutboxes_.count(srcDevice) != 0) {
+            failProtocol();
+            return;
+          }
           void* mapped = nullptr;
-          int rc = HipIpcImports::get().open(device, h, &mapped);
+          int rc = HipIpcImports::get().acquire(device, peer, outboxId, h, &mapped);
           if (rc != 0) {
             setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
             return;
           }
           remoteOutboxes_[srcDevice] = mapped;
+          imports_.push_back(Import{device, peer, outboxId});
         }
         const uint32_t slotIdx = r.u32();
         const uint64_t offset = r.u64();
@@ -748,6 +772,13 @@ class ChannelImpl final : public ChannelImplBase {
   std::map<int, bool> outboxAnnounced_;
   std::map<uint64_t, void*> remoteAllocations_;
   std::map<int, void*> remoteOutboxes_;
+  // What this channel holds in the process-wide import table.
+  struct Import {
+    int device;
+    std::string peer;
+    uint64_t id;
+  };
+  std::vector<Import> imports_;
 };
 
 class IpcChannel final : public ChannelHandle<ChannelImpl>, public BatchedChannel {

@@ -703,7 +703,14 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     writeControl(std::move(w.bytes()));
     if (connectionsAwaited_ == 0) {
       createServerChannels();
+      return;
     }
+    // While the client opens the channel connections nothing else would be
+    // reading the primary connection, and a client that goes away now would
+    // never be noticed: keep a read posted. Whatever it delivers before the
+    // pipe is established waits in earlyPacket_.
+    awaitingChannelConnections_ = true;
+    pumpPackets();
   }
 
   void onRequestedConnection(
@@ -739,7 +746,13 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
 
   void establish() {
     established_ = true;
+    awaitingChannelConnections_ = false;
     TP_VLOG(2) << "Pipe " << id_ << " is established with " << channels_.size() << " channel(s)";
+    if (haveEarlyPacket_) {
+      haveEarlyPacket_ = false;
+      onPacket(std::move(earlyPacket_));
+      earlyPacket_.clear();
+    }
     pumpPackets();
     advanceWrites();
   }
@@ -777,13 +790,21 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   // the most recent descriptor have not been claimed by a read() call: those
   // are the next messages on the connection and go straight to user memory.
   void pumpPackets() {
-    if (!established_ || error_ || packetReadOutstanding_ || payloadsUnclaimed_) {
+    if ((!established_ && !awaitingChannelConnections_) || error_ || packetReadOutstanding_ ||
+        payloadsUnclaimed_ || haveEarlyPacket_) {
       return;
     }
     packetReadOutstanding_ = true;
     readControl([this](std::vector<uint8_t> bytes) {
       packetReadOutstanding_ = false;
       if (error_) {
+        return;
+      }
+      if (!established_) {
+        // A descriptor may be followed by payloads that only read() can
+        // place, so nothing more is taken off the connection until then.
+        earlyPacket_ = std::move(bytes);
+        haveEarlyPacket_ = true;
         return;
       }
       onPacket(std::move(bytes));
@@ -1328,6 +1349,10 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   uint64_t childKey_{0};
   Error error_;
   bool established_{false};
+  // Server side, between the brochure answer and the last channel connection.
+  bool awaitingChannelConnections_{false};
+  bool haveEarlyPacket_{false};
+  std::vector<uint8_t> earlyPacket_;
 
   std::unordered_map<std::string, std::shared_ptr<channel::Channel>> channels_;
   DevicePairMap channelForDevicePair_;

@@ -1,0 +1,535 @@
+// Channel-level tests of hip_xth, hip_ipc and hip_basic, driven through the
+// plugin surface itself: channel::Context::createChannel over raw transport
+// connections, then Channel::send / recv with Buffer{HipBuffer|CpuBuffer}.
+//
+//   channel_tests --suite hip_xth|hip_ipc|hip_basic|basic|xth [--case SUBSTRING] [--list]
+//
+// hip_xth and xth run both endpoints as two threads of this process; hip_ipc,
+// hip_basic and basic run them as two processes. The CPU channels (basic, xth)
+// go through the same cases with host memory. Each case prints one
+// "RESULT <role> <case> OK|FAIL ..." line per endpoint.
+//
+// Cases and data follow the reference's suites:
+//   tensorpipe/test/channel/channel_test.cc:19-336        (generic)
+//   tensorpipe/test/channel/channel_test_cuda.cc:19-139   (stream ordering, offsets)
+//   tensorpipe/test/channel/channel_test_cuda_xdtt.cc:19-195 (CPU <-> GPU)
+//   tensorpipe/test/channel/cuda_ipc/cuda_ipc_test.cc:37-57
+//   tensorpipe/test/channel/cuda_basic/cuda_basic_test.cc:40-62
+#include "support.h"
+
+using namespace tptest;
+
+namespace {
+
+std::string gSuite;
+bool gGpu = true; // whether the suite's tensors live on the GPU
+
+bool knownSuite(const std::string& s) {
+  return s == "hip_xth" || s == "hip_ipc" || s == "hip_basic" || s == "basic" || s == "xth";
+}
+
+bool twoProcessSuite(const std::string& s) {
+  return s == "hip_ipc" || s == "hip_basic" || s == "basic";
+}
+
+Buffer nullBuffer() {
+  if (gGpu) {
+    return HipBuffer{nullptr, nullptr};
+  }
+  return CpuBuffer{nullptr};
+}
+
+std::shared_ptr<channel::Context> makeContext() {
+  if (gSuite == "hip_xth") {
+    return channel::hip_xth::create();
+  }
+  if (gSuite == "hip_ipc") {
+    return channel::hip_ipc::create();
+  }
+  if (gSuite == "hip_basic") {
+    return channel::hip_basic::create(channel::basic::create());
+  }
+  if (gSuite == "basic") {
+    return channel::basic::create();
+  }
+  if (gSuite == "xth") {
+    return channel::xth::create();
+  }
+  throw Fatal("unknown suite " + gSuite);
+}
+
+struct Opened {
+  std::shared_ptr<channel::Context> ctx;
+  std::shared_ptr<channel::Channel> ch;
+  // Channel first, then the context (joined), as the reference's harness does.
+  ~Opened() {
+    ch.reset();
+    if (ctx) {
+      ctx->join();
+    }
+  }
+};
+
+std::unique_ptr<Opened> open(Endpoint& ep) {
+  auto o = std::make_unique<Opened>();
+  o->ctx = makeContext();
+  o->ctx->setId(std::string(roleName(ep.role())) + "_ctx");
+  if (!o->ctx->isViable()) {
+    throw Fatal("context is not viable");
+  }
+  auto conns = ep.openConnections(o->ctx->numConnectionsNeeded());
+  o->ch = o->ctx->createChannel(
+      std::move(conns), ep.isServer() ? channel::Endpoint::kListen : channel::Endpoint::kConnect);
+  return o;
+}
+
+std::future<Error> sendF(channel::Channel& ch, Buffer b, size_t n) {
+  auto p = std::make_shared<std::promise<Error>>();
+  auto f = p->get_future();
+  ch.send(std::move(b), n, [p](const Error& e) { p->set_value(e); });
+  return f;
+}
+
+std::future<Error> recvF(channel::Channel& ch, Buffer b, size_t n) {
+  auto p = std::make_shared<std::promise<Error>>();
+  auto f = p->get_future();
+  ch.recv(std::move(b), n, [p](const Error& e) { p->set_value(e); });
+  return f;
+}
+
+void expectBytes(Data& d, const std::vector<uint8_t>& want, const char* what) {
+  std::vector<uint8_t> got = d.bytes();
+  if (got.size() != want.size()) {
+    failures().add(std::string(what) + ": size differs");
+    return;
+  }
+  for (size_t i = 0; i < got.size(); ++i) {
+    if (got[i] != want[i]) {
+      failures().add(
+          std::string(what) + ": byte " + std::to_string(i) + " is " + std::to_string(got[i]) +
+          ", expected " + std::to_string(want[i]));
+      return;
+    }
+  }
+}
+
+// A transfer of `data` from the sending endpoint to the receiving one.
+void sender(Endpoint& ep, bool gpu, const std::vector<uint8_t>& data) {
+  auto o = open(ep);
+  auto d = makeData(gpu, data);
+  auto f = sendF(*o->ch, d->buffer(), d->size());
+  EXPECT_OK(waitFor(f, "send"));
+  ep.barrier();
+}
+
+void receiver(Endpoint& ep, bool gpu, const std::vector<uint8_t>& want) {
+  auto o = open(ep);
+  auto d = makeData(gpu, want.size());
+  auto f = recvF(*o->ch, d->buffer(), d->size());
+  EXPECT_OK(waitFor(f, "recv"));
+  expectBytes(*d, want, "received data");
+  ep.barrier();
+}
+
+std::vector<Case> makeCases() {
+  std::vector<Case> cases;
+  const bool staged = gSuite == "hip_basic";
+
+  // channel_test.cc:19-43
+  auto descriptors = [](Endpoint&) {
+    auto c1 = makeContext();
+    auto c2 = makeContext();
+    const auto& d1 = c1->deviceDescriptors();
+    const auto& d2 = c2->deviceDescriptors();
+    EXPECT_FALSE(d1.empty());
+    EXPECT_EQ(d1.size(), d2.size());
+    EXPECT_EQ(d1.count(gGpu ? Device{kHipDeviceType, 0} : Device{kCpuDeviceType, 0}), size_t(1));
+    for (auto& kv : d1) {
+      EXPECT_FALSE(kv.second.empty());
+      EXPECT_EQ(d2.count(kv.first), size_t(1));
+      if (d2.count(kv.first) == 1) {
+        EXPECT_EQ(kv.second, d2.at(kv.first));
+      }
+    }
+    c1->join();
+    c2->join();
+  };
+  cases.push_back({"DeviceDescriptors", descriptors, descriptors});
+
+  // channel_test.cc:45-125: 256 sequential bytes, each direction.
+  cases.push_back({"ServerToClient",
+                   [](Endpoint& ep) { sender(ep, gGpu, iota(256)); },
+                   [](Endpoint& ep) { receiver(ep, gGpu, iota(256)); }});
+  cases.push_back({"ClientToServer",
+                   [](Endpoint& ep) { receiver(ep, gGpu, iota(256)); },
+                   [](Endpoint& ep) { sender(ep, gGpu, iota(256)); }});
+
+  // channel_test.cc:127-189: 100 tensors of 256 KiB holding i % 256, all posted
+  // before any is awaited.
+  cases.push_back(
+      {"SendMultipleTensors",
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         auto d = makeData(gGpu, iota(256 * 1024));
+         std::vector<std::future<Error>> fs;
+         for (int i = 0; i < 100; ++i) {
+           fs.push_back(sendF(*o->ch, d->buffer(), d->size()));
+         }
+         for (auto& f : fs) {
+           EXPECT_OK(waitFor(f, "send"));
+         }
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         std::vector<std::unique_ptr<Data>> ds;
+         std::vector<std::future<Error>> fs;
+         for (int i = 0; i < 100; ++i) {
+           ds.push_back(makeData(gGpu, 256 * 1024));
+           fs.push_back(recvF(*o->ch, ds.back()->buffer(), ds.back()->size()));
+         }
+         for (auto& f : fs) {
+           EXPECT_OK(waitFor(f, "recv"));
+         }
+         const auto want = iota(256 * 1024);
+         for (auto& d : ds) {
+           expectBytes(*d, want, "tensor");
+         }
+         ep.barrier();
+       }});
+
+  // channel_test.cc:191-259: one send and one recv in flight on each side.
+  auto bothWays = [](Endpoint& ep) {
+    auto o = open(ep);
+    std::vector<uint8_t> mine(256, ep.isServer() ? 0x11 : 0x22);
+    std::vector<uint8_t> theirs(256, ep.isServer() ? 0x22 : 0x11);
+    auto out = makeData(gGpu, mine);
+    auto in = makeData(gGpu, 256);
+    auto fs = sendF(*o->ch, out->buffer(), out->size());
+    auto fr = recvF(*o->ch, in->buffer(), in->size());
+    EXPECT_OK(waitFor(fs, "send"));
+    EXPECT_OK(waitFor(fr, "recv"));
+    expectBytes(*in, theirs, "received data");
+    ep.barrier();
+  };
+  cases.push_back({"SendTensorsBothWays", bothWays, bothWays});
+
+  // channel_test.cc:262-293: zero bytes at a null pointer complete at once.
+  cases.push_back({"EmptyTensor",
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     auto f = sendF(*o->ch, nullBuffer(), 0);
+                     EXPECT_OK(waitFor(f, "send"));
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     auto f = recvF(*o->ch, nullBuffer(), 0);
+                     EXPECT_OK(waitFor(f, "recv"));
+                     ep.barrier();
+                   }});
+
+  // channel_test.cc:295-336: lengths 1, 0, 1 keep their order.
+  cases.push_back(
+      {"EmptyAndNonEmptyTensors",
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         auto a = makeData(gGpu, std::vector<uint8_t>{0xA1});
+         auto c = makeData(gGpu, std::vector<uint8_t>{0xC3});
+         auto f1 = sendF(*o->ch, a->buffer(), 1);
+         auto f2 = sendF(*o->ch, nullBuffer(), 0);
+         auto f3 = sendF(*o->ch, c->buffer(), 1);
+         EXPECT_OK(waitFor(f1, "send 1"));
+         EXPECT_OK(waitFor(f2, "send 2"));
+         EXPECT_OK(waitFor(f3, "send 3"));
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         auto a = makeData(gGpu, 1);
+         auto c = makeData(gGpu, 1);
+         auto f1 = recvF(*o->ch, a->buffer(), 1);
+         auto f2 = recvF(*o->ch, nullBuffer(), 0);
+         auto f3 = recvF(*o->ch, c->buffer(), 1);
+         EXPECT_OK(waitFor(f1, "recv 1"));
+         EXPECT_OK(waitFor(f2, "recv 2"));
+         EXPECT_OK(waitFor(f3, "recv 3"));
+         expectBytes(*a, {0xA1}, "first");
+         expectBytes(*c, {0xC3}, "third");
+         ep.barrier();
+       }});
+
+  if (gGpu) {
+  // channel_test_cuda.cc:19-94: the source is still being produced on the send
+  // stream when send() is called (a slow kernel scribbles over it, then a fill
+  // writes 0x42); the receiver must see the 0x42s.
+  cases.push_back(
+      {"ReceiverWaitsForStartEvent",
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         GpuData d(1024);
+         HIP_OK(tphip_test_slow_kernel(0, d.ptr(), 1024, d.stream()));
+         HIP_OK(tphip_fill(0, d.ptr(), 0x42, 1024, d.stream()));
+         auto f = sendF(*o->ch, d.buffer(), 1024);
+         EXPECT_OK(waitFor(f, "send"));
+         ep.barrier();
+       },
+       [](Endpoint& ep) { receiver(ep, true, std::vector<uint8_t>(1024, 0x42)); }});
+
+  // channel_test_cuda.cc:96-139: the tensor starts 128 bytes into its
+  // allocation (matters for handles that name the allocation base).
+  cases.push_back({"SendOffsetAllocation",
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     GpuData d(std::vector<uint8_t>(256, 0x42), /*offset=*/128);
+                     auto f = sendF(*o->ch, d.buffer(), 256);
+                     EXPECT_OK(waitFor(f, "send"));
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) { receiver(ep, true, std::vector<uint8_t>(256, 0x42)); }});
+  } // gGpu
+
+  // Sizes around the chunking and vector-width boundaries of the copy paths.
+  for (size_t n : {size_t(1), size_t(15), size_t(4097), size_t(1) << 20, (size_t(8) << 20) + 5,
+                   size_t(20) << 20}) {
+    std::vector<uint8_t> v(n);
+    uint64_t x = 0x9E3779B97F4A7C15ull * (n + 1);
+    for (size_t i = 0; i < n; ++i) {
+      x ^= x << 13;
+      x ^= x >> 7;
+      x ^= x << 17;
+      v[i] = static_cast<uint8_t>(x);
+    }
+    cases.push_back({"Size" + std::to_string(n),
+                     [v](Endpoint& ep) { sender(ep, gGpu, v); },
+                     [v](Endpoint& ep) { receiver(ep, gGpu, v); }});
+  }
+
+  if (staged) {
+    // channel_test_cuda_xdtt.cc:19-143: 1024 bytes of 0x42 across device types.
+    cases.push_back({"SendFromCpuToGpu",
+                     [](Endpoint& ep) { sender(ep, false, std::vector<uint8_t>(1024, 0x42)); },
+                     [](Endpoint& ep) { receiver(ep, true, std::vector<uint8_t>(1024, 0x42)); }});
+    cases.push_back({"SendFromGpuToCpu",
+                     [](Endpoint& ep) { sender(ep, true, std::vector<uint8_t>(1024, 0x42)); },
+                     [](Endpoint& ep) { receiver(ep, false, std::vector<uint8_t>(1024, 0x42)); }});
+    // cuda_basic_test.cc:40-62: a pair of CPU endpoints is left to CPU channels.
+    auto cpuToCpu = [](Endpoint&) {
+      auto c = makeContext();
+      const auto& d = c->deviceDescriptors();
+      const Device cpu{kCpuDeviceType, 0};
+      const Device gpu{kHipDeviceType, 0};
+      EXPECT_EQ(d.count(cpu), size_t(1));
+      EXPECT_EQ(d.count(gpu), size_t(1));
+      if (d.count(cpu) == 1 && d.count(gpu) == 1) {
+        EXPECT_FALSE(c->canCommunicateWithRemote(d.at(cpu), d.at(cpu)));
+        EXPECT_TRUE(c->canCommunicateWithRemote(d.at(cpu), d.at(gpu)));
+        EXPECT_TRUE(c->canCommunicateWithRemote(d.at(gpu), d.at(cpu)));
+        EXPECT_TRUE(c->canCommunicateWithRemote(d.at(gpu), d.at(gpu)));
+      }
+      c->join();
+    };
+    cases.push_back({"CannotCommunicateCpuToCpu", cpuToCpu, cpuToCpu});
+  }
+
+  if (gSuite == "hip_ipc") {
+    // cuda_ipc_test.cc:37-57: two contexts of one process must not pick IPC.
+    auto sameProcess = [](Endpoint&) {
+      auto c1 = makeContext();
+      auto c2 = makeContext();
+      const Device gpu{kHipDeviceType, 0};
+      const auto& d1 = c1->deviceDescriptors();
+      const auto& d2 = c2->deviceDescriptors();
+      EXPECT_EQ(d1.count(gpu), size_t(1));
+      EXPECT_EQ(d2.count(gpu), size_t(1));
+      if (d1.count(gpu) == 1 && d2.count(gpu) == 1) {
+        EXPECT_FALSE(c1->canCommunicateWithRemote(d1.at(gpu), d2.at(gpu)));
+      }
+      c1->join();
+      c2->join();
+    };
+    cases.push_back({"CannotCommunicateInSameProcess", sameProcess, sameProcess});
+  }
+
+  if (gSuite == "hip_xth") {
+    auto sameProcess = [](Endpoint&) {
+      auto c1 = makeContext();
+      auto c2 = makeContext();
+      const Device gpu{kHipDeviceType, 0};
+      EXPECT_TRUE(c1->canCommunicateWithRemote(
+          c1->deviceDescriptors().at(gpu), c2->deviceDescriptors().at(gpu)));
+      // Same boot, another process: refused.
+      std::string other = c2->deviceDescriptors().at(gpu) + "9";
+      EXPECT_FALSE(c1->canCommunicateWithRemote(c1->deviceDescriptors().at(gpu), other));
+      c1->join();
+      c2->join();
+    };
+    cases.push_back({"CommunicatesOnlyInSameProcess", sameProcess, sameProcess});
+  }
+
+  // channel_test_cpu.cc:44-109: the callback does not run inside send()/recv()
+  // on the caller's stack (it would deadlock on the caller's mutex here). The
+  // reference asks this of its CPU channels only. hip_basic is left out: its
+  // recv callback means "copy enqueued", which can be true before recv()
+  // returns when the sender's chunk notice is already waiting.
+  if (!staged)
+  cases.push_back(
+      {"CallbacksAreDeferred",
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         auto d = makeData(gGpu, iota(256));
+         auto p = std::make_shared<std::promise<Error>>();
+         auto f = p->get_future();
+         auto mutex = std::make_shared<std::mutex>();
+         {
+           std::unique_lock<std::mutex> callerLock(*mutex);
+           o->ch->send(d->buffer(), 256, [p, mutex](const Error& e) {
+             std::unique_lock<std::mutex> calleeLock(*mutex);
+             p->set_value(e);
+           });
+         }
+         EXPECT_OK(waitFor(f, "send"));
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto o = open(ep);
+         auto d = makeData(gGpu, 256);
+         auto p = std::make_shared<std::promise<Error>>();
+         auto f = p->get_future();
+         auto mutex = std::make_shared<std::mutex>();
+         {
+           std::unique_lock<std::mutex> callerLock(*mutex);
+           o->ch->recv(d->buffer(), 256, [p, mutex](const Error& e) {
+             std::unique_lock<std::mutex> calleeLock(*mutex);
+             p->set_value(e);
+           });
+         }
+         EXPECT_OK(waitFor(f, "recv"));
+         expectBytes(*d, iota(256), "received data");
+         ep.barrier();
+       }});
+
+  // ---- closing and errors (channel_impl_boilerplate.h:189-192, error.h:18-37) --
+
+  // After close() every new operation fails with ChannelClosedError, through
+  // its callback, exactly once. The server closes first; the client, whose
+  // channel may already have seen the server go away, fails with whichever
+  // error came first (the first error latches).
+  auto closedChannel = [](Endpoint& ep) {
+    auto o = open(ep);
+    ep.barrier(); // both channels exist
+    if (!ep.isServer()) {
+      ep.barrier(); // the server has closed and checked
+    }
+    o->ch->close();
+    auto d = makeData(gGpu, 64);
+    auto fs = sendF(*o->ch, d->buffer(), 64);
+    auto fr = recvF(*o->ch, d->buffer(), 64);
+    Error es = waitFor(fs, "send after close");
+    Error er = waitFor(fr, "recv after close");
+    EXPECT_TRUE(static_cast<bool>(es));
+    EXPECT_TRUE(static_cast<bool>(er));
+    if (ep.isServer()) {
+      EXPECT_TRUE(es.isOfType<channel::ChannelClosedError>());
+      EXPECT_TRUE(er.isOfType<channel::ChannelClosedError>());
+      ep.barrier();
+    }
+    ep.barrier();
+  };
+  cases.push_back({"OperationsAfterCloseFail", closedChannel, closedChannel});
+
+  // Closing the context closes its channels.
+  auto closedContext = [](Endpoint& ep) {
+    auto o = open(ep);
+    ep.barrier();
+    o->ctx->close();
+    auto d = makeData(gGpu, 64);
+    auto fs = sendF(*o->ch, d->buffer(), 64);
+    Error es = waitFor(fs, "send after context close");
+    EXPECT_TRUE(static_cast<bool>(es));
+    ep.barrier();
+  };
+  cases.push_back({"ContextCloseFailsOperations", closedContext, closedContext});
+
+  // A receive that can never be matched fails once the peer has gone away.
+  cases.push_back({"PeerCloseFailsPendingRecv",
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     auto d = makeData(gGpu, 4096);
+                     auto f = recvF(*o->ch, d->buffer(), 4096);
+                     ep.barrier(); // recv posted; the client closes now
+                     Error e = waitFor(f, "recv that must fail");
+                     EXPECT_TRUE(static_cast<bool>(e));
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     ep.barrier();
+                     o->ch->close();
+                     o.reset();
+                     ep.barrier();
+                   }});
+
+  // channel/context_boilerplate.h:147-149: a context that is dropped without
+  // join() cleans up after itself (the destructor joins).
+  cases.push_back({"ContextIsNotJoined",
+                   [](Endpoint& ep) {
+                     auto ctx = makeContext();
+                     auto conns = ep.openConnections(ctx->numConnectionsNeeded());
+                     auto ch = ctx->createChannel(std::move(conns), channel::Endpoint::kListen);
+                     auto d = makeData(gGpu, iota(256));
+                     auto f = sendF(*ch, d->buffer(), 256);
+                     EXPECT_OK(waitFor(f, "send"));
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     auto ctx = makeContext();
+                     auto conns = ep.openConnections(ctx->numConnectionsNeeded());
+                     auto ch = ctx->createChannel(std::move(conns), channel::Endpoint::kConnect);
+                     auto d = makeData(gGpu, 256);
+                     auto f = recvF(*ch, d->buffer(), 256);
+                     EXPECT_OK(waitFor(f, "recv"));
+                     expectBytes(*d, iota(256), "received data");
+                     ep.barrier();
+                   }});
+
+  return cases;
+}
+
+} // namespace
+
+int main(int argc, char** argv) {
+  Args args = parseArgs(argc, argv);
+  if (!knownSuite(args.suite)) {
+    std::fprintf(
+        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_basic|basic|xth [--case S] [--list]\n",
+        argv[0]);
+    return 2;
+  }
+  gSuite = args.suite;
+  gGpu = gSuite.rfind("hip_", 0) == 0;
+  std::vector<Case> cases = makeCases();
+  if (args.list) {
+    for (auto& c : cases) {
+      std::printf("%s\n", c.name.c_str());
+    }
+    return 0;
+  }
+  const std::string addr =
+      args.addr.empty() ? "tptest_" + std::to_string(::getpid()) + "_" + gSuite : args.addr;
+  if (args.role == "server") {
+    return runSingleRole(Role::kServer, cases, args.filter, addr, args.readyFd);
+  }
+  if (args.role == "client") {
+    return runSingleRole(Role::kClient, cases, args.filter, addr, -1);
+  }
+  if (!twoProcessSuite(gSuite)) {
+    return runBoth(cases, args.filter, addr);
+  }
+  std::vector<std::string> pass = {"--suite", gSuite};
+  if (!args.filter.empty()) {
+    pass.push_back("--case");
+    pass.push_back(args.filter);
+  }
+  return orchestrate(argv[0], pass, addr);
+}

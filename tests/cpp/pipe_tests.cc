@@ -1,0 +1,344 @@
+// Pipe-level tests of messages that mix CPU and GPU tensors, through
+// Context::registerChannel + Pipe::write / readDescriptor / read, with the
+// channel set and priorities of the reference's test context
+// (tensorpipe/test/core/pipe_test.h:292-316): basic 100, hip_basic 10,
+// hip_ipc 11, hip_xth 12 over the shm transport.
+//
+//   pipe_tests --suite [cpu_]two_process|[cpu_]same_process [--case SUBSTRING] [--list]
+//
+// The cpu_ suites run the same messages with every tensor in host memory and
+// only the CPU channels (basic 100, xth 101) registered.
+//
+// The messages are those of tensorpipe/test/core/pipe_cuda_test.cc:13-262:
+// three payloads "payload #k", tensors "tensor #k" with per-item metadata,
+// sources and targets on cpu:0 / the GPU in every combination, received into
+// freshly allocated buffers on the devices the test names; checked as
+// expectDescriptorAndStorageMatchMessage does (pipe_test.h:225-280).
+#include "support.h"
+
+using namespace tptest;
+
+namespace {
+
+// Without a GPU (the cpu_* suites) every "GPU" tensor of the messages below
+// becomes a CPU tensor and only the CPU channels are registered.
+bool gHaveGpu = true;
+const Device kCpu{kCpuDeviceType, 0};
+Device kGpu{kHipDeviceType, 0};
+
+struct InlineTensor {
+  std::string data;
+  std::string metadata;
+  Device device;
+  optional<Device> target;
+};
+
+struct InlineMessage {
+  std::vector<std::pair<std::string, std::string>> payloads; // data, metadata
+  std::vector<InlineTensor> tensors;
+  std::string metadata;
+};
+
+std::shared_ptr<Context> makeContext(const char* name) {
+  auto ctx = std::make_shared<Context>(ContextOptions().name(name));
+  ctx->registerTransport(1, "shm", transport::shm::create());
+  ctx->registerChannel(100, "basic", channel::basic::create());
+  ctx->registerChannel(101, "xth", channel::xth::create());
+  if (!gHaveGpu) {
+    return ctx;
+  }
+  ctx->registerChannel(10, "hip_basic", channel::hip_basic::create(channel::basic::create()));
+  ctx->registerChannel(11, "hip_ipc", channel::hip_ipc::create());
+  ctx->registerChannel(12, "hip_xth", channel::hip_xth::create());
+  return ctx;
+}
+
+std::vector<uint8_t> toBytes(const std::string& s) {
+  return std::vector<uint8_t>(s.begin(), s.end());
+}
+
+// Owns the memory a Message refers to.
+struct Storage {
+  std::vector<std::vector<uint8_t>> payloads;
+  std::vector<std::unique_ptr<Data>> tensors;
+};
+
+Message buildMessage(const InlineMessage& im, Storage* storage) {
+  Message m;
+  m.metadata = im.metadata;
+  for (auto& p : im.payloads) {
+    storage->payloads.push_back(toBytes(p.first));
+    Message::Payload mp;
+    mp.data = storage->payloads.back().data();
+    mp.length = storage->payloads.back().size();
+    mp.metadata = p.second;
+    m.payloads.push_back(std::move(mp));
+  }
+  for (auto& t : im.tensors) {
+    storage->tensors.push_back(makeData(gHaveGpu && t.device == kGpu, toBytes(t.data)));
+    Message::Tensor mt;
+    mt.buffer = storage->tensors.back()->buffer();
+    mt.length = t.data.size();
+    mt.targetDevice = t.target;
+    mt.metadata = t.metadata;
+    m.tensors.push_back(std::move(mt));
+  }
+  return m;
+}
+
+void writeMessage(Pipe& pipe, const InlineMessage& im) {
+  Storage storage;
+  Message m = buildMessage(im, &storage);
+  auto p = std::make_shared<std::promise<Error>>();
+  auto f = p->get_future();
+  pipe.write(std::move(m), [p](const Error& e) { p->set_value(e); });
+  EXPECT_OK(waitFor(f, "write"));
+}
+
+// readDescriptor, allocate on `devices`, read, compare with `im`.
+void readAndCheck(Pipe& pipe, const InlineMessage& im, const std::vector<Device>& devices) {
+  auto pd = std::make_shared<std::promise<std::pair<Error, Descriptor>>>();
+  auto fd = pd->get_future();
+  pipe.readDescriptor([pd](const Error& e, Descriptor d) { pd->set_value({e, std::move(d)}); });
+  auto rd = waitFor(fd, "readDescriptor");
+  EXPECT_OK(rd.first);
+  if (rd.first) {
+    return;
+  }
+  const Descriptor& d = rd.second;
+  EXPECT_EQ(d.metadata, im.metadata);
+  EXPECT_EQ(d.payloads.size(), im.payloads.size());
+  EXPECT_EQ(d.tensors.size(), im.tensors.size());
+  EXPECT_EQ(d.tensors.size(), devices.size());
+  if (failures().any()) {
+    throw Fatal("descriptor does not match the message; not reading");
+  }
+
+  Storage storage;
+  Allocation a;
+  for (auto& p : d.payloads) {
+    storage.payloads.emplace_back(p.length, 0);
+    Allocation::Payload ap;
+    ap.data = storage.payloads.back().data();
+    a.payloads.push_back(ap);
+  }
+  for (size_t i = 0; i < d.tensors.size(); ++i) {
+    storage.tensors.push_back(makeData(gHaveGpu && devices[i] == kGpu, d.tensors[i].length));
+    Allocation::Tensor at;
+    at.buffer = storage.tensors.back()->buffer();
+    a.tensors.push_back(std::move(at));
+  }
+  auto pr = std::make_shared<std::promise<Error>>();
+  auto fr = pr->get_future();
+  pipe.read(std::move(a), [pr](const Error& e) { pr->set_value(e); });
+  EXPECT_OK(waitFor(fr, "read"));
+
+  for (size_t i = 0; i < im.payloads.size(); ++i) {
+    EXPECT_EQ(d.payloads[i].metadata, im.payloads[i].second);
+    EXPECT_EQ(d.payloads[i].length, im.payloads[i].first.size());
+    EXPECT_EQ(std::string(storage.payloads[i].begin(), storage.payloads[i].end()), im.payloads[i].first);
+  }
+  for (size_t i = 0; i < im.tensors.size(); ++i) {
+    EXPECT_TRUE(d.tensors[i].sourceDevice == im.tensors[i].device);
+    EXPECT_EQ(d.tensors[i].metadata, im.tensors[i].metadata);
+    EXPECT_EQ(d.tensors[i].targetDevice.has_value(), im.tensors[i].target.has_value());
+    if (d.tensors[i].targetDevice.has_value() && im.tensors[i].target.has_value()) {
+      EXPECT_TRUE(*d.tensors[i].targetDevice == *im.tensors[i].target);
+      EXPECT_TRUE(*im.tensors[i].target == devices[i]);
+    }
+    EXPECT_EQ(d.tensors[i].length, im.tensors[i].data.size());
+    std::vector<uint8_t> got = storage.tensors[i]->bytes();
+    EXPECT_EQ(std::string(got.begin(), got.end()), im.tensors[i].data);
+  }
+}
+
+struct PipeEnd {
+  std::shared_ptr<Context> ctx;
+  std::shared_ptr<Listener> listener;
+  std::shared_ptr<Pipe> pipe;
+  ~PipeEnd() {
+    pipe.reset();
+    listener.reset();
+    if (ctx) {
+      ctx->join();
+    }
+  }
+};
+
+std::unique_ptr<PipeEnd> openPipe(Endpoint& ep) {
+  auto e = std::make_unique<PipeEnd>();
+  const std::string url = "shm://" + ep.freshAddr();
+  if (ep.isServer()) {
+    e->ctx = makeContext("server");
+    e->listener = e->ctx->listen({url});
+    ep.signalListening();
+    auto p = std::make_shared<std::promise<std::pair<Error, std::shared_ptr<Pipe>>>>();
+    auto f = p->get_future();
+    e->listener->accept([p](const Error& err, std::shared_ptr<Pipe> pipe) {
+      p->set_value({err, std::move(pipe)});
+    });
+    auto r = waitFor(f, "accept");
+    if (r.first) {
+      throw Fatal("accept failed: " + r.first.what());
+    }
+    e->pipe = std::move(r.second);
+  } else {
+    e->ctx = makeContext("client");
+    ep.awaitListening();
+    e->pipe = e->ctx->connect(url);
+  }
+  return e;
+}
+
+InlineMessage messageWith(std::vector<InlineTensor> tensors) {
+  InlineMessage im;
+  im.payloads = {{"payload #1", "payload metadata #1"},
+                 {"payload #2", "payload metadata #2"},
+                 {"payload #3", "payload metadata #3"}};
+  im.tensors = std::move(tensors);
+  im.metadata = "pipe metadata";
+  return im;
+}
+
+// The server writes `im`; the client reads it onto `devices`.
+Case oneWay(std::string name, InlineMessage im, std::vector<Device> devices) {
+  return Case{std::move(name),
+              [im](Endpoint& ep) {
+                auto e = openPipe(ep);
+                writeMessage(*e->pipe, im);
+                ep.barrier();
+              },
+              [im, devices](Endpoint& ep) {
+                auto e = openPipe(ep);
+                readAndCheck(*e->pipe, im, devices);
+                ep.barrier();
+              }};
+}
+
+std::vector<Case> makeCases() {
+  std::vector<Case> cases;
+
+  // pipe_cuda_test.cc:13-81
+  cases.push_back(oneWay(
+      "SimpleWriteReadWithAllTargetDevices",
+      messageWith({{"tensor #1", "tensor metadata #1", kGpu, kGpu},
+                   {"tensor #2", "tensor metadata #2", kCpu, kGpu},
+                   {"tensor #3", "tensor metadata #3", kGpu, kCpu},
+                   {"tensor #4", "tensor metadata #4", kCpu, kCpu}}),
+      {kGpu, kGpu, kCpu, kCpu}));
+
+  // pipe_cuda_test.cc:83-142
+  cases.push_back(oneWay(
+      "SimpleWriteReadWithSomeTargetDevices",
+      messageWith({{"tensor #1", "tensor metadata #1", kGpu, kGpu},
+                   {"tensor #2", "tensor metadata #2", kGpu, nullopt},
+                   {"tensor #3", "tensor metadata #3", kCpu, nullopt}}),
+      {kGpu, kCpu, kCpu}));
+
+  // pipe_cuda_test.cc:144-208
+  cases.push_back(oneWay(
+      "SimpleWriteReadWithoutTargetDevice",
+      messageWith({{"tensor #1", "tensor metadata #1", kCpu, nullopt},
+                   {"tensor #2", "tensor metadata #2", kCpu, nullopt},
+                   {"tensor #3", "tensor metadata #3", kGpu, nullopt},
+                   {"tensor #4", "tensor metadata #4", kGpu, nullopt}}),
+      {kCpu, kGpu, kCpu, kGpu}));
+
+  // Several messages back to back, each answered, with tensors large enough to
+  // go through more than one staging slot.
+  cases.push_back(
+      {"MixedMessagesBothDirections",
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         for (int k = 0; k < 5; ++k) {
+           InlineMessage out = messageWith(
+               {{std::string(3 * 1024 * 1024 + k, char('a' + k)), "big", kGpu, kGpu},
+                {std::string(100 + k, char('A' + k)), "small", kCpu, nullopt},
+                {"", "empty", kGpu, nullopt}});
+           writeMessage(*e->pipe, out);
+           InlineMessage in = messageWith(
+               {{std::string(2 * 1024 * 1024 + k, char('k' + k)), "reply", kGpu, nullopt}});
+           readAndCheck(*e->pipe, in, {kCpu});
+         }
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         for (int k = 0; k < 5; ++k) {
+           InlineMessage in = messageWith(
+               {{std::string(3 * 1024 * 1024 + k, char('a' + k)), "big", kGpu, kGpu},
+                {std::string(100 + k, char('A' + k)), "small", kCpu, nullopt},
+                {"", "empty", kGpu, nullopt}});
+           readAndCheck(*e->pipe, in, {kGpu, kGpu, kGpu});
+           InlineMessage out = messageWith(
+               {{std::string(2 * 1024 * 1024 + k, char('k' + k)), "reply", kGpu, nullopt}});
+           writeMessage(*e->pipe, out);
+         }
+         ep.barrier();
+       }});
+
+  // A pipe that is closed fails what is pending and what comes later.
+  cases.push_back({"CloseFailsPendingRead",
+                   [](Endpoint& ep) {
+                     auto e = openPipe(ep);
+                     auto pd = std::make_shared<std::promise<Error>>();
+                     auto fd = pd->get_future();
+                     e->pipe->readDescriptor(
+                         [pd](const Error& err, Descriptor) { pd->set_value(err); });
+                     ep.barrier(); // the client closes its end now
+                     Error err = waitFor(fd, "readDescriptor that must fail");
+                     EXPECT_TRUE(static_cast<bool>(err));
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     auto e = openPipe(ep);
+                     // make sure the pipe is fully established before closing
+                     ep.barrier();
+                     e->pipe->close();
+                     ep.barrier();
+                   }});
+
+  return cases;
+}
+
+} // namespace
+
+int main(int argc, char** argv) {
+  Args args = parseArgs(argc, argv);
+  const bool cpuOnly = args.suite.rfind("cpu_", 0) == 0;
+  const std::string shape = cpuOnly ? args.suite.substr(4) : args.suite;
+  if (shape != "two_process" && shape != "same_process") {
+    std::fprintf(
+        stderr, "usage: %s --suite [cpu_]two_process|[cpu_]same_process [--case S] [--list]\n",
+        argv[0]);
+    return 2;
+  }
+  if (cpuOnly) {
+    gHaveGpu = false;
+    kGpu = kCpu;
+  }
+  std::vector<Case> cases = makeCases();
+  if (args.list) {
+    for (auto& c : cases) {
+      std::printf("%s\n", c.name.c_str());
+    }
+    return 0;
+  }
+  const std::string addr =
+      args.addr.empty() ? "tppipe_" + std::to_string(::getpid()) + "_" + args.suite : args.addr;
+  if (args.role == "server") {
+    return runSingleRole(Role::kServer, cases, args.filter, addr, args.readyFd);
+  }
+  if (args.role == "client") {
+    return runSingleRole(Role::kClient, cases, args.filter, addr, -1);
+  }
+  if (shape == "same_process") {
+    return runBoth(cases, args.filter, addr);
+  }
+  std::vector<std::string> pass = {"--suite", args.suite};
+  if (!args.filter.empty()) {
+    pass.push_back("--case");
+    pass.push_back(args.filter);
+  }
+  return orchestrate(argv[0], pass, addr);
+}

@@ -1,0 +1,78 @@
+"""Runs the C++ test programs under tests/cpp and reports every case as a test.
+
+The programs drive the product's C++ API directly: channel::Context::createChannel +
+Channel::send/recv (channel_tests) and Context/Listener/Pipe with mixed CPU/GPU messages
+(pipe_tests), following the reference's own suites (tensorpipe/test/channel/*.cc,
+tensorpipe/test/core/pipe_cuda_test.cc). Each suite is started once; every endpoint of
+every case prints a "RESULT <role> <case> OK|FAIL ..." line that is checked here.
+"""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "bin")
+
+CPU_SUITES = [("channel_tests", "basic"), ("channel_tests", "xth"),
+              ("pipe_tests", "cpu_same_process"), ("pipe_tests", "cpu_two_process")]
+GPU_SUITES = [("channel_tests", "hip_xth"), ("channel_tests", "hip_ipc"), ("channel_tests", "hip_basic"),
+              ("pipe_tests", "same_process"), ("pipe_tests", "two_process")]
+
+_results = {}
+
+
+def _binary(program):
+    path = os.path.join(BIN, program)
+    if not os.path.exists(path):
+        pytest.fail(f"{path} is not built (run __graft_entry__.build())")
+    return path
+
+
+def list_cases(program, suite):
+    path = os.path.join(BIN, program)
+    if not os.path.exists(path):
+        return ["<not built>"]
+    out = subprocess.run([path, "--suite", suite, "--list"], stdout=subprocess.PIPE, text=True, timeout=30)
+    return out.stdout.split()
+
+
+def run_suite(program, suite):
+    """One run per suite and session; returns {case: [(role, ok, detail), ...]}."""
+    key = (program, suite)
+    if key not in _results:
+        print(f"running {program} --suite {suite}", flush=True)
+        proc = subprocess.run([_binary(program), "--suite", suite], stdout=subprocess.PIPE,
+                              stderr=subprocess.PIPE, text=True, timeout=600)
+        per_case = {}
+        for line in proc.stdout.splitlines():
+            parts = line.split(" ", 4)
+            if len(parts) >= 4 and parts[0] == "RESULT":
+                role, case, verdict = parts[1], parts[2], parts[3]
+                per_case.setdefault(case, []).append((role, verdict == "OK", line))
+        _results[key] = (proc.returncode, per_case, proc.stdout[-4000:], proc.stderr[-4000:])
+    return _results[key]
+
+
+def check_case(program, suite, case):
+    rc, per_case, out, err = run_suite(program, suite)
+    assert case in per_case, f"no result for {case}; exit code {rc}\n{out}\n{err}"
+    bad = [line for _, ok, line in per_case[case] if not ok]
+    assert not bad, "\n".join(bad) + "\n" + err
+    two_process = suite in ("basic", "hip_ipc", "hip_basic", "two_process", "cpu_two_process")
+    assert len(per_case[case]) == (2 if two_process else 1), per_case[case]
+
+
+def _params(suites):
+    return [pytest.param(p, s, c, id=f"{s}-{c}") for p, s in suites for c in list_cases(p, s)]
+
+
+@pytest.mark.parametrize("program,suite,case", _params(CPU_SUITES))
+def test_cpu_suite(program, suite, case):
+    check_case(program, suite, case)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("program,suite,case", _params(GPU_SUITES))
+def test_gpu_suite(program, suite, case):
+    check_case(program, suite, case)
