@@ -305,6 +305,34 @@ std::vector<Case> makeCases() {
                      [v](Endpoint& ep) { receiver(ep, gGpu, v); }});
   }
 
+  // Memory that is freed and allocated again between sends (the allocator
+  // tends to hand the same address back): the receiver must see the bytes of
+  // the allocation that is live now, never those of a mapping it kept from an
+  // earlier one.
+  cases.push_back({"SourceFreedAndAllocatedAgain",
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     for (int k = 0; k < 12; ++k) {
+                       auto d = makeData(gGpu, std::vector<uint8_t>((1 << 20) + 64 * k, uint8_t(k + 1)));
+                       auto f = sendF(*o->ch, d->buffer(), d->size());
+                       EXPECT_OK(waitFor(f, "send"));
+                       ep.barrier(); // the receiver has checked; free the source now
+                     }
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     auto o = open(ep);
+                     for (int k = 0; k < 12; ++k) {
+                       const size_t n = (1 << 20) + 64 * k;
+                       auto d = makeData(gGpu, n);
+                       auto f = recvF(*o->ch, d->buffer(), n);
+                       EXPECT_OK(waitFor(f, "recv"));
+                       expectBytes(*d, std::vector<uint8_t>(n, uint8_t(k + 1)), "round");
+                       ep.barrier();
+                     }
+                     ep.barrier();
+                   }});
+
   if (staged) {
     // channel_test_cuda_xdtt.cc:19-143: 1024 bytes of 0x42 across device types.
     cases.push_back({"SendFromCpuToGpu",
