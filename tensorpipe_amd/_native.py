@@ -28,6 +28,40 @@ def _load(name, mode=ctypes.DEFAULT_MODE):
     return ctypes.CDLL(path, mode=mode)
 
 
+_hip_runtime_pinned = False
+
+
+def _share_hip_runtime_with_torch():
+    """One HIP runtime per process.
+
+    PyTorch wheels bundle their own libamdhip64.so and link it by file name, while
+    libtphip.so links the runtime by its soname (libamdhip64.so.7). If libtphip.so is
+    loaded first, the system runtime comes in under the soname and a later `import torch`
+    loads the bundled file as well: two runtimes, each blind to the other's allocations
+    (pointer queries and hipIpcOpenMemHandle then fail with "invalid argument"). Loading
+    the bundled runtime first, by path, makes both names resolve to that one object.
+    Processes without torch simply get the system runtime.
+    """
+    global _hip_runtime_pinned
+    if _hip_runtime_pinned:
+        return
+    _hip_runtime_pinned = True
+    import importlib.util
+    import sys
+
+    if "torch" in sys.modules:
+        return  # already loaded; libtphip.so binds to the same soname
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.origin:
+        return
+    bundled = os.path.join(os.path.dirname(spec.origin), "lib", "libamdhip64.so")
+    if os.path.exists(bundled):
+        ctypes.CDLL(bundled, mode=ctypes.RTLD_GLOBAL)
+
+
 class CopyDesc(ctypes.Structure):
     """Mirror of tphip_copy_desc (include/tphip.h)."""
 
@@ -42,6 +76,7 @@ _tpc = None
 def tphip():
     global _tphip
     if _tphip is None:
+        _share_hip_runtime_with_torch()
         lib = _load("libtphip.so", mode=ctypes.RTLD_GLOBAL)
         vp, i32, u32, u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64
         P = ctypes.POINTER

@@ -170,39 +170,69 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
   const uint32_t total = sPrefix[n];
   constexpr uint32_t kChunk = kBlockThreads * U;
 
-  for (uint32_t g = wave; g * kWave < n; g += nwaves) {
-    copy_edges(descs, n, g, lane);
-  }
-
-  uint32_t t = 0; // entry containing the start of the previous chunk
-#pragma clang loop unroll(disable)
-  for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    const uint32_t c0 = c * kChunk;
-    const uint32_t cEnd = total - c0 < kChunk ? total : c0 + kChunk;
-    // Largest entry index with prefix <= c0; chunks only move forward.
-    uint32_t lo = t, hi = n;
+  // Entry that holds vector `first` (largest index with prefix <= first),
+  // searched from `from` onwards: a workgroup's chunks only move forward.
+  auto locate = [&](uint32_t first, uint32_t from) -> uint32_t {
+    uint32_t lo = from, hi = n;
     while (hi - lo > 1) {
       const uint32_t mid = (lo + hi) >> 1;
-      if (sPrefix[mid] <= c0) {
+      if (sPrefix[mid] <= first) {
         lo = mid;
       } else {
         hi = mid;
       }
     }
-    t = __builtin_amdgcn_readfirstlane(lo);
-    const uint32_t tBegin = sPrefix[t];
-    const uint32_t tEnd = sPrefix[t + 1];
+    return __builtin_amdgcn_readfirstlane(lo);
+  };
+
+  // Where a chunk lives: entry, addresses of its first vector, vector count and
+  // whether it lies inside one entry. Resolving costs a chain of dependent LDS
+  // reads, so the NEXT chunk is resolved while the loads of the current one are
+  // in flight (LDS and global memory have separate wait counters); only the
+  // first resolve of a workgroup is exposed.
+  struct Where {
+    const char* s;
+    char* d;
+    uint32_t c0;
+    uint32_t cnt;
+    uint32_t t;
+    bool inside;
+  };
+  auto resolve = [&](uint32_t c, uint32_t from) -> Where {
+    Where w;
+    w.c0 = c * kChunk;
+    const uint32_t cEnd = total - w.c0 < kChunk ? total : w.c0 + kChunk;
+    w.cnt = cEnd - w.c0;
+    w.t = locate(w.c0, from);
+    const uint32_t tBegin = sPrefix[w.t];
+    w.inside = cEnd <= sPrefix[w.t + 1];
+    const uint64_t off = static_cast<uint64_t>(w.c0 - tBegin) * 16;
+    w.s = body[w.t].src + off;
+    w.d = body[w.t].dst + off;
+    return w;
+  };
+
+  Where cur{};
+  if (blockIdx.x < nchunks) {
+    cur = resolve(blockIdx.x, 0);
+  }
+#pragma clang loop unroll(disable)
+  for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+    const uint32_t cNext = c + gridDim.x;
+    Where nxt = cur;
     u32x4 v[U];
-    if (cEnd <= tEnd) {
+    if (cur.inside) {
       // Whole chunk inside one entry: uniform base, contiguous addresses.
-      const uint64_t off = static_cast<uint64_t>(c0 - tBegin) * 16;
-      const char* s = body[t].src + off;
-      char* d = body[t].dst + off;
-      const uint32_t cnt = cEnd - c0;
+      const char* s = cur.s;
+      char* d = cur.d;
+      const uint32_t cnt = cur.cnt;
       if (cnt == kChunk) {
 #pragma unroll
         for (int j = 0; j < U; ++j) {
           v[j] = load16<NT>(s + (static_cast<size_t>(j) * kBlockThreads + threadIdx.x) * 16);
+        }
+        if (cNext < nchunks) {
+          nxt = resolve(cNext, cur.t);
         }
 #pragma unroll
         for (int j = 0; j < U; ++j) {
@@ -216,6 +246,9 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
           const uint32_t idx = j * kBlockThreads + threadIdx.x;
           v[j] = load16<NT>(s + static_cast<size_t>(idx < cnt ? idx : cnt - 1) * 16);
         }
+        if (cNext < nchunks) {
+          nxt = resolve(cNext, cur.t);
+        }
 #pragma unroll
         for (int j = 0; j < U; ++j) {
           const uint32_t idx = j * kBlockThreads + threadIdx.x;
@@ -226,13 +259,13 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
       }
     } else {
       // Chunk straddles entries: per-lane lookup packs small tensors tightly.
-      const uint32_t cnt = cEnd - c0;
+      const uint32_t cnt = cur.cnt;
       char* dp[U];
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint32_t idx = j * kBlockThreads + threadIdx.x;
-        const uint32_t vv = c0 + (idx < cnt ? idx : cnt - 1);
-        uint32_t l = t, h = n;
+        const uint32_t vv = cur.c0 + (idx < cnt ? idx : cnt - 1);
+        uint32_t l = cur.t, h = n;
         while (h - l > 1) {
           const uint32_t m = (l + h) >> 1;
           if (sPrefix[m] <= vv) {
@@ -245,6 +278,9 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
         v[j] = load16<NT>(body[l].src + off);
         dp[j] = body[l].dst + off;
       }
+      if (cNext < nchunks) {
+        nxt = resolve(cNext, cur.t);
+      }
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         if (j * kBlockThreads + threadIdx.x < cnt) {
@@ -252,6 +288,14 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
         }
       }
     }
+    cur = nxt;
+  }
+
+  // Heads and tails last, on the waves at the far end of the grid (they run
+  // out of chunks first): the byte-wise gather is latency-bound and would
+  // otherwise delay the chunks of the workgroup that does it.
+  for (uint32_t g = nwaves - 1 - wave; g * kWave < n; g += nwaves) {
+    copy_edges(descs, n, g, lane);
   }
 }
 

@@ -533,7 +533,7 @@ class ChannelImpl final : public ChannelImplBase {
       const int device = stagePending_.front().device;
       std::vector<tphip_copy_desc> table;
       std::vector<std::shared_ptr<SendChunk>> chunks;
-      const size_t cap = batchCap(bctx_->numSlots);
+      const size_t cap = batchCap(bctx_->numSlots, bctx_->slotBytes);
       for (auto it = stagePending_.begin(); it != stagePending_.end() && table.size() < cap;) {
         if (it->stream == stream && it->device == device) {
           table.push_back(it->desc);
@@ -559,21 +559,38 @@ class ChannelImpl final : public ChannelImplBase {
 
   // Chunks per launch. One launch for the whole ring would put the two ends in
   // lock step (the sender stages all slots, then idles while the receiver
-  // drains all of them); half the ring (a quarter for deep rings) lets one end
-  // fill slots while the other drains the rest.
-  static size_t batchCap(size_t numSlots) {
-    const size_t quarter = std::max<size_t>(numSlots / 4, 2);
-    return std::max<size_t>(1, std::min(numSlots / 2, quarter));
+  // drains all of them); a quarter of the ring per launch keeps both ends busy
+  // on different slots. Measured, 256 MiB each way: 4 x 1 MiB slots 29 GB/s with
+  // one slot per launch against 22 with two and 20 with four; 16 x 1 MiB 29.5
+  // with four per launch against 28.5 with one; 4 MiB slots are best alone (36).
+  static size_t batchCap(size_t numSlots, size_t slotBytes) {
+    static const long forced = [] {
+      const char* e = std::getenv("TP_HIP_BASIC_BATCH_CAP");
+      return e != nullptr ? std::atol(e) : 0L;
+    }();
+    if (forced > 0) {
+      return static_cast<size_t>(forced);
+    }
+    if (slotBytes >= (2u << 20)) {
+      return 1; // a slot this large amortises its launch by itself
+    }
+    return std::max<size_t>(1, numSlots / 4);
   }
 
   // A copy with one end in pinned host memory: the host link saturates with
-  // about 32 workgroups, more only add contention (50 vs 42 GB/s reading).
+  // about 32 workgroups, more only add contention (50 vs 42 GB/s reading
+  // alone; with the other direction busy 64 workgroups lose 1-5 GB/s).
   bool launchHostLinkCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table) {
     size_t off = 0;
     while (off < table.size()) {
       const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
+      static const long forcedBlocks = [] {
+        const char* e = std::getenv("TP_HIP_BASIC_BLOCKS");
+        return e != nullptr ? std::atol(e) : 0L;
+      }();
+      const uint32_t blocks = forcedBlocks > 0 ? static_cast<uint32_t>(forcedBlocks) : 32;
       int rc = tphip_batched_copy_tuned(
-          device, table.data() + off, static_cast<uint32_t>(n), stream, 4, 32, 3);
+          device, table.data() + off, static_cast<uint32_t>(n), stream, 4, blocks, 3);
       if (rc != 0) {
         setError(TP_CREATE_ERROR(HipError, "tphip_batched_copy", rc));
         return false;
@@ -758,7 +775,7 @@ class ChannelImpl final : public ChannelImplBase {
       std::vector<tphip_copy_desc> table;
       std::vector<uint32_t> slots;
       std::vector<std::shared_ptr<Op>> ops;
-      const size_t cap = batchCap(remoteNumSlots_);
+      const size_t cap = batchCap(remoteNumSlots_, remoteSlotBytes_);
       for (auto it = ringPending_.begin(); it != ringPending_.end() && table.size() < cap;) {
         if (it->stream == stream && it->device == device) {
           table.push_back(it->desc);

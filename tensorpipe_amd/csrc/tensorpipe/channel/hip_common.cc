@@ -171,18 +171,26 @@ int HipIpcImports::acquire(
     return 0;
   }
   // Same handle bytes under another identifier: stale, unmap before mapping anew.
+  size_t staleClosed = 0;
   for (auto& kv : entries_) {
     if (std::get<0>(kv.first) == device && kv.second.mapped && kv.second.handle == handle) {
-      tphip_ipc_mem_close(device, kv.second.ptr);
+      int crc = tphip_ipc_mem_close(device, kv.second.ptr);
+      TP_VLOG(5) << "IPC imports: unmapped stale " << std::get<1>(kv.first) << "#"
+                 << std::get<2>(kv.first) << " (rc " << crc << ") for #" << id;
       kv.second.mapped = false;
       kv.second.ptr = nullptr;
+      ++staleClosed;
     }
   }
   void* ptr = nullptr;
   int rc = tphip_ipc_mem_open(device, handle.data(), &ptr);
   if (rc != 0) {
+    TP_LOG_WARNING() << "IPC imports: cannot map " << peer << "#" << id << ": " << tphip_strerror(rc)
+                     << " (" << entries_.size() << " entries, " << staleClosed
+                     << " stale unmapped, re-acquire of a known id: " << (it != entries_.end()) << ")";
     return rc;
   }
+  TP_VLOG(5) << "IPC imports: mapped " << peer << "#" << id << " at " << ptr;
   Entry& e = entries_[key];
   e.ptr = ptr;
   e.handle = handle;

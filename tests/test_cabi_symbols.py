@@ -39,3 +39,22 @@ def test_copy_desc_layout():
 
     assert ctypes.sizeof(_native.CopyDesc) == 24
     assert _native.CopyDesc.dst.offset == 8 and _native.CopyDesc.bytes.offset == 16
+
+
+def test_one_hip_runtime_per_process():
+    """Loading the native library before torch must not leave two HIP runtimes in the process
+    (each would be blind to the other's allocations)."""
+    import subprocess
+    import sys
+
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "from tensorpipe_amd import _native\n"
+        "_native.tphip()\n"
+        "import torch\n"
+        "libs = sorted({l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l})\n"
+        "print(len(libs), libs)\n" % ROOT
+    )
+    out = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, text=True, timeout=300)
+    assert out.returncode == 0
+    assert out.stdout.split()[0] == "1", out.stdout
