@@ -81,7 +81,7 @@ def build_host(jobs=8):
          f"-L{LIB}", "-ltphip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"])
 
 
-CPP_TESTS = ["channel_tests", "pipe_tests"]
+CPP_TESTS = ["channel_tests", "pipe_tests", "unit_tests"]
 
 
 def build_cpp_tests():

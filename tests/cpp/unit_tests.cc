@@ -1,0 +1,160 @@
+// Host-only unit checks of the small building blocks under the channels; no
+// GPU needed. Driven by tests/test_cpp_units.py.
+//
+//   unit_tests allocator <slots> <ev> <ev> ...   ev = a<k> | r<slot> | c
+//       replays the events on SlotAllocator and prints "k:slot" per grant in
+//       the order the grants happen (slot -1 = failed by close), so the caller
+//       can compare with the golden trace (tensorpipe/common/allocator.cc:26-79).
+//   unit_tests basics
+//       Buffer / Device / Error / wire helpers; prints "OK" or the failures.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include <tensorpipe/common/buffer.h>
+#include <tensorpipe/common/cpu_buffer.h>
+#include <tensorpipe/common/device.h>
+#include <tensorpipe/common/error.h>
+#include <tensorpipe/common/hip_buffer.h>
+#include <tensorpipe/common/slot_allocator.h>
+#include <tensorpipe/common/wire.h>
+#include <tensorpipe/channel/error.h>
+
+using namespace tensorpipe;
+
+static int runAllocator(int argc, char** argv) {
+  const size_t slots = std::strtoul(argv[2], nullptr, 10);
+  const size_t slotSize = 64;
+  std::vector<uint8_t> slab(slots * slotSize);
+  SlotAllocator alloc(slab.data(), slots, slotSize);
+  std::map<size_t, SlotAllocator::TSlot> held; // slot index -> grant
+  for (int i = 3; i < argc; ++i) {
+    const char op = argv[i][0];
+    const long arg = argv[i][1] != 0 ? std::strtol(argv[i] + 1, nullptr, 10) : 0;
+    if (op == 'a') {
+      alloc.alloc([&, arg](const Error& e, SlotAllocator::TSlot s) {
+        if (e) {
+          std::printf("%ld:-1%s ", arg, e.isOfType<AllocatorClosedError>() ? "" : "?");
+          return;
+        }
+        const size_t idx = alloc.slotIndex(s.get());
+        std::printf("%ld:%zu ", arg, idx);
+        held[idx] = std::move(s);
+      });
+    } else if (op == 'r') {
+      auto it = held.find(static_cast<size_t>(arg));
+      if (it == held.end()) {
+        std::printf("\nslot %ld is not held\n", arg);
+        return 1;
+      }
+      SlotAllocator::TSlot s = std::move(it->second);
+      held.erase(it);
+      s.reset(); // returns the slot; a waiter may be served inside this call
+    } else if (op == 'c') {
+      alloc.close();
+    } else {
+      std::printf("\nbad event %s\n", argv[i]);
+      return 2;
+    }
+  }
+  std::printf("\n");
+  return 0;
+}
+
+#define CHECK(cond)                                         \
+  do {                                                      \
+    if (!(cond)) {                                          \
+      std::printf("FAILED line %d: %s\n", __LINE__, #cond); \
+      ++failed;                                             \
+    }                                                       \
+  } while (0)
+
+static int runBasics() {
+  int failed = 0;
+  // Device: value semantics, printing, hashing (tensorpipe/common/device.h:17-64).
+  Device cpu{kCpuDeviceType, 0};
+  Device gpu0{kHipDeviceType, 0};
+  Device gpu1{kHipDeviceType, 1};
+  CHECK(cpu.toString() == "cpu:0");
+  CHECK(gpu1.toString() == "cuda:1");
+  CHECK(gpu0 == Device(kCudaDeviceType, 0));
+  CHECK(gpu0 != gpu1);
+  CHECK(std::hash<Device>{}(gpu0) == std::hash<Device>{}(Device{kHipDeviceType, 0}));
+  CHECK(std::hash<Device>{}(gpu0) != std::hash<Device>{}(gpu1));
+
+  // Buffer: type erasure over CpuBuffer / HipBuffer (tensorpipe/common/buffer.h:21-133).
+  int x = 0;
+  Buffer b = CpuBuffer{&x};
+  CHECK(b.device() == cpu);
+  CHECK(b.unwrap<CpuBuffer>().ptr == &x);
+  bool threw = false;
+  try {
+    (void)b.unwrap<HipBuffer>();
+  } catch (const std::runtime_error&) {
+    threw = true;
+  }
+  CHECK(threw);
+  Buffer copy = b;
+  CHECK(copy.unwrap<CpuBuffer>().ptr == &x);
+  Buffer h = HipBuffer{reinterpret_cast<void*>(0x1000), reinterpret_cast<void*>(0x2000)};
+  CHECK(h.unwrap<HipBuffer>().stream == reinterpret_cast<void*>(0x2000));
+  copy = h;
+  CHECK(copy.unwrap<HipBuffer>().ptr == reinterpret_cast<void*>(0x1000));
+  Buffer dflt;
+  CHECK(dflt.unwrap<CpuBuffer>().ptr == nullptr);
+
+  // Error: falsy when empty, what() names the origin (tensorpipe/common/error.h:38-80).
+  Error ok;
+  CHECK(!ok);
+  CHECK(ok.what() == "success");
+  Error closed = TP_CREATE_ERROR(channel::ChannelClosedError);
+  CHECK(static_cast<bool>(closed));
+  CHECK(closed.isOfType<channel::ChannelClosedError>());
+  CHECK(!closed.isOfType<channel::ContextClosedError>());
+  CHECK(closed.what().find("unit_tests.cc") != std::string::npos);
+  Error sys = TP_CREATE_ERROR(SystemError, "connect", 111);
+  CHECK(sys.what().find("connect") != std::string::npos);
+
+  // Wire helpers: round trip and refusal to read past the end.
+  WireWriter w;
+  w.u8(7);
+  w.u32(0xdeadbeef);
+  w.u64(0x0123456789abcdefull);
+  w.str("hello");
+  w.str("");
+  std::vector<uint8_t> bytes = w.bytes();
+  CHECK(bytes.size() == 1 + 4 + 8 + 4 + 5 + 4);
+  CHECK(bytes[1] == 0xef && bytes[4] == 0xde); // little endian
+  WireReader r(bytes.data(), bytes.size());
+  CHECK(r.u8() == 7);
+  CHECK(r.u32() == 0xdeadbeef);
+  CHECK(r.u64() == 0x0123456789abcdefull);
+  CHECK(r.str() == "hello");
+  std::string e = "x";
+  r.str(&e);
+  CHECK(e.empty());
+  CHECK(r.ok() && r.atEnd());
+  CHECK(r.u32() == 0 && !r.ok());
+  const uint8_t lying[] = {0xff, 0xff, 0xff, 0x7f, 'a'}; // length far beyond the buffer
+  WireReader bad(lying, sizeof(lying));
+  CHECK(bad.str().empty() && !bad.ok());
+
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
+int main(int argc, char** argv) {
+  if (argc >= 3 && std::strcmp(argv[1], "allocator") == 0) {
+    return runAllocator(argc, argv);
+  }
+  if (argc == 2 && std::strcmp(argv[1], "basics") == 0) {
+    return runBasics();
+  }
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics\n", argv[0]);
+  return 2;
+}

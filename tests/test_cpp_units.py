@@ -1,0 +1,60 @@
+"""Host-only unit checks of the C++ building blocks (tests/cpp/unit_tests.cc)."""
+import json
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "bin", "unit_tests")
+with open(os.path.join(ROOT, "tests", "golden", "reference_vectors.json")) as f:
+    GOLDEN = json.load(f)
+
+
+def run(*args):
+    if not os.path.exists(BIN):
+        pytest.fail(f"{BIN} is not built (run __graft_entry__.build())")
+    out = subprocess.run([BIN, *args], stdout=subprocess.PIPE, text=True, timeout=60)
+    return out.returncode, out.stdout
+
+
+def replay(slots, events):
+    rc, out = run("allocator", str(slots), *[op + (str(arg) if op != "c" else "") for op, arg in events])
+    assert rc == 0, out
+    return [tuple(int(x) for x in tok.split(":")) for tok in out.split()]
+
+
+def test_slot_allocator_matches_the_golden_trace():
+    g = GOLDEN["allocator"]
+    assert replay(g["slots"], g["events"]) == [tuple(x) for x in g["grants"]]
+
+
+def test_slot_allocator_matches_the_oracle(oracle):
+    import random
+
+    rng = random.Random(1234)
+    for trial in range(50):
+        slots = rng.randint(1, 6)
+        events, held, waiting, req = [], [], 0, 0
+        for _ in range(rng.randint(1, 40)):
+            if held and rng.random() < 0.45:
+                s = held.pop(rng.randrange(len(held)))
+                events.append(("r", s))
+                if waiting:
+                    waiting -= 1
+                    held.append(s)  # the oldest waiter takes exactly the slot that came back
+            else:
+                events.append(("a", req))
+                req += 1
+                free = [i for i in range(slots) if i not in held]
+                if free and not waiting:
+                    held.append(min(free))
+                else:
+                    waiting += 1
+        events.append(("c", 0))
+        assert replay(slots, events) == oracle.allocator_trace(slots, events), (trial, slots, events)
+
+
+def test_basics():
+    rc, out = run("basics")
+    assert rc == 0 and out.strip() == "OK", out
