@@ -71,12 +71,20 @@ __device__ __forceinline__ uint64_t shfl64(uint64_t v, int srcLane) {
   return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// One wavefront moves the heads and tails of entries [64*group, 64*group+64).
+// Entries whose heads and tails one wavefront moves. The gather below is a
+// chain of dependent byte loads and stores (about one memory latency per 64
+// bytes), so a group is kept small and the groups spread over many waves: 64
+// entries per wave left one workgroup busy for microseconds after every other
+// one had finished.
+constexpr uint32_t kEdgeGroup = 8;
+
+// One wavefront moves the heads and tails of entries
+// [kEdgeGroup*group, kEdgeGroup*(group+1)); all 64 lanes share the byte copies.
 __device__ __forceinline__ void copy_edges(
     const tphip_copy_desc* __restrict__ descs, uint32_t n, uint32_t group, uint32_t lane) {
-  uint32_t t = group * kWave + lane;
+  uint32_t t = group * kEdgeGroup + lane;
   uint64_t src = 0, dst = 0, bytes = 0;
-  if (t < n) {
+  if (lane < kEdgeGroup && t < n) {
     src = reinterpret_cast<uint64_t>(descs[t].src);
     dst = reinterpret_cast<uint64_t>(descs[t].dst);
     bytes = descs[t].bytes;
@@ -294,7 +302,7 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
   // Heads and tails last, on the waves at the far end of the grid (they run
   // out of chunks first): the byte-wise gather is latency-bound and would
   // otherwise delay the chunks of the workgroup that does it.
-  for (uint32_t g = nwaves - 1 - wave; g * kWave < n; g += nwaves) {
+  for (uint32_t g = nwaves - 1 - wave; g * kEdgeGroup < n; g += nwaves) {
     copy_edges(descs, n, g, lane);
   }
 }

@@ -350,7 +350,8 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
 
     const uint64_t chunk = uint64_t(kBlockThreads) * unroll;
     const uint32_t nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
-    const uint32_t edgeBlocks = (n + kBlockThreads - 1) / kBlockThreads;
+    // one wave per kEdgeGroup entries for the heads and tails
+    const uint32_t edgeBlocks = (n + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
     const uint32_t grid = pickBlocks(st, nchunks, edgeBlocks, blocks, true);
     const size_t lds = prefixBytes + (n <= kLdsBodies ? bodyBytes : 0);
     const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
