@@ -127,7 +127,11 @@ def bench_d2d(steps, warmup):
         "profiled_pass_ms_per_step": prof_total_s / steps * 1e3,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBPS,
+            # HBM bytes per launch from the two rocprofv3 --pmc passes over this command (FETCH_SIZE x 2.000
+            # + WRITE_SIZE x 1.000, in KiB; see the profile named below): 1.001 x the algorithmic bytes.
+            "traffic": 131203 * 1024,
+            "traffic_source": "profiles/single_copy_kernel_d2d_64MiB_pmc_fetch_write.txt",
             "kernel": "tphip::single_copy_kernel<4, 2>", "kernel_avg_us": kernel_us,
             "algorithmic_bytes_per_launch": 2 * nbytes,
         },
