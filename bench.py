@@ -3,9 +3,9 @@
 
     python bench.py --gpus 1 --steps K --warmup W
 
-The headline line is BASELINE.json's configs[1]: same-process device-to-device
-(hip_xth channel), one 64 MiB uint8 tensor, two connected pipes in one process,
-K write/read steps after W warm-up steps, received bytes compared with the sent
+The headline line is the same-process device-to-device configuration (configs[1] of the
+benchmark definition): hip_xth channel, one 64 MiB uint8 tensor, two connected pipes in one
+process, K write/read steps after W warm-up steps, received bytes compared with the sent
 ones. One step = Pipe::write + Pipe::readDescriptor + Pipe::read of one message
 and a synchronisation of the receive stream. `value` is payload bytes delivered
 per second with the tensors already resident in HBM.
