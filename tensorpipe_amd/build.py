@@ -90,7 +90,7 @@ def build_cpp_tests():
     bin_dir = os.path.join(src_dir, "bin")
     os.makedirs(bin_dir, exist_ok=True)
     for name in CPP_TESTS:
-        run(["g++", "-O1", "-g", "-std=c++17", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
+        run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
              f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(src_dir, name + ".cc"),
              "-o", os.path.join(bin_dir, name), f"-L{LIB}", "-ltensorpipe_amd", "-ltphip",
              "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib"])

@@ -108,7 +108,10 @@ class ChannelImpl final : public ChannelImplBase {
   void handleError() override {
     descriptorConnection_->close();
     completionConnection_->close();
-    // Every pending callback fires now, in order, with the error.
+    // Every pending callback fires now, in order, with the error -- except for
+    // receives whose copy is already running: that kernel sits on the sender's
+    // stream and keeps writing into the receive buffer, so its callback waits
+    // for the event behind the copy (the watcher finishes the op).
     auto sends = std::move(sendOps_);
     sendOps_.clear();
     for (auto& op : sends) {
@@ -117,7 +120,9 @@ class ChannelImpl final : public ChannelImplBase {
     auto recvs = std::move(recvOps_);
     recvOps_.clear();
     for (auto& op : recvs) {
-      finishRecv(op);
+      if (op->copiesInFlight == 0) {
+        finishRecv(op);
+      }
     }
   }
 
@@ -261,7 +266,6 @@ class ChannelImpl final : public ChannelImplBase {
         }
         g->table.push_back(tphip_copy_desc{src, hb.ptr, len});
       }
-      op->copiesInFlight = groups.size();
       decodeTimer.reset();
       for (auto& g : groups) {
         StageScope launchTimer(Stage::kXthLaunch);
@@ -283,10 +287,17 @@ class ChannelImpl final : public ChannelImplBase {
         auto done = xctx_->events.get(g.src.device);
         done->record(g.src.stream);
         auto self = shared_from_this();
+        // Counted per launch: if a later launch of this op fails, the error
+        // path still waits for exactly the copies that are running.
+        ++op->copiesInFlight;
         xctx_->poller.watch(std::move(done), &xctx_->events, [this, self, op](const Error& error) {
           ctx_->defer([this, self, op, error] {
             setError(error);
-            if (error_ || --op->copiesInFlight > 0) {
+            if (--op->copiesInFlight > 0) {
+              return;
+            }
+            if (error_) {
+              finishRecv(op); // no longer in recvOps_: the error path left it to us
               return;
             }
             TP_VLOG(6) << "Channel " << id_ << " done copying payload (#" << op->seq << ")";
@@ -297,6 +308,11 @@ class ChannelImpl final : public ChannelImplBase {
       }
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " copy failed: " << ex.what();
+      // A copy may have been launched without an event behind it: wait for the
+      // source streams before the receive buffers are handed back.
+      for (auto& g : groups) {
+        tphip_stream_sync(g.src.device, g.src.stream);
+      }
       setError(TP_CREATE_ERROR(HipError, "hip_xth copy", TPHIP_ERR_INVALID_ARG));
     }
   }

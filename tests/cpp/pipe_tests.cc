@@ -215,6 +215,129 @@ Case oneWay(std::string name, InlineMessage im, std::vector<Device> devices) {
               }};
 }
 
+
+// ---- many messages in flight ----------------------------------------------------
+
+// Deterministic content of tensor `t` of message `m` travelling in direction `dir`.
+std::vector<uint8_t> patterned(uint32_t dir, uint32_t m, uint32_t t, size_t n) {
+  std::vector<uint8_t> v(n);
+  uint64_t x = 0x9E3779B97F4A7C15ull * (1 + dir + 7 * m + 131 * t) + n;
+  for (size_t i = 0; i < n; ++i) {
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    v[i] = static_cast<uint8_t>(x >> 11);
+  }
+  return v;
+}
+
+// Shape of message `m` in direction `dir`: tensor lengths and devices, derived
+// from the indices alone so that both endpoints agree without talking.
+struct Shape {
+  std::vector<size_t> lengths;
+  std::vector<bool> gpu;
+};
+
+Shape shapeOf(uint32_t dir, uint32_t m) {
+  Shape s;
+  uint64_t x = 0xD1B54A32D192ED03ull * (3 + dir + 2 * m);
+  const uint32_t n = static_cast<uint32_t>((x >> 60) % 6); // 0..5 tensors
+  for (uint32_t t = 0; t < n; ++t) {
+    x = x * 6364136223846793005ull + 1442695040888963407ull;
+    const uint32_t cls = static_cast<uint32_t>((x >> 33) % 5);
+    size_t len = 0;
+    switch (cls) {
+      case 0: len = 0; break;
+      case 1: len = 1 + (x >> 40) % 63; break;
+      case 2: len = 4096 + (x >> 40) % 4096; break;
+      case 3: len = (256u << 10) + (x >> 40) % 1000; break;
+      default: len = (2u << 20) + (x >> 40) % 100000; break;
+    }
+    s.lengths.push_back(len);
+    s.gpu.push_back(((x >> 20) & 1) != 0);
+  }
+  return s;
+}
+
+// Writes `count` messages without waiting in between and reads `count`
+// messages of the opposite direction at the same time; every callback must
+// fire exactly once, in order, with the right bytes.
+void exchangeMany(Pipe& pipe, uint32_t myDir, uint32_t count) {
+  struct Outgoing {
+    Storage storage;
+    std::future<Error> done;
+  };
+  std::vector<std::unique_ptr<Outgoing>> outs;
+  auto writeFires = std::make_shared<std::vector<int>>(count, 0);
+  for (uint32_t m = 0; m < count; ++m) {
+    Shape sh = shapeOf(myDir, m);
+    auto o = std::make_unique<Outgoing>();
+    Message msg;
+    msg.metadata = "m" + std::to_string(m);
+    for (size_t t = 0; t < sh.lengths.size(); ++t) {
+      o->storage.tensors.push_back(
+          makeData(gHaveGpu && sh.gpu[t], patterned(myDir, m, static_cast<uint32_t>(t), sh.lengths[t])));
+      Message::Tensor mt;
+      mt.buffer = o->storage.tensors.back()->buffer();
+      mt.length = sh.lengths[t];
+      mt.metadata = "t" + std::to_string(t);
+      msg.tensors.push_back(std::move(mt));
+    }
+    auto p = std::make_shared<std::promise<Error>>();
+    o->done = p->get_future();
+    pipe.write(std::move(msg), [p, writeFires, m](const Error& e) {
+      if (++(*writeFires)[m] == 1) {
+        p->set_value(e);
+      }
+    });
+    outs.push_back(std::move(o));
+  }
+
+  const uint32_t theirDir = 1 - myDir;
+  for (uint32_t m = 0; m < count; ++m) {
+    Shape sh = shapeOf(theirDir, m);
+    auto pd = std::make_shared<std::promise<std::pair<Error, Descriptor>>>();
+    auto fd = pd->get_future();
+    pipe.readDescriptor([pd](const Error& e, Descriptor d) { pd->set_value({e, std::move(d)}); });
+    auto rd = waitFor(fd, "readDescriptor");
+    EXPECT_OK(rd.first);
+    if (rd.first) {
+      throw Fatal("readDescriptor failed in the middle of the exchange");
+    }
+    const Descriptor& d = rd.second;
+    EXPECT_EQ(d.metadata, "m" + std::to_string(m)); // messages arrive in the order written
+    EXPECT_EQ(d.tensors.size(), sh.lengths.size());
+    if (d.tensors.size() != sh.lengths.size()) {
+      throw Fatal("unexpected message shape");
+    }
+    Storage storage;
+    Allocation a;
+    for (size_t t = 0; t < d.tensors.size(); ++t) {
+      EXPECT_EQ(d.tensors[t].length, sh.lengths[t]);
+      // receive on the other kind of device than the one it was sent from
+      storage.tensors.push_back(makeData(gHaveGpu && !sh.gpu[t], d.tensors[t].length));
+      Allocation::Tensor at;
+      at.buffer = storage.tensors.back()->buffer();
+      a.tensors.push_back(std::move(at));
+    }
+    auto pr = std::make_shared<std::promise<Error>>();
+    auto fr = pr->get_future();
+    pipe.read(std::move(a), [pr](const Error& e) { pr->set_value(e); });
+    EXPECT_OK(waitFor(fr, "read"));
+    for (size_t t = 0; t < d.tensors.size(); ++t) {
+      if (storage.tensors[t]->bytes() != patterned(theirDir, m, static_cast<uint32_t>(t), sh.lengths[t])) {
+        failures().add("message " + std::to_string(m) + " tensor " + std::to_string(t) + " differs");
+      }
+    }
+  }
+  for (uint32_t m = 0; m < count; ++m) {
+    EXPECT_OK(waitFor(outs[m]->done, "write"));
+  }
+  for (uint32_t m = 0; m < count; ++m) {
+    EXPECT_EQ((*writeFires)[m], 1);
+  }
+}
+
 std::vector<Case> makeCases() {
   std::vector<Case> cases;
 
@@ -273,6 +396,88 @@ std::vector<Case> makeCases() {
            InlineMessage out = messageWith(
                {{std::string(2 * 1024 * 1024 + k, char('k' + k)), "reply", kGpu, nullopt}});
            writeMessage(*e->pipe, out);
+         }
+         ep.barrier();
+       }});
+
+  // Sixty messages of random shape each way, all writes issued up front.
+  cases.push_back({"ManyMessagesBothDirections",
+                   [](Endpoint& ep) {
+                     auto e = openPipe(ep);
+                     exchangeMany(*e->pipe, 0, 60);
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     auto e = openPipe(ep);
+                     exchangeMany(*e->pipe, 1, 60);
+                     ep.barrier();
+                   }});
+
+  // Writes that are still queued or in flight when the pipe is closed complete
+  // with an error or with success, but every one of them completes, once.
+  cases.push_back(
+      {"CloseWithWritesInFlight",
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         ep.barrier();
+         const int count = 40;
+         auto fires = std::make_shared<std::vector<std::atomic<int>>>(count);
+         auto remaining = std::make_shared<std::atomic<int>>(count);
+         auto all = std::make_shared<std::promise<void>>();
+         auto fAll = all->get_future();
+         std::vector<std::unique_ptr<Data>> keep;
+         for (int m = 0; m < count; ++m) {
+           keep.push_back(makeData(gHaveGpu && (m & 1), patterned(0, m, 0, (1u << 20) + m)));
+           Message msg;
+           Message::Tensor mt;
+           mt.buffer = keep.back()->buffer();
+           mt.length = keep.back()->size();
+           msg.tensors.push_back(std::move(mt));
+           e->pipe->write(std::move(msg), [fires, remaining, all, m](const Error&) {
+             (*fires)[m].fetch_add(1);
+             if (remaining->fetch_sub(1) == 1) {
+               all->set_value();
+             }
+           });
+           if (m == count / 2) {
+             e->pipe->close();
+           }
+         }
+         if (fAll.wait_for(std::chrono::seconds(kWaitSeconds)) != std::future_status::ready) {
+           throw Fatal("not every write callback fired after close");
+         }
+         for (int m = 0; m < count; ++m) {
+           EXPECT_EQ((*fires)[m].load(), 1);
+         }
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         ep.barrier();
+         // Read whatever arrives until the pipe fails.
+         for (;;) {
+           auto pd = std::make_shared<std::promise<std::pair<Error, Descriptor>>>();
+           auto fd = pd->get_future();
+           e->pipe->readDescriptor(
+               [pd](const Error& err, Descriptor d) { pd->set_value({err, std::move(d)}); });
+           auto rd = waitFor(fd, "readDescriptor");
+           if (rd.first) {
+             break;
+           }
+           Storage storage;
+           Allocation a;
+           for (auto& t : rd.second.tensors) {
+             storage.tensors.push_back(makeData(gHaveGpu, t.length));
+             Allocation::Tensor at;
+             at.buffer = storage.tensors.back()->buffer();
+             a.tensors.push_back(std::move(at));
+           }
+           auto pr = std::make_shared<std::promise<Error>>();
+           auto fr = pr->get_future();
+           e->pipe->read(std::move(a), [pr](const Error& err) { pr->set_value(err); });
+           if (waitFor(fr, "read")) {
+             break;
+           }
          }
          ep.barrier();
        }});
