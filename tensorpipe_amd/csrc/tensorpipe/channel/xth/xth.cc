@@ -47,6 +47,7 @@ class ChannelImpl final : public ChannelImplBase {
     size_t length;
     std::function<void(const Error&)> cb;
     bool done{false};
+    bool copying{false}; // handed to the copier thread, which still writes to ptr
   };
 
   void sendFromLoop(uint64_t seq, Buffer buffer, size_t length, TSendCallback cb) override {
@@ -59,8 +60,12 @@ class ChannelImpl final : public ChannelImplBase {
     WireWriter w;
     w.u64(reinterpret_cast<uint64_t>(op->ptr));
     w.u64(length);
+    TP_VLOG(6) << "Channel " << id_ << " is writing descriptor (#" << seq << ")";
     writeMessage(*descriptorConnection_, std::move(w.bytes()));
-    completionConnection_->read(nullptr, 0, onRead([this, op] { finish(op); }));
+    completionConnection_->read(nullptr, 0, onRead([this, op] {
+      TP_VLOG(6) << "Channel " << id_ << " done reading completion (#" << op->seq << ")";
+      finish(op);
+    }));
   }
 
   void recvFromLoop(uint64_t seq, Buffer buffer, size_t length, TRecvCallback cb) override {
@@ -70,7 +75,9 @@ class ChannelImpl final : public ChannelImplBase {
     }
     auto op = std::make_shared<Op>(Op{seq, buffer.unwrap<CpuBuffer>().ptr, length, std::move(cb)});
     ops_.push_back(op);
+    TP_VLOG(6) << "Channel " << id_ << " is reading descriptor (#" << seq << ")";
     descriptorConnection_->read(onReadMessage([this, op](std::vector<uint8_t> bytes) {
+      TP_VLOG(6) << "Channel " << id_ << " done reading descriptor (#" << op->seq << ")";
       if (error_) {
         finish(op);
         return;
@@ -84,9 +91,12 @@ class ChannelImpl final : public ChannelImplBase {
         return;
       }
       auto self = shared_from_this();
+      op->copying = true;
       xctx_->copier.defer([this, self, op, src] {
         std::memcpy(op->ptr, src, op->length);
         ctx_->defer([this, self, op] {
+          TP_VLOG(6) << "Channel " << id_ << " done copying payload (#" << op->seq << ")";
+          op->copying = false;
           finish(op);
           if (!error_) {
             completionConnection_->write(nullptr, 0, onWritten([] {}));
@@ -99,10 +109,14 @@ class ChannelImpl final : public ChannelImplBase {
   void handleError() override {
     descriptorConnection_->close();
     completionConnection_->close();
+    // A receive that the copier thread is working on keeps its buffer until
+    // the copy has ended; the copier's completion finishes it.
     auto ops = std::move(ops_);
     ops_.clear();
     for (auto& op : ops) {
-      finish(op);
+      if (!op->copying) {
+        finish(op);
+      }
     }
   }
 

@@ -76,6 +76,20 @@ int spinMicros() {
   return v;
 }
 
+// ThreadSanitizer keys its happens-before edges on virtual addresses, and the
+// two ends of a ring inside ONE process see the same counters at different
+// addresses; tell it about the hand-off through one process-wide token.
+#if defined(__SANITIZE_THREAD__)
+extern "C" void __tsan_acquire(void* addr);
+extern "C" void __tsan_release(void* addr);
+char gTsanRingToken;
+#define TP_TSAN_RING_RELEASE() __tsan_release(&gTsanRingToken)
+#define TP_TSAN_RING_ACQUIRE() __tsan_acquire(&gTsanRingToken)
+#else
+#define TP_TSAN_RING_RELEASE() ((void)0)
+#define TP_TSAN_RING_ACQUIRE() ((void)0)
+#endif
+
 struct RingHeader {
   alignas(64) std::atomic<uint64_t> head; // bytes ever produced
   alignas(64) std::atomic<uint64_t> tail; // bytes ever consumed
@@ -147,6 +161,7 @@ class Ring {
     const uint64_t cap = hdr_->capacity;
     const uint64_t head = hdr_->head.load(std::memory_order_relaxed);
     const uint64_t tail = hdr_->tail.load(std::memory_order_acquire);
+    TP_TSAN_RING_ACQUIRE();
     const uint64_t space = cap - (head - tail);
     if (n > space) {
       n = space;
@@ -160,6 +175,7 @@ class Ring {
     if (n > first) {
       std::memcpy(data_, src + first, n - first);
     }
+    TP_TSAN_RING_RELEASE();
     hdr_->head.store(head + n, std::memory_order_release);
     return n;
   }
@@ -178,6 +194,7 @@ class Ring {
     const uint64_t cap = hdr_->capacity;
     const uint64_t tail = hdr_->tail.load(std::memory_order_relaxed);
     const uint64_t head = hdr_->head.load(std::memory_order_acquire);
+    TP_TSAN_RING_ACQUIRE();
     const uint64_t avail = head - tail;
     if (n > avail) {
       n = avail;
@@ -191,6 +208,7 @@ class Ring {
     if (n > first) {
       std::memcpy(dst + first, data_, n - first);
     }
+    TP_TSAN_RING_RELEASE();
     hdr_->tail.store(tail + n, std::memory_order_release);
     return n;
   }

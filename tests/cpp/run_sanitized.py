@@ -1,0 +1,61 @@
+#!/usr/bin/env python3
+"""Builds the host library and the C++ test programs with a sanitizer and runs the CPU suites.
+
+    python tests/cpp/run_sanitized.py thread|address [build_dir]
+
+Host code only (g++ -fsanitize=...); libtphip.so is used as built. Not collected by pytest: a
+full pass takes several minutes. The shm transport tells ThreadSanitizer about the hand-off
+through its rings (two mappings of one segment inside a process), so a clean run reports
+nothing; any "WARNING: ThreadSanitizer" / "ERROR: AddressSanitizer" line fails the run.
+"""
+import os
+import subprocess
+import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from tensorpipe_amd import build as tp_build  # noqa: E402
+
+SUITES = [("channel_tests", "xth"), ("channel_tests", "basic"),
+          ("pipe_tests", "cpu_same_process"), ("pipe_tests", "cpu_two_process")]
+
+
+def main():
+    san = sys.argv[1] if len(sys.argv) > 1 else "thread"
+    out = sys.argv[2] if len(sys.argv) > 2 else tempfile.mkdtemp(prefix=f"tp_{san}_")
+    os.makedirs(out, exist_ok=True)
+    flags = ["-O1", "-g", "-std=c++17", "-fPIC", f"-fsanitize={san}", "-fno-omit-frame-pointer", "-pthread",
+             f"-I{tp_build.INCLUDE}", f"-I{tp_build.CSRC}"]
+    objs = [os.path.join(out, s.replace("/", "_") + ".o") for s in tp_build.HOST_SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        subprocess.run(["g++", *flags, "-c", os.path.join(tp_build.CSRC, src), "-o", obj], check=True)
+
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        list(pool.map(compile_one, zip(tp_build.HOST_SOURCES, objs)))
+    lib = os.path.join(out, "libtensorpipe_amd.so")
+    subprocess.run(["g++", "-shared", f"-fsanitize={san}", "-pthread", "-o", lib, *objs, f"-L{tp_build.LIB}",
+                    "-ltphip", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
+    for prog in sorted({p for p, _ in SUITES}):
+        subprocess.run(["g++", *flags, os.path.join(ROOT, "tests", "cpp", prog + ".cc"), "-o",
+                        os.path.join(out, prog), f"-L{out}", "-ltensorpipe_amd", f"-L{tp_build.LIB}", "-ltphip",
+                        f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
+    bad = 0
+    for prog, suite in SUITES:
+        proc = subprocess.run([os.path.join(out, prog), "--suite", suite], stdout=subprocess.PIPE,
+                              stderr=subprocess.STDOUT, text=True, timeout=1800)
+        results = [l for l in proc.stdout.splitlines() if l.startswith("RESULT")]
+        failed = [l for l in results if " OK" not in l]
+        reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+        print(f"{prog} --suite {suite}: {len(results)} results, {len(failed)} failed, {len(reports)} sanitizer reports")
+        for l in failed + reports[:5]:
+            print("   ", l[:200])
+        bad += len(failed) + len(reports) + (0 if results else 1)
+    sys.exit(1 if bad else 0)
+
+
+if __name__ == "__main__":
+    main()
