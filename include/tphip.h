@@ -131,9 +131,11 @@ int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], 
 
 /* ---- data movement ------------------------------------------------------- */
 
-/* The hot path. Enqueue on `stream` ONE kernel launch that performs every copy
+/* The hot path. Enqueue on `stream` ONE copy kernel that performs every copy
  * of `table[0..n)`; `table` is host memory and may be reused as soon as the
- * call returns. Any mix of device, mapped-pinned-host and peer-mapped (IPC)
+ * call returns. Tables of up to 64 entries travel in the kernel arguments (one
+ * launch in all); larger ones are written to a pinned plan ring and moved to
+ * device memory by a small staging kernel enqueued ahead of the copy kernel. Any mix of device, mapped-pinned-host and peer-mapped (IPC)
  * addresses is accepted as long as the device can address them. n == 0 or an
  * all-empty table enqueues nothing. n > TPHIP_MAX_BATCH returns
  * TPHIP_ERR_TOO_LARGE. Replaces one cudaMemcpyAsync per tensor at the three

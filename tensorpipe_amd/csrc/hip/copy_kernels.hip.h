@@ -150,27 +150,15 @@ constexpr uint32_t kLdsBodies = 1024;
 // bodies if n <= kLdsBodies. A chunk's lookup then costs LDS reads only; a
 // dependent global load per chunk used to stall every workgroup for the best
 // part of a microsecond.
+// The work of a table copy once the plan is where the workgroup can read it
+// cheaply: sPrefix (and normally body) in LDS, descs wherever they are.
 template <int U, int NT>
-__global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
-    const uint32_t* __restrict__ prefix,
-    const CopyBody* __restrict__ bodies,
-    const tphip_copy_desc* __restrict__ descs,
+__device__ __forceinline__ void table_copy(
+    const uint32_t* sPrefix,
+    const CopyBody* body,
+    const tphip_copy_desc* descs,
     uint32_t n,
     uint32_t nchunks) {
-  extern __shared__ __align__(16) uint32_t sPrefix[];
-  const bool cached = n <= kLdsBodies;
-  CopyBody* sBodies = reinterpret_cast<CopyBody*>(sPrefix + ((n + 1 + 3) & ~3u));
-  for (uint32_t i = threadIdx.x; i <= n; i += kBlockThreads) {
-    sPrefix[i] = prefix[i];
-  }
-  if (cached) {
-    for (uint32_t i = threadIdx.x; i < n; i += kBlockThreads) {
-      sBodies[i] = bodies[i];
-    }
-  }
-  __syncthreads();
-  const CopyBody* body = cached ? sBodies : bodies;
-
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t waveInBlock = threadIdx.x >> 6;
   const uint32_t wave = blockIdx.x * kWavesPerBlock + waveInBlock;
@@ -305,6 +293,55 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
   for (uint32_t g = nwaves - 1 - wave; g * kEdgeGroup < n; g += nwaves) {
     copy_edges(descs, n, g, lane);
   }
+}
+
+template <int U, int NT>
+__global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
+    const uint32_t* __restrict__ prefix,
+    const CopyBody* __restrict__ bodies,
+    const tphip_copy_desc* __restrict__ descs,
+    uint32_t n,
+    uint32_t nchunks) {
+  extern __shared__ __align__(16) uint32_t sPrefix[];
+  const bool cached = n <= kLdsBodies;
+  CopyBody* sBodies = reinterpret_cast<CopyBody*>(sPrefix + ((n + 1 + 3) & ~3u));
+  for (uint32_t i = threadIdx.x; i <= n; i += kBlockThreads) {
+    sPrefix[i] = prefix[i];
+  }
+  if (cached) {
+    for (uint32_t i = threadIdx.x; i < n; i += kBlockThreads) {
+      sBodies[i] = bodies[i];
+    }
+  }
+  __syncthreads();
+  table_copy<U, NT>(sPrefix, cached ? sBodies : bodies, descs, n, nchunks);
+}
+
+// Small tables travel in the kernel arguments: no plan upload, no staging
+// kernel, nothing to recycle afterwards -- one launch is the whole cost. The
+// struct is a plain array of 32-bit words so that every lane can fetch its
+// share with one indexed load.
+constexpr uint32_t kInlineEntries = 64;
+
+struct InlinePlan {
+  uint32_t n;
+  uint32_t nchunks;
+  uint32_t prefix[kInlineEntries + 2]; // n+1 used; padded to keep 8-byte alignment below
+  CopyBody bodies[kInlineEntries];
+  tphip_copy_desc descs[kInlineEntries];
+};
+static_assert(sizeof(InlinePlan) % 4 == 0 && sizeof(InlinePlan) <= 3072, "kernel argument budget");
+
+template <int U, int NT>
+__global__ __launch_bounds__(kBlockThreads) void inline_copy_kernel(const InlinePlan plan) {
+  __shared__ __align__(16) InlinePlan sPlan;
+  const uint32_t* in = reinterpret_cast<const uint32_t*>(&plan);
+  uint32_t* out = reinterpret_cast<uint32_t*>(&sPlan);
+  for (uint32_t i = threadIdx.x; i < sizeof(InlinePlan) / 4; i += kBlockThreads) {
+    out[i] = in[i];
+  }
+  __syncthreads();
+  table_copy<U, NT>(sPlan.prefix, sPlan.bodies, sPlan.descs, sPlan.n, sPlan.nchunks);
 }
 
 // Single-entry variant: the descriptor travels in the kernel arguments, no

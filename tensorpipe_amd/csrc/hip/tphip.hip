@@ -145,6 +145,12 @@ int planViaKernel() {
   return v;
 }
 
+// TPHIP_INLINE_PLANS=0 sends small tables through the plan ring as well (A/B switch).
+bool inlinePlansEnabled() {
+  static const bool v = envInt("TPHIP_INLINE_PLANS", 1) != 0;
+  return v;
+}
+
 int getDevice(int dev, DeviceState** out) {
   if (dev < 0 || dev >= kMaxDevices) {
     return TPHIP_ERR_INVALID_ARG;
@@ -240,6 +246,20 @@ int launchTable(int unroll, uint32_t blocks, size_t lds, hipStream_t stream,
   }
 }
 
+template <int NT>
+int launchInline(int unroll, uint32_t blocks, hipStream_t stream, const InlinePlan& plan) {
+  switch (unroll) {
+    case 1:
+      return launchKernel(inline_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+    case 2:
+      return launchKernel(inline_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+    case 8:
+      return launchKernel(inline_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+    default:
+      return launchKernel(inline_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+  }
+}
+
 // Workgroups for `units` work units of one workgroup-iteration each: enough to
 // give every unit a workgroup, capped at blocksPerCu * CUs (or `blocks`).
 uint32_t pickBlocks(const DeviceState& st, uint64_t units, uint32_t minBlocks, uint32_t blocks,
@@ -292,13 +312,50 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
   if (unroll == 0) {
     unroll = defaultUnroll(true);
   }
-  if (nt < 0) {
-    uint64_t payload = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-      payload += table[i].bytes;
-    }
-    nt = defaultNontemporal(payload);
+  uint64_t payloadBytes = 0;
+  for (uint32_t i = 0; i < n; ++i) {
+    payloadBytes += table[i].bytes;
   }
+  if (nt < 0) {
+    nt = defaultNontemporal(payloadBytes);
+  }
+
+  if (n <= kInlineEntries && inlinePlansEnabled()) {
+    // The whole plan fits the kernel arguments.
+    InlinePlan plan;
+    memset(&plan, 0, sizeof(plan));
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+      plan.prefix[i] = static_cast<uint32_t>(total);
+      const uint64_t bytes = table[i].bytes;
+      uint64_t head = (0 - reinterpret_cast<uintptr_t>(table[i].dst)) & 15u;
+      if (head > bytes) {
+        head = bytes;
+      }
+      plan.bodies[i].src = static_cast<const char*>(table[i].src) + head;
+      plan.bodies[i].dst = static_cast<char*>(table[i].dst) + head;
+      plan.descs[i] = table[i];
+      total += (bytes - head) >> 4;
+    }
+    plan.prefix[n] = static_cast<uint32_t>(total);
+    const uint64_t chunk = uint64_t(kBlockThreads) * unroll;
+    plan.n = n;
+    plan.nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
+    const uint32_t edgeBlocks = (n + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
+    const uint32_t grid = pickBlocks(st, plan.nchunks, edgeBlocks, blocks, true);
+    ProfileScope prof(st, stream, payloadBytes);
+    switch (nt & 3) {
+      case 0:
+        return launchInline<0>(unroll, grid, stream, plan);
+      case 1:
+        return launchInline<1>(unroll, grid, stream, plan);
+      case 2:
+        return launchInline<2>(unroll, grid, stream, plan);
+      default:
+        return launchInline<3>(unroll, grid, stream, plan);
+    }
+  }
+
   const size_t prefixBytes = ((size_t(n) + 1) * sizeof(uint32_t) + 15) / 16 * 16;
   const size_t bodyBytes = size_t(n) * sizeof(CopyBody);
   const size_t planBytes = prefixBytes + bodyBytes + size_t(n) * sizeof(tphip_copy_desc);
@@ -360,11 +417,7 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
         reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes + bodyBytes);
     int rc;
     {
-      uint64_t payload = 0;
-      for (uint32_t i = 0; i < n; ++i) {
-        payload += table[i].bytes;
-      }
-      ProfileScope prof(st, stream, payload);
+      ProfileScope prof(st, stream, payloadBytes);
       switch (nt & 3) {
         case 0:
           rc = launchTable<0>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, n, nchunks);

@@ -122,10 +122,30 @@ def test_launch_shapes(oracle, unroll, nt):
 
 
 def test_plan_ring_reuse(oracle):
-    # more launches than plan slots on one stream, all checked
+    # more launches than plan slots on one stream, all checked; 70 entries each, so that the
+    # plans go through the ring (tables of up to 64 entries travel in the kernel arguments)
     for k in range(70):
-        sizes = [1000 + k, 17, 4096 + k]
+        sizes = [1000 + k, 17, 4096 + k] + [64 + (i * 37 + k) % 900 for i in range(67)]
         _run_case(oracle, _pack(sizes, lambda i: (i + k) % 16, lambda i: (i * 3 + k) % 16), seed=k)
+
+
+@pytest.mark.parametrize("n", [2, 3, 31, 63, 64, 65, 66, 130])
+def test_inline_plan_boundary(oracle, n):
+    # either side of the largest table that travels in the kernel arguments, default and tuned launches
+    rng = np.random.default_rng(1000 + n)
+    sizes = [int(x) for x in rng.integers(0, 70000, n)]
+    sizes[0] = (2 << 20) + 3
+    layout = _pack(sizes, lambda i: int(rng.integers(0, 16)), lambda i: int(rng.integers(0, 16)), gap=3)
+    _run_case(oracle, layout, seed=n)
+    for tuned in ((1, 0, 3), (2, 1, 0), (4, 5, 2), (8, 300, 1)):
+        _run_case(oracle, layout, seed=n + 1, tuned=tuned)
+
+
+def test_many_inline_launches_back_to_back(oracle):
+    # the arguments of a launch belong to that launch alone: 200 different small tables in a row
+    for k in range(200):
+        sizes = [100 + k, 4096 + 3 * k, 0, 15 + k % 17]
+        _run_case(oracle, _pack(sizes, lambda i: (i + k) % 16, lambda i: (i * 5 + k) % 16), seed=300 + k)
 
 
 def test_full_size_roundtrip_property():
