@@ -352,7 +352,7 @@ def cpu_baseline():
         return json.loads(r.stdout.strip().splitlines()[-1])
 
     def suite(exe):
-        same = run(exe, 64 * MIB, 0, 2, 40)    # the headline workload's tensor, bounded sample
+        same = run(exe, 64 * MIB, 0, 2, 400)   # the headline workload's tensor, bounded sample (~5 s)
         cfg1 = run(exe, 1 * MIB, 64, 5, 1000)  # configs[0]
         rtt = run(exe, 4096, 64, 5, 2000)      # 4 KiB round trip
         return {"payload_GBps_64MiB": same["payload_GBps"],
@@ -380,7 +380,7 @@ def cpu_baseline():
         return {"error": "neither oracle/cpu_shm_basic nor oracle/_ref/ref_pipe_bench is built"}
     return {
         "value": main_["payload_GBps_64MiB"], "unit": "GB/s", "cores": cores, "kind": kind,
-        "sample": "40 ping-pong round trips (80 transfers) of one 64 MiB CPU tensor through "
+        "sample": "400 ping-pong round trips (800 transfers, 53.7 GB) of one 64 MiB CPU tensor through "
                   "Pipe + shm transport + basic channel; " + threads,
         "config1_1MiB_rtt_p50_us": main_["config1_1MiB_rtt_p50_us"],
         "config1_payload_GBps": main_["config1_payload_GBps"],
