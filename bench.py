@@ -150,8 +150,8 @@ def bench_rpc_message(messages=500, warmup=20):
 
     sizes = [int(s) for s in datagen.loguniform_sizes(datagen.SEED_BASE + 5, 256, 4 * MIB, 256)]
     total = sum(sizes)
-    arena_src = torch.empty(total + 16 * len(sizes), dtype=torch.uint8, device="cuda")
-    arena_dst = torch.zeros_like(arena_src)
+    arena_src = torch.zeros(total + 16 * len(sizes), dtype=torch.uint8, device="cuda")
+    arena_dst = torch.zeros_like(arena_src)  # the padding between tensors stays zero in both
     st, rt, off = [], [], 0
     for i, n in enumerate(sizes):
         h = datagen.normal(1000 + i, n // 2, "f16", sigma=0.02).view(np.uint8)
@@ -174,6 +174,19 @@ def bench_rpc_message(messages=500, warmup=20):
     torch.cuda.synchronize()
     ok = bool(torch.equal(arena_src[:off], arena_dst[:off])) and bytes(pout) == bytes(payload)
     destroy(objs)
+
+    # the same message between two processes (hip_ipc), as a round trip
+    arena_dst.zero_()
+    peer = PeerRun("basic:0,hip_ipc:11")
+    try:
+        torch.cuda.synchronize()
+        ipc_us, _ = peer.pingpong(st, rt, sizes, "gpu", 10, 200)
+        torch.cuda.synchronize()
+        ipc_ok = bool(torch.equal(arena_src[:off], arena_dst[:off]))
+    finally:
+        peer.close()
+    ipc_us.sort()
+    ipc_p50 = float(ipc_us[int(0.5 * len(ipc_us))])
     per_us.sort()
     kernel_us = kernel_ms / max(launches, 1) * 1e3
     return {
@@ -185,6 +198,9 @@ def bench_rpc_message(messages=500, warmup=20):
         "kernel_hbm_GBps": 2.0 * total / (kernel_us * 1e-6) / 1e9,
         "kernel_hbm_frac": 2.0 * total / (kernel_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
         "byte_exact": ok,
+        "ipc_round_trip_p50_us": ipc_p50,
+        "ipc_payload_GBps": 2.0 * total / (ipc_p50 * 1e-6) / 1e9,
+        "ipc_byte_exact": ipc_ok,
     }
 
 

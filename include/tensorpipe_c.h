@@ -61,7 +61,7 @@ typedef struct tpc_payload {
 typedef struct tpc_descriptor {
   uint32_t num_payloads;
   uint32_t num_tensors;
-  char metadata[256];
+  char metadata[8192];
   uint64_t payload_lengths[64];
   uint64_t tensor_lengths[TPC_MAX_DESC_ITEMS];
   int32_t tensor_source_type[TPC_MAX_DESC_ITEMS];

@@ -35,7 +35,7 @@ class Descriptor(ctypes.Structure):
     _fields_ = [
         ("num_payloads", ctypes.c_uint32),
         ("num_tensors", ctypes.c_uint32),
-        ("metadata", ctypes.c_char * 256),
+        ("metadata", ctypes.c_char * 8192),
         ("payload_lengths", ctypes.c_uint64 * 64),
         ("tensor_lengths", ctypes.c_uint64 * MAX_DESC_ITEMS),
         ("tensor_source_type", ctypes.c_int32 * MAX_DESC_ITEMS),
