@@ -517,9 +517,21 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     bool finished{false};
   };
 
+  // What read() needs to know about a tensor once the descriptor itself has
+  // been handed (moved) to the user: devices are indices into ReadOp::devices.
+  struct TensorShape {
+    size_t length;
+    uint16_t source;
+    uint16_t target; // kNoDevice = the receiver chooses
+  };
+  static constexpr uint16_t kNoDevice = 0xffff;
+
   struct ReadOp {
     uint64_t seq;
-    Descriptor descriptor;
+    Descriptor descriptor; // until delivered
+    std::vector<Device> devices;
+    std::vector<TensorShape> shapes;
+    std::vector<size_t> payloadLengths;
     bool delivered{false};
     bool readCalled{false};
     Allocation allocation;
@@ -827,17 +839,33 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         Descriptor::Payload p;
         p.length = r.u64();
         p.metadata = r.str();
+        op->payloadLengths.push_back(p.length);
         d.payloads.push_back(std::move(p));
       }
       const uint32_t nT = r.u32();
       // every tensor takes at least 9 bytes on the wire
       bool wellFormed = nT <= r.remaining() / 9;
       d.tensors.reserve(wellFormed ? nT : 0); // no reallocation below: prevTarget points inside
+      op->shapes.reserve(wellFormed ? nT : 0);
       const Device* prevTarget = nullptr;
+      uint16_t prevSourceIdx = kNoDevice;
+      uint16_t prevTargetIdx = kNoDevice;
+      // Index of `dev` in op->devices (a handful of entries at most).
+      auto intern = [&op](const Device& dev) -> uint16_t {
+        for (size_t k = 0; k < op->devices.size(); ++k) {
+          if (op->devices[k] == dev) {
+            return static_cast<uint16_t>(k);
+          }
+        }
+        op->devices.push_back(dev);
+        return static_cast<uint16_t>(op->devices.size() - 1);
+      };
       for (uint32_t i = 0; wellFormed && i < nT && r.ok(); ++i) {
         d.tensors.emplace_back();
         Descriptor::Tensor& t = d.tensors.back();
+        TensorShape shape{0, kNoDevice, kNoDevice};
         t.length = r.u64();
+        shape.length = t.length;
         const uint8_t flags = r.u8();
         if (flags & kTensorSameSource) {
           if (i == 0) {
@@ -847,7 +875,9 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
           t.sourceDevice = d.tensors[i - 1].sourceDevice;
         } else {
           getDevice(r, &t.sourceDevice);
+          prevSourceIdx = op->devices.size() < kNoDevice ? intern(t.sourceDevice) : kNoDevice;
         }
+        shape.source = prevSourceIdx;
         if (flags & kTensorHasTarget) {
           if (flags & kTensorSameTarget) {
             if (prevTarget == nullptr) {
@@ -858,20 +888,27 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
           } else {
             t.targetDevice.emplace();
             getDevice(r, &*t.targetDevice);
+            prevTargetIdx = op->devices.size() < kNoDevice ? intern(*t.targetDevice) : kNoDevice;
           }
           prevTarget = &*t.targetDevice;
+          shape.target = prevTargetIdx;
         }
         if (flags & kTensorHasMetadata) {
           r.str(&t.metadata);
         }
+        if (shape.source == kNoDevice) {
+          wellFormed = false; // more distinct devices than an index can name
+          break;
+        }
+        op->shapes.push_back(shape);
       }
       if (!r.ok() || !wellFormed) {
         setError(TP_CREATE_ERROR(LogicError, "malformed descriptor"));
         return;
       }
       bool hasPayloadBytes = false;
-      for (auto& p : d.payloads) {
-        hasPayloadBytes |= p.length > 0;
+      for (size_t len : op->payloadLengths) {
+        hasPayloadBytes |= len > 0;
       }
       if (hasPayloadBytes) {
         payloadsUnclaimed_ = true;
@@ -921,7 +958,9 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       descriptorWaiters_.pop_front();
       TP_VLOG(3) << "Pipe " << id_ << " is calling a readDescriptor callback (#" << next->seq
                  << ")";
-      fn(Error::kSuccess, next->descriptor);
+      // The op keeps shapes, devices and payload lengths; the descriptor
+      // itself goes to the user without another copy.
+      fn(Error::kSuccess, std::move(next->descriptor));
     }
   }
 
@@ -946,18 +985,18 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     op->readCalled = true;
     op->fn = std::move(fn);
     op->allocation = std::move(allocation);
-    const Descriptor& d = op->descriptor;
+    const std::vector<TensorShape>& shapes = op->shapes;
     // checkAllocationCompatibility, tensorpipe/core/pipe_impl.cc:49-65
-    TP_THROW_ASSERT_IF(op->allocation.payloads.size() != d.payloads.size());
-    TP_THROW_ASSERT_IF(op->allocation.tensors.size() != d.tensors.size());
-    const size_t nT = d.tensors.size();
+    TP_THROW_ASSERT_IF(op->allocation.payloads.size() != op->payloadLengths.size());
+    TP_THROW_ASSERT_IF(op->allocation.tensors.size() != shapes.size());
+    const size_t nT = shapes.size();
     bool needsReply = false;
     std::vector<Device> targets;
     targets.reserve(nT);
     for (size_t i = 0; i < nT; ++i) {
       targets.push_back(op->allocation.tensors[i].buffer.device());
-      if (d.tensors[i].targetDevice.has_value()) {
-        TP_THROW_ASSERT_IF(d.tensors[i].length > 0 && !(targets[i] == *d.tensors[i].targetDevice));
+      if (shapes[i].target != kNoDevice) {
+        TP_THROW_ASSERT_IF(shapes[i].length > 0 && !(targets[i] == op->devices[shapes[i].target]));
       } else {
         needsReply = true;
       }
@@ -966,15 +1005,15 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     // Payloads: the next messages on the connection.
     auto self = shared_from_this();
     bool claimed = false;
-    for (size_t i = 0; i < d.payloads.size(); ++i) {
-      if (d.payloads[i].length == 0) {
+    for (size_t i = 0; i < op->payloadLengths.size(); ++i) {
+      if (op->payloadLengths[i] == 0) {
         continue;
       }
       claimed = true;
       ++op->pendingPayloads;
       connection_->read(
           op->allocation.payloads[i].data,
-          d.payloads[i].length,
+          op->payloadLengths[i],
           [self, op](const Error& error, const void*, size_t) {
             self->ctx_->defer([self, op, error] {
               self->setError(error);
@@ -1003,12 +1042,12 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     std::vector<ChannelGroup> groups;
     ChannelLookup lookup(channelForDevicePair_);
     for (size_t i = 0; i < nT; ++i) {
-      const std::string* name = lookup.find(targets[i], d.tensors[i].sourceDevice);
+      const Device& source = op->devices[shapes[i].source];
+      const std::string* name = lookup.find(targets[i], source);
       if (name == nullptr) {
         setError(TP_CREATE_ERROR(
             LogicError,
-            "no channel between " + targets[i].toString() + " and " +
-                d.tensors[i].sourceDevice.toString()));
+            "no channel between " + targets[i].toString() + " and " + source.toString()));
         return;
       }
       addToGroup(groups, name, i, nT);
@@ -1027,7 +1066,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         std::vector<channel::BatchEntry> entries;
         entries.reserve(g.second.size());
         for (size_t i : g.second) {
-          entries.push_back({op->allocation.tensors[i].buffer, d.tensors[i].length});
+          entries.push_back({op->allocation.tensors[i].buffer, shapes[i].length});
         }
         ++op->pendingRecvs;
         TP_VLOG(9) << "Pipe " << id_ << " expects " << entries.size() << " tensors from channel "
@@ -1036,7 +1075,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       } else {
         for (size_t i : g.second) {
           ++op->pendingRecvs;
-          ch->recv(op->allocation.tensors[i].buffer, d.tensors[i].length, done);
+          ch->recv(op->allocation.tensors[i].buffer, shapes[i].length, done);
         }
       }
     }
