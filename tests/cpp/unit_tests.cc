@@ -22,6 +22,7 @@
 #include <tensorpipe/common/slot_allocator.h>
 #include <tensorpipe/common/wire.h>
 #include <tensorpipe/channel/error.h>
+#include <tensorpipe/tensorpipe_cuda.h>
 
 using namespace tensorpipe;
 
@@ -141,6 +142,17 @@ static int runBasics() {
   const uint8_t lying[] = {0xff, 0xff, 0xff, 0x7f, 'a'}; // length far beyond the buffer
   WireReader bad(lying, sizeof(lying));
   CHECK(bad.str().empty() && !bad.ok());
+
+  // The reference's names resolve to the HIP side (tensorpipe/tensorpipe_cuda.h).
+  CudaBuffer cb{reinterpret_cast<void*>(0x3000), nullptr};
+  Buffer viaAlias = cb;
+  CHECK(viaAlias.unwrap<HipBuffer>().ptr == reinterpret_cast<void*>(0x3000));
+  std::shared_ptr<channel::Context> (*makeXth)() = &channel::cuda_xth::create;
+  std::shared_ptr<channel::Context> (*makeIpc)() = &channel::cuda_ipc::create;
+  std::shared_ptr<channel::Context> (*makeBasic)(std::shared_ptr<channel::Context>) =
+      &channel::cuda_basic::create;
+  CHECK(makeXth != nullptr && makeIpc != nullptr && makeBasic != nullptr);
+  CHECK(kCudaDeviceType == "cuda");
 
   if (failed == 0) {
     std::printf("OK\n");
