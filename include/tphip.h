@@ -6,7 +6,8 @@
  * Conventions: every function returns 0 on success or a positive hipError_t
  * value (negative values are errors detected by this library itself, see
  * tphip_strerror). No exceptions, no C++ types, no reliance on the caller's
- * current device: every call that needs a device takes its index explicitly.
+ * current device: every call that needs a device takes its index explicitly,
+ * makes it current for its own duration and puts the caller's device back.
  * Streams and events are passed as void* (hipStream_t / hipEvent_t values).
  * All functions are thread-safe.
  *

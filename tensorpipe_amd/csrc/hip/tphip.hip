@@ -145,6 +145,45 @@ int planViaKernel() {
   return v;
 }
 
+// Makes `dev` the calling thread's current device for the lifetime of the
+// object and puts the previous one back afterwards, so that no entry point
+// leaves the caller on another device (the role of CudaDeviceGuard,
+// tensorpipe/common/cuda.h:168-179).
+class DeviceScope {
+ public:
+  explicit DeviceScope(int dev) {
+    err_ = hipGetDevice(&prev_);
+    if (err_ == hipSuccess && prev_ != dev) {
+      err_ = hipSetDevice(dev);
+      changed_ = err_ == hipSuccess;
+    }
+    if (err_ != hipSuccess) {
+      (void)hipGetLastError();
+    }
+  }
+  ~DeviceScope() {
+    if (changed_) {
+      (void)hipSetDevice(prev_);
+    }
+  }
+  DeviceScope(const DeviceScope&) = delete;
+  DeviceScope& operator=(const DeviceScope&) = delete;
+  int error() const {
+    return static_cast<int>(err_);
+  }
+
+ private:
+  int prev_{0};
+  bool changed_{false};
+  hipError_t err_{hipSuccess};
+};
+
+#define TPHIP_ON_DEVICE(dev)          \
+  DeviceScope deviceScope_(dev);      \
+  if (deviceScope_.error() != 0) {    \
+    return deviceScope_.error();      \
+  }
+
 // TPHIP_INLINE_PLANS=0 sends small tables through the plan ring as well (A/B switch).
 bool inlinePlansEnabled() {
   static const bool v = envInt("TPHIP_INLINE_PLANS", 1) != 0;
@@ -156,7 +195,7 @@ int getDevice(int dev, DeviceState** out) {
     return TPHIP_ERR_INVALID_ARG;
   }
   DeviceState& st = gDevices[dev];
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   std::call_once(st.once, [&] {
     hipError_t e = hipDeviceGetAttribute(&st.numCus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e == hipSuccess) {
@@ -456,6 +495,10 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
   if (!(unroll == 0 || unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8)) {
     return TPHIP_ERR_INVALID_ARG;
   }
+  if (dev < 0 || dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
   DeviceState* st = nullptr;
   int rc = getDevice(dev, &st);
   if (rc != 0) {
@@ -643,13 +686,13 @@ int tphip_mem_buffer_id(const void* ptr, uint64_t* id) {
 }
 
 int tphip_malloc(int dev, size_t bytes, void** ptr) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipMalloc(ptr, bytes));
   return 0;
 }
 
 int tphip_free(int dev, void* ptr) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipFree(ptr));
   return 0;
 }
@@ -658,7 +701,7 @@ int tphip_host_alloc(int dev, size_t bytes, void** host_ptr, void** dev_ptr) {
   if (host_ptr == nullptr) {
     return TPHIP_ERR_INVALID_ARG;
   }
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipHostMalloc(host_ptr, bytes, hipHostMallocMapped | hipHostMallocPortable));
   if (dev_ptr != nullptr) {
     TPHIP_TRY(hipHostGetDevicePointer(dev_ptr, *host_ptr, 0));
@@ -672,7 +715,7 @@ int tphip_host_free(void* host_ptr) {
 }
 
 int tphip_stream_create(int dev, void** stream) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipStream_t s;
   TPHIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   *stream = s;
@@ -680,19 +723,19 @@ int tphip_stream_create(int dev, void** stream) {
 }
 
 int tphip_stream_destroy(int dev, void* stream) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(stream)));
   return 0;
 }
 
 int tphip_stream_sync(int dev, void* stream) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   return 0;
 }
 
 int tphip_stream_query(int dev, void* stream, int* done) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
   if (e == hipErrorNotReady) {
     (void)hipGetLastError();
@@ -705,7 +748,7 @@ int tphip_stream_query(int dev, void* stream, int* done) {
 }
 
 int tphip_event_create(int dev, int interprocess, void** event) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipEvent_t e;
   unsigned flags = hipEventDisableTiming;
   if (interprocess) {
@@ -717,7 +760,7 @@ int tphip_event_create(int dev, int interprocess, void** event) {
 }
 
 int tphip_event_create_timed(int dev, void** event) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipEvent_t e;
   TPHIP_TRY(hipEventCreate(&e));
   *event = e;
@@ -725,26 +768,26 @@ int tphip_event_create_timed(int dev, void** event) {
 }
 
 int tphip_event_destroy(int dev, void* event) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
   return 0;
 }
 
 int tphip_event_record(int dev, void* event, void* stream) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
   return 0;
 }
 
 int tphip_stream_wait_event(int dev, void* stream, void* event) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(
       hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
   return 0;
 }
 
 int tphip_event_query(int dev, void* event, int* done) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
   if (e == hipErrorNotReady) {
     (void)hipGetLastError();
@@ -757,7 +800,7 @@ int tphip_event_query(int dev, void* event, int* done) {
 }
 
 int tphip_event_sync(int dev, void* event) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)));
   return 0;
 }
@@ -771,7 +814,7 @@ int tphip_stream_on_complete(int dev, void* stream, tphip_host_fn fn, void* arg)
   if (fn == nullptr) {
     return TPHIP_ERR_INVALID_ARG;
   }
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   HostFnThunk* t = new HostFnThunk{fn, arg};
   hipError_t e = hipStreamAddCallback(static_cast<hipStream_t>(stream), hostFnTrampoline, t, 0);
   if (e != hipSuccess) {
@@ -783,7 +826,7 @@ int tphip_stream_on_complete(int dev, void* stream, tphip_host_fn fn, void* arg)
 
 int tphip_ipc_mem_export(int dev, void* base, uint8_t out[TPHIP_IPC_HANDLE_BYTES]) {
   static_assert(sizeof(hipIpcMemHandle_t) == TPHIP_IPC_HANDLE_BYTES, "handle size");
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipIpcMemHandle_t h;
   TPHIP_TRY(hipIpcGetMemHandle(&h, base));
   memcpy(out, &h, sizeof(h));
@@ -791,7 +834,7 @@ int tphip_ipc_mem_export(int dev, void* base, uint8_t out[TPHIP_IPC_HANDLE_BYTES
 }
 
 int tphip_ipc_mem_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], void** ptr) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipIpcMemHandle_t h;
   memcpy(&h, handle, sizeof(h));
   TPHIP_TRY(hipIpcOpenMemHandle(ptr, h, hipIpcMemLazyEnablePeerAccess));
@@ -799,14 +842,14 @@ int tphip_ipc_mem_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], vo
 }
 
 int tphip_ipc_mem_close(int dev, void* ptr) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipIpcCloseMemHandle(ptr));
   return 0;
 }
 
 int tphip_ipc_event_export(int dev, void* event, uint8_t out[TPHIP_IPC_HANDLE_BYTES]) {
   static_assert(sizeof(hipIpcEventHandle_t) == TPHIP_IPC_HANDLE_BYTES, "handle size");
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipIpcEventHandle_t h;
   TPHIP_TRY(hipIpcGetEventHandle(&h, static_cast<hipEvent_t>(event)));
   memcpy(out, &h, sizeof(h));
@@ -814,7 +857,7 @@ int tphip_ipc_event_export(int dev, void* event, uint8_t out[TPHIP_IPC_HANDLE_BY
 }
 
 int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], void** event) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   hipIpcEventHandle_t h;
   memcpy(&h, handle, sizeof(h));
   hipEvent_t e;
@@ -838,6 +881,10 @@ int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, 
 }
 
 int tphip_profile_start(int dev, uint32_t max_launches) {
+  if (dev < 0 || dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
   DeviceState* st = nullptr;
   int rc = getDevice(dev, &st);
   if (rc != 0) {
@@ -866,6 +913,10 @@ int tphip_profile_start(int dev, uint32_t max_launches) {
 }
 
 int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* total_bytes) {
+  if (dev < 0 || dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
   DeviceState* st = nullptr;
   int rc = getDevice(dev, &st);
   if (rc != 0) {
@@ -910,7 +961,7 @@ int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* 
 }
 
 int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, static_cast<hipStream_t>(stream)));
   return 0;
 }
@@ -919,7 +970,7 @@ int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream) {
   if (bytes == 0) {
     return 0;
   }
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   uint64_t blocks = (bytes + kBlockThreads - 1) / kBlockThreads;
   if (blocks > 2048) {
     blocks = 2048;
@@ -930,7 +981,7 @@ int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream) {
 }
 
 int tphip_test_slow_kernel(int dev, void* ptr, uint64_t n, void* stream) {
-  TPHIP_TRY(hipSetDevice(dev));
+  TPHIP_ON_DEVICE(dev);
   return launchKernel(slow_kernel, dim3(128), dim3(128), 0, static_cast<hipStream_t>(stream),
                       static_cast<volatile unsigned char*>(ptr), n);
 }
