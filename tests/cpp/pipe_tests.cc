@@ -400,6 +400,98 @@ std::vector<Case> makeCases() {
          ep.barrier();
        }});
 
+  // context_test.cc:384-466 (ClientPingInline): read() issued from inside the
+  // readDescriptor callback, on the library's thread.
+  cases.push_back(
+      {"ReadInsideDescriptorCallback",
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         auto done = std::make_shared<std::promise<Error>>();
+         auto fDone = done->get_future();
+         auto storage = std::make_shared<Storage>();
+         auto got = std::make_shared<Descriptor>();
+         Pipe* pipe = e->pipe.get();
+         pipe->readDescriptor([pipe, done, storage, got](const Error& err, Descriptor d) {
+           if (err) {
+             done->set_value(err);
+             return;
+           }
+           Allocation a;
+           for (auto& p : d.payloads) {
+             storage->payloads.emplace_back(p.length, 0);
+             Allocation::Payload ap;
+             ap.data = storage->payloads.back().data();
+             a.payloads.push_back(ap);
+           }
+           for (auto& t : d.tensors) {
+             storage->tensors.push_back(makeData(gHaveGpu && t.sourceDevice == kGpu, t.length));
+             Allocation::Tensor at;
+             at.buffer = storage->tensors.back()->buffer();
+             a.tensors.push_back(std::move(at));
+           }
+           *got = std::move(d);
+           pipe->read(std::move(a), [done](const Error& err2) { done->set_value(err2); });
+         });
+         EXPECT_OK(waitFor(fDone, "read chained to readDescriptor"));
+         EXPECT_EQ(got->tensors.size(), size_t(2));
+         if (got->tensors.size() == 2) {
+           std::vector<uint8_t> b0 = storage->tensors[0]->bytes();
+           std::vector<uint8_t> b1 = storage->tensors[1]->bytes();
+           EXPECT_EQ(std::string(b0.begin(), b0.end()), std::string("tensor #1"));
+           EXPECT_EQ(std::string(b1.begin(), b1.end()), std::string("tensor #2"));
+         }
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         writeMessage(*e->pipe, messageWith({{"tensor #1", "tensor metadata #1", kGpu, nullopt},
+                                              {"tensor #2", "tensor metadata #2", kCpu, nullopt}}));
+         ep.barrier();
+       }});
+
+  // pipe_test.cc:525-600 (WriteFromBothThenRead): each endpoint writes before it
+  // reads; neither write may wait for the local read.
+  auto writeThenRead = [](Endpoint& ep) {
+    auto e = openPipe(ep);
+    const char mine = ep.isServer() ? 'S' : 'C';
+    const char theirs = ep.isServer() ? 'C' : 'S';
+    InlineMessage out = messageWith({{std::string(300000, mine), "from me", kGpu, nullopt},
+                                     {std::string(17, mine), "small", kCpu, nullopt}});
+    InlineMessage in = messageWith({{std::string(300000, theirs), "from me", kGpu, nullopt},
+                                    {std::string(17, theirs), "small", kCpu, nullopt}});
+    Storage storage;
+    Message m = buildMessage(out, &storage);
+    auto p = std::make_shared<std::promise<Error>>();
+    auto f = p->get_future();
+    e->pipe->write(std::move(m), [p](const Error& err) { p->set_value(err); });
+    readAndCheck(*e->pipe, in, {kGpu, kCpu});
+    EXPECT_OK(waitFor(f, "write"));
+    ep.barrier();
+  };
+  cases.push_back({"WriteFromBothThenRead", writeThenRead, writeThenRead});
+
+  // listener_test.cc:21-60 (ClosingAbortsOperations): an accept that is pending
+  // when the listener closes fails, once.
+  auto listenerClose = [](Endpoint& ep) {
+    auto ctx = makeContext(ep.isServer() ? "server" : "client");
+    auto listener = ctx->listen({"shm://" + ep.freshAddr() + (ep.isServer() ? "_s" : "_c")});
+    auto fires = std::make_shared<std::atomic<int>>(0);
+    auto p = std::make_shared<std::promise<Error>>();
+    auto f = p->get_future();
+    listener->accept([p, fires](const Error& err, std::shared_ptr<Pipe>) {
+      if (fires->fetch_add(1) == 0) {
+        p->set_value(err);
+      }
+    });
+    listener->close();
+    Error err = waitFor(f, "accept that must fail");
+    EXPECT_TRUE(static_cast<bool>(err));
+    listener.reset();
+    ctx->join();
+    EXPECT_EQ(fires->load(), 1);
+  };
+  cases.push_back({"ListenerClosingAbortsAccept", listenerClose, listenerClose});
+
   // Sixty messages of random shape each way, all writes issued up front.
   cases.push_back({"ManyMessagesBothDirections",
                    [](Endpoint& ep) {
