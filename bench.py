@@ -329,6 +329,34 @@ def bench_staged(iters=50, warmup=3, nbytes=256 * MIB):
     return out
 
 
+def bench_cpu_path():
+    """configs[0] on this library's own CPU side (Pipe + shm transport + basic channel, two
+    processes): the control plane the device channels ride on, next to the reference's."""
+    import numpy as np
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    out = {}
+    peer = PeerRun("basic:0")
+    try:
+        for name, n, iters in (("4KiB", 4096, 2000), ("1MiB", MIB, 1000), ("64MiB", 64 * MIB, 40)):
+            src = datagen.uniform_u8(datagen.SEED_BASE + 1, n)
+            dst = np.zeros(n, np.uint8)
+            payload = datagen.bench_pattern(64)
+            pout = np.zeros(64, np.uint8)
+            per_us, _ = peer.pingpong([tp.make_tensor(src)], [tp.make_tensor(dst)], [n], "cpu", 5, iters,
+                                      payloads=[payload], recv_payloads=[pout])
+            per_us.sort()
+            p50 = float(per_us[int(0.5 * len(per_us))])
+            out[name] = {"rtt_p50_us": p50, "payload_GBps": 2.0 * n / (p50 * 1e-6) / 1e9,
+                         "byte_exact": bool((src == dst).all()) and bytes(pout) == bytes(payload)}
+            log(f"  own CPU path {name}: rtt p50 {p50:.1f} us  exact={out[name]['byte_exact']}")
+    finally:
+        peer.close()
+    return out
+
+
 def bench_link_ceiling(nbytes=256 * MIB):
     """Pinned D2H / H2D: the copy kernel against the runtime's copy engine path."""
     import torch
@@ -414,6 +442,7 @@ LEGS = {
     "ipc": bench_ipc,
     "staged": bench_staged,
     "host_link": bench_link_ceiling,
+    "cpu_path": bench_cpu_path,
 }
 
 
@@ -468,6 +497,8 @@ def main():
         log("[bench] host-staged 256 MiB")
         extra["staged"] = run_leg("staged")
         extra["host_link"] = run_leg("host_link")
+        log("[bench] this library's CPU path (shm + basic)")
+        extra["cpu_path"] = run_leg("cpu_path")
     log("[bench] CPU baseline (port of shm + basic)")
     cpu = cpu_baseline()
     extra["bench_wall_s"] = time.time() - t_start
