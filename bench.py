@@ -117,6 +117,25 @@ def bench_d2d(steps, warmup):
     memcpy_us = e0.elapsed_ms(e1) / 50 * 1e3
     destroy(objs)
 
+    # The timed loop sends the same source every step, and 64 MiB stays resident in the 256 MiB
+    # Infinity Cache between steps. The same kernel over ten rotating 64 MiB source/destination
+    # pairs (1.25 GiB working set) shows what it does when every byte comes from HBM.
+    pairs = [(torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(),
+              torch.empty(nbytes, dtype=torch.uint8, device="cuda")) for _ in range(10)]
+    torch.cuda.synchronize()
+
+    def rotate():
+        for _ in range(4):
+            for a, b in pairs:
+                hip.copy(b, a, nbytes)
+        torch.cuda.synchronize()
+
+    rotate()
+    _, cold_n, cold_ms, _ = profiled(rotate, 64)
+    cold_us = cold_ms / max(cold_n, 1) * 1e3
+    assert all(torch.equal(a, b) for a, b in pairs[:2])
+    del pairs
+
     kernel_us = kernel_ms / launches * 1e3
     achieved = 2.0 * nbytes / (kernel_us * 1e-6) / 1e9
     per_us.sort()
@@ -135,6 +154,8 @@ def bench_d2d(steps, warmup):
             "kernel": "tphip::single_copy_kernel<4, 2>", "kernel_avg_us": kernel_us,
             "algorithmic_bytes_per_launch": 2 * nbytes,
         },
+        "cold_source_kernel_us": cold_us,
+        "cold_source_hbm_GBps": 2.0 * nbytes / (cold_us * 1e-6) / 1e9,
         "hipMemcpyAsync_d2d_us": memcpy_us,
         "hipMemcpyAsync_d2d_hbm_GBps": 2.0 * nbytes / (memcpy_us * 1e-6) / 1e9,
     }
@@ -283,6 +304,15 @@ def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
             out["sizes"][str(size)] = {
                 "rtt_p50_us": p50, "payload_GBps": gbps, "hbm_GBps": 2 * gbps,
                 "hbm_frac": 2 * gbps / HBM_PEAK_GBPS, "byte_exact": ok, "iters": n_it}
+            if size >= 64 * MIB:
+                # the copy kernel alone (this side launches the copies of the echo direction)
+                _, launches, kernel_ms, _ = profiled(
+                    lambda: peer.pingpong(st, rt, [size], "gpu", 1, 10), 16)
+                k_us = kernel_ms / max(launches, 1) * 1e3
+                out["sizes"][str(size)].update({
+                    "kernel_avg_us": k_us,
+                    "kernel_hbm_GBps": 2.0 * size / (k_us * 1e-6) / 1e9,
+                    "kernel_hbm_frac": 2.0 * size / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBPS})
             log(f"  ipc {size:>11d} B  rtt p50 {p50:10.1f} us  payload {gbps:8.1f} GB/s  exact={ok}")
             del src, dst
             size *= 4
@@ -486,6 +516,9 @@ def main():
     extra = {
         "d2d_step_p50_us": d2d["step_p50_us"],
         "d2d_profiled_pass_ms_per_step": d2d["profiled_pass_ms_per_step"],
+        "d2d_cold_source_kernel_us": d2d["cold_source_kernel_us"],
+        "d2d_cold_source_hbm_GBps": d2d["cold_source_hbm_GBps"],
+        "d2d_cold_source_hbm_frac": d2d["cold_source_hbm_GBps"] / HBM_PEAK_GBPS,
         "hipMemcpyAsync_d2d_us": d2d["hipMemcpyAsync_d2d_us"],
         "hipMemcpyAsync_d2d_hbm_GBps": d2d["hipMemcpyAsync_d2d_hbm_GBps"],
     }
