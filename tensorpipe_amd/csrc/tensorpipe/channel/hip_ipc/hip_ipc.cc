@@ -31,7 +31,9 @@
 
 #include <tensorpipe/channel/hip_ipc/factory.h>
 
+#include <algorithm>
 #include <array>
+#include <cstdlib>
 #include <deque>
 #include <map>
 #include <mutex>
@@ -49,11 +51,25 @@ namespace hip_ipc {
 
 namespace {
 
-// Staging geometry of the outbox path, as
-// tensorpipe/channel/cuda_ipc/constants.h:22-24.
-constexpr size_t kSlotSize = 8 * 1024 * 1024;
-constexpr size_t kNumSlots = 4;
-constexpr size_t kStagingAreaSize = kSlotSize * kNumSlots;
+// Staging geometry of the outbox path. The reference uses 4 slots of 8 MiB
+// (tensorpipe/channel/cuda_ipc/constants.h:22-24); every chunk costs two host
+// round trips here (there are no cross-process events to let the GPU order the
+// two copies), so the defaults are larger -- 8 slots of 32 MiB, 256 MiB of a
+// 288 GB device, allocated when the path is first used -- and both are
+// settable per context (TP_HIP_IPC_SLOT_BYTES, TP_HIP_IPC_NUM_SLOTS). The
+// sender's geometry travels with the first chunk it announces.
+constexpr size_t kDefaultSlotBytes = 32u << 20;
+constexpr size_t kDefaultNumSlots = 8;
+constexpr size_t kMaxNumSlots = 1024;
+
+size_t envSize(const char* name, size_t fallback) {
+  const char* e = std::getenv(name);
+  if (e == nullptr || *e == 0) {
+    return fallback;
+  }
+  const unsigned long long v = std::strtoull(e, nullptr, 10);
+  return v > 0 ? static_cast<size_t>(v) : fallback;
+}
 
 // Read when a context is created, so that one process can host contexts of
 // both kinds.
@@ -134,8 +150,8 @@ class ExportRegistry {
 
 // Per-device staging slab of the outbox path, created on first use.
 struct Outbox {
-  explicit Outbox(int device)
-      : slab(device, kStagingAreaSize), allocator(slab.ptr(), kNumSlots, kSlotSize) {
+  Outbox(int device, size_t slotBytes, size_t numSlots)
+      : slab(device, slotBytes * numSlots), allocator(slab.ptr(), numSlots, slotBytes) {
     TP_HIP_CHECK(tphip_ipc_mem_export(device, slab.ptr(), handle.data()));
   }
   HipDeviceSlab slab;
@@ -149,6 +165,9 @@ class IpcContextCore final : public ContextCore {
   HipEventPool events;
   HipEventPoller poller;
   const bool forceOutbox{outboxForcedByEnv()};
+  // 16-byte multiples keep every slot vector-aligned.
+  const size_t slotBytes{(envSize("TP_HIP_IPC_SLOT_BYTES", kDefaultSlotBytes) + 15) / 16 * 16};
+  const size_t numSlots{std::min(envSize("TP_HIP_IPC_NUM_SLOTS", kDefaultNumSlots), kMaxNumSlots)};
 
   // Loop only.
   Outbox& outbox(int device) {
@@ -156,7 +175,7 @@ class IpcContextCore final : public ContextCore {
       outboxes_.resize(device + 1);
     }
     if (!outboxes_[device]) {
-      outboxes_[device] = std::make_unique<Outbox>(device);
+      outboxes_[device] = std::make_unique<Outbox>(device, slotBytes, numSlots);
     }
     return *outboxes_[device];
   }
@@ -298,8 +317,8 @@ class ChannelImpl final : public ChannelImplBase {
     bool ready{false};
   };
 
-  static size_t numChunks(size_t length) {
-    return (length + kSlotSize - 1) / kSlotSize;
+  size_t numChunks(size_t length) const {
+    return (length + ictx_->slotBytes - 1) / ictx_->slotBytes;
   }
 
   // ---- send -----------------------------------------------------------------
@@ -409,8 +428,8 @@ class ChannelImpl final : public ChannelImplBase {
         const int device = hipDeviceForPointer(hb.ptr);
         const size_t chunks = numChunks(live[i].length);
         for (size_t k = 0; k < chunks; ++k) {
-          const size_t offset = k * kSlotSize;
-          const size_t len = std::min(live[i].length - offset, kSlotSize);
+          const size_t offset = k * ictx_->slotBytes;
+          const size_t len = std::min(live[i].length - offset, ictx_->slotBytes);
           auto unit = std::make_shared<WireUnit>();
           wireQueue_.push_back(unit);
           ++op->pending; // staged copy of this chunk finished
@@ -463,6 +482,8 @@ class ChannelImpl final : public ChannelImplBase {
       if (announce) {
         w.str(processIdentity());
         w.u64(outbox.id);
+        w.u64(ictx_->slotBytes);
+        w.u32(static_cast<uint32_t>(ictx_->numSlots));
         w.raw(outbox.handle.data(), outbox.handle.size());
       }
       w.u32(static_cast<uint32_t>(slotIdx));
@@ -621,9 +642,12 @@ class ChannelImpl final : public ChannelImplBase {
         if (announce) {
           const std::string peer = r.str();
           const uint64_t outboxId = r.u64();
+          const uint64_t remoteSlotBytes = r.u64();
+          const uint32_t remoteNumSlots = r.u32();
           HandleBytes h;
           r.raw(h.data(), h.size());
-          if (!r.ok() || remoteOutboxes_.count(srcDevice) != 0) {
+          if (!r.ok() || remoteOutboxes_.count(srcDevice) != 0 || remoteSlotBytes == 0 ||
+              remoteNumSlots == 0 || remoteNumSlots > kMaxNumSlots) {
             failProtocol();
             return;
           }
@@ -633,22 +657,22 @@ class ChannelImpl final : public ChannelImplBase {
             setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
             return;
           }
-          remoteOutboxes_[srcDevice] = mapped;
+          remoteOutboxes_[srcDevice] = RemoteOutbox{mapped, remoteSlotBytes, remoteNumSlots};
           imports_.push_back(Import{device, peer, outboxId});
         }
         const uint32_t slotIdx = r.u32();
         const uint64_t offset = r.u64();
         const uint64_t len = r.u64();
         auto it = remoteOutboxes_.find(srcDevice);
-        if (!r.ok() || it == remoteOutboxes_.end() || slotIdx >= kNumSlots || len > kSlotSize ||
-            offset + len > op->entries[index].length) {
+        if (!r.ok() || it == remoteOutboxes_.end() || slotIdx >= it->second.numSlots ||
+            len > it->second.slotBytes || offset + len > op->entries[index].length) {
           failProtocol();
           return;
         }
         int rc = tphip_copy(
             device,
             static_cast<uint8_t*>(hb.ptr) + offset,
-            static_cast<const uint8_t*>(it->second) + slotIdx * kSlotSize,
+            static_cast<const uint8_t*>(it->second.ptr) + slotIdx * it->second.slotBytes,
             len,
             hb.stream);
         if (rc != 0) {
@@ -771,7 +795,12 @@ class ChannelImpl final : public ChannelImplBase {
   std::set<uint64_t> announced_;
   std::map<int, bool> outboxAnnounced_;
   std::map<uint64_t, void*> remoteAllocations_;
-  std::map<int, void*> remoteOutboxes_;
+  struct RemoteOutbox {
+    void* ptr;
+    uint64_t slotBytes;
+    uint32_t numSlots;
+  };
+  std::map<int, RemoteOutbox> remoteOutboxes_;
   // What this channel holds in the process-wide import table.
   struct Import {
     int device;

@@ -246,9 +246,28 @@ def ipc_peer():
 
 @pytest.fixture(scope="module")
 def ipc_outbox_peer():
+    # the reference's staging geometry (4 slots of 8 MiB), so that the sizes below cross slot
+    # boundaries and reuse slots
+    env = {"TP_HIP_IPC_MODE": "outbox", "TP_HIP_IPC_SLOT_BYTES": str(8 << 20), "TP_HIP_IPC_NUM_SLOTS": "4"}
+    os.environ.update(env)
+    try:
+        peer = Peer("basic:0,hip_ipc:11", env=env)
+    finally:
+        for k in env:
+            del os.environ[k]
+    yield peer
+    peer.close()
+
+
+@pytest.fixture(scope="module")
+def ipc_outbox_default_peer():
+    # default geometry on this side, a small odd one on the peer's: each receiver follows the
+    # geometry the sender announced
     os.environ["TP_HIP_IPC_MODE"] = "outbox"
     try:
-        peer = Peer("basic:0,hip_ipc:11", env={"TP_HIP_IPC_MODE": "outbox"})
+        peer = Peer("basic:0,hip_ipc:11", env={"TP_HIP_IPC_MODE": "outbox",
+                                               "TP_HIP_IPC_SLOT_BYTES": str((1 << 20) + 48),
+                                               "TP_HIP_IPC_NUM_SLOTS": "3"})
     finally:
         del os.environ["TP_HIP_IPC_MODE"]
     yield peer
@@ -329,6 +348,12 @@ def test_ipc_outbox_sizes(oracle, ipc_outbox_peer):
     # multi-chunk (> 8 MiB) and slot reuse (> 4 chunks in flight) included
     _ipc_cases(oracle, ipc_outbox_peer, 8 << 20,
                [256, 1 << 20, (8 << 20) - 1, 8 << 20, (8 << 20) + 1, (40 << 20) + 7, 0])
+
+
+def test_ipc_outbox_mixed_geometries(oracle, ipc_outbox_default_peer):
+    # 32 MiB slots this way, 1 MiB + 48 B slots (three of them) on the way back
+    _ipc_cases(oracle, ipc_outbox_default_peer, 32 << 20,
+               [4096, (1 << 20) + 48, (1 << 20) + 49, (32 << 20) + 5, (70 << 20) + 1, 0])
 
 
 def test_ipc_refuses_same_process():
