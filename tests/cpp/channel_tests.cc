@@ -2,7 +2,7 @@
 // plugin surface itself: channel::Context::createChannel over raw transport
 // connections, then Channel::send / recv with Buffer{HipBuffer|CpuBuffer}.
 //
-//   channel_tests --suite hip_xth|hip_ipc|hip_basic|basic|xth [--case SUBSTRING] [--list]
+//   channel_tests --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_basic|basic|xth [--case SUBSTRING] [--list]
 //
 // hip_xth and xth run both endpoints as two threads of this process; hip_ipc,
 // hip_basic and basic run them as two processes. The CPU channels (basic, xth)
@@ -25,11 +25,12 @@ std::string gSuite;
 bool gGpu = true; // whether the suite's tensors live on the GPU
 
 bool knownSuite(const std::string& s) {
-  return s == "hip_xth" || s == "hip_ipc" || s == "hip_basic" || s == "basic" || s == "xth";
+  return s == "hip_xth" || s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_basic" ||
+      s == "basic" || s == "xth";
 }
 
 bool twoProcessSuite(const std::string& s) {
-  return s == "hip_ipc" || s == "hip_basic" || s == "basic";
+  return s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_basic" || s == "basic";
 }
 
 Buffer nullBuffer() {
@@ -43,7 +44,7 @@ std::shared_ptr<channel::Context> makeContext() {
   if (gSuite == "hip_xth") {
     return channel::hip_xth::create();
   }
-  if (gSuite == "hip_ipc") {
+  if (gSuite == "hip_ipc" || gSuite == "hip_ipc_outbox") {
     return channel::hip_ipc::create();
   }
   if (gSuite == "hip_basic") {
@@ -360,7 +361,7 @@ std::vector<Case> makeCases() {
     cases.push_back({"CannotCommunicateCpuToCpu", cpuToCpu, cpuToCpu});
   }
 
-  if (gSuite == "hip_ipc") {
+  if (gSuite == "hip_ipc" || gSuite == "hip_ipc_outbox") {
     // cuda_ipc_test.cc:37-57: two contexts of one process must not pick IPC.
     auto sameProcess = [](Endpoint&) {
       auto c1 = makeContext();
@@ -530,12 +531,19 @@ int main(int argc, char** argv) {
   Args args = parseArgs(argc, argv);
   if (!knownSuite(args.suite)) {
     std::fprintf(
-        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_basic|basic|xth [--case S] [--list]\n",
+        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_basic|basic|xth [--case S] [--list]\n",
         argv[0]);
     return 2;
   }
   gSuite = args.suite;
   gGpu = gSuite.rfind("hip_", 0) == 0;
+  if (gSuite == "hip_ipc_outbox") {
+    // The reference's algorithm (every tensor staged through the outbox), with
+    // slots small enough for the sizes of this suite to span and reuse them.
+    ::setenv("TP_HIP_IPC_MODE", "outbox", 1);
+    ::setenv("TP_HIP_IPC_SLOT_BYTES", "1048576", 1);
+    ::setenv("TP_HIP_IPC_NUM_SLOTS", "3", 1);
+  }
   std::vector<Case> cases = makeCases();
   if (args.list) {
     for (auto& c : cases) {
