@@ -478,15 +478,17 @@ LEGS = {
     "rpc_message": bench_rpc_message,
     "ipc": bench_ipc,
     "staged": bench_staged,
+    "staged_short": lambda: bench_staged(iters=20),
     "host_link": bench_link_ceiling,
     "cpu_path": bench_cpu_path,
     "cold_copy": bench_cold_copy,
 }
 
 
-def run_leg(name, timeout_s=600):
+def run_leg(name, timeout_s=600, env=None):
     proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--leg", name],
-                          stdout=subprocess.PIPE, timeout=timeout_s)
+                          stdout=subprocess.PIPE, timeout=timeout_s,
+                          env=dict(os.environ, **(env or {})))
     if proc.returncode != 0:
         raise RuntimeError(f"bench leg {name} failed with exit code {proc.returncode}")
     return json.loads(proc.stdout.decode().strip().splitlines()[-1])
@@ -534,6 +536,8 @@ def main():
         extra["ipc"] = run_leg("ipc")
         log("[bench] host-staged 256 MiB")
         extra["staged"] = run_leg("staged")
+        # the same transfers with the runtime's hipMemcpyAsync instead of the copy kernel
+        extra["staged_hipMemcpyAsync"] = run_leg("staged_short", env={"TP_HIP_BASIC_ENGINE": "sdma"})
         extra["host_link"] = run_leg("host_link")
         extra["d2d_cold_source"] = run_leg("cold_copy")
         log("[bench] this library's CPU path (shm + basic)")

@@ -543,7 +543,7 @@ class ChannelImpl final : public ChannelImplBase {
           ++it;
         }
       }
-      if (!launchHostLinkCopy(device, stream, table)) {
+      if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/true)) {
         return;
       }
       auto ev = bctx_->events.get(device);
@@ -580,7 +580,41 @@ class ChannelImpl final : public ChannelImplBase {
   // A copy with one end in pinned host memory: the host link saturates with
   // about 32 workgroups, more only add contention (50 vs 42 GB/s reading
   // alone; with the other direction busy 64 workgroups lose 1-5 GB/s).
-  bool launchHostLinkCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table) {
+  // TP_HIP_BASIC_ENGINE chooses who moves the bytes, for comparison: "kernel"
+  // (default: the copy kernel in both directions), "sdma" (the runtime's
+  // hipMemcpyAsync in both) or "mixed" (kernel towards the host, the runtime's
+  // copy from it).
+  enum class Engine { kKernel, kSdma, kMixed };
+  static Engine engine() {
+    static const Engine chosen = [] {
+      const char* e = std::getenv("TP_HIP_BASIC_ENGINE");
+      if (e != nullptr && std::strcmp(e, "sdma") == 0) {
+        return Engine::kSdma;
+      }
+      if (e != nullptr && std::strcmp(e, "mixed") == 0) {
+        return Engine::kMixed;
+      }
+      return Engine::kKernel;
+    }();
+    return chosen;
+  }
+
+  bool launchHostLinkCopy(
+      int device,
+      void* stream,
+      const std::vector<tphip_copy_desc>& table,
+      bool towardsHost) {
+    const Engine how = engine();
+    if (how == Engine::kSdma || (how == Engine::kMixed && !towardsHost)) {
+      for (const auto& d : table) {
+        int rc = tphip_memcpy_async(device, d.dst, d.src, d.bytes, stream);
+        if (rc != 0) {
+          setError(TP_CREATE_ERROR(HipError, "tphip_memcpy_async", rc));
+          return false;
+        }
+      }
+      return true;
+    }
     size_t off = 0;
     while (off < table.size()) {
       const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
@@ -786,7 +820,7 @@ class ChannelImpl final : public ChannelImplBase {
           ++it;
         }
       }
-      if (!launchHostLinkCopy(device, stream, table)) {
+      if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/false)) {
         return;
       }
       auto ev = bctx_->events.get(device);
@@ -884,7 +918,8 @@ class ChannelImpl final : public ChannelImplBase {
             {tphip_copy_desc{
                 rring.devAddress(chunk->slot.get()),
                 static_cast<uint8_t*>(hb.ptr) + chunk->offset,
-                chunk->length}})) {
+                chunk->length}},
+            /*towardsHost=*/false)) {
       return;
     }
     auto ev = bctx_->events.get(device);
