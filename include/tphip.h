@@ -165,7 +165,8 @@ int tphip_profile_start(int dev, uint32_t max_launches);
 int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* total_bytes);
 
 /* Runtime copy engine path (hipMemcpyAsync), kept only as the A/B comparison
- * for the kernel-driven copies; never used by the channels' data path. */
+ * for the kernel-driven copies; the channels use it only when asked to
+ * (TP_HIP_BASIC_ENGINE=sdma|mixed), never by default. */
 int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream);
 
 /* Fill `bytes` bytes at `ptr` with `value` using a kernel (safe to capture in
@@ -176,6 +177,13 @@ int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream);
  * leaving garbage behind; lets a test detect a missing event wait. HIP
  * counterpart of slowKernel, tensorpipe/test/channel/kernel.cu:11-22. */
 int tphip_test_slow_kernel(int dev, void* ptr, uint64_t n, void* stream);
+
+/* Test hook: the largest number of 16-byte vectors one table launch may
+ * carry (its prefix sums are 32-bit); a table beyond it is cut into several
+ * launches and an entry beyond it goes to the single-entry kernel. 0 restores
+ * the built-in limit (just under 2^32 vectors = 64 GiB). Lets a test drive
+ * the cut with small tables. The reference has no counterpart. */
+int tphip_test_set_table_limit(uint64_t vectors);
 
 #ifdef __cplusplus
 }

@@ -116,6 +116,7 @@ def tphip():
         lib.tphip_memcpy_async.argtypes = [i32, vp, vp, u64, vp]
         lib.tphip_fill.argtypes = [i32, vp, i32, u64, vp]
         lib.tphip_test_slow_kernel.argtypes = [i32, vp, u64, vp]
+        lib.tphip_test_set_table_limit.argtypes = [u64]
         _tphip = lib
     return _tphip
 

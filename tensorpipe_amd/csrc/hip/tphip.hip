@@ -38,6 +38,7 @@ constexpr size_t kPlanSlotBytes =
 // Plans for small tables are packed into sub-slots so that a burst of
 // messages does not wait for a slot.
 constexpr uint64_t kMaxTableVectors = 0xFFFFFFFFull - 64ull * 8ull;
+std::atomic<uint64_t> gTableLimit{kMaxTableVectors}; // lowered by tests only
 
 struct DeviceState {
   std::once_flag once;
@@ -542,12 +543,13 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
 
   // Cut into launches whose body vector total fits the 32-bit prefix; entries
   // too large for that go through the single-entry kernel (64-bit counts).
+  const uint64_t limit = gTableLimit.load(std::memory_order_relaxed);
   uint32_t begin = 0;
   uint64_t acc = 0;
   for (uint32_t i = 0; i <= m; ++i) {
     const uint64_t vecs = i < m ? (cur[i].bytes >> 4) : 0;
-    const bool huge = i < m && vecs > kMaxTableVectors;
-    if (i == m || huge || acc + vecs > kMaxTableVectors) {
+    const bool huge = i < m && vecs > limit;
+    if (i == m || huge || acc + vecs > limit) {
       const uint32_t cnt = i - begin;
       if (cnt == 1) {
         rc = copySingle(*st, cur[begin], stream, unroll, blocks, nt);
@@ -986,6 +988,14 @@ int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream) {
   return launchKernel(fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlockThreads), 0,
                       static_cast<hipStream_t>(stream), static_cast<unsigned char*>(ptr),
                       static_cast<unsigned char>(value), bytes);
+}
+
+int tphip_test_set_table_limit(uint64_t vectors) {
+  if (vectors > kMaxTableVectors) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  gTableLimit.store(vectors == 0 ? kMaxTableVectors : vectors, std::memory_order_relaxed);
+  return 0;
 }
 
 int tphip_test_slow_kernel(int dev, void* ptr, uint64_t n, void* stream) {

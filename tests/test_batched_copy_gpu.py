@@ -148,6 +148,50 @@ def test_many_inline_launches_back_to_back(oracle):
         _run_case(oracle, _pack(sizes, lambda i: (i + k) % 16, lambda i: (i * 5 + k) % 16), seed=300 + k)
 
 
+@pytest.mark.parametrize("limit", [1, 64, 1000, 70000])
+def test_table_cut_into_several_launches(oracle, limit):
+    # a table whose 16-byte vector total exceeds what one launch carries is cut into several
+    # launches, and an entry above the limit goes to the single-entry kernel; driven here with a
+    # lowered limit (the real one is just under 64 GiB) on tables with both kinds of entry
+    lib = _native.tphip()
+    rng = np.random.default_rng(4000 + limit)
+    sizes = [int(x) for x in rng.integers(0, 40000, 90)] + [0, 15, 16 * limit, 16 * limit + 16,
+                                                            16 * limit - 1, 3 << 20]
+    order = rng.permutation(len(sizes))
+    sizes = [sizes[i] for i in order]
+    layout = _pack(sizes, lambda i: (i * 7) % 16, lambda i: (i * 3) % 16)
+    _native.check(lib.tphip_test_set_table_limit(limit))
+    try:
+        _run_case(oracle, layout, seed=limit)
+        _run_case(oracle, layout, seed=limit + 1, tuned=(2, 9, 3))
+    finally:
+        _native.check(lib.tphip_test_set_table_limit(0))
+    assert lib.tphip_test_set_table_limit(1 << 33) == -1
+
+
+def test_entry_larger_than_4GiB():
+    # 64-bit byte counts in the single-entry kernel and in a table next to small entries: 5 GiB + 3
+    # with unaligned ends, checked on the device
+    import torch
+
+    n = (5 << 30) + 3
+    a = torch.empty((n + 16 + 7) // 8, dtype=torch.int64, device="cuda").random_().view(torch.uint8)
+    b = torch.full((n + 32,), FILL, dtype=torch.uint8, device="cuda")
+    hip.batched_copy([(a.data_ptr() + 1, b.data_ptr() + 7, n)])
+    torch.cuda.synchronize()
+    assert torch.equal(a[1:1 + n], b[7:7 + n])
+    assert bool((b[:7] == FILL).all()) and bool((b[7 + n:] == FILL).all())
+    b.fill_(FILL)
+    small = torch.arange(1000, dtype=torch.int32, device="cuda").view(torch.uint8)
+    out = torch.zeros(4000 + 8, dtype=torch.uint8, device="cuda")
+    hip.batched_copy([(small, out.data_ptr() + 3, 4000), (a.data_ptr() + 1, b.data_ptr() + 7, n),
+                      (small.data_ptr() + 5, out.data_ptr() + 4003, 2)])
+    torch.cuda.synchronize()
+    assert torch.equal(a[1:1 + n], b[7:7 + n])
+    assert torch.equal(out[3:4003], small) and torch.equal(out[4003:4005], small[5:7])
+    assert bool((b[:7] == FILL).all()) and bool((b[7 + n:] == FILL).all())
+
+
 def test_full_size_roundtrip_property():
     # 1 GiB single tensor and the ~105 MiB many-tensor message at full size:
     # checked on the device (copy twice, compare), not against the CPU oracle.
