@@ -78,6 +78,12 @@ bool outboxForcedByEnv() {
   return e != nullptr && std::string(e) == "outbox";
 }
 
+// Allocations of this size or more are not exported but staged through the
+// outbox: mapping an allocation of 2 GiB or more in another process has been
+// seen never to return on the deployment this was built for. Settable per
+// context (TP_HIP_IPC_MAX_EXPORT_BYTES) where larger mappings are known to work.
+constexpr size_t kDefaultMaxExportBytes = size_t(2) << 30;
+
 // Allocations this process has exported, keyed by base address. Process-wide:
 // a handle describes an allocation, not a context.
 struct ExportedAllocation {
@@ -95,7 +101,12 @@ class ExportRegistry {
   }
 
   // Returns false if the allocation containing ptr cannot be exported.
-  bool lookup(int device, const void* ptr, ExportedAllocation* out, uint64_t* offset) {
+  bool lookup(
+      int device,
+      const void* ptr,
+      size_t maxExportBytes,
+      ExportedAllocation* out,
+      uint64_t* offset) {
     // Common case first: ptr falls inside an allocation exported before. One
     // runtime query (the allocation's identifier) confirms that the address
     // range still belongs to that allocation.
@@ -108,7 +119,8 @@ class ExportRegistry {
         --it;
         const uint8_t* base = static_cast<const uint8_t*>(it->first);
         const uint8_t* p = static_cast<const uint8_t*>(ptr);
-        if (p < base + it->second.size && it->second.bufferId == bufferId) {
+        if (p < base + it->second.size && it->second.bufferId == bufferId &&
+            it->second.size < maxExportBytes) {
           *out = it->second;
           *offset = static_cast<uint64_t>(p - base);
           return true;
@@ -117,7 +129,7 @@ class ExportRegistry {
     }
     void* base = nullptr;
     size_t size = 0;
-    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr) {
+    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr || size >= maxExportBytes) {
       return false;
     }
     uint64_t bufferId = 0;
@@ -165,6 +177,7 @@ class IpcContextCore final : public ContextCore {
   HipEventPool events;
   HipEventPoller poller;
   const bool forceOutbox{outboxForcedByEnv()};
+  const size_t maxExportBytes{envSize("TP_HIP_IPC_MAX_EXPORT_BYTES", kDefaultMaxExportBytes)};
   // 16-byte multiples keep every slot vector-aligned.
   const size_t slotBytes{(envSize("TP_HIP_IPC_SLOT_BYTES", kDefaultSlotBytes) + 15) / 16 * 16};
   const size_t numSlots{std::min(envSize("TP_HIP_IPC_NUM_SLOTS", kDefaultNumSlots), kMaxNumSlots)};
@@ -358,7 +371,8 @@ class ChannelImpl final : public ChannelImplBase {
         const int device = hipDeviceForPointer(hb.ptr);
         TP_THROW_ASSERT_IF(device < 0);
         DirectItem item;
-        if (!ictx_->forceOutbox && ExportRegistry::get().lookup(device, hb.ptr, &item.alloc, &item.offset)) {
+        if (!ictx_->forceOutbox && ExportRegistry::get().lookup(
+                device, hb.ptr, ictx_->maxExportBytes, &item.alloc, &item.offset)) {
           item.length = live[i].length;
           item.index = i;
           direct.push_back(item);

@@ -380,6 +380,48 @@ std::vector<Case> makeCases() {
     cases.push_back({"CannotCommunicateInSameProcess", sameProcess, sameProcess});
   }
 
+  if (gSuite == "hip_ipc") {
+    // An allocation at or above the export limit is not mapped by the peer but
+    // staged through the outbox. The two routes are told apart by when the send
+    // completes: a staged send once its bytes sit in the outbox, before the
+    // peer has posted its recv; a direct send only after the peer's copy.
+    const size_t big = 256 * 1024, small = 4096;
+    auto pattern = [](size_t n, uint8_t salt) {
+      std::vector<uint8_t> v(n);
+      for (size_t i = 0; i < n; ++i) {
+        v[i] = static_cast<uint8_t>((i >> 8) ^ (i & 0xff) ^ salt);
+      }
+      return v;
+    };
+    auto sendSide = [=](Endpoint& ep) {
+      ::setenv("TP_HIP_IPC_MAX_EXPORT_BYTES", "65536", 1);
+      auto o = open(ep);
+      ::unsetenv("TP_HIP_IPC_MAX_EXPORT_BYTES");
+      GpuData above(pattern(big, 1));
+      GpuData below(pattern(small, 2));
+      auto fa = sendF(*o->ch, above.buffer(), above.size());
+      EXPECT_OK(waitFor(fa, "staged send before the peer's recv"));
+      auto fb = sendF(*o->ch, below.buffer(), below.size());
+      EXPECT_TRUE(fb.wait_for(std::chrono::milliseconds(300)) == std::future_status::timeout);
+      ep.barrier(); // the peer posts its recvs now
+      EXPECT_OK(waitFor(fb, "direct send"));
+      ep.barrier();
+    };
+    auto recvSide = [=](Endpoint& ep) {
+      auto o = open(ep);
+      GpuData a(big), b(small);
+      ep.barrier();
+      auto fa = recvF(*o->ch, a.buffer(), a.size());
+      auto fb = recvF(*o->ch, b.buffer(), b.size());
+      EXPECT_OK(waitFor(fa, "recv of the staged tensor"));
+      EXPECT_OK(waitFor(fb, "recv of the direct tensor"));
+      expectBytes(a, pattern(big, 1), "staged tensor");
+      expectBytes(b, pattern(small, 2), "direct tensor");
+      ep.barrier();
+    };
+    cases.push_back({"AllocationsAboveExportLimitAreStaged", sendSide, recvSide});
+  }
+
   if (gSuite == "hip_xth") {
     auto sameProcess = [](Endpoint&) {
       auto c1 = makeContext();
