@@ -32,6 +32,7 @@ extern "C" {
 #define TPHIP_ERR_TOO_LARGE (-2)
 #define TPHIP_ERR_OVERLAP (-3)
 #define TPHIP_ERR_NO_DEVICE (-4)
+#define TPHIP_ERR_CAPTURING (-5)
 
 /* One entry of the copy table: `bytes` bytes from `src` to `dst`. Any
  * alignment, any length (including 0). Ranges of different entries must not
@@ -139,7 +140,11 @@ int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], 
  * device memory by a small staging kernel enqueued ahead of the copy kernel. Any mix of device, mapped-pinned-host and peer-mapped (IPC)
  * addresses is accepted as long as the device can address them. n == 0 or an
  * all-empty table enqueues nothing. n > TPHIP_MAX_BATCH returns
- * TPHIP_ERR_TOO_LARGE. Replaces one cudaMemcpyAsync per tensor at the three
+ * TPHIP_ERR_TOO_LARGE. A call whose plan travels in the kernel arguments (up
+ * to 64 non-empty entries; tphip_copy always) may be captured into a HIP
+ * graph: every replay copies between the same addresses. A larger table on a
+ * capturing stream returns TPHIP_ERR_CAPTURING and enqueues nothing, because
+ * the plan ring is rewritten by later calls. Replaces one cudaMemcpyAsync per tensor at the three
  * call sites listed for tphip_copy_desc. */
 int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* stream);
 
@@ -150,7 +155,8 @@ int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream
 /* Same as tphip_batched_copy with explicit launch shape, for tuning sweeps:
  * `unroll` in {1,2,4,8} 16-byte vectors in flight per lane, `blocks` workgroups
  * of 256 threads (0 = default: one per CU), `nontemporal` a mask (bit 0 =
- * nontemporal loads, bit 1 = nontemporal stores; the default is 3). */
+ * nontemporal loads, bit 1 = nontemporal stores; negative = the default, which
+ * goes by the bytes of the launch: 0 up to 64 MiB, 2 up to 512 MiB, 3 above). */
 int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                              int unroll, uint32_t blocks, int nontemporal);
 

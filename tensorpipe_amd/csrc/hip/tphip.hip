@@ -404,6 +404,16 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     }
   }
 
+  // The plan ring is rewritten by later calls: a graph that captured this
+  // launch would replay it over someone else's plan.
+  if (stream != nullptr) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    TPHIP_TRY(hipStreamIsCapturing(stream, &capture));
+    if (capture != hipStreamCaptureStatusNone) {
+      return TPHIP_ERR_CAPTURING;
+    }
+  }
+
   const size_t prefixBytes = ((size_t(n) + 1) * sizeof(uint32_t) + 15) / 16 * 16;
   const size_t bodyBytes = size_t(n) * sizeof(CopyBody);
   const size_t planBytes = prefixBytes + bodyBytes + size_t(n) * sizeof(tphip_copy_desc);
@@ -602,6 +612,8 @@ const char* tphip_strerror(int err) {
       return "tphip: overlapping ranges in copy table";
     case TPHIP_ERR_NO_DEVICE:
       return "tphip: no usable GPU";
+    case TPHIP_ERR_CAPTURING:
+      return "tphip: a table of more than 64 entries cannot be captured into a graph";
     default:
       return hipGetErrorString(static_cast<hipError_t>(err));
   }

@@ -192,6 +192,59 @@ def test_entry_larger_than_4GiB():
     assert bool((b[:7] == FILL).all()) and bool((b[7 + n:] == FILL).all())
 
 
+def test_graph_capture_and_replay(oracle):
+    # launches whose plan travels in the kernel arguments can be captured; every replay must copy
+    # what the sources hold at that moment. Eager work and synchronisation between the replays.
+    import torch
+
+    lib = _native.tphip()
+    rng = np.random.default_rng(77)
+    sizes = [int(x) for x in rng.integers(1, 50000, 40)] + [0, 1, 15, 17, 1 << 20]
+    layout = _pack(sizes, lambda i: (i * 3) % 16, lambda i: (i * 11) % 16)
+    src_size = max(s + n for s, _, n in layout) + 64
+    dst_size = max(d + n for _, d, n in layout) + 64
+    one = (5 << 20) + 13
+    src = torch.zeros(src_size, dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(dst_size, dtype=torch.uint8, device="cuda")
+    big_src = torch.zeros(one + 16, dtype=torch.uint8, device="cuda")
+    big_dst = torch.zeros(one + 16, dtype=torch.uint8, device="cuda")
+    entries = [(src.data_ptr() + s, dst.data_ptr() + d, n) for s, d, n in layout]
+    many = [(src.data_ptr() + i, dst.data_ptr() + i, 1) for i in range(70)]
+    many_table, many_n = hip.make_table(many)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hip.batched_copy(entries)
+        hip.copy(big_dst.data_ptr() + 3, big_src.data_ptr() + 1, one)
+        # more entries than fit the kernel arguments: refused while capturing, nothing enqueued
+        stream = torch.cuda.current_stream().cuda_stream
+        assert lib.tphip_batched_copy(0, many_table, many_n, ctypes.c_void_p(stream)) == -5
+    assert b"graph" in lib.tphip_strerror(-5)
+
+    for replay in range(4):
+        host_src = datagen.uniform_u8(900 + replay, src_size)
+        host_big = datagen.uniform_u8(950 + replay, one + 16)
+        src.copy_(torch.from_numpy(host_src))
+        big_src.copy_(torch.from_numpy(host_big))
+        dst.fill_(FILL)
+        big_dst.fill_(FILL)
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = np.full(dst_size, FILL, dtype=np.uint8)
+        oracle.xth_message([(host_src[s:], ref[d:], n) for s, d, n in layout])
+        assert (dst.cpu().numpy() == ref).all(), f"replay {replay}: table copy differs"
+        got = big_dst.cpu().numpy()
+        assert (got[3:3 + one] == host_big[1:1 + one]).all(), f"replay {replay}: single copy differs"
+        assert (got[:3] == FILL).all() and (got[3 + one:] == FILL).all()
+        # eager launches between replays, through the plan ring as well
+        _run_case(oracle, _pack([100 + replay] * 70), seed=replay)
+    # outside capture the large table goes through as before
+    _native.check(lib.tphip_batched_copy(0, many_table, many_n, None))
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:70], src[:70])
+
+
 def test_full_size_roundtrip_property():
     # 1 GiB single tensor and the ~105 MiB many-tensor message at full size:
     # checked on the device (copy twice, compare), not against the CPU oracle.
