@@ -65,6 +65,9 @@ struct DeviceState {
 // and end, so their distance is the kernel's execution time.
 thread_local hipEvent_t tlsProfStart = nullptr;
 thread_local hipEvent_t tlsProfStop = nullptr;
+// Event to attach to the next copy-kernel launch of this thread as its
+// completion signal (instead of a marker of its own behind the kernel).
+thread_local hipEvent_t tlsSignal = nullptr;
 
 class ProfileScope {
  public:
@@ -246,6 +249,12 @@ int launchKernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, h
                            tlsProfStart, tlsProfStop, 0);
     tlsProfStart = nullptr;
     tlsProfStop = nullptr;
+  } else if (tlsSignal != nullptr) {
+    e = hipExtLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream,
+                           nullptr, tlsSignal, 0);
+    if (e == hipSuccess) {
+      tlsSignal = nullptr; // attached
+    }
   } else {
     e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream);
   }
@@ -453,12 +462,15 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     if (planViaKernel()) {
       const uint32_t nv = static_cast<uint32_t>(planBytesPadded / 16);
       const uint32_t sb = (nv + kBlockThreads - 1) / kBlockThreads;
+      hipEvent_t heldSignal = tlsSignal; // belongs to the copy kernel, not to this one
+      tlsSignal = nullptr;
       int src = launchKernel(stage_plan_kernel, dim3(sb < 8 ? sb : 8), dim3(kBlockThreads), 0,
                              stream, reinterpret_cast<const u32x4*>(hostDev),
                              reinterpret_cast<u32x4*>(devp), nv);
       if (src != 0) {
         return src;
       }
+      tlsSignal = heldSignal;
     } else {
       TPHIP_TRY(hipMemcpyAsync(devp, host, planBytesPadded, hipMemcpyHostToDevice, stream));
     }
@@ -500,12 +512,34 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
 }
 
 int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* streamPtr,
-                    int unroll, uint32_t blocks, int nt) {
+                    int unroll, uint32_t blocks, int nt, hipEvent_t signal = nullptr) {
+  if (table == nullptr && n != 0) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  if (signal != nullptr) {
+    // Validate before anything is enqueued, then make sure the event ends up
+    // behind whatever this call enqueues, on every path that succeeds.
+    if (n > TPHIP_MAX_BATCH ||
+        !(unroll == 0 || unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8) || dev < 0 ||
+        dev >= kMaxDevices) {
+      return batchedCopyImpl(dev, table, n, streamPtr, unroll, blocks, nt);
+    }
+    struct Disarm {
+      ~Disarm() {
+        tlsSignal = nullptr;
+      }
+    } disarm;
+    tlsSignal = signal;
+    int rc = batchedCopyImpl(dev, table, n, streamPtr, unroll, blocks, nt);
+    if (rc == 0 && tlsSignal != nullptr) {
+      // Nothing was launched, or the launch carried profiling events: a marker of its own.
+      TPHIP_ON_DEVICE(dev);
+      TPHIP_TRY(hipEventRecord(signal, static_cast<hipStream_t>(streamPtr)));
+    }
+    return rc;
+  }
   if (n == 0) {
     return 0;
-  }
-  if (table == nullptr) {
-    return TPHIP_ERR_INVALID_ARG;
   }
   if (n > TPHIP_MAX_BATCH) {
     return TPHIP_ERR_TOO_LARGE;
@@ -554,6 +588,10 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
   // Cut into launches whose body vector total fits the 32-bit prefix; entries
   // too large for that go through the single-entry kernel (64-bit counts).
   const uint64_t limit = gTableLimit.load(std::memory_order_relaxed);
+  // A completion event rides on the last launch of the call only.
+  hipEvent_t heldSignal = tlsSignal;
+  tlsSignal = nullptr;
+  bool armed = false;
   uint32_t begin = 0;
   uint64_t acc = 0;
   for (uint32_t i = 0; i <= m; ++i) {
@@ -561,6 +599,10 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
     const bool huge = i < m && vecs > limit;
     if (i == m || huge || acc + vecs > limit) {
       const uint32_t cnt = i - begin;
+      if (cnt >= 1 && i == m) {
+        tlsSignal = heldSignal;
+        armed = true;
+      }
       if (cnt == 1) {
         rc = copySingle(*st, cur[begin], stream, unroll, blocks, nt);
       } else if (cnt > 1) {
@@ -572,6 +614,10 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
       begin = i;
       acc = 0;
       if (huge) {
+        if (i + 1 == m) {
+          tlsSignal = heldSignal;
+          armed = true;
+        }
         rc = copySingle(*st, cur[i], stream, unroll, blocks, nt);
         if (rc != 0) {
           return rc;
@@ -581,6 +627,9 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
       }
     }
     acc += vecs;
+  }
+  if (!armed) {
+    tlsSignal = heldSignal; // not attached: the caller records it behind the copies
   }
   return 0;
 }
@@ -890,6 +939,15 @@ int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], 
 
 int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* stream) {
   return batchedCopyImpl(dev, table, n, stream, 0, 0, -1);
+}
+
+int tphip_batched_copy_signal(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
+                              void* event, int unroll, uint32_t blocks, int nontemporal) {
+  if (event == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  return batchedCopyImpl(dev, table, n, stream, unroll, blocks,
+                         nontemporal < 0 ? -1 : (nontemporal & 3), static_cast<hipEvent_t>(event));
 }
 
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {

@@ -543,11 +543,10 @@ class ChannelImpl final : public ChannelImplBase {
           ++it;
         }
       }
-      if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/true)) {
+      auto ev = bctx_->events.get(device);
+      if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/true, *ev)) {
         return;
       }
-      auto ev = bctx_->events.get(device);
-      ev->record(stream);
       watch(std::move(ev), [this, chunks{std::move(chunks)}] {
         for (auto& c : chunks) {
           c->ready = true;
@@ -599,37 +598,33 @@ class ChannelImpl final : public ChannelImplBase {
     return chosen;
   }
 
+  // `done` ends up behind the copy on `stream`.
   bool launchHostLinkCopy(
       int device,
       void* stream,
       const std::vector<tphip_copy_desc>& table,
-      bool towardsHost) {
+      bool towardsHost,
+      HipEvent& done) {
     const Engine how = engine();
-    if (how == Engine::kSdma || (how == Engine::kMixed && !towardsHost)) {
-      for (const auto& d : table) {
-        int rc = tphip_memcpy_async(device, d.dst, d.src, d.bytes, stream);
-        if (rc != 0) {
-          setError(TP_CREATE_ERROR(HipError, "tphip_memcpy_async", rc));
-          return false;
+    try {
+      if (how == Engine::kSdma || (how == Engine::kMixed && !towardsHost)) {
+        for (const auto& d : table) {
+          TP_HIP_CHECK(tphip_memcpy_async(device, d.dst, d.src, d.bytes, stream));
         }
+        done.record(stream);
+        return true;
       }
-      return true;
-    }
-    size_t off = 0;
-    while (off < table.size()) {
-      const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
       static const long forcedBlocks = [] {
         const char* e = std::getenv("TP_HIP_BASIC_BLOCKS");
         return e != nullptr ? std::atol(e) : 0L;
       }();
       const uint32_t blocks = forcedBlocks > 0 ? static_cast<uint32_t>(forcedBlocks) : 32;
-      int rc = tphip_batched_copy_tuned(
-          device, table.data() + off, static_cast<uint32_t>(n), stream, 4, blocks, 3);
-      if (rc != 0) {
-        setError(TP_CREATE_ERROR(HipError, "tphip_batched_copy", rc));
-        return false;
-      }
-      off += n;
+      // a marker behind the kernel: signalling from the kernel gains nothing measurable per chunk
+      hipBatchedCopy(device, stream, table, done, /*signalOnKernel=*/false, blocks, 3);
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " host-link copy failed: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "hip_basic copy", TPHIP_ERR_INVALID_ARG));
+      return false;
     }
     return true;
   }
@@ -783,13 +778,15 @@ class ChannelImpl final : public ChannelImplBase {
         setError(TP_CREATE_ERROR(HipError, "tphip_stream_create", TPHIP_ERR_INVALID_ARG));
         return;
       }
-      int rc = tphip_copy(0, rring.devAddress(local.get()), remote, len, stream);
-      if (rc != 0) {
-        setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+      auto ev = bctx_->events.get(0);
+      if (!launchHostLinkCopy(
+              0,
+              stream,
+              {tphip_copy_desc{remote, rring.devAddress(local.get()), len}},
+              /*towardsHost=*/true,
+              *ev)) {
         return;
       }
-      auto ev = bctx_->events.get(0);
-      ev->record(stream);
       watch(std::move(ev), [this, op, slot, offset, len, local] {
         if (error_) {
           return;
@@ -820,11 +817,10 @@ class ChannelImpl final : public ChannelImplBase {
           ++it;
         }
       }
-      if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/false)) {
+      auto ev = bctx_->events.get(device);
+      if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/false, *ev)) {
         return;
       }
-      auto ev = bctx_->events.get(device);
-      ev->record(stream);
       // The slots go back to the sender when the copy has read them.
       watch(std::move(ev), [this, slots{std::move(slots)}] { ackSlots(slots); });
       for (auto& op : ops) {
@@ -912,6 +908,7 @@ class ChannelImpl final : public ChannelImplBase {
     const HipBuffer hb = chunk->op->buffer.unwrap<HipBuffer>();
     PinnedRing& rring = bctx_->recvRing();
     const int device = hipDeviceForPointer(hb.ptr);
+    auto ev = bctx_->events.get(device);
     if (!launchHostLinkCopy(
             device,
             hb.stream,
@@ -919,11 +916,10 @@ class ChannelImpl final : public ChannelImplBase {
                 rring.devAddress(chunk->slot.get()),
                 static_cast<uint8_t*>(hb.ptr) + chunk->offset,
                 chunk->length}},
-            /*towardsHost=*/false)) {
+            /*towardsHost=*/false,
+            *ev)) {
       return;
     }
-    auto ev = bctx_->events.get(device);
-    ev->record(hb.stream);
     // The slot goes back to the ring when the copy has read it.
     watch(std::move(ev), [chunk] { chunk->slot.reset(); });
     chunkLanded(chunk->op);

@@ -1,5 +1,6 @@
 #include <tensorpipe/channel/hip_common.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cstdlib>
 #include <fstream>
@@ -224,6 +225,41 @@ void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>
     TP_HIP_CHECK(tphip_batched_copy(device, table.data() + off, static_cast<uint32_t>(n), stream));
     off += n;
   }
+}
+
+void hipBatchedCopy(
+    int device,
+    void* stream,
+    const std::vector<tphip_copy_desc>& table,
+    HipEvent& done,
+    bool signalOnKernel,
+    uint32_t blocks,
+    int nontemporal) {
+  static const bool onKernel = [] {
+    const char* e = std::getenv("TP_HIP_SIGNAL_ON_KERNEL");
+    return e == nullptr || std::atoi(e) != 0;
+  }();
+  const bool tuned = blocks != 0 || nontemporal >= 0;
+  if (!signalOnKernel || !onKernel || table.size() > TPHIP_MAX_BATCH || done.device() != device) {
+    size_t off = 0;
+    while (off < table.size()) {
+      const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
+      if (tuned) {
+        TP_HIP_CHECK(tphip_batched_copy_tuned(
+            device, table.data() + off, static_cast<uint32_t>(n), stream, 4, blocks,
+            nontemporal < 0 ? 3 : nontemporal));
+      } else {
+        TP_HIP_CHECK(
+            tphip_batched_copy(device, table.data() + off, static_cast<uint32_t>(n), stream));
+      }
+      off += n;
+    }
+    done.record(stream);
+    return;
+  }
+  TP_HIP_CHECK(tphip_batched_copy_signal(
+      device, table.data(), static_cast<uint32_t>(table.size()), stream, done.raw(),
+      tuned ? 4 : 0, blocks, nontemporal));
 }
 
 } // namespace channel

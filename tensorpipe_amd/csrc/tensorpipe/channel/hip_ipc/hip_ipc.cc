@@ -481,9 +481,18 @@ class ChannelImpl final : public ChannelImplBase {
         return;
       }
       const size_t slotIdx = outbox.allocator.slotIndex(slot.get());
-      int rc = tphip_copy(device, slot.get(), static_cast<const uint8_t*>(hb.ptr) + offset, len, hb.stream);
-      if (rc != 0) {
-        setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
+      std::unique_ptr<HipEvent> ev;
+      try {
+        ev = ictx_->events.get(device);
+        hipBatchedCopy(
+            device,
+            hb.stream,
+            {tphip_copy_desc{static_cast<const uint8_t*>(hb.ptr) + offset, slot.get(), len}},
+            *ev,
+            /*signalOnKernel=*/false);
+      } catch (const std::exception& ex) {
+        TP_LOG_WARNING() << "Channel " << id_ << " staging failed: " << ex.what();
+        setError(TP_CREATE_ERROR(HipError, "hip_ipc staging", TPHIP_ERR_INVALID_ARG));
         return;
       }
       WireWriter w;
@@ -505,8 +514,6 @@ class ChannelImpl final : public ChannelImplBase {
       w.u64(len);
       unit->bytes = std::move(w.bytes());
       unit->onReply = [slot]() mutable { slot.reset(); }; // reply frees the slot
-      auto ev = ictx_->events.get(device);
-      ev->record(hb.stream);
       watch(std::move(ev), [this, op, unit] {
         unit->ready = true;
         flushWire();
@@ -578,7 +585,7 @@ class ChannelImpl final : public ChannelImplBase {
                << op->seq << ")";
     auto reply = std::make_shared<ReplyUnit>();
     replyQueue_.push_back(reply);
-    std::vector<StreamRef> touched;
+    std::vector<std::unique_ptr<HipEvent>> launched; // one event per copy launch
     try {
       if (kind == kDirect) {
         const uint32_t n = r.u32();
@@ -638,8 +645,9 @@ class ChannelImpl final : public ChannelImplBase {
           ++op->unitsSeen;
         }
         for (auto& g : groups) {
-          hipBatchedCopy(g.dst.device, g.dst.stream, g.table);
-          touched.push_back(g.dst);
+          auto ev = ictx_->events.get(g.dst.device);
+          hipBatchedCopy(g.dst.device, g.dst.stream, g.table, *ev, /*signalOnKernel=*/false);
+          launched.push_back(std::move(ev));
         }
         op->unitsExpected += n;
       } else if (kind == kChunk) {
@@ -683,17 +691,17 @@ class ChannelImpl final : public ChannelImplBase {
           failProtocol();
           return;
         }
-        int rc = tphip_copy(
+        auto ev = ictx_->events.get(device);
+        hipBatchedCopy(
             device,
-            static_cast<uint8_t*>(hb.ptr) + offset,
-            static_cast<const uint8_t*>(it->second.ptr) + slotIdx * it->second.slotBytes,
-            len,
-            hb.stream);
-        if (rc != 0) {
-          setError(TP_CREATE_ERROR(HipError, "tphip_copy", rc));
-          return;
-        }
-        touched.push_back(StreamRef{hb.stream, device});
+            hb.stream,
+            {tphip_copy_desc{
+                static_cast<const uint8_t*>(it->second.ptr) + slotIdx * it->second.slotBytes,
+                static_cast<uint8_t*>(hb.ptr) + offset,
+                len}},
+            *ev,
+            /*signalOnKernel=*/false);
+        launched.push_back(std::move(ev));
         // A staged tensor counts as seen when its last chunk arrived.
         if (offset + len == op->entries[index].length) {
           ++op->unitsSeen;
@@ -713,10 +721,8 @@ class ChannelImpl final : public ChannelImplBase {
 
     TP_VLOG(6) << "Channel " << id_ << " enqueued the copies (#" << op->seq << ")";
     // Reply once the copies of this unit have finished.
-    auto remaining = std::make_shared<size_t>(touched.size());
-    for (auto& s : touched) {
-      auto ev = ictx_->events.get(s.device);
-      ev->record(s.stream);
+    auto remaining = std::make_shared<size_t>(launched.size());
+    for (auto& ev : launched) {
       watch(std::move(ev), [this, reply, remaining] {
         if (--*remaining == 0) {
           reply->ready = true;

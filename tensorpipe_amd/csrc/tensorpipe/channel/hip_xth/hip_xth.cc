@@ -282,10 +282,9 @@ class ChannelImpl final : public ChannelImplBase {
           }
         }
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
-        hipBatchedCopy(g.src.device, g.src.stream, g.table);
-        TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
         auto done = xctx_->events.get(g.src.device);
-        done->record(g.src.stream);
+        hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*signalOnKernel=*/true);
+        TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
         auto self = shared_from_this();
         // Counted per launch: if a later launch of this op fails, the error
         // path still waits for exactly the copies that are running.

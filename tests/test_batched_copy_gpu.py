@@ -192,6 +192,62 @@ def test_entry_larger_than_4GiB():
     assert bool((b[:7] == FILL).all()) and bool((b[7 + n:] == FILL).all())
 
 
+def test_copy_with_completion_event(oracle):
+    # tphip_batched_copy_signal: the event covers everything the call enqueued, whichever kernel
+    # (or none) the call ends with. The copies run on a non-blocking stream that nothing else waits
+    # for, so only the event orders the read-back after them.
+    import torch
+
+    lib = _native.tphip()
+    stream = ctypes.c_void_p()
+    _native.check(lib.tphip_stream_create(0, ctypes.byref(stream)))
+    event = ctypes.c_void_p()
+    _native.check(lib.tphip_event_create(0, 0, ctypes.byref(event)))
+    rng = np.random.default_rng(321)
+
+    def run(sizes, seed, tuned=(0, 0, -1), limit=0):
+        layout = _pack(sizes, lambda i: (i * 5) % 16, lambda i: (i * 9) % 16)
+        src_size = max([s + n for s, _, n in layout] + [0]) + 64
+        dst_size = max([d + n for _, d, n in layout] + [0]) + 64
+        host_src = datagen.uniform_u8(seed, src_size)
+        dev_src = torch.from_numpy(host_src).cuda()
+        dev_dst = torch.full((dst_size,), FILL, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        table, n = hip.make_table([(dev_src.data_ptr() + s, dev_dst.data_ptr() + d, k)
+                                   for s, d, k in layout])
+        _native.check(lib.tphip_test_set_table_limit(limit))
+        try:
+            _native.check(lib.tphip_batched_copy_signal(0, table, n, stream, event, *tuned))
+        finally:
+            _native.check(lib.tphip_test_set_table_limit(0))
+        _native.check(lib.tphip_event_sync(0, event))
+        done = ctypes.c_int(0)
+        _native.check(lib.tphip_event_query(0, event, ctypes.byref(done)))
+        assert done.value == 1
+        got = dev_dst.cpu().numpy()  # on torch's stream: ordered after the copies by the event alone
+        ref = np.full(dst_size, FILL, dtype=np.uint8)
+        oracle.xth_message([(host_src[s:], ref[d:], k) for s, d, k in layout])
+        assert (got == ref).all()
+
+    run([(96 << 20) + 5], 1)                                        # single-entry kernel
+    run([int(x) for x in rng.integers(1, 3 << 20, 30)], 2)          # plan in the kernel arguments
+    run([int(x) for x in rng.integers(1, 1 << 20, 200)], 3)         # plan ring: stage kernel + copy kernel
+    run([int(x) for x in rng.integers(1, 1 << 20, 200)], 4, tuned=(4, 32, 3))
+    run([], 5)                                                      # nothing to enqueue
+    run([0, 0, 0], 6)
+    run([int(x) for x in rng.integers(1, 200000, 50)] + [16 * 5000 + 16], 7, limit=5000)  # ends with a lone large entry
+    run([16 * 5000 + 16] + [int(x) for x in rng.integers(1, 60000, 50)], 8, limit=5000)   # several launches
+    # with launch profiling on, the event is recorded as a marker of its own
+    _native.check(lib.tphip_profile_start(0, 8))
+    run([(32 << 20) + 1], 9)
+    launches, ms, nbytes = ctypes.c_uint32(), ctypes.c_double(), ctypes.c_uint64()
+    _native.check(lib.tphip_profile_stop(0, ctypes.byref(launches), ctypes.byref(ms), ctypes.byref(nbytes)))
+    assert launches.value == 1 and nbytes.value == (32 << 20) + 1
+    assert lib.tphip_batched_copy_signal(0, None, 0, stream, None, 0, 0, -1) == -1
+    _native.check(lib.tphip_event_destroy(0, event))
+    _native.check(lib.tphip_stream_destroy(0, stream))
+
+
 def test_graph_capture_and_replay(oracle):
     # launches whose plan travels in the kernel arguments can be captured; every replay must copy
     # what the sources hold at that moment. Eager work and synchronisation between the replays.
