@@ -4,7 +4,9 @@
 #pragma once
 
 #include <array>
+#include <chrono>
 #include <condition_variable>
+#include <cstdlib>
 #include <atomic>
 #include <deque>
 #include <functional>
@@ -67,11 +69,6 @@ class HipEventPoller {
 
 using HandleBytes = std::array<uint8_t, TPHIP_IPC_HANDLE_BYTES>;
 
-// Allocations of other processes mapped into this one, keyed by device and
-// handle bytes. Mappings stay open for the life of the process: opening takes
-// about 0.2 ms, a handle may be shared by several channels, and the reference
-// keeps its opened handles until the context closes for the same reasons
-// (tensorpipe/channel/cuda_ipc/context_impl.cc:388-418).
 // Process-wide identifiers for things this process exports to peers (tensor
 // allocations, staging slabs, pinned rings). A peer keys its mapping on
 // (exporting process, identifier), never on the handle bytes: an address that
@@ -103,6 +100,50 @@ class HipIpcImports {
   using Key = std::tuple<int, std::string, uint64_t>;
   std::mutex mutex_;
   std::map<Key, Entry> entries_;
+};
+
+// "Is there anything pending on this stream?", asked only while asking is
+// cheap. hipStreamQuery answers in about 0.1 us when the last thing on the
+// stream was an event marker that has completed (a ping-pong through these
+// channels: the stream's last work was the channel's own copy and marker), and
+// lets a channel skip an event round trip of about 10 us. When the last thing
+// was a kernel -- finished or not -- the runtime has to enqueue a marker of
+// its own to find out: the call takes about 12 us and answers "busy" anyway.
+// A stream whose query turned out slow and said "busy" is therefore treated as
+// busy, without asking, for the next 63 calls. Use from one loop.
+class StreamIdleProbe {
+ public:
+  bool idle(int device, void* stream) {
+    State& st = states_[std::make_pair(device, stream)];
+    if (st.skip > 0) {
+      --st.skip;
+      return false;
+    }
+    const auto t0 = std::chrono::steady_clock::now();
+    int idle = 0;
+    const int rc = tphip_stream_query(device, stream, &idle);
+    const auto took = std::chrono::steady_clock::now() - t0;
+    const bool isIdle = rc == 0 && idle != 0;
+    if (!isIdle && took > std::chrono::microseconds(6)) {
+      st.skip = skipCount();
+    }
+    return isIdle;
+  }
+
+ private:
+  // TP_HIP_IDLE_PROBE_SKIP: calls answered "busy" without asking after a slow
+  // query (default 63; 0 asks every time).
+  static uint32_t skipCount() {
+    static const uint32_t v = [] {
+      const char* e = std::getenv("TP_HIP_IDLE_PROBE_SKIP");
+      return e != nullptr ? static_cast<uint32_t>(std::atoi(e)) : 63u;
+    }();
+    return v;
+  }
+  struct State {
+    uint32_t skip{0};
+  };
+  std::map<std::pair<int, void*>, State> states_;
 };
 
 // Enqueue one batched copy on (device, stream); throws on a failed launch.

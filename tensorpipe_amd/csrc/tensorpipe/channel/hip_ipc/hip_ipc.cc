@@ -176,6 +176,7 @@ class IpcContextCore final : public ContextCore {
  public:
   HipEventPool events;
   HipEventPoller poller;
+  StreamIdleProbe idleProbe; // loop only
   const bool forceOutbox{outboxForcedByEnv()};
   const size_t maxExportBytes{envSize("TP_HIP_IPC_MAX_EXPORT_BYTES", kDefaultMaxExportBytes)};
   // 16-byte multiples keep every slot vector-aligned.
@@ -415,8 +416,7 @@ class ChannelImpl final : public ChannelImplBase {
         // Streams with nothing pending need no event at all.
         std::vector<StreamRef> busy;
         for (auto& s : directStreams) {
-          int idle = 0;
-          if (tphip_stream_query(s.device, s.stream, &idle) != 0 || !idle) {
+          if (!ictx_->idleProbe.idle(s.device, s.stream)) {
             busy.push_back(s);
           }
         }

@@ -43,6 +43,7 @@ class XthContextCore final : public ContextCore {
  public:
   HipEventPool events;
   HipEventPoller poller;
+  StreamIdleProbe idleProbe; // loop only
   void joinImpl() override {
     poller.join();
   }
@@ -272,9 +273,7 @@ class ChannelImpl final : public ChannelImplBase {
         // The copy may only touch a destination once everything the receiver
         // enqueued before recv() on that buffer's stream is done.
         for (auto& d : g.dstStreams) {
-          int idle = 0;
-          TP_HIP_CHECK(tphip_stream_query(d.device, d.stream, &idle));
-          if (!idle) {
+          if (!xctx_->idleProbe.idle(d.device, d.stream)) {
             auto ev = xctx_->events.get(d.device);
             ev->record(d.stream);
             ev->wait(g.src.stream, g.src.device);
