@@ -232,7 +232,7 @@ void hipBatchedCopy(
     void* stream,
     const std::vector<tphip_copy_desc>& table,
     HipEvent& done,
-    bool signalOnKernel,
+    HipEventPool* markerPool,
     uint32_t blocks,
     int nontemporal) {
   static const bool onKernel = [] {
@@ -240,7 +240,7 @@ void hipBatchedCopy(
     return e == nullptr || std::atoi(e) != 0;
   }();
   const bool tuned = blocks != 0 || nontemporal >= 0;
-  if (!signalOnKernel || !onKernel || table.size() > TPHIP_MAX_BATCH || done.device() != device) {
+  if (markerPool == nullptr || !onKernel || table.size() > TPHIP_MAX_BATCH || done.device() != device) {
     size_t off = 0;
     while (off < table.size()) {
       const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
@@ -260,6 +260,9 @@ void hipBatchedCopy(
   TP_HIP_CHECK(tphip_batched_copy_signal(
       device, table.data(), static_cast<uint32_t>(table.size()), stream, done.raw(),
       tuned ? 4 : 0, blocks, nontemporal));
+  auto marker = markerPool->get(device);
+  marker->record(stream);
+  markerPool->put(std::move(marker)); // nobody waits for it; recording it again later is fine
 }
 
 } // namespace channel

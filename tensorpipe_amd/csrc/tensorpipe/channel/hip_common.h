@@ -149,22 +149,25 @@ class StreamIdleProbe {
 // Enqueue one batched copy on (device, stream); throws on a failed launch.
 void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table);
 
-// The same, and `done` is recorded behind the copy. With `signalOnKernel` the
+// The same, and `done` is recorded behind the copy. With a `markerPool` the
 // event is the completion signal of the copy kernel itself where possible: a
 // polling host sees it about 2.5 us sooner than a marker enqueued after the
-// kernel. The price: the runtime then does not know the stream is idle until
-// it is asked, and the next hipStreamQuery on that stream takes about 12 us
-// and answers "busy" once; channels that ask streams whether they are idle
-// (hip_ipc does, before announcing a tensor) record the marker instead.
-// TP_HIP_SIGNAL_ON_KERNEL=0 records the marker everywhere. `blocks` workgroups
-// (0 = the library's choice) and `nontemporal` mask (-1 = the library's
-// choice) as for tphip_batched_copy_tuned.
+// kernel. A marker (an event of the pool, recorded and handed straight back,
+// never polled) still follows the kernel: without one the runtime does not
+// know when the stream has drained, and the user's next hipStreamQuery or
+// hipStreamSynchronize on it would take 12-20 us instead of 0.1. The marker
+// completes about 4 us after the kernel's signal; until then the stream reads
+// as busy, which is why channels that ask a stream whether it is idle right
+// after their own copy (hip_ipc, before announcing a tensor) pass no pool and
+// poll the marker itself. TP_HIP_SIGNAL_ON_KERNEL=0 does that everywhere.
+// `blocks` workgroups (0 = the library's choice) and `nontemporal` mask (-1 =
+// the library's choice) as for tphip_batched_copy_tuned.
 void hipBatchedCopy(
     int device,
     void* stream,
     const std::vector<tphip_copy_desc>& table,
     HipEvent& done,
-    bool signalOnKernel,
+    HipEventPool* markerPool,
     uint32_t blocks = 0,
     int nontemporal = -1);
 

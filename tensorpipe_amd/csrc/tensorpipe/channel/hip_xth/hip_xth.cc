@@ -282,7 +282,7 @@ class ChannelImpl final : public ChannelImplBase {
         }
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
         auto done = xctx_->events.get(g.src.device);
-        hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*signalOnKernel=*/true);
+        hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*markerPool=*/&xctx_->events);
         TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
         auto self = shared_from_this();
         // Counted per launch: if a later launch of this op fails, the error
