@@ -192,6 +192,32 @@ def test_entry_larger_than_4GiB():
     assert bool((b[:7] == FILL).all()) and bool((b[7 + n:] == FILL).all())
 
 
+def test_random_tables_against_oracle(oracle):
+    # randomised tables (hypothesis, fixed seed): sizes over six orders of magnitude, every alignment,
+    # empty entries anywhere, random launch shapes; each compared byte for byte with the oracle
+    from hypothesis import given, settings, strategies as st, seed, HealthCheck
+
+    size = st.one_of(
+        st.integers(0, 48), st.integers(49, 5000), st.integers(5001, 300000),
+        st.integers(300001, 3 << 20))
+    entry = st.tuples(size, st.integers(0, 15), st.integers(0, 15))
+    shape = st.one_of(
+        st.none(),
+        st.tuples(st.sampled_from([1, 2, 4, 8]), st.sampled_from([0, 1, 3, 64, 500, 2048]),
+                  st.integers(0, 3)))
+
+    @seed(20240611)
+    @settings(max_examples=150, deadline=None, derandomize=True, database=None,
+              suppress_health_check=list(HealthCheck))
+    @given(st.lists(entry, min_size=0, max_size=150), shape, st.integers(0, 1 << 30))
+    def check(entries, tuned, data_seed):
+        sizes = [e[0] for e in entries]
+        layout = _pack(sizes, lambda i: entries[i][1], lambda i: entries[i][2], gap=1)
+        _run_case(oracle, layout, seed=data_seed, tuned=tuned)
+
+    check()
+
+
 def test_copy_with_completion_event(oracle):
     # tphip_batched_copy_signal: the event covers everything the call enqueued, whichever kernel
     # (or none) the call ends with. The copies run on a non-blocking stream that nothing else waits
