@@ -14,6 +14,8 @@
 // sources and targets on cpu:0 / the GPU in every combination, received into
 // freshly allocated buffers on the devices the test names; checked as
 // expectDescriptorAndStorageMatchMessage does (pipe_test.h:225-280).
+#include <thread>
+
 #include "support.h"
 
 using namespace tptest;
@@ -262,7 +264,9 @@ Shape shapeOf(uint32_t dir, uint32_t m) {
 // Writes `count` messages without waiting in between and reads `count`
 // messages of the opposite direction at the same time; every callback must
 // fire exactly once, in order, with the right bytes.
-void exchangeMany(Pipe& pipe, uint32_t myDir, uint32_t count) {
+// `lane` separates the contents of pipes that run side by side.
+void exchangeMany(Pipe& pipe, uint32_t myRole, uint32_t count, uint32_t lane = 0) {
+  const uint32_t myDir = myRole + 2 * lane;
   struct Outgoing {
     Storage storage;
     std::future<Error> done;
@@ -293,7 +297,7 @@ void exchangeMany(Pipe& pipe, uint32_t myDir, uint32_t count) {
     outs.push_back(std::move(o));
   }
 
-  const uint32_t theirDir = 1 - myDir;
+  const uint32_t theirDir = (1 - myRole) + 2 * lane;
   for (uint32_t m = 0; m < count; ++m) {
     Shape sh = shapeOf(theirDir, m);
     auto pd = std::make_shared<std::promise<std::pair<Error, Descriptor>>>();
@@ -504,6 +508,98 @@ std::vector<Case> makeCases() {
                      exchangeMany(*e->pipe, 1, 60);
                      ep.barrier();
                    }});
+
+  // Four pipes between the same two contexts, each exchanging messages of
+  // random shape both ways from a thread of its own: the channels of a context
+  // share its staging slots, pinned rings, mapped peer allocations and event
+  // poller.
+  cases.push_back(
+      {"SeveralPipesAtOnce",
+       [](Endpoint& ep) {
+         const uint32_t lanes = 4, count = 25;
+         PipeEnd e;
+         const std::string url = "shm://" + ep.freshAddr();
+         e.ctx = makeContext("server");
+         e.listener = e.ctx->listen({url});
+         ep.signalListening();
+         // Pipes are accepted in any order: the first message names the lane.
+         std::vector<std::shared_ptr<Pipe>> pipes(lanes);
+         for (uint32_t k = 0; k < lanes; ++k) {
+           auto p = std::make_shared<std::promise<std::pair<Error, std::shared_ptr<Pipe>>>>();
+           auto f = p->get_future();
+           e.listener->accept([p](const Error& err, std::shared_ptr<Pipe> pipe) {
+             p->set_value({err, std::move(pipe)});
+           });
+           auto r = waitFor(f, "accept");
+           if (r.first) {
+             throw Fatal("accept failed: " + r.first.what());
+           }
+           auto pd = std::make_shared<std::promise<std::pair<Error, Descriptor>>>();
+           auto fd = pd->get_future();
+           r.second->readDescriptor(
+               [pd](const Error& err, Descriptor d) { pd->set_value({err, std::move(d)}); });
+           auto rd = waitFor(fd, "lane announcement");
+           if (rd.first) {
+             throw Fatal("lane announcement failed: " + rd.first.what());
+           }
+           auto pr = std::make_shared<std::promise<Error>>();
+           auto fr = pr->get_future();
+           r.second->read(Allocation{}, [pr](const Error& err) { pr->set_value(err); });
+           EXPECT_OK(waitFor(fr, "read of the lane announcement"));
+           const uint32_t lane = static_cast<uint32_t>(std::stoul(rd.second.metadata));
+           if (lane >= lanes || pipes[lane]) {
+             throw Fatal("unexpected lane " + rd.second.metadata);
+           }
+           pipes[lane] = std::move(r.second);
+         }
+         std::vector<std::thread> threads;
+         for (uint32_t k = 0; k < lanes; ++k) {
+           threads.emplace_back([&pipes, k] {
+             try {
+               exchangeMany(*pipes[k], 0, count, k);
+             } catch (const std::exception& ex) {
+               failures().add("lane " + std::to_string(k) + ": " + ex.what());
+             }
+           });
+         }
+         for (auto& t : threads) {
+           t.join();
+         }
+         ep.barrier();
+         pipes.clear();
+       },
+       [](Endpoint& ep) {
+         const uint32_t lanes = 4, count = 25;
+         PipeEnd e;
+         const std::string url = "shm://" + ep.freshAddr();
+         e.ctx = makeContext("client");
+         ep.awaitListening();
+         std::vector<std::shared_ptr<Pipe>> pipes;
+         for (uint32_t k = 0; k < lanes; ++k) {
+           pipes.push_back(e.ctx->connect(url));
+           Message msg;
+           msg.metadata = std::to_string(k);
+           auto p = std::make_shared<std::promise<Error>>();
+           auto f = p->get_future();
+           pipes.back()->write(std::move(msg), [p](const Error& err) { p->set_value(err); });
+           EXPECT_OK(waitFor(f, "lane announcement"));
+         }
+         std::vector<std::thread> threads;
+         for (uint32_t k = 0; k < lanes; ++k) {
+           threads.emplace_back([&pipes, k] {
+             try {
+               exchangeMany(*pipes[k], 1, count, k);
+             } catch (const std::exception& ex) {
+               failures().add("lane " + std::to_string(k) + ": " + ex.what());
+             }
+           });
+         }
+         for (auto& t : threads) {
+           t.join();
+         }
+         ep.barrier();
+         pipes.clear();
+       }});
 
   // Writes that are still queued or in flight when the pipe is closed complete
   // with an error or with success, but every one of them completes, once.
