@@ -105,6 +105,13 @@ def bench_d2d(steps, warmup):
     assert torch.equal(src, dst), "received bytes differ from sent bytes after the profiled loop"
     assert launches == steps and kernel_bytes == steps * nbytes, (launches, kernel_bytes)
 
+    # two more uninstrumented passes of K steps: how much one pass varies on this box
+    repeats = [total_s / steps * 1e3]
+    for _ in range(2):
+        _, again_s = tp.bench_transfer(cpipe, spipe, st, rt, warmup=0, iters=steps)
+        repeats.append(again_s / steps * 1e3)
+    torch.cuda.synchronize()
+
     # practical ceiling: the runtime's own D2D copy of the same size, same timing method
     e0, e1 = hip.TimedEvent(), hip.TimedEvent()
     for _ in range(5):
@@ -125,6 +132,7 @@ def bench_d2d(steps, warmup):
         "ms_per_step": total_s / steps * 1e3,
         "step_p50_us": float(per_us[int(0.5 * len(per_us))]),
         "profiled_pass_ms_per_step": prof_total_s / steps * 1e3,
+        "ms_per_step_repeats": repeats,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
@@ -539,6 +547,8 @@ def main():
     extra = {
         "d2d_step_p50_us": d2d["step_p50_us"],
         "d2d_profiled_pass_ms_per_step": d2d["profiled_pass_ms_per_step"],
+        # the timed pass (= ms_per_step) and two more passes of the same K steps
+        "d2d_ms_per_step_repeats": d2d["ms_per_step_repeats"],
         "hipMemcpyAsync_d2d_us": d2d["hipMemcpyAsync_d2d_us"],
         "hipMemcpyAsync_d2d_hbm_GBps": d2d["hipMemcpyAsync_d2d_hbm_GBps"],
     }
