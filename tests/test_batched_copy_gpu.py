@@ -277,8 +277,12 @@ def test_copy_with_completion_event(oracle):
 def test_graph_capture_and_replay(oracle):
     # launches whose plan travels in the kernel arguments can be captured; every replay must copy
     # what the sources hold at that moment. Eager work and synchronisation between the replays.
+    import os
+
     import torch
 
+    if os.environ.get("TPHIP_INLINE_PLANS") == "0":
+        pytest.skip("plans in the kernel arguments are switched off: no table can be captured")
     lib = _native.tphip()
     rng = np.random.default_rng(77)
     sizes = [int(x) for x in rng.integers(1, 50000, 40)] + [0, 1, 15, 17, 1 << 20]
