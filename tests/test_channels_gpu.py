@@ -308,6 +308,16 @@ def basic_small_ring_peer():
     peer.close()
 
 
+@pytest.fixture(scope="module")
+def basic_mixed_ring_peer():
+    # the default ring on this side (16 x 1 MiB), 3 slots of 256 KiB + 48 B on the peer's: the two
+    # ends agree on the smaller slot as chunk size, and each ring keeps its own depth
+    peer = Peer("basic:0,hip_basic:10", env={"TP_HIP_BASIC_SLOT_BYTES": str((256 << 10) + 48),
+                                             "TP_HIP_BASIC_NUM_SLOTS": "3"})
+    yield peer
+    peer.close()
+
+
 def _ipc_cases(oracle, peer, slot, sizes):
     for k, n in enumerate(sizes):
         host = datagen.normal(datagen.SEED_BASE + 3 + k, max(n // 4, 1), "f32").view(np.uint8)
@@ -401,6 +411,12 @@ def test_basic_staged_small_ring(oracle, basic_small_ring_peer):
         [tp.make_tensor(s, target=(tp.HIP, 0)) for s in srcs], "gpu")
     for o, h in zip(outs, hosts):
         _check_echo(o, h, h.size)
+
+
+def test_basic_staged_mixed_geometries(oracle, basic_mixed_ring_peer):
+    chunk = (256 << 10) + 48
+    _staged_cases(oracle, basic_mixed_ring_peer, [1024, chunk, chunk + 1, (3 << 20) + 7, 0],
+                  slot=chunk, num_slots=3)
 
 
 def test_basic_cross_device_types(oracle, basic_peer):
