@@ -26,6 +26,8 @@ def echo_peer(url, channels, env, ready, errors):
             meta = d.metadata.decode()
             if meta == "quit":
                 break
+            if meta == "die":
+                os._exit(3)  # the process vanishes with the message half read
             places = meta.split(",") if meta else []
             bufs, tensors = [], []
             for i in range(d.num_tensors):

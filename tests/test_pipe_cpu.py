@@ -141,6 +141,51 @@ def test_context_close_fails_pipes(pair):
         cpipe.read_descriptor(timeout_ms=5000)
 
 
+def test_peer_process_dies_mid_message():
+    # the other process disappears (no close, no goodbye) after it has seen a descriptor and before
+    # it has read the tensor: what is pending here fails, later operations fail too, nothing hangs
+    import multiprocessing as mp
+
+    from tests import peer_process
+
+    ctx = tp.Context("main", channels="basic:0")
+    listener = ctx.listen()
+    spawn = mp.get_context("spawn")
+    ready, errors = spawn.Event(), spawn.Queue()
+    proc = spawn.Process(target=peer_process.echo_peer,
+                         args=(listener.url(), "basic:0", {}, ready, errors))
+    proc.start()
+    try:
+        assert ready.wait(120), "peer did not start"
+        pipe = listener.accept(60000)
+        a = np.arange(100000, dtype=np.uint8)
+        w = pipe.write([tp.make_tensor(a)], metadata="cpu")
+        d = pipe.read_descriptor(60000)
+        out = np.zeros(d.tensor_lengths[0], np.uint8)
+        pipe.read([tp.make_tensor(out)], []).wait(60000)
+        w.wait(60000)
+        assert (out == a).all()
+        big = np.zeros(8 << 20, np.uint8)  # larger than the transport's ring: cannot complete alone
+        w = pipe.write([tp.make_tensor(big)], metadata="die")
+        with pytest.raises(tp.PipeError) as failed:
+            pipe.read_descriptor(timeout_ms=20000)
+        assert "timed out" not in str(failed.value)  # an error was delivered, not a time-out
+        with pytest.raises(tp.PipeError) as failed:
+            w.wait(20000)
+        assert "timed out" not in str(failed.value)
+        with pytest.raises(tp.PipeError) as failed:
+            pipe.write([tp.make_tensor(a)], metadata="cpu").wait(20000)
+        assert "timed out" not in str(failed.value)
+        proc.join(30)
+        assert proc.exitcode == 3
+    finally:
+        if proc.is_alive():
+            proc.kill()
+        pipe.destroy()
+        listener.destroy()
+        ctx.destroy()
+
+
 def test_unknown_channel_and_missing_gpu():
     with pytest.raises(tp.PipeError):
         tp.Context("x", channels="nope:0")
