@@ -447,3 +447,52 @@ def test_basic_refuses_cpu_to_cpu():
         cpipe.write([tp.make_tensor(a, target=(tp.CPU, 0))]).wait()
     for o in (cpipe, spipe, listener, other, ctx):
         o.destroy()
+
+
+def test_contexts_come_and_go_without_leaking_device_memory():
+    # contexts with every HIP channel, pipes and transfers, created and destroyed over and over:
+    # device memory in use must not grow (staging slabs, events and mappings are given back)
+    import torch
+
+    def one_round(k, peer_rounds):
+        server = tp.Context("server", channels="basic:0,hip_xth:10,hip_ipc:11,hip_basic:12")
+        client = tp.Context("client", channels="basic:0,hip_xth:10,hip_ipc:11,hip_basic:12")
+        listener = server.listen()
+        cpipe = client.connect(listener.url())
+        spipe = listener.accept()
+        src = torch.full((1 << 20,), k % 251, dtype=torch.uint8, device="cuda")
+        dst = torch.zeros_like(src)
+        w = cpipe.write([tp.make_tensor(src, target=(tp.HIP, 0))])
+        spipe.read_descriptor()
+        spipe.read([tp.make_tensor(dst)]).wait()
+        w.wait()
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        for o in (cpipe, spipe, listener, client, server):
+            o.destroy()
+        if peer_rounds:
+            # a second process, every tensor through the staging slab of hip_ipc
+            env = {"TP_HIP_IPC_MODE": "outbox"}
+            os.environ.update(env)
+            try:
+                peer = Peer("basic:0,hip_ipc:11,hip_basic:10", env=env)
+            finally:
+                del os.environ["TP_HIP_IPC_MODE"]
+            host = datagen.uniform_u8(k, (3 << 20) + 1)
+            keep = _gpu(host)
+            outs, _ = peer.echo([tp.make_tensor(keep, target=(tp.HIP, 0))], "gpu")
+            _check_echo(outs[0], host, host.size)
+            outs, _ = peer.echo([tp.make_tensor(host, target=(tp.HIP, 0))], "gpu")  # hip_basic
+            _check_echo(outs[0], host, host.size)
+            peer.close()
+
+    one_round(0, True)  # first use creates what lives as long as the process (copy plan ring)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    free_before, _ = torch.cuda.mem_get_info()
+    for k in range(1, 25):
+        one_round(k, k % 8 == 0)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_before - free_after < (32 << 20), (free_before, free_after)

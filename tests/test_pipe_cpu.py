@@ -186,6 +186,33 @@ def test_peer_process_dies_mid_message():
         ctx.destroy()
 
 
+def test_contexts_come_and_go_without_leaking_descriptors_or_threads():
+    # every context brings a reactor thread, sockets, an epoll set and ring segments:
+    # all of it must be gone after destroy()
+    import os
+    import threading
+
+    def one_round(k):
+        server = tp.Context("server", channels="xth:5,basic:0")
+        client = tp.Context("client", channels="xth:5,basic:0")
+        listener = server.listen()
+        cpipe = client.connect(listener.url())
+        spipe = listener.accept()
+        outs, _ = _roundtrip(cpipe, spipe, [np.full(70000 + k, k % 251, np.uint8)])
+        assert (outs[0] == k % 251).all()
+        for o in (cpipe, spipe, listener, client, server):
+            o.destroy()
+
+    one_round(0)
+    fds_before = len(os.listdir("/proc/self/fd"))
+    threads_before = len(os.listdir("/proc/self/task"))
+    for k in range(1, 40):
+        one_round(k)
+    assert len(os.listdir("/proc/self/fd")) <= fds_before
+    assert len(os.listdir("/proc/self/task")) <= threads_before
+    assert threading.active_count() >= 1
+
+
 def test_unknown_channel_and_missing_gpu():
     with pytest.raises(tp.PipeError):
         tp.Context("x", channels="nope:0")
