@@ -1,5 +1,7 @@
 #include <tensorpipe/channel/hip_common.h>
 
+#include <tensorpipe/common/loop.h>
+
 #include <algorithm>
 #include <chrono>
 #include <cstdlib>
@@ -75,6 +77,7 @@ int pollGapNanos() {
 } // namespace
 
 void HipEventPoller::run() {
+  thisIsLibraryThread() = true;
   using Clock = std::chrono::steady_clock;
   std::deque<Item> active;
   auto lastBusy = Clock::now();

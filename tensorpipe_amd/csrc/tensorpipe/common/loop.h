@@ -2,11 +2,23 @@
 // inside one loop, so no per-object locks are needed.
 //
 //  OnDemandLoop : no thread of its own. defer() enqueues; if nobody is
-//                 draining the queue the caller drains it (and anything that
-//                 gets enqueued meanwhile) before returning. Keeps the send /
-//                 recv fast path on the calling thread, without a hop.
+//                 draining the queue the caller drains it before returning.
+//                 Keeps the send / recv fast path on the calling thread,
+//                 without a hop.
 //  ThreadLoop   : same queue, drained by a dedicated thread that sleeps on a
 //                 condition variable.
+//
+// Whose tasks a draining thread runs depends on whose thread it is. A thread
+// the library created (transport reactor, event poller, ThreadLoop) runs
+// whatever is queued, also what other threads add meanwhile. A thread of the
+// application that entered through send/recv/write/read runs only what it
+// queued itself: a completion that a library thread queues at that moment
+// would otherwise run the application's callback on the application's own
+// stack, inside the very call that started the operation -- and a caller that
+// holds a lock its callback also takes would deadlock (the reference checks
+// for exactly that: tensorpipe/test/channel/channel_test_cpu.cc:44-109). The
+// library thread instead waits the few microseconds until the application's
+// thread has left the loop and drains the queue itself.
 #pragma once
 
 #include <atomic>
@@ -22,28 +34,72 @@ TP_AMD_NAMESPACE_BEGIN
 
 using TTask = std::function<void()>;
 
+// Set once by every thread the library starts.
+inline bool& thisIsLibraryThread() {
+  static thread_local bool flag = false;
+  return flag;
+}
+
 class OnDemandLoop {
  public:
   void defer(TTask fn) {
+    const std::thread::id me = std::this_thread::get_id();
+    bool wait = false;
     {
       std::unique_lock<std::mutex> lock(mutex_);
-      queue_.push_back(std::move(fn));
+      queue_.push_back(Item{std::move(fn), me});
       if (draining_) {
-        return;
+        if (drainer_ == me || !guestDrainer_) {
+          return; // the draining thread will get to it
+        }
+        // An application thread is draining: it leaves our task alone.
+        ++waiters_;
+        wait = true;
+      } else {
+        draining_ = true;
+        drainer_ = me;
+        guestDrainer_ = !thisIsLibraryThread();
       }
-      draining_ = true;
     }
-    owner_.store(std::this_thread::get_id(), std::memory_order_relaxed);
+    if (wait) {
+      for (unsigned spins = 0;; ++spins) {
+        {
+          std::unique_lock<std::mutex> lock(mutex_);
+          if (!draining_) {
+            --waiters_;
+            draining_ = true;
+            drainer_ = me;
+            guestDrainer_ = !thisIsLibraryThread();
+            break;
+          }
+          if (!guestDrainer_) {
+            --waiters_;
+            return; // a library thread took over and will run it
+          }
+        }
+        if (spins < 2000) {
+#if defined(__x86_64__)
+          __builtin_ia32_pause();
+#endif
+        } else {
+          std::this_thread::yield();
+        }
+      }
+    }
+    owner_.store(me, std::memory_order_relaxed);
     for (;;) {
       TTask task;
       {
         std::unique_lock<std::mutex> lock(mutex_);
-        if (queue_.empty()) {
+        // A guest stops at the first task that is not its own when that task's
+        // owner is waiting to take over; with nobody waiting it carries on, so
+        // that no task is left behind.
+        if (queue_.empty() || (guestDrainer_ && queue_.front().from != me && waiters_ > 0)) {
           owner_.store(std::thread::id(), std::memory_order_relaxed);
           draining_ = false;
           return;
         }
-        task = std::move(queue_.front());
+        task = std::move(queue_.front().fn);
         queue_.pop_front();
       }
       task();
@@ -55,9 +111,16 @@ class OnDemandLoop {
   }
 
  private:
+  struct Item {
+    TTask fn;
+    std::thread::id from;
+  };
   std::mutex mutex_;
-  std::deque<TTask> queue_;
+  std::deque<Item> queue_;
   bool draining_{false};
+  bool guestDrainer_{false}; // the draining thread belongs to the application
+  std::thread::id drainer_;
+  unsigned waiters_{0}; // threads waiting for a guest drainer to leave
   std::atomic<std::thread::id> owner_{std::thread::id()};
 };
 
@@ -100,6 +163,7 @@ class ThreadLoop {
 
  private:
   void run() {
+    thisIsLibraryThread() = true;
     std::unique_lock<std::mutex> lock(mutex_);
     for (;;) {
       cv_.wait(lock, [this] { return stopping_ || !queue_.empty(); });

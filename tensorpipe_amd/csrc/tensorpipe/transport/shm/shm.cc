@@ -42,6 +42,7 @@
 #include <unistd.h>
 
 #include <tensorpipe/common/defs.h>
+#include <tensorpipe/common/loop.h>
 #include <tensorpipe/transport/connection.h>
 #include <tensorpipe/transport/error.h>
 #include <tensorpipe/transport/listener.h>
@@ -1116,6 +1117,7 @@ void ContextImpl::pollFds(int timeoutMs) {
 }
 
 void ContextImpl::run() {
+  thisIsLibraryThread() = true;
   using Clock = std::chrono::steady_clock;
   auto lastProgress = Clock::now();
   auto lastFdPoll = Clock::now();
