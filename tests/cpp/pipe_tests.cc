@@ -14,6 +14,7 @@
 // sources and targets on cpu:0 / the GPU in every combination, received into
 // freshly allocated buffers on the devices the test names; checked as
 // expectDescriptorAndStorageMatchMessage does (pipe_test.h:225-280).
+#include <algorithm>
 #include <thread>
 
 #include "support.h"
@@ -57,6 +58,17 @@ std::shared_ptr<Context> makeContext(const char* name) {
 
 std::vector<uint8_t> toBytes(const std::string& s) {
   return std::vector<uint8_t>(s.begin(), s.end());
+}
+
+// The same kind of buffer as `d`'s, `offset` bytes further into its memory.
+Buffer subBuffer(Data& d, size_t offset) {
+  Buffer whole = d.buffer();
+  if (whole.device().type == kCpuDeviceType) {
+    return CpuBuffer{static_cast<uint8_t*>(whole.unwrap<CpuBuffer>().ptr) + offset};
+  }
+  HipBuffer hb = whole.unwrap<HipBuffer>();
+  hb.ptr = static_cast<uint8_t*>(hb.ptr) + offset;
+  return hb;
 }
 
 // Owns the memory a Message refers to.
@@ -508,6 +520,81 @@ std::vector<Case> makeCases() {
                      exchangeMany(*e->pipe, 1, 60);
                      ep.barrier();
                    }});
+
+  // One message with more tensors than a copy table holds (4096): the channels
+  // cut it into several launches, the pipe into nothing. 5000 tensors of 1 to
+  // 200 bytes, carved at odd offsets out of one allocation on each side.
+  {
+    const uint32_t count = 5000;
+    auto lengthOf = [](uint32_t t) { return size_t(1 + (t * 37u) % 200u); };
+    auto layout = [lengthOf](std::vector<size_t>* offsets) {
+      size_t off = 3;
+      for (uint32_t t = 0; t < count; ++t) {
+        offsets->push_back(off);
+        off += lengthOf(t) + 1 + (t % 5);
+      }
+      return off;
+    };
+    cases.push_back(
+        {"FiveThousandTensorsInOneMessage",
+         [lengthOf, layout](Endpoint& ep) {
+           auto e = openPipe(ep);
+           std::vector<size_t> offsets;
+           const size_t total = layout(&offsets);
+           auto arena = makeData(gHaveGpu, patterned(0, 0, 0, total));
+           Message msg;
+           msg.metadata = "many";
+           for (uint32_t t = 0; t < count; ++t) {
+             Message::Tensor mt;
+             mt.buffer = subBuffer(*arena, offsets[t]);
+             mt.length = lengthOf(t);
+             msg.tensors.push_back(std::move(mt));
+           }
+           auto p = std::make_shared<std::promise<Error>>();
+           auto f = p->get_future();
+           e->pipe->write(std::move(msg), [p](const Error& err) { p->set_value(err); });
+           EXPECT_OK(waitFor(f, "write"));
+           ep.barrier();
+         },
+         [lengthOf, layout](Endpoint& ep) {
+           auto e = openPipe(ep);
+           std::vector<size_t> offsets;
+           const size_t total = layout(&offsets);
+           auto pd = std::make_shared<std::promise<std::pair<Error, Descriptor>>>();
+           auto fd = pd->get_future();
+           e->pipe->readDescriptor(
+               [pd](const Error& err, Descriptor d) { pd->set_value({err, std::move(d)}); });
+           auto rd = waitFor(fd, "readDescriptor");
+           EXPECT_OK(rd.first);
+           EXPECT_EQ(rd.second.tensors.size(), size_t(count));
+           if (rd.first || rd.second.tensors.size() != count) {
+             throw Fatal("unexpected descriptor");
+           }
+           auto arena = makeData(gHaveGpu, std::vector<uint8_t>(total, 0xEE));
+           Allocation a;
+           for (uint32_t t = 0; t < count; ++t) {
+             EXPECT_EQ(rd.second.tensors[t].length, lengthOf(t));
+             Allocation::Tensor at;
+             at.buffer = subBuffer(*arena, offsets[t]);
+             a.tensors.push_back(std::move(at));
+           }
+           auto pr = std::make_shared<std::promise<Error>>();
+           auto fr = pr->get_future();
+           e->pipe->read(std::move(a), [pr](const Error& err) { pr->set_value(err); });
+           EXPECT_OK(waitFor(fr, "read"));
+           // every tensor arrived, and the gaps between them are untouched
+           std::vector<uint8_t> want(total, 0xEE);
+           const std::vector<uint8_t> sent = patterned(0, 0, 0, total);
+           for (uint32_t t = 0; t < count; ++t) {
+             std::copy(sent.begin() + offsets[t], sent.begin() + offsets[t] + lengthOf(t),
+                       want.begin() + offsets[t]);
+           }
+           if (arena->bytes() != want) {
+             failures().add("received arena differs");
+           }
+           ep.barrier();
+         }});
+  }
 
   // Four pipes between the same two contexts, each exchanging messages of
   // random shape both ways from a thread of its own: the channels of a context
