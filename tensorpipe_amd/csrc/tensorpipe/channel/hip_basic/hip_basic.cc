@@ -200,6 +200,8 @@ class ChannelImpl final : public ChannelImplBase {
     if (exported) {
       w.u64(bctx_->sendRingId);
       w.raw(bctx_->sendRingHandle().data(), TPHIP_IPC_HANDLE_BYTES);
+      w.u64(reinterpret_cast<uint64_t>(bctx_->sendRing().slab.host()));
+      w.u64(bctx_->sendRing().slab.size());
     }
     writeMessage(*controlConnection_, std::move(w.bytes()));
     readControl();
@@ -362,11 +364,13 @@ class ChannelImpl final : public ChannelImplBase {
         const uint64_t ringId = r.u64();
         HandleBytes h;
         r.raw(h.data(), h.size());
+        const uint64_t ringBase = r.u64();
+        const uint64_t ringSize = r.u64();
         // Map the peer's send ring if it lives on this machine in another
         // process; otherwise its chunks come through the inner channel.
         if (r.ok() && bctx_->shareRing && boot == bootIdentity() && process != processIdentity()) {
           void* ptr = nullptr;
-          if (HipIpcImports::get().acquire(0, process, ringId, h, &ptr) == 0) {
+          if (HipIpcImports::get().acquire(0, process, ringId, h, ringBase, ringSize, &ptr) == 0) {
             remoteRingPeer_ = process;
             remoteRingId_ = ringId;
             remoteRing_ = static_cast<uint8_t*>(ptr);

@@ -165,6 +165,8 @@ int HipIpcImports::acquire(
     const std::string& peer,
     uint64_t id,
     const HandleBytes& handle,
+    uint64_t base,
+    uint64_t size,
     void** out) {
   std::lock_guard<std::mutex> lock(mutex_);
   const Key key{device, peer, id};
@@ -174,10 +176,12 @@ int HipIpcImports::acquire(
     *out = it->second.ptr;
     return 0;
   }
-  // Same handle bytes under another identifier: stale, unmap before mapping anew.
+  // The same address range of the same process under another identifier:
+  // stale, unmap before mapping anew.
   size_t staleClosed = 0;
   for (auto& kv : entries_) {
-    if (std::get<0>(kv.first) == device && kv.second.mapped && kv.second.handle == handle) {
+    if (std::get<0>(kv.first) == device && std::get<1>(kv.first) == peer && kv.second.mapped &&
+        kv.second.base < base + size && base < kv.second.base + kv.second.size) {
       int crc = tphip_ipc_mem_close(device, kv.second.ptr);
       TP_VLOG(5) << "IPC imports: unmapped stale " << std::get<1>(kv.first) << "#"
                  << std::get<2>(kv.first) << " (rc " << crc << ") for #" << id;
@@ -197,7 +201,8 @@ int HipIpcImports::acquire(
   TP_VLOG(5) << "IPC imports: mapped " << peer << "#" << id << " at " << ptr;
   Entry& e = entries_[key];
   e.ptr = ptr;
-  e.handle = handle;
+  e.base = base;
+  e.size = size;
   e.mapped = true;
   ++e.refs;
   *out = ptr;

@@ -83,17 +83,28 @@ class HipIpcImports {
  public:
   static HipIpcImports& get();
   // `peer` is the exporter's processIdentity(), `id` its nextExportId() value
-  // for the allocation, `handle` what tphip_ipc_mem_export gave it. Returns a
-  // tphip error code. An older mapping with the same handle bytes belongs to
-  // memory the exporter has freed since (two live allocations never share a
-  // handle) and is unmapped first.
-  int acquire(int device, const std::string& peer, uint64_t id, const HandleBytes& handle, void** out);
+  // for the allocation, `handle` what tphip_ipc_mem_export gave it, `base` and
+  // `size` the allocation's address range in the exporter. Returns a tphip
+  // error code. An older mapping from the same process whose range overlaps
+  // the new one belongs to memory the exporter has freed since (two live
+  // allocations of a process never overlap) and is unmapped first; the handle
+  // bytes themselves cannot tell, their tail differs from one export of the
+  // same allocation to the next.
+  int acquire(
+      int device,
+      const std::string& peer,
+      uint64_t id,
+      const HandleBytes& handle,
+      uint64_t base,
+      uint64_t size,
+      void** out);
   void release(int device, const std::string& peer, uint64_t id);
 
  private:
   struct Entry {
     void* ptr{nullptr};
-    HandleBytes handle;
+    uint64_t base{0};
+    uint64_t size{0};
     size_t refs{0};
     bool mapped{false};
   };

@@ -89,6 +89,7 @@ constexpr size_t kDefaultMaxExportBytes = size_t(2) << 30;
 struct ExportedAllocation {
   uint64_t id;
   HandleBytes handle;
+  uint64_t base;
   size_t size;
   uint64_t bufferId;
 };
@@ -148,6 +149,7 @@ class ExportRegistry {
       return false;
     }
     e.id = nextExportId();
+    e.base = reinterpret_cast<uint64_t>(base);
     e.size = size;
     e.bufferId = bufferId;
     exports_[base] = e;
@@ -402,6 +404,8 @@ class ChannelImpl final : public ChannelImplBase {
           if (announce) {
             w.str(processIdentity());
             w.raw(d.alloc.handle.data(), d.alloc.handle.size());
+            w.u64(d.alloc.base);
+            w.u64(d.alloc.size);
           }
           w.u64(d.offset);
           w.u64(d.length);
@@ -508,6 +512,8 @@ class ChannelImpl final : public ChannelImplBase {
         w.u64(ictx_->slotBytes);
         w.u32(static_cast<uint32_t>(ictx_->numSlots));
         w.raw(outbox.handle.data(), outbox.handle.size());
+        w.u64(reinterpret_cast<uint64_t>(outbox.slab.ptr()));
+        w.u64(outbox.slab.size());
       }
       w.u32(static_cast<uint32_t>(slotIdx));
       w.u64(offset);
@@ -609,12 +615,15 @@ class ChannelImpl final : public ChannelImplBase {
             const std::string peer = r.str();
             HandleBytes h;
             r.raw(h.data(), h.size());
+            const uint64_t remoteBase = r.u64();
+            const uint64_t remoteSize = r.u64();
             if (!r.ok() || remoteAllocations_.count(exportId) != 0) {
               failProtocol();
               return;
             }
             void* mapped = nullptr;
-            int rc = HipIpcImports::get().acquire(device, peer, exportId, h, &mapped);
+            int rc = HipIpcImports::get().acquire(
+                device, peer, exportId, h, remoteBase, remoteSize, &mapped);
             if (rc != 0) {
               setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
               return;
@@ -668,13 +677,16 @@ class ChannelImpl final : public ChannelImplBase {
           const uint32_t remoteNumSlots = r.u32();
           HandleBytes h;
           r.raw(h.data(), h.size());
+          const uint64_t remoteBase = r.u64();
+          const uint64_t remoteSize = r.u64();
           if (!r.ok() || remoteOutboxes_.count(srcDevice) != 0 || remoteSlotBytes == 0 ||
               remoteNumSlots == 0 || remoteNumSlots > kMaxNumSlots) {
             failProtocol();
             return;
           }
           void* mapped = nullptr;
-          int rc = HipIpcImports::get().acquire(device, peer, outboxId, h, &mapped);
+          int rc = HipIpcImports::get().acquire(
+              device, peer, outboxId, h, remoteBase, remoteSize, &mapped);
           if (rc != 0) {
             setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
             return;

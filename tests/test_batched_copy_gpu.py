@@ -192,6 +192,43 @@ def test_entry_larger_than_4GiB():
     assert bool((b[:7] == FILL).all()) and bool((b[7 + n:] == FILL).all())
 
 
+def test_stream_completion_callback():
+    # tphip_stream_on_complete (the role of CudaLoop::addCallback, tensorpipe/common/cuda_loop.cc:86-124):
+    # the function runs once, with status 0, after the work enqueued before it -- here a 64 MiB copy
+    # behind a fill -- and the copied bytes are complete by then
+    import threading
+
+    import torch
+
+    lib = _native.tphip()
+    host_fn = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_int)
+    lib.tphip_stream_on_complete.argtypes = [ctypes.c_int, ctypes.c_void_p, host_fn, ctypes.c_void_p]
+    stream = ctypes.c_void_p()
+    _native.check(lib.tphip_stream_create(0, ctypes.byref(stream)))
+    n = 64 << 20
+    src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    calls, fired = [], threading.Event()
+
+    def on_done(arg, status):
+        calls.append((arg, status))
+        fired.set()
+
+    keep = host_fn(on_done)  # must outlive the call
+    _native.check(lib.tphip_fill(0, src.data_ptr(), 0x5A, n, stream))
+    _native.check(lib.tphip_copy(0, dst.data_ptr(), src.data_ptr(), n, stream))
+    _native.check(lib.tphip_stream_on_complete(0, stream, keep, ctypes.c_void_p(1234)))
+    assert fired.wait(30), "completion callback did not run"
+    # read back on torch's stream: only the callback orders this after the copy
+    got = dst.cpu()
+    assert bool((got == 0x5A).all())
+    assert calls == [(1234, 0)]
+    assert lib.tphip_stream_on_complete(0, stream, host_fn(), None) == -1  # null function
+    _native.check(lib.tphip_stream_sync(0, stream))
+    _native.check(lib.tphip_stream_destroy(0, stream))
+
+
 def test_random_tables_against_oracle(oracle):
     # randomised tables (hypothesis, fixed seed): sizes over six orders of magnitude, every alignment,
     # empty entries anywhere, random launch shapes; each compared byte for byte with the oracle
