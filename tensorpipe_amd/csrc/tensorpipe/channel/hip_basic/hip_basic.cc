@@ -368,7 +368,9 @@ class ChannelImpl final : public ChannelImplBase {
         const uint64_t ringSize = r.u64();
         // Map the peer's send ring if it lives on this machine in another
         // process; otherwise its chunks come through the inner channel.
-        if (r.ok() && bctx_->shareRing && boot == bootIdentity() && process != processIdentity()) {
+        // (a ring smaller than the geometry it was announced with is not mapped)
+        if (r.ok() && bctx_->shareRing && boot == bootIdentity() && process != processIdentity() &&
+            remoteSlots != 0 && remoteSlot <= ringSize / remoteSlots) {
           void* ptr = nullptr;
           if (HipIpcImports::get().acquire(0, process, ringId, h, ringBase, ringSize, &ptr) == 0) {
             remoteRingPeer_ = process;

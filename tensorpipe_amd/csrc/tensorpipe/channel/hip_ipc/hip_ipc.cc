@@ -628,13 +628,16 @@ class ChannelImpl final : public ChannelImplBase {
               setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
               return;
             }
-            remoteAllocations_[exportId] = mapped;
+            remoteAllocations_[exportId] = RemoteAllocation{mapped, remoteSize};
             imports_.push_back(Import{device, peer, exportId});
           }
           const uint64_t offset = r.u64();
           const uint64_t length = r.u64();
           auto it = remoteAllocations_.find(exportId);
-          if (!r.ok() || it == remoteAllocations_.end() || length != op->entries[index].length) {
+          // The range must lie inside the allocation the peer announced: the
+          // copy kernel would fault on anything else.
+          if (!r.ok() || it == remoteAllocations_.end() || length != op->entries[index].length ||
+              offset > it->second.size || length > it->second.size - offset) {
             failProtocol();
             return;
           }
@@ -650,7 +653,7 @@ class ChannelImpl final : public ChannelImplBase {
             g = &groups.back();
           }
           g->table.push_back(
-              tphip_copy_desc{static_cast<const uint8_t*>(it->second) + offset, hb.ptr, length});
+              tphip_copy_desc{static_cast<const uint8_t*>(it->second.ptr) + offset, hb.ptr, length});
           ++op->unitsSeen;
         }
         for (auto& g : groups) {
@@ -680,7 +683,8 @@ class ChannelImpl final : public ChannelImplBase {
           const uint64_t remoteBase = r.u64();
           const uint64_t remoteSize = r.u64();
           if (!r.ok() || remoteOutboxes_.count(srcDevice) != 0 || remoteSlotBytes == 0 ||
-              remoteNumSlots == 0 || remoteNumSlots > kMaxNumSlots) {
+              remoteNumSlots == 0 || remoteNumSlots > kMaxNumSlots ||
+              remoteSlotBytes > remoteSize / remoteNumSlots) {
             failProtocol();
             return;
           }
@@ -826,7 +830,11 @@ class ChannelImpl final : public ChannelImplBase {
   std::deque<std::shared_ptr<ReplyUnit>> replyQueue_;
   std::set<uint64_t> announced_;
   std::map<int, bool> outboxAnnounced_;
-  std::map<uint64_t, void*> remoteAllocations_;
+  struct RemoteAllocation {
+    void* ptr;
+    uint64_t size;
+  };
+  std::map<uint64_t, RemoteAllocation> remoteAllocations_;
   struct RemoteOutbox {
     void* ptr;
     uint64_t slotBytes;
