@@ -39,7 +39,7 @@ def main():
     lib = os.path.join(out, "libtensorpipe_amd.so")
     subprocess.run(["g++", "-shared", f"-fsanitize={san}", "-pthread", "-o", lib, *objs, f"-L{tp_build.LIB}",
                     "-ltphip", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
-    for prog in sorted({p for p, _ in SUITES}):
+    for prog in sorted({p for p, _ in SUITES} | {"unit_tests"}):
         subprocess.run(["g++", *flags, os.path.join(ROOT, "tests", "cpp", prog + ".cc"), "-o",
                         os.path.join(out, prog), f"-L{out}", "-ltensorpipe_amd", f"-L{tp_build.LIB}", "-ltphip",
                         f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
@@ -54,6 +54,16 @@ def main():
         for l in failed + reports[:5]:
             print("   ", l[:200])
         bad += len(failed) + len(reports) + (0 if results else 1)
+    # random bytes where a pipe's first packets belong
+    for seed in (11, 12, 13):
+        proc = subprocess.run([os.path.join(out, "unit_tests"), "garbage", str(seed), "150"],
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+        reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+        ok = proc.returncode == 0 and proc.stdout.strip().endswith("OK")
+        print(f"unit_tests garbage {seed}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
+        for l in reports[:5]:
+            print("   ", l[:200])
+        bad += (0 if ok else 1) + len(reports)
     sys.exit(1 if bad else 0)
 
 

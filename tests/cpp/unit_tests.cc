@@ -7,12 +7,22 @@
 //       can compare with the golden trace (tensorpipe/common/allocator.cc:26-79).
 //   unit_tests basics
 //       Buffer / Device / Error / wire helpers; prints "OK" or the failures.
+//   unit_tests garbage <seed> <connections>
+//       opens raw transport connections to a listening context and writes
+//       random bytes where a pipe's first packets belong; the context must
+//       survive all of them and still serve a proper pipe afterwards.
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <future>
 #include <map>
+#include <random>
 #include <string>
+#include <thread>
 #include <vector>
+
+#include <unistd.h>
 
 #include <tensorpipe/common/buffer.h>
 #include <tensorpipe/common/cpu_buffer.h>
@@ -22,7 +32,9 @@
 #include <tensorpipe/common/slot_allocator.h>
 #include <tensorpipe/common/wire.h>
 #include <tensorpipe/channel/error.h>
+#include <tensorpipe/tensorpipe.h>
 #include <tensorpipe/tensorpipe_cuda.h>
+#include <tensorpipe/transport/connection.h>
 
 using namespace tensorpipe;
 
@@ -160,13 +172,126 @@ static int runBasics() {
   return failed == 0 ? 0 : 1;
 }
 
+// Random bytes where the first packets of a pipe belong.
+static int runGarbage(int argc, char** argv) {
+  const unsigned seed = static_cast<unsigned>(std::strtoul(argv[2], nullptr, 10));
+  const int connections = std::atoi(argv[3]);
+  std::mt19937 rng(seed);
+  auto server = std::make_shared<Context>(ContextOptions().name("server"));
+  server->registerTransport(1, "shm", transport::shm::create());
+  server->registerChannel(1, "basic", channel::basic::create());
+  const std::string addr = "tp_unit_garbage_" + std::to_string(::getpid()) + "_" + std::to_string(seed);
+  auto listener = server->listen({"shm://" + addr});
+  auto rawTransport = transport::shm::create();
+  std::vector<std::shared_ptr<transport::Connection>> keep;
+  for (int c = 0; c < connections; ++c) {
+    auto conn = rawTransport->connect(addr);
+    const int messages = 1 + static_cast<int>(rng() % 4);
+    for (int m = 0; m < messages; ++m) {
+      auto bytes = std::make_shared<std::vector<uint8_t>>(rng() % 300);
+      for (auto& b : *bytes) {
+        b = static_cast<uint8_t>(rng());
+      }
+      if (!bytes->empty() && rng() % 2 == 0) {
+        (*bytes)[0] = static_cast<uint8_t>(1 + rng() % 2); // looks like a hello of either kind
+      }
+      conn->write(bytes->data(), bytes->size(), [bytes](const Error&) {});
+    }
+    if (rng() % 3 == 0) {
+      conn->close();
+    } else {
+      keep.push_back(std::move(conn));
+    }
+  }
+  // Pipes the garbage may have created are accepted and dropped; then a proper one.
+  auto client = std::make_shared<Context>(ContextOptions().name("client"));
+  client->registerTransport(1, "shm", transport::shm::create());
+  client->registerChannel(1, "basic", channel::basic::create());
+  auto pipe = client->connect("shm://" + addr);
+  std::vector<uint8_t> data(100000);
+  for (size_t i = 0; i < data.size(); ++i) {
+    data[i] = static_cast<uint8_t>(i * 7);
+  }
+  Message msg;
+  msg.metadata = "proper";
+  Message::Tensor t;
+  t.buffer = CpuBuffer{data.data()};
+  t.length = data.size();
+  msg.tensors.push_back(std::move(t));
+  auto written = std::make_shared<std::promise<Error>>();
+  auto fWritten = written->get_future();
+  pipe->write(std::move(msg), [written](const Error& e) { written->set_value(e); });
+
+  std::vector<uint8_t> got(data.size());
+  auto done = std::make_shared<std::promise<std::string>>();
+  auto fDone = done->get_future();
+  auto fulfilled = std::make_shared<std::atomic<bool>>(false);
+  std::function<void()> acceptNext;
+  std::vector<std::shared_ptr<Pipe>> accepted;
+  acceptNext = [&] {
+    listener->accept([&](const Error& e, std::shared_ptr<Pipe> p) {
+      if (e) {
+        if (!fulfilled->exchange(true)) {
+          done->set_value("accept failed: " + e.what());
+        }
+        return;
+      }
+      accepted.push_back(p);
+      p->readDescriptor([&, p](const Error& e2, Descriptor d) {
+        if (e2 || d.metadata != "proper") {
+          return; // one of the garbage pipes: it fails or never speaks; ignore it
+        }
+        Allocation a;
+        Allocation::Tensor at;
+        at.buffer = CpuBuffer{got.data()};
+        a.tensors.push_back(std::move(at));
+        p->read(std::move(a), [&](const Error& e3) {
+          if (!fulfilled->exchange(true)) {
+            done->set_value(e3 ? "read failed: " + e3.what() : std::string());
+          }
+        });
+      });
+      acceptNext();
+    });
+  };
+  acceptNext();
+  int rc = 0;
+  if (fDone.wait_for(std::chrono::seconds(30)) != std::future_status::ready) {
+    std::printf("the proper pipe did not get through\n");
+    rc = 1;
+  } else {
+    const std::string problem = fDone.get();
+    if (!problem.empty() || got != data) {
+      std::printf("proper pipe: %s\n", problem.empty() ? "bytes differ" : problem.c_str());
+      rc = 1;
+    }
+  }
+  if (rc == 0 && (fWritten.wait_for(std::chrono::seconds(30)) != std::future_status::ready || fWritten.get())) {
+    std::printf("the proper write did not complete\n");
+    rc = 1;
+  }
+  keep.clear();
+  pipe.reset();
+  accepted.clear();
+  listener.reset();
+  client->join();
+  server->join();
+  if (rc == 0) {
+    std::printf("OK\n");
+  }
+  return rc;
+}
+
 int main(int argc, char** argv) {
+  if (argc == 4 && std::strcmp(argv[1], "garbage") == 0) {
+    return runGarbage(argc, argv);
+  }
   if (argc >= 3 && std::strcmp(argv[1], "allocator") == 0) {
     return runAllocator(argc, argv);
   }
   if (argc == 2 && std::strcmp(argv[1], "basics") == 0) {
     return runBasics();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics\n", argv[0]);
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | garbage <seed> <n>\n", argv[0]);
   return 2;
 }

@@ -58,3 +58,11 @@ def test_slot_allocator_matches_the_oracle(oracle):
 def test_basics():
     rc, out = run("basics")
     assert rc == 0 and out.strip() == "OK", out
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_garbage_on_new_connections(seed):
+    # random bytes where the first packets of a pipe belong: the listening context survives them
+    # and still serves a proper pipe
+    out = subprocess.run([BIN, "garbage", str(seed), "100"], stdout=subprocess.PIPE, text=True, timeout=120)
+    assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
