@@ -478,6 +478,7 @@ def cpu_baseline():
         "config1_payload_GBps": main_["config1_payload_GBps"],
         "rtt_4KiB_p50_us": main_["rtt_4KiB_p50_us"],
         "host_cpus": os.cpu_count(),
+        "affinity_cpus": sorted(os.sched_getaffinity(0)),
         "reference": ref, "port": port,
     }
 
