@@ -213,6 +213,25 @@ def test_contexts_come_and_go_without_leaking_descriptors_or_threads():
     assert threading.active_count() >= 1
 
 
+def test_idle_contexts_do_not_spin(pair):
+    # the reactor threads busy-poll only while traffic flows (a 200 us window); an open, idle pipe
+    # costs no CPU
+    import resource
+    import time
+
+    cpipe, spipe = pair()
+    _roundtrip(cpipe, spipe, [np.arange(1000, dtype=np.uint8)])
+    time.sleep(0.2)
+    before = resource.getrusage(resource.RUSAGE_SELF)
+    time.sleep(1.0)
+    after = resource.getrusage(resource.RUSAGE_SELF)
+    used = (after.ru_utime - before.ru_utime) + (after.ru_stime - before.ru_stime)
+    assert used < 0.2, f"{used:.3f} CPU seconds in one idle second"
+    # and it still works afterwards (the threads wake up)
+    outs, _ = _roundtrip(cpipe, spipe, [np.arange(77, dtype=np.uint8)])
+    assert (outs[0] == np.arange(77, dtype=np.uint8)).all()
+
+
 def test_unknown_channel_and_missing_gpu():
     with pytest.raises(tp.PipeError):
         tp.Context("x", channels="nope:0")
