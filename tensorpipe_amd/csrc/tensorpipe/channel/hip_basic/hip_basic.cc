@@ -56,7 +56,8 @@ namespace {
 size_t slotBytesFromEnv() {
   const char* e = std::getenv("TP_HIP_BASIC_SLOT_BYTES");
   size_t b = e != nullptr ? std::strtoull(e, nullptr, 10) : (1u << 20);
-  return b < 4096 ? size_t(4096) : b;
+  b = b < 4096 ? size_t(4096) : b;
+  return b > (size_t(1) << 30) ? (size_t(1) << 30) : b; // see numSlots below
 }
 
 size_t numSlotsFromEnv() {
@@ -86,7 +87,10 @@ class BasicContextCore final : public ContextCore {
   HipEventPool events;
   HipEventPoller poller;
   const size_t slotBytes{slotBytesFromEnv()};
-  const size_t numSlots{numSlotsFromEnv()};
+  // A ring is mapped by the peer: the whole of it stays below 2 GiB (larger
+  // mappings in a second process have been seen never to return).
+  const size_t numSlots{std::max<size_t>(
+      1, std::min<size_t>(numSlotsFromEnv(), ((size_t(2) << 30) - 1) / slotBytesFromEnv()))};
   const bool shareRing{!ringSharingDisabled()};
 
   // Loop only. The send ring exists from the first channel on (its handle is

@@ -182,8 +182,16 @@ class IpcContextCore final : public ContextCore {
   const bool forceOutbox{outboxForcedByEnv()};
   const size_t maxExportBytes{envSize("TP_HIP_IPC_MAX_EXPORT_BYTES", kDefaultMaxExportBytes)};
   // 16-byte multiples keep every slot vector-aligned.
-  const size_t slotBytes{(envSize("TP_HIP_IPC_SLOT_BYTES", kDefaultSlotBytes) + 15) / 16 * 16};
-  const size_t numSlots{std::min(envSize("TP_HIP_IPC_NUM_SLOTS", kDefaultNumSlots), kMaxNumSlots)};
+  const size_t slotBytes{
+      (std::min<size_t>(envSize("TP_HIP_IPC_SLOT_BYTES", kDefaultSlotBytes), size_t(1) << 30) + 15) / 16 *
+      16};
+  // The slab is mapped by the peer: the whole of it stays below 2 GiB, like
+  // everything else this channel lets a peer map.
+  const size_t numSlots{std::max<size_t>(
+      1,
+      std::min(
+          std::min(envSize("TP_HIP_IPC_NUM_SLOTS", kDefaultNumSlots), kMaxNumSlots),
+          ((size_t(2) << 30) - 1) / slotBytes))};
 
   // Loop only.
   Outbox& outbox(int device) {
