@@ -4,10 +4,15 @@
 //
 //  direct  The sender exports the allocation that contains the tensor
 //          (hipIpcGetMemHandle on its base, cached per allocation) and sends
-//          {export id, handle the first time, offset, length}. The receiver
+//          {export id, handle, address range} of every allocation a message
+//          touches, then {allocation, offset, length} per tensor. The receiver
 //          maps the allocation (cached) and its batched copy kernel reads the
 //          sender's memory directly: one read and one write per payload byte,
-//          all tensors of a message in one launch.
+//          all tensors of a message in one launch. Because every message
+//          carries the handles it needs, the receiver may drop a mapping
+//          whenever no copy reads from it: it keeps the most recently used
+//          ones up to TP_HIP_IPC_MAX_MAPPED_BYTES (a mapping keeps the memory
+//          alive after the sender has freed it).
 //  outbox  What the reference does for every transfer
 //          (tensorpipe/channel/cuda_ipc/channel_impl.cc:107-136,238-252,
 //          431-467, context_impl.cc:173-195,341-418): the tensor is cut into
@@ -83,6 +88,11 @@ bool outboxForcedByEnv() {
 // seen never to return on the deployment this was built for. Settable per
 // context (TP_HIP_IPC_MAX_EXPORT_BYTES) where larger mappings are known to work.
 constexpr size_t kDefaultMaxExportBytes = size_t(2) << 30;
+
+// Peer allocations a channel keeps mapped: least recently used ones go once
+// their sizes add up to more than this, or there are more than this many.
+constexpr size_t kDefaultMaxMappedBytes = size_t(64) << 30;
+constexpr size_t kMaxMappedAllocations = 1024;
 
 // Allocations this process has exported, keyed by base address. Process-wide:
 // a handle describes an allocation, not a context.
@@ -181,6 +191,7 @@ class IpcContextCore final : public ContextCore {
   StreamIdleProbe idleProbe; // loop only
   const bool forceOutbox{outboxForcedByEnv()};
   const size_t maxExportBytes{envSize("TP_HIP_IPC_MAX_EXPORT_BYTES", kDefaultMaxExportBytes)};
+  const size_t maxMappedBytes{envSize("TP_HIP_IPC_MAX_MAPPED_BYTES", kDefaultMaxMappedBytes)};
   // 16-byte multiples keep every slot vector-aligned.
   const size_t slotBytes{
       (std::min<size_t>(envSize("TP_HIP_IPC_SLOT_BYTES", kDefaultSlotBytes), size_t(1) << 30) + 15) / 16 *
@@ -239,6 +250,9 @@ class ChannelImpl final : public ChannelImplBase {
   ~ChannelImpl() override {
     for (auto& i : imports_) {
       HipIpcImports::get().release(i.device, i.peer, i.id);
+    }
+    for (auto& kv : remoteAllocations_) {
+      HipIpcImports::get().release(kv.second.device, peerIdentity_, kv.first);
     }
   }
 
@@ -401,22 +415,40 @@ class ChannelImpl final : public ChannelImplBase {
       }
 
       if (!direct.empty()) {
-        WireWriter w;
-        w.u8(kDirect);
-        w.u32(static_cast<uint32_t>(direct.size()));
-        for (auto& d : direct) {
-          w.u32(d.index);
-          w.u64(d.alloc.id);
-          const bool announce = announced_.insert(d.alloc.id).second;
-          w.u8(announce ? 1 : 0);
-          if (announce) {
-            w.str(processIdentity());
-            w.raw(d.alloc.handle.data(), d.alloc.handle.size());
-            w.u64(d.alloc.base);
-            w.u64(d.alloc.size);
+        // The distinct allocations of the unit, then the tensors by reference.
+        std::vector<const ExportedAllocation*> allocs;
+        std::vector<uint32_t> allocOf(direct.size());
+        for (size_t k = 0; k < direct.size(); ++k) {
+          uint32_t a = 0;
+          while (a < allocs.size() && allocs[a]->id != direct[k].alloc.id) {
+            ++a;
           }
-          w.u64(d.offset);
-          w.u64(d.length);
+          if (a == allocs.size()) {
+            allocs.push_back(&direct[k].alloc);
+          }
+          allocOf[k] = a;
+        }
+        WireWriter w;
+        w.reserve(64 + 96 * allocs.size() + 24 * direct.size());
+        w.u8(kDirect);
+        w.u8(identitySent_ ? 0 : 1);
+        if (!identitySent_) {
+          w.str(processIdentity());
+          identitySent_ = true;
+        }
+        w.u32(static_cast<uint32_t>(allocs.size()));
+        for (const ExportedAllocation* a : allocs) {
+          w.u64(a->id);
+          w.raw(a->handle.data(), a->handle.size());
+          w.u64(a->base);
+          w.u64(a->size);
+        }
+        w.u32(static_cast<uint32_t>(direct.size()));
+        for (size_t k = 0; k < direct.size(); ++k) {
+          w.u32(direct[k].index);
+          w.u32(allocOf[k]);
+          w.u64(direct[k].offset);
+          w.u64(direct[k].length);
         }
         auto unit = std::make_shared<WireUnit>();
         unit->bytes = std::move(w.bytes());
@@ -600,54 +632,79 @@ class ChannelImpl final : public ChannelImplBase {
     auto reply = std::make_shared<ReplyUnit>();
     replyQueue_.push_back(reply);
     std::vector<std::unique_ptr<HipEvent>> launched; // one event per copy launch
+    std::vector<uint64_t> inUse; // peer allocations the copies of this unit read from
     try {
       if (kind == kDirect) {
+        if (r.u8() != 0) {
+          peerIdentity_ = r.str();
+        }
+        const uint32_t nAllocs = r.u32();
+        // every allocation takes 88 bytes on the wire
+        if (!r.ok() || peerIdentity_.empty() || nAllocs > r.remaining() / 88) {
+          failProtocol();
+          return;
+        }
+        struct Announced {
+          uint64_t id;
+          HandleBytes handle;
+          uint64_t base;
+          uint64_t size;
+        };
+        std::vector<Announced> announced(nAllocs);
+        for (auto& a : announced) {
+          a.id = r.u64();
+          r.raw(a.handle.data(), a.handle.size());
+          a.base = r.u64();
+          a.size = r.u64();
+        }
         const uint32_t n = r.u32();
+        if (!r.ok() || n == 0 || n > r.remaining() / 24) {
+          failProtocol();
+          return;
+        }
         struct Group {
           StreamRef dst;
           std::vector<tphip_copy_desc> table;
         };
         std::vector<Group> groups;
+        std::vector<RemoteAllocation*> mappedOf(nAllocs, nullptr);
         for (uint32_t k = 0; k < n; ++k) {
           const uint32_t index = r.u32();
-          const uint64_t exportId = r.u64();
-          const bool announce = r.u8() != 0;
-          if (!r.ok() || index >= op->entries.size()) {
+          const uint32_t allocIdx = r.u32();
+          const uint64_t offset = r.u64();
+          const uint64_t length = r.u64();
+          if (!r.ok() || index >= op->entries.size() || allocIdx >= nAllocs) {
             failProtocol();
             return;
           }
           const HipBuffer& hb = op->entries[index].buffer.unwrap<HipBuffer>();
           const int device = hipDeviceForPointer(hb.ptr);
           TP_THROW_ASSERT_IF(device < 0);
-          if (announce) {
-            const std::string peer = r.str();
-            HandleBytes h;
-            r.raw(h.data(), h.size());
-            const uint64_t remoteBase = r.u64();
-            const uint64_t remoteSize = r.u64();
-            if (!r.ok() || remoteAllocations_.count(exportId) != 0) {
-              failProtocol();
-              return;
-            }
-            void* mapped = nullptr;
-            int rc = HipIpcImports::get().acquire(
-                device, peer, exportId, h, remoteBase, remoteSize, &mapped);
-            if (rc != 0) {
-              setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
-              return;
-            }
-            remoteAllocations_[exportId] = RemoteAllocation{mapped, remoteSize};
-            imports_.push_back(Import{device, peer, exportId});
-          }
-          const uint64_t offset = r.u64();
-          const uint64_t length = r.u64();
-          auto it = remoteAllocations_.find(exportId);
+          const Announced& a = announced[allocIdx];
           // The range must lie inside the allocation the peer announced: the
           // copy kernel would fault on anything else.
-          if (!r.ok() || it == remoteAllocations_.end() || length != op->entries[index].length ||
-              offset > it->second.size || length > it->second.size - offset) {
+          if (length != op->entries[index].length || offset > a.size || length > a.size - offset) {
             failProtocol();
             return;
+          }
+          if (mappedOf[allocIdx] == nullptr) {
+            auto it = remoteAllocations_.find(a.id);
+            if (it == remoteAllocations_.end()) {
+              void* mapped = nullptr;
+              int rc = HipIpcImports::get().acquire(
+                  device, peerIdentity_, a.id, a.handle, a.base, a.size, &mapped);
+              if (rc != 0) {
+                setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
+                return;
+              }
+              it = remoteAllocations_.emplace(a.id, RemoteAllocation{mapped, a.size, device, 0, 0}).first;
+              mappedBytes_ += a.size;
+            } else if (it->second.size != a.size) {
+              failProtocol(); // one identifier, one allocation
+              return;
+            }
+            it->second.lastUse = ++useCounter_;
+            mappedOf[allocIdx] = &it->second;
           }
           StreamRef ref{hb.stream, device};
           Group* g = nullptr;
@@ -660,9 +717,16 @@ class ChannelImpl final : public ChannelImplBase {
             groups.push_back(Group{ref, {}});
             g = &groups.back();
           }
-          g->table.push_back(
-              tphip_copy_desc{static_cast<const uint8_t*>(it->second.ptr) + offset, hb.ptr, length});
+          g->table.push_back(tphip_copy_desc{
+              static_cast<const uint8_t*>(mappedOf[allocIdx]->ptr) + offset, hb.ptr, length});
           ++op->unitsSeen;
+        }
+        // From here until the copies have finished the mappings must stay.
+        for (uint32_t a = 0; a < nAllocs; ++a) {
+          if (mappedOf[a] != nullptr) {
+            ++mappedOf[a]->inFlight;
+            inUse.push_back(announced[a].id);
+          }
         }
         for (auto& g : groups) {
           auto ev = ictx_->events.get(g.dst.device);
@@ -747,8 +811,15 @@ class ChannelImpl final : public ChannelImplBase {
     // Reply once the copies of this unit have finished.
     auto remaining = std::make_shared<size_t>(launched.size());
     for (auto& ev : launched) {
-      watch(std::move(ev), [this, reply, remaining] {
+      watch(std::move(ev), [this, reply, remaining, inUse] {
         if (--*remaining == 0) {
+          for (uint64_t id : inUse) {
+            auto it = remoteAllocations_.find(id);
+            if (it != remoteAllocations_.end() && it->second.inFlight > 0) {
+              --it->second.inFlight;
+            }
+          }
+          dropLeastRecentlyUsedMappings();
           reply->ready = true;
           flushReplies();
         }
@@ -761,6 +832,28 @@ class ChannelImpl final : public ChannelImplBase {
       finishRecv(op);
     } else {
       readNextUnit(op);
+    }
+  }
+
+  // Mappings nobody reads from go, oldest use first, while this channel holds
+  // more than it may. (On an error the watchers still run and the destructor
+  // releases what is left.)
+  void dropLeastRecentlyUsedMappings() {
+    while (mappedBytes_ > ictx_->maxMappedBytes || remoteAllocations_.size() > kMaxMappedAllocations) {
+      auto victim = remoteAllocations_.end();
+      for (auto it = remoteAllocations_.begin(); it != remoteAllocations_.end(); ++it) {
+        if (it->second.inFlight == 0 &&
+            (victim == remoteAllocations_.end() || it->second.lastUse < victim->second.lastUse)) {
+          victim = it;
+        }
+      }
+      if (victim == remoteAllocations_.end()) {
+        return; // everything mapped is being read
+      }
+      TP_VLOG(5) << "Channel " << id_ << " drops its mapping of peer allocation #" << victim->first;
+      HipIpcImports::get().release(victim->second.device, peerIdentity_, victim->first);
+      mappedBytes_ -= victim->second.size;
+      remoteAllocations_.erase(victim);
     }
   }
 
@@ -836,20 +929,27 @@ class ChannelImpl final : public ChannelImplBase {
   std::deque<std::shared_ptr<RecvOp>> recvOps_;
   std::deque<std::shared_ptr<WireUnit>> wireQueue_;
   std::deque<std::shared_ptr<ReplyUnit>> replyQueue_;
-  std::set<uint64_t> announced_;
+  bool identitySent_{false};
   std::map<int, bool> outboxAnnounced_;
+  // Peer allocations this channel keeps mapped (direct route), by export id.
   struct RemoteAllocation {
     void* ptr;
     uint64_t size;
+    int device;
+    uint64_t lastUse;
+    uint32_t inFlight; // units whose copies may still read from it
   };
   std::map<uint64_t, RemoteAllocation> remoteAllocations_;
+  std::string peerIdentity_; // the peer's processIdentity(), from its first direct unit
+  uint64_t mappedBytes_{0};
+  uint64_t useCounter_{0};
   struct RemoteOutbox {
     void* ptr;
     uint64_t slotBytes;
     uint32_t numSlots;
   };
   std::map<int, RemoteOutbox> remoteOutboxes_;
-  // What this channel holds in the process-wide import table.
+  // The peer's outboxes this channel holds in the process-wide import table.
   struct Import {
     int device;
     std::string peer;

@@ -422,6 +422,60 @@ std::vector<Case> makeCases() {
     cases.push_back({"AllocationsAboveExportLimitAreStaged", sendSide, recvSide});
   }
 
+  if (gSuite == "hip_ipc") {
+    // A receiver keeps the peer allocations it has mapped up to a limit and
+    // drops the least recently used ones beyond it; a tensor out of an
+    // allocation that was dropped is mapped again when it comes by. Thirty
+    // allocations of 512 KiB, all alive at once, against a limit of 1 MiB.
+    const size_t bytes = 512 * 1024;
+    const int allocations = 30;
+    auto pattern = [](size_t n, uint8_t salt) {
+      std::vector<uint8_t> v(n);
+      for (size_t i = 0; i < n; ++i) {
+        v[i] = static_cast<uint8_t>((i * 13) ^ (i >> 9) ^ salt);
+      }
+      return v;
+    };
+    // the order both sides follow: every allocation once, then back to old ones
+    auto order = [allocations] {
+      std::vector<int> o;
+      for (int i = 0; i < allocations; ++i) {
+        o.push_back(i);
+      }
+      for (int i : {0, 1, 29, 0, 15, 2}) {
+        o.push_back(i);
+      }
+      return o;
+    };
+    auto sendSide = [=](Endpoint& ep) {
+      auto o = open(ep);
+      std::vector<std::unique_ptr<GpuData>> sources;
+      for (int i = 0; i < allocations; ++i) {
+        sources.push_back(std::make_unique<GpuData>(pattern(bytes, static_cast<uint8_t>(i))));
+      }
+      ep.barrier();
+      for (int i : order()) {
+        auto f = sendF(*o->ch, sources[i]->buffer(), bytes);
+        EXPECT_OK(waitFor(f, "send"));
+      }
+      ep.barrier();
+    };
+    auto recvSide = [=](Endpoint& ep) {
+      ::setenv("TP_HIP_IPC_MAX_MAPPED_BYTES", "1048576", 1);
+      auto o = open(ep);
+      ::unsetenv("TP_HIP_IPC_MAX_MAPPED_BYTES");
+      ep.barrier();
+      GpuData d(bytes);
+      for (int i : order()) {
+        auto f = recvF(*o->ch, d.buffer(), bytes);
+        EXPECT_OK(waitFor(f, "recv"));
+        expectBytes(d, pattern(bytes, static_cast<uint8_t>(i)), "received data");
+      }
+      ep.barrier();
+    };
+    cases.push_back({"MappingsBeyondTheLimitAreDropped", sendSide, recvSide});
+  }
+
   if (gSuite == "hip_xth") {
     auto sameProcess = [](Endpoint&) {
       auto c1 = makeContext();

@@ -496,3 +496,41 @@ def test_contexts_come_and_go_without_leaking_device_memory():
     torch.cuda.empty_cache()
     free_after, _ = torch.cuda.mem_get_info()
     assert free_before - free_after < (32 << 20), (free_before, free_after)
+
+
+def test_ipc_peer_mappings_do_not_pin_freed_memory():
+    # sixty tensors, each out of its own 64 MiB allocation; all sixty stay alive until the last echo
+    # is back (so that every one has an address of its own) and are freed together. The peer has
+    # mapped every one of them; with a limit on what it keeps mapped (256 MiB here) the freed
+    # memory goes back to the device instead of staying alive through the peer's mappings.
+    import ctypes
+
+    import torch
+
+    lib = _native.tphip()
+    peer = Peer("basic:0,hip_ipc:11", env={"TP_HIP_IPC_MAX_MAPPED_BYTES": str(256 << 20)})
+    held = []
+    try:
+        n = 64 << 20
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        free_before, _ = torch.cuda.mem_get_info()
+        for k in range(60):
+            p = ctypes.c_void_p()
+            _native.check(lib.tphip_malloc(0, n, ctypes.byref(p)))
+            held.append(p)
+            _native.check(lib.tphip_fill(0, p, k + 1, n, None))
+            _native.check(lib.tphip_stream_sync(0, None))
+            outs, _ = peer.echo([tp.make_tensor(p.value, nbytes=n, device=tp.HIP, target=(tp.HIP, 0))], "gpu")
+            assert int(outs[0][32]) == k + 1 and int(outs[0][32 + n - 1]) == k + 1
+            del outs
+        while held:
+            _native.check(lib.tphip_free(0, held.pop()))
+        torch.cuda.empty_cache()
+        free_after, _ = torch.cuda.mem_get_info()
+        # without the limit the peer would still hold 60 x 64 MiB = 3.75 GiB of what was just freed
+        assert free_before - free_after < (1 << 30), (free_before, free_after)
+    finally:
+        while held:
+            lib.tphip_free(0, held.pop())
+        peer.close()
