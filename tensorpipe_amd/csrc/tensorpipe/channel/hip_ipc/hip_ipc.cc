@@ -164,11 +164,31 @@ class ExportRegistry {
     e.bufferId = bufferId;
     exports_[base] = e;
     *out = e;
+    forgetFreedAllocations();
     return true;
   }
 
  private:
+  // Entries of allocations that no longer exist are dropped now and then (each
+  // time the table has doubled), so that a process that keeps allocating and
+  // freeing does not grow it for ever. Called with the mutex held.
+  void forgetFreedAllocations() {
+    if (exports_.size() < purgeAt_) {
+      return;
+    }
+    for (auto it = exports_.begin(); it != exports_.end();) {
+      uint64_t now = 0;
+      if (tphip_mem_buffer_id(it->first, &now) != 0 || now != it->second.bufferId) {
+        it = exports_.erase(it);
+      } else {
+        ++it;
+      }
+    }
+    purgeAt_ = std::max<size_t>(1024, 2 * exports_.size());
+  }
+
   std::mutex mutex_;
+  size_t purgeAt_{1024};
   std::map<void*, ExportedAllocation> exports_;
 };
 

@@ -534,3 +534,38 @@ def test_ipc_peer_mappings_do_not_pin_freed_memory():
         while held:
             lib.tphip_free(0, held.pop())
         peer.close()
+
+
+def test_ipc_one_message_out_of_many_allocations(ipc_peer):
+    # 1100 tensors in one message, each out of an allocation of its own: more allocations than the
+    # sender's export table holds before it looks for freed ones (1024) and more than a receiving
+    # channel keeps mapped (1024); the message names every one of them
+    import ctypes
+
+    import torch
+
+    lib = _native.tphip()
+    count, n = 1100, 4096
+    held = []
+    try:
+        for k in range(count):
+            p = ctypes.c_void_p()
+            _native.check(lib.tphip_malloc(0, n, ctypes.byref(p)))
+            held.append(p)
+            _native.check(lib.tphip_fill(0, p, k % 251 + 1, n, None))
+        _native.check(lib.tphip_stream_sync(0, None))
+        tensors = [tp.make_tensor(p.value + 16 * (k % 3), nbytes=n - 64, device=tp.HIP, target=(tp.HIP, 0))
+                   for k, p in enumerate(held)]
+        outs, _ = ipc_peer.echo(tensors, "gpu")
+        torch.cuda.synchronize()
+        for k, o in enumerate(outs):
+            got = o.cpu().numpy()
+            assert (got[32:32 + n - 64] == k % 251 + 1).all(), k
+            assert (got[:32] == FILL).all() and (got[32 + n - 64:] == FILL).all(), k
+        # and again, now that the peer has dropped some of the mappings
+        outs, _ = ipc_peer.echo(tensors[:40], "gpu")
+        for k, o in enumerate(outs):
+            assert (o.cpu().numpy()[32:32 + n - 64] == k % 251 + 1).all(), k
+    finally:
+        while held:
+            lib.tphip_free(0, held.pop())
