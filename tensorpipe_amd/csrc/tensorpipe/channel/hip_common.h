@@ -125,6 +125,9 @@ class HipIpcImports {
 class StreamIdleProbe {
  public:
   bool idle(int device, void* stream) {
+    if (states_.size() > 256) {
+      states_.clear(); // streams come and go; what is remembered here is only a hint
+    }
     State& st = states_[std::make_pair(device, stream)];
     if (st.skip > 0) {
       --st.skip;
