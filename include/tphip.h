@@ -30,7 +30,7 @@ extern "C" {
 /* Errors raised by the library itself (all negative). */
 #define TPHIP_ERR_INVALID_ARG (-1)
 #define TPHIP_ERR_TOO_LARGE (-2)
-#define TPHIP_ERR_OVERLAP (-3)
+/* (-3 is not in use) */
 #define TPHIP_ERR_NO_DEVICE (-4)
 #define TPHIP_ERR_CAPTURING (-5)
 

@@ -657,8 +657,6 @@ const char* tphip_strerror(int err) {
       return "tphip: invalid argument";
     case TPHIP_ERR_TOO_LARGE:
       return "tphip: table larger than TPHIP_MAX_BATCH";
-    case TPHIP_ERR_OVERLAP:
-      return "tphip: overlapping ranges in copy table";
     case TPHIP_ERR_NO_DEVICE:
       return "tphip: no usable GPU";
     case TPHIP_ERR_CAPTURING:

@@ -107,8 +107,8 @@ struct StageTable {
     static const char* const kNames[] = {
         "pipe: encode descriptor", "pipe: write descriptor+payloads", "pipe: issue tensors",
         "pipe: parse descriptor",  "pipe: read request",               "hip_xth: encode descriptor",
-        "hip_xth: decode+group",   "hip_xth: launch",                  "hip_xth: copy in flight",
-        "harness: make message",   "harness: stream sync"};
+        "hip_xth: decode+group",   "hip_xth: launch",                  "harness: make message",
+        "harness: stream sync"};
     for (int i = 0; i < static_cast<int>(Stage::kCount); ++i) {
       const uint64_t c = calls[i].load();
       if (c != 0) {

@@ -21,7 +21,6 @@ enum class Stage : int {
   kXthEncode,
   kXthDecode,
   kXthLaunch,
-  kXthCopyInFlight,
   kHarnessMakeMessage,
   kHarnessSync,
   kCount
