@@ -148,6 +148,46 @@ def bench_d2d(steps, warmup):
     }
 
 
+def bench_d2d_in_flight(depth=4, transfers=400):
+    """configs[1]'s tensor with several transfers in flight on the same pipes: `depth` chains of
+    write/read run side by side (one caller thread each), every chain with a receive buffer and
+    stream of its own; all copies are queued on the sender's one stream."""
+    import threading
+
+    import torch
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    nbytes = 64 * MIB
+    src = torch.from_numpy(datagen.uniform_u8(datagen.SEED_BASE + 2, nbytes)).cuda()
+    dsts = [torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(depth)]
+    objs = make_pair("basic:0,hip_xth:10")
+    cpipe, spipe = objs[0], objs[1]
+    send_stream = torch.cuda.Stream()
+    recv_streams = [torch.cuda.Stream() for _ in range(depth)]
+    st = [tp.make_tensor(src, stream=send_stream, target=(tp.HIP, 0))]
+    rts = [[tp.make_tensor(d, stream=s)] for d, s in zip(dsts, recv_streams)]
+    torch.cuda.synchronize()
+    tp.bench_transfer(cpipe, spipe, st, rts[0], warmup=0, iters=20)
+    per_chain = transfers // depth
+    threads = [threading.Thread(target=tp.bench_transfer, args=(cpipe, spipe, st, rts[k]),
+                                kwargs={"warmup": 0, "iters": per_chain}) for k in range(depth)]
+    t0 = time.perf_counter()
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ok = all(bool(torch.equal(src, d)) for d in dsts)
+    destroy(objs)
+    done = per_chain * depth
+    return {"in_flight": depth, "transfers": done, "us_per_transfer": dt / done * 1e6,
+            "payload_GBps": nbytes * done / dt / 1e9,
+            "hbm_frac": 2.0 * nbytes * done / dt / 1e9 / HBM_PEAK_GBPS, "byte_exact": ok}
+
+
 def bench_rpc_message(messages=500, warmup=20):
     """configs[4]: 256 fp16 tensors, log-uniform sizes, 4 KiB payload, one launch per message."""
     import numpy as np
@@ -488,6 +528,7 @@ def cpu_baseline():
 # runtime does on later launches, which shifts small-transfer latencies by microseconds).
 LEGS = {
     "rpc_message": bench_rpc_message,
+    "d2d_in_flight": bench_d2d_in_flight,
     "ipc": bench_ipc,
     "staged": bench_staged,
     "staged_short": lambda: bench_staged(iters=20),
@@ -563,6 +604,8 @@ def main():
         # the same transfers with the runtime's hipMemcpyAsync instead of the copy kernel
         extra["staged_hipMemcpyAsync"] = extra_leg("staged_short", env={"TP_HIP_BASIC_ENGINE": "sdma"})
         extra["host_link"] = extra_leg("host_link")
+        # the headline's tensor with four transfers in flight instead of one
+        extra["d2d_in_flight"] = extra_leg("d2d_in_flight")
         extra["d2d_cold_source"] = extra_leg("cold_copy")
         log("[bench] this library's CPU path (shm + basic)")
         extra["cpu_path"] = extra_leg("cpu_path")

@@ -630,7 +630,7 @@ class ChannelImpl final : public ChannelImplBase {
       }();
       const uint32_t blocks = forcedBlocks > 0 ? static_cast<uint32_t>(forcedBlocks) : 32;
       // a marker behind the kernel: signalling from the kernel gains nothing measurable per chunk
-      hipBatchedCopy(device, stream, table, done, /*markerPool=*/nullptr, blocks, 3);
+      hipBatchedCopy(device, stream, table, done, /*signalOnKernel=*/false, blocks, 3);
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " host-link copy failed: " << ex.what();
       setError(TP_CREATE_ERROR(HipError, "hip_basic copy", TPHIP_ERR_INVALID_ARG));

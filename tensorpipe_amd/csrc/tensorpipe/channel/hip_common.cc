@@ -235,12 +235,12 @@ void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>
   }
 }
 
-void hipBatchedCopy(
+bool hipBatchedCopy(
     int device,
     void* stream,
     const std::vector<tphip_copy_desc>& table,
     HipEvent& done,
-    HipEventPool* markerPool,
+    bool signalOnKernel,
     uint32_t blocks,
     int nontemporal) {
   static const bool onKernel = [] {
@@ -248,7 +248,8 @@ void hipBatchedCopy(
     return e == nullptr || std::atoi(e) != 0;
   }();
   const bool tuned = blocks != 0 || nontemporal >= 0;
-  if (markerPool == nullptr || !onKernel || table.size() > TPHIP_MAX_BATCH || done.device() != device) {
+  if (!signalOnKernel || !onKernel || table.empty() || table.size() > TPHIP_MAX_BATCH ||
+      done.device() != device) {
     size_t off = 0;
     while (off < table.size()) {
       const size_t n = std::min<size_t>(table.size() - off, TPHIP_MAX_BATCH);
@@ -263,14 +264,12 @@ void hipBatchedCopy(
       off += n;
     }
     done.record(stream);
-    return;
+    return false;
   }
   TP_HIP_CHECK(tphip_batched_copy_signal(
       device, table.data(), static_cast<uint32_t>(table.size()), stream, done.raw(),
       tuned ? 4 : 0, blocks, nontemporal));
-  auto marker = markerPool->get(device);
-  marker->record(stream);
-  markerPool->put(std::move(marker)); // nobody waits for it; recording it again later is fine
+  return true;
 }
 
 } // namespace channel

@@ -163,27 +163,100 @@ class StreamIdleProbe {
 // Enqueue one batched copy on (device, stream); throws on a failed launch.
 void hipBatchedCopy(int device, void* stream, const std::vector<tphip_copy_desc>& table);
 
-// The same, and `done` is recorded behind the copy. With a `markerPool` the
+// The same, and `done` is recorded behind the copy. With `signalOnKernel` the
 // event is the completion signal of the copy kernel itself where possible: a
 // polling host sees it about 2.5 us sooner than a marker enqueued after the
-// kernel. A marker (an event of the pool, recorded and handed straight back,
-// never polled) still follows the kernel: without one the runtime does not
-// know when the stream has drained, and the user's next hipStreamQuery or
-// hipStreamSynchronize on it would take 12-20 us instead of 0.1. The marker
-// completes about 4 us after the kernel's signal; until then the stream reads
-// as busy, which is why channels that ask a stream whether it is idle right
-// after their own copy (hip_ipc, before announcing a tensor) pass no pool and
-// poll the marker itself. TP_HIP_SIGNAL_ON_KERNEL=0 does that everywhere.
-// `blocks` workgroups (0 = the library's choice) and `nontemporal` mask (-1 =
-// the library's choice) as for tphip_batched_copy_tuned.
-void hipBatchedCopy(
+// kernel. Returns true when that is what happened. A marker must then still
+// follow on the stream at some point: after a kernel without one the runtime
+// does not know when the stream has drained, and the next hipStreamQuery or
+// hipStreamSynchronize on it (the user's, or a channel's idle check) takes
+// 12-20 us instead of 0.1. StreamMarkers below decides when. Channels that ask a
+// stream whether it is idle right after their own copy (hip_ipc, before
+// announcing a tensor) pass false and poll a marker, recorded at once.
+// TP_HIP_SIGNAL_ON_KERNEL=0 does that everywhere. `blocks` workgroups (0 = the
+// library's choice) and `nontemporal` mask (-1 = the library's choice) as for
+// tphip_batched_copy_tuned.
+bool hipBatchedCopy(
     int device,
     void* stream,
     const std::vector<tphip_copy_desc>& table,
     HipEvent& done,
-    HipEventPool* markerPool,
+    bool signalOnKernel,
     uint32_t blocks = 0,
     int nontemporal = -1);
+
+// When the marker behind a kernel whose own signal is polled gets recorded. On
+// a quiet stream: at once, right behind the kernel, off everybody's path (the
+// kernel is still running). When the stream already has an unfinished copy of
+// ours in front -- several transfers in flight -- not yet: a marker between
+// two queued kernels would only hold the second one back (24-26 us instead of
+// ~21 per 64 MiB copy); the thread that sees the kernel finish records it
+// then, if nothing newer has been launched on the stream meanwhile. Shared
+// between the loop (launched) and the poller thread (finished).
+class StreamMarkers {
+ public:
+  struct Launch {
+    uint64_t id{0};
+    bool markerOwed{false}; // not recorded at launch: due when the kernel has finished
+  };
+
+  // Loop: a kernel without a marker behind it has just been launched.
+  Launch launched(int device, void* stream, HipEventPool& pool) {
+    Launch l;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      if (streams_.size() > 256) {
+        for (auto it = streams_.begin(); it != streams_.end();) {
+          it = it->second.outstanding == 0 ? streams_.erase(it) : std::next(it);
+        }
+      }
+      State& st = streams_[std::make_pair(device, stream)];
+      l.id = ++st.last;
+      l.markerOwed = st.outstanding > 0;
+      ++st.outstanding;
+    }
+    if (!l.markerOwed) {
+      record(device, stream, pool);
+    }
+    return l;
+  }
+
+  // Any thread: that kernel has finished.
+  void finished(int device, void* stream, const Launch& l, HipEventPool& pool) {
+    bool due = false;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      auto it = streams_.find(std::make_pair(device, stream));
+      if (it != streams_.end()) {
+        if (it->second.outstanding > 0) {
+          --it->second.outstanding;
+        }
+        due = l.markerOwed && it->second.last == l.id;
+      }
+    }
+    if (due) {
+      record(device, stream, pool);
+    }
+  }
+
+ private:
+  static void record(int device, void* stream, HipEventPool& pool) {
+    try {
+      auto marker = pool.get(device);
+      marker->record(stream);
+      pool.put(std::move(marker)); // nobody waits for it
+    } catch (const std::exception&) {
+      // without the marker the next query of the stream is slow, nothing more
+    }
+  }
+
+  struct State {
+    uint64_t last{0};
+    uint32_t outstanding{0};
+  };
+  std::mutex mutex_;
+  std::map<std::pair<int, void*>, State> streams_;
+};
 
 } // namespace channel
 TP_AMD_NAMESPACE_END

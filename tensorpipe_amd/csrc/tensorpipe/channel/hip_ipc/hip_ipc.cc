@@ -553,7 +553,7 @@ class ChannelImpl final : public ChannelImplBase {
             hb.stream,
             {tphip_copy_desc{static_cast<const uint8_t*>(hb.ptr) + offset, slot.get(), len}},
             *ev,
-            /*markerPool=*/nullptr);
+            /*signalOnKernel=*/false);
       } catch (const std::exception& ex) {
         TP_LOG_WARNING() << "Channel " << id_ << " staging failed: " << ex.what();
         setError(TP_CREATE_ERROR(HipError, "hip_ipc staging", TPHIP_ERR_INVALID_ARG));
@@ -750,7 +750,7 @@ class ChannelImpl final : public ChannelImplBase {
         }
         for (auto& g : groups) {
           auto ev = ictx_->events.get(g.dst.device);
-          hipBatchedCopy(g.dst.device, g.dst.stream, g.table, *ev, /*markerPool=*/nullptr);
+          hipBatchedCopy(g.dst.device, g.dst.stream, g.table, *ev, /*signalOnKernel=*/false);
           launched.push_back(std::move(ev));
         }
         op->unitsExpected += n;
@@ -808,7 +808,7 @@ class ChannelImpl final : public ChannelImplBase {
                 static_cast<uint8_t*>(hb.ptr) + offset,
                 len}},
             *ev,
-            /*markerPool=*/nullptr);
+            /*signalOnKernel=*/false);
         launched.push_back(std::move(ev));
         // A staged tensor counts as seen when its last chunk arrived.
         if (offset + len == op->entries[index].length) {

@@ -44,6 +44,7 @@ class XthContextCore final : public ContextCore {
   HipEventPool events;
   HipEventPoller poller;
   StreamIdleProbe idleProbe; // loop only
+  StreamMarkers markers;
   void joinImpl() override {
     poller.join();
   }
@@ -282,13 +283,24 @@ class ChannelImpl final : public ChannelImplBase {
         }
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
         auto done = xctx_->events.get(g.src.device);
-        hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*markerPool=*/&xctx_->events);
+        const bool onKernel =
+            hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*signalOnKernel=*/true);
+        StreamMarkers::Launch launch;
+        if (onKernel) {
+          launch = xctx_->markers.launched(g.src.device, g.src.stream, xctx_->events);
+        }
         TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
         auto self = shared_from_this();
         // Counted per launch: if a later launch of this op fails, the error
         // path still waits for exactly the copies that are running.
         ++op->copiesInFlight;
-        xctx_->poller.watch(std::move(done), &xctx_->events, [this, self, op](const Error& error) {
+        const StreamRef src = g.src;
+        xctx_->poller.watch(std::move(done), &xctx_->events, [this, self, op, src, onKernel, launch](
+                                                                 const Error& error) {
+          if (onKernel) {
+            // before anybody hears of the completion: the stream is still the sender's to keep
+            xctx_->markers.finished(src.device, src.stream, launch, xctx_->events);
+          }
           ctx_->defer([this, self, op, error] {
             setError(error);
             if (--op->copiesInFlight > 0) {
