@@ -171,11 +171,17 @@ def bench_d2d_in_flight(depth=4, transfers=400):
     torch.cuda.synchronize()
     tp.bench_transfer(cpipe, spipe, st, rts[0], warmup=0, iters=20)
     per_chain = transfers // depth
-    threads = [threading.Thread(target=tp.bench_transfer, args=(cpipe, spipe, st, rts[k]),
-                                kwargs={"warmup": 0, "iters": per_chain}) for k in range(depth)]
-    t0 = time.perf_counter()
+    lined_up = threading.Barrier(depth + 1)
+
+    def chain(k):
+        lined_up.wait()
+        tp.bench_transfer(cpipe, spipe, st, rts[k], warmup=0, iters=per_chain)
+
+    threads = [threading.Thread(target=chain, args=(k,)) for k in range(depth)]
     for t in threads:
         t.start()
+    lined_up.wait()  # every caller thread is up: the clock starts with the first write
+    t0 = time.perf_counter()
     for t in threads:
         t.join()
     torch.cuda.synchronize()
