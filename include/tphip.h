@@ -154,7 +154,8 @@ int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* 
  * by a polling host, and no second submission). Where that is not possible
  * (nothing to enqueue, launch profiling on) the event is recorded plainly, so
  * after a successful call `event` always covers everything the call enqueued
- * and all earlier work of `stream`. `unroll`, `blocks` and `nontemporal` as
+ * and all earlier work of `stream`. Not for a stream that is being captured
+ * into a graph (an event has no meaning there). `unroll`, `blocks` and `nontemporal` as
  * for tphip_batched_copy_tuned; 0, 0 and -1 select the defaults. The pair it
  * replaces: cudaMemcpyAsync +
  * cudaEventRecord at tensorpipe/channel/cuda_xth/channel_impl.cc:69-74,
