@@ -65,6 +65,27 @@ def test_send_multiple_tensors(pair, channels, targets):
         assert (o == src).all()
 
 
+def test_some_tensors_name_a_target_device(pair):
+    # tensorpipe/test/core/pipe_test.cc:281-359 (SimpleWriteReadWithSomeTargetDevices): the first
+    # tensor names the device it is to land on, the second leaves it to the receiver; the descriptor
+    # tells the receiver which is which
+    cpipe, spipe = pair()
+    a = np.frombuffer(b"tensor #1", np.uint8).copy()
+    b = np.frombuffer(b"tensor #2", np.uint8).copy()
+    w = cpipe.write([tp.make_tensor(a, target=(tp.CPU, 0)), tp.make_tensor(b)],
+                    payloads=[b"payload #1"], metadata="pipe metadata")
+    d = spipe.read_descriptor()
+    assert d.metadata.decode() == "pipe metadata" and d.num_tensors == 2 and d.num_payloads == 1
+    assert (d.tensor_target_type[0], d.tensor_target_index[0]) == (tp.CPU, 0)
+    assert d.tensor_target_type[1] == -1  # no target named
+    assert d.tensor_source_type[0] == tp.CPU and d.tensor_source_type[1] == tp.CPU
+    outs = [np.zeros(d.tensor_lengths[i], np.uint8) for i in range(2)]
+    pout = np.zeros(d.payload_lengths[0], np.uint8)
+    spipe.read([tp.make_tensor(o) for o in outs], [pout]).wait()
+    w.wait()
+    assert bytes(outs[0]) == b"tensor #1" and bytes(outs[1]) == b"tensor #2" and bytes(pout) == b"payload #1"
+
+
 def test_payloads_and_empty_tensors(pair):
     cpipe, spipe = pair()
     a, z, b = np.array([7], np.uint8), np.zeros(0, np.uint8), np.array([9], np.uint8)
