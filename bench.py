@@ -11,8 +11,11 @@ and a synchronisation of the receive stream. `value` is payload bytes delivered
 per second with the tensors already resident in HBM.
 
 The other configurations (cross-process IPC size sweep and 4 KiB round trip,
-host-staged 256 MiB, 256-tensor RPC-style message) and the CPU baseline are
-reported under "extra" / "cpu_baseline" of the same JSON line.
+host-staged 256 MiB with the copy kernel and with hipMemcpyAsync, 256-tensor RPC-style
+message), the headline's tensor with four transfers in flight and with a source that is
+not in the Infinity Cache, the host link's ceilings and the CPU baseline are reported
+under "extra" / "cpu_baseline" of the same JSON line; each runs in a process of its own
+(`--leg`), and one that fails is reported in its place without taking the line with it.
 """
 import argparse
 import json
