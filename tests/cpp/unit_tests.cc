@@ -17,11 +17,14 @@
 #include <cstring>
 #include <future>
 #include <map>
+#include <mutex>
 #include <random>
 #include <string>
 #include <thread>
 #include <vector>
 
+#include <execinfo.h>
+#include <signal.h>
 #include <unistd.h>
 
 #include <tensorpipe/common/buffer.h>
@@ -227,6 +230,7 @@ static int runGarbage(int argc, char** argv) {
   auto fDone = done->get_future();
   auto fulfilled = std::make_shared<std::atomic<bool>>(false);
   std::function<void()> acceptNext;
+  std::mutex acceptedMutex;
   std::vector<std::shared_ptr<Pipe>> accepted;
   acceptNext = [&] {
     listener->accept([&](const Error& e, std::shared_ptr<Pipe> p) {
@@ -234,9 +238,12 @@ static int runGarbage(int argc, char** argv) {
         if (!fulfilled->exchange(true)) {
           done->set_value("accept failed: " + e.what());
         }
-        return;
+        return; // also how the chain ends when the context closes
       }
-      accepted.push_back(p);
+      {
+        std::lock_guard<std::mutex> lock(acceptedMutex);
+        accepted.push_back(p);
+      }
       p->readDescriptor([&, p](const Error& e2, Descriptor d) {
         if (e2 || d.metadata != "proper") {
           return; // one of the garbage pipes: it fails or never speaks; ignore it
@@ -270,19 +277,35 @@ static int runGarbage(int argc, char** argv) {
     std::printf("the proper write did not complete\n");
     rc = 1;
   }
+  // The accept chain above runs on the server's threads and uses `listener` and
+  // `accepted`: the contexts are joined (no callback runs after that) before
+  // either goes away.
   keep.clear();
   pipe.reset();
-  accepted.clear();
-  listener.reset();
   client->join();
   server->join();
+  accepted.clear();
+  listener.reset();
   if (rc == 0) {
     std::printf("OK\n");
   }
   return rc;
 }
 
+// A crash names its stack before the process dies.
+static void onFatalSignal(int sig) {
+  void* frames[48];
+  const int n = backtrace(frames, 48);
+  const char msg[] = "fatal signal, stack:\n";
+  (void)!write(2, msg, sizeof(msg) - 1);
+  backtrace_symbols_fd(frames, n, 2);
+  signal(sig, SIG_DFL);
+  raise(sig);
+}
+
 int main(int argc, char** argv) {
+  signal(SIGSEGV, onFatalSignal);
+  signal(SIGABRT, onFatalSignal);
   if (argc == 4 && std::strcmp(argv[1], "garbage") == 0) {
     return runGarbage(argc, argv);
   }
