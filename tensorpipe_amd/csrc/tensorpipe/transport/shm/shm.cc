@@ -536,7 +536,10 @@ class ConnectionImpl final : public FdHandler,
 
   void close() {
     auto self = shared_from_this();
-    ctx_->defer([self] { self->fail(TP_CREATE_ERROR(ConnectionClosedError)); });
+    ctx_->defer([self] {
+      self->peerGone_ = false; // closed here: nothing more is handed over
+      self->fail(TP_CREATE_ERROR(ConnectionClosedError));
+    });
   }
 
   // Reactor thread: move bytes; returns whether anything happened.
@@ -599,6 +602,7 @@ class ConnectionImpl final : public FdHandler,
       // Peer went away: deliver what is already in the inbox, fail the rest.
       if (established_) {
         pumpReads();
+        peerGone_ = true;
       }
       fail(TP_CREATE_ERROR(EOFError));
     } else if (established_ && (events & EPOLLIN)) {
@@ -606,6 +610,7 @@ class ConnectionImpl final : public FdHandler,
       ssize_t rc = ::recv(sock_, &b, 1, MSG_DONTWAIT);
       if (rc == 0) {
         pumpReads();
+        peerGone_ = true;
         fail(TP_CREATE_ERROR(EOFError));
       }
     }
@@ -696,6 +701,20 @@ class ConnectionImpl final : public FdHandler,
   }
 
   void enqueueRead(ReadOp op) {
+    if (error_ && peerGone_ && reads_.empty()) {
+      // The peer wrote and left before this read was posted: what it wrote is
+      // still in the inbox, and a stream hands over what arrived before it
+      // reports the end. Whole messages only; the rest fails as before.
+      reads_.push_back(std::move(op));
+      pumpReads(/*afterPeerLeft=*/true);
+      if (reads_.empty()) {
+        return;
+      }
+      // A message cut short: the stream has no boundary to resume from.
+      op = std::move(reads_.front());
+      reads_.clear();
+      peerGone_ = false;
+    }
     if (error_) {
       op.fn(error_, nullptr, 0);
       return;
@@ -761,9 +780,9 @@ class ConnectionImpl final : public FdHandler,
     return progress;
   }
 
-  bool pumpReads() {
+  bool pumpReads(bool afterPeerLeft = false) {
     bool progress = false;
-    while (!reads_.empty() && !error_) {
+    while (!reads_.empty() && (!error_ || afterPeerLeft)) {
       ReadOp& op = reads_.front();
       if (!op.haveLen) {
         if (inbox_.available() < kLenPrefix) {
@@ -825,6 +844,9 @@ class ConnectionImpl final : public FdHandler,
   std::string id_{"N/A"};
   int sock_{-1};
   int peerWakeFd_{-1};
+  // The error is the peer's departure (not a local close or a protocol error):
+  // the inbox may still hold messages it sent before.
+  bool peerGone_{false};
   const bool connecting_;
   bool established_{false};
   Error error_;

@@ -64,6 +64,15 @@ def main():
         for l in reports[:5]:
             print("   ", l[:200])
         bad += (0 if ok else 1) + len(reports)
+    # a peer that wrote and left before the reads were posted
+    proc = subprocess.run([os.path.join(out, "unit_tests"), "departed_peer"],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+    ok = proc.returncode == 0 and proc.stdout.strip().endswith("OK")
+    print(f"unit_tests departed_peer: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
+    for l in reports[:5]:
+        print("   ", l[:200])
+    bad += (0 if ok else 1) + len(reports)
     sys.exit(1 if bad else 0)
 
 

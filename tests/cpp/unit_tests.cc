@@ -11,6 +11,9 @@
 //       opens raw transport connections to a listening context and writes
 //       random bytes where a pipe's first packets belong; the context must
 //       survive all of them and still serve a proper pipe afterwards.
+//   unit_tests departed_peer
+//       a peer writes two messages and goes away before the reader posts its
+//       reads: both messages are handed over, the third read reports the end.
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -38,6 +41,7 @@
 #include <tensorpipe/tensorpipe.h>
 #include <tensorpipe/tensorpipe_cuda.h>
 #include <tensorpipe/transport/connection.h>
+#include <tensorpipe/transport/listener.h>
 
 using namespace tensorpipe;
 
@@ -169,6 +173,63 @@ static int runBasics() {
   CHECK(makeXth != nullptr && makeIpc != nullptr && makeBasic != nullptr);
   CHECK(kCudaDeviceType == "cuda");
 
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
+// What a stream owes its reader when the writer left first: everything that
+// arrived, then the end (a two-process harness whose last step is "write a
+// byte, read a byte, exit" depends on exactly this).
+static int runDepartedPeer() {
+  int failed = 0;
+  auto serverSide = transport::shm::create();
+  const std::string addr = "tp_unit_departed_" + std::to_string(::getpid());
+  auto listener = serverSide->listen(addr);
+  std::promise<std::shared_ptr<transport::Connection>> acceptedP;
+  listener->accept([&](const Error& e, std::shared_ptr<transport::Connection> c) {
+    acceptedP.set_value(e ? nullptr : std::move(c));
+  });
+  auto clientSide = transport::shm::create();
+  auto conn = clientSide->connect(addr);
+  auto accepted = acceptedP.get_future().get();
+  CHECK(accepted != nullptr);
+  if (!accepted) {
+    return 1;
+  }
+  const std::string first = "first message";
+  const std::string second(5000, 'x');
+  std::promise<void> wroteP;
+  conn->write(first.data(), first.size(), [](const Error&) {});
+  conn->write(second.data(), second.size(), [&](const Error&) { wroteP.set_value(); });
+  wroteP.get_future().get();
+  conn.reset();
+  clientSide->join(); // the writer is gone, its socket closed
+  clientSide.reset();
+  // Let the reader's reactor see the hang-up before any read exists.
+  std::this_thread::sleep_for(std::chrono::milliseconds(200));
+  for (int i = 0; i < 3; ++i) {
+    std::promise<std::pair<bool, std::string>> gotP;
+    accepted->read([&](const Error& e, const void* ptr, size_t len) {
+      gotP.set_value({static_cast<bool>(e), e ? e.what() : std::string(static_cast<const char*>(ptr), len)});
+    });
+    auto got = gotP.get_future().get();
+    if (i == 0) {
+      CHECK(!got.first && got.second == first);
+    } else if (i == 1) {
+      CHECK(!got.first && got.second == second);
+    } else {
+      CHECK(got.first && got.second.find("eof") != std::string::npos);
+    }
+  }
+  // A connection that was closed on this side hands over nothing more.
+  accepted->close();
+  std::promise<bool> afterCloseP;
+  accepted->read([&](const Error& e, const void*, size_t) { afterCloseP.set_value(static_cast<bool>(e)); });
+  CHECK(afterCloseP.get_future().get());
+  listener->close();
+  serverSide->join();
   if (failed == 0) {
     std::printf("OK\n");
   }
@@ -315,6 +376,9 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "basics") == 0) {
     return runBasics();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | garbage <seed> <n>\n", argv[0]);
+  if (argc == 2 && std::strcmp(argv[1], "departed_peer") == 0) {
+    return runDepartedPeer();
+  }
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | garbage <seed> <n>\n", argv[0]);
   return 2;
 }

@@ -60,6 +60,13 @@ def test_basics():
     assert rc == 0 and out.strip() == "OK", out
 
 
+def test_messages_of_a_departed_peer_are_delivered():
+    # the writer exits before the reader posts its reads: the stream hands over what arrived,
+    # then reports the end
+    rc, out = run("departed_peer")
+    assert rc == 0 and out.strip() == "OK", out
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_garbage_on_new_connections(seed):
     # random bytes where the first packets of a pipe belong: the listening context survives them
