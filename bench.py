@@ -299,7 +299,10 @@ class PeerRun:
 
     def close(self):
         try:
-            self.pipe.write([], metadata=json.dumps({"op": "quit"})).wait(10000)
+            try:
+                self.pipe.write([], metadata=json.dumps({"op": "quit"})).wait(10000)
+            except self.tp.PipeError:
+                pass  # the peer read it and left before the write's callback ran
             self.proc.wait(30)
         finally:
             if self.proc.poll() is None:

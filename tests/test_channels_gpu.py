@@ -219,7 +219,12 @@ class Peer:
 
     def close(self):
         try:
-            self.pipe.write([], metadata="quit").wait(10000)
+            try:
+                self.pipe.write([], metadata="quit").wait(10000)
+            except tp.PipeError:
+                # the peer may read the message and exit before this side's write callback has
+                # run; a pipe whose peer is gone fails what is still pending, as the reference's does
+                pass
             self.proc.join(30)
         finally:
             if self.proc.is_alive():
@@ -228,6 +233,7 @@ class Peer:
             self.listener.destroy()
             self.ctx.destroy()
         self._check()
+        assert self.proc.exitcode == 0, f"peer exited with {self.proc.exitcode}"
 
 
 def _check_echo(out, host, length):
