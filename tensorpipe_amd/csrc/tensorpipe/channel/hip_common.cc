@@ -81,10 +81,11 @@ void HipEventPoller::run() {
   using Clock = std::chrono::steady_clock;
   std::deque<Item> active;
   auto lastBusy = Clock::now();
+  const auto hot = std::chrono::microseconds(runsOnOneCpu() ? 0 : 300);
   for (;;) {
     // Idle and hot: watch one flag, leave the mutex to the threads that post.
     if (active.empty() && !incomingPending_.load(std::memory_order_acquire) &&
-        Clock::now() - lastBusy < std::chrono::microseconds(300)) {
+        Clock::now() - lastBusy < hot) {
 #if defined(__x86_64__)
       __builtin_ia32_pause();
 #endif
@@ -96,7 +97,7 @@ void HipEventPoller::run() {
         // Stay hot for a short while after the last event: in a ping-pong the
         // next one arrives within microseconds and a sleeping thread would add
         // its wake-up time to every transfer.
-        if (Clock::now() - lastBusy < std::chrono::microseconds(300)) {
+        if (Clock::now() - lastBusy < hot) {
           lock.unlock();
 #if defined(__x86_64__)
           __builtin_ia32_pause();
@@ -140,6 +141,11 @@ void HipEventPoller::run() {
     if (!any) {
       // Leave the runtime's locks alone for a moment between rounds: the
       // threads that launch the next copies need them too.
+      if (runsOnOneCpu()) {
+        // The copy's launcher and the callbacks' consumers need this CPU.
+        ::sched_yield();
+        continue;
+      }
       const auto until = Clock::now() + std::chrono::nanoseconds(pollGapNanos());
       do {
 #if defined(__x86_64__)

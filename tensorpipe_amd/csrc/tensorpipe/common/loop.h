@@ -28,6 +28,8 @@
 #include <mutex>
 #include <thread>
 
+#include <sched.h>
+
 #include <tensorpipe/common/defs.h>
 
 TP_AMD_NAMESPACE_BEGIN
@@ -38,6 +40,18 @@ using TTask = std::function<void()>;
 inline bool& thisIsLibraryThread() {
   static thread_local bool flag = false;
   return flag;
+}
+
+// Whether this process may run on one CPU only (affinity mask, cgroup-pinned
+// containers): there a thread that spins keeps the thread it waits for off
+// the CPU, so the loops that stay hot after an event go to sleep at once.
+inline bool runsOnOneCpu() {
+  static const bool one = [] {
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    return ::sched_getaffinity(0, sizeof(set), &set) == 0 && CPU_COUNT(&set) < 2;
+  }();
+  return one;
 }
 
 class OnDemandLoop {

@@ -72,7 +72,12 @@ size_t ringBytes() {
 int spinMicros() {
   static const int v = [] {
     const char* e = std::getenv("TP_SHM_SPIN_US");
-    return e != nullptr ? std::atoi(e) : 200;
+    if (e != nullptr) {
+      return std::atoi(e);
+    }
+    // With one CPU to run on, a spinning reactor only keeps the thread it
+    // waits for off that CPU (4 KiB round trip: 870 us spinning, 46 sleeping).
+    return runsOnOneCpu() ? 0 : 200;
   }();
   return v;
 }
