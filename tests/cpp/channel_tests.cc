@@ -215,7 +215,8 @@ std::vector<Case> makeCases() {
   };
   cases.push_back({"SendTensorsBothWays", bothWays, bothWays});
 
-  // channel_test.cc:262-293: zero bytes at a null pointer complete at once.
+  // channel_test.cc:262-293 and channel_test_cpu.cc:19-43 (NullPointer): zero
+  // bytes at a null pointer complete at once.
   cases.push_back({"EmptyTensor",
                    [](Endpoint& ep) {
                      auto o = open(ep);

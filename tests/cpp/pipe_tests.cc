@@ -383,6 +383,135 @@ std::vector<Case> makeCases() {
                    {"tensor #4", "tensor metadata #4", kGpu, nullopt}}),
       {kCpu, kGpu, kCpu, kGpu}));
 
+  // pipe_test.cc:72-105: a message of payloads alone.
+  {
+    InlineMessage im = messageWith({});
+    cases.push_back(oneWay("SimpleWriteReadPayloadsOnly", im, {}));
+  }
+
+  // pipe_test.cc:107-160: a message of tensors alone.
+  {
+    InlineMessage im = messageWith({{"tensor #1", "tensor metadata #1", kGpu, nullopt},
+                                    {"tensor #2", "tensor metadata #2", kCpu, nullopt}});
+    im.payloads.clear();
+    cases.push_back(oneWay("SimpleWriteReadTensorsOnly", im, {kGpu, kCpu}));
+  }
+
+  // context_test.cc:468-632 (ServerPingPongTwice): two pings written back to
+  // back; every later step (readDescriptor, read, the pong's write) is issued
+  // from inside the callback of the one before, and the rounds finish in order.
+  {
+    struct Round {
+      Storage out;
+      Storage in;
+      Descriptor descriptor;
+    };
+    auto pingPong = [](Endpoint& ep) {
+      auto e = openPipe(ep);
+      const bool server = ep.isServer();
+      const InlineMessage im = messageWith({{"tensor #1", "tensor metadata #1", kGpu, nullopt},
+                                            {"tensor #2", "tensor metadata #2", kCpu, nullopt}});
+      Pipe* pipe = e->pipe.get();
+      auto rounds = std::make_shared<std::vector<Round>>(2);
+      auto finished = std::make_shared<std::atomic<int>>(0);
+      auto done = std::make_shared<std::promise<std::string>>();
+      auto fDone = done->get_future();
+      auto settle = [done, finished](int i, const Error& err, const char* what) {
+        // a failure ends the case at once; success needs both rounds, in order
+        if (err) {
+          try {
+            done->set_value(std::string(what) + ": " + err.what());
+          } catch (const std::future_error&) {
+          }
+          return false;
+        }
+        (void)i;
+        return true;
+      };
+      // readDescriptor -> read, then `then(i)`
+      auto readOne = [pipe, rounds, settle](int i, std::function<void(int)> then) {
+        pipe->readDescriptor([pipe, rounds, settle, i, then](const Error& err, Descriptor d) {
+          if (!settle(i, err, "readDescriptor")) {
+            return;
+          }
+          Round& r = (*rounds)[i];
+          Allocation a;
+          for (auto& p : d.payloads) {
+            r.in.payloads.emplace_back(p.length, 0);
+            Allocation::Payload ap;
+            ap.data = r.in.payloads.back().data();
+            a.payloads.push_back(ap);
+          }
+          for (auto& t : d.tensors) {
+            r.in.tensors.push_back(makeData(gHaveGpu && t.sourceDevice == kGpu, t.length));
+            Allocation::Tensor at;
+            at.buffer = r.in.tensors.back()->buffer();
+            a.tensors.push_back(std::move(at));
+          }
+          r.descriptor = std::move(d);
+          pipe->read(std::move(a), [settle, i, then](const Error& err2) {
+            if (settle(i, err2, "read")) {
+              then(i);
+            }
+          });
+        });
+      };
+      auto roundOver = [finished, done](int i) {
+        const int before = finished->fetch_add(1);
+        if (before != i) {
+          try {
+            done->set_value("round " + std::to_string(i) + " finished out of order");
+          } catch (const std::future_error&) {
+          }
+        } else if (before == 1) {
+          try {
+            done->set_value("");
+          } catch (const std::future_error&) {
+          }
+        }
+      };
+      for (int i = 0; i < 2; ++i) {
+        if (server) {
+          // ping; from its callback: read the pong
+          Message m = buildMessage(im, &(*rounds)[i].out);
+          pipe->write(std::move(m), [settle, readOne, roundOver, i](const Error& err) {
+            if (settle(i, err, "write")) {
+              readOne(i, roundOver);
+            }
+          });
+        } else {
+          // read the ping; from the read's callback: write the pong
+          readOne(i, [pipe, rounds, im, settle, roundOver](int k) {
+            Message m = buildMessage(im, &(*rounds)[k].out);
+            pipe->write(std::move(m), [settle, roundOver, k](const Error& err) {
+              if (settle(k, err, "write")) {
+                roundOver(k);
+              }
+            });
+          });
+        }
+      }
+      const std::string problem = waitFor(fDone, "two chained rounds");
+      EXPECT_EQ(problem, std::string());
+      for (int i = 0; i < 2 && problem.empty(); ++i) {
+        Round& r = (*rounds)[i];
+        EXPECT_EQ(r.descriptor.metadata, im.metadata);
+        EXPECT_EQ(r.descriptor.payloads.size(), im.payloads.size());
+        EXPECT_EQ(r.descriptor.tensors.size(), im.tensors.size());
+        for (size_t k = 0; k < r.in.payloads.size() && k < im.payloads.size(); ++k) {
+          EXPECT_EQ(std::string(r.in.payloads[k].begin(), r.in.payloads[k].end()), im.payloads[k].first);
+        }
+        for (size_t k = 0; k < r.in.tensors.size() && k < im.tensors.size(); ++k) {
+          std::vector<uint8_t> got = r.in.tensors[k]->bytes();
+          EXPECT_EQ(std::string(got.begin(), got.end()), im.tensors[k].data);
+          EXPECT_EQ(r.descriptor.tensors[k].metadata, im.tensors[k].metadata);
+        }
+      }
+      ep.barrier();
+    };
+    cases.push_back({"ServerPingPongTwice", pingPong, pingPong});
+  }
+
   // Several messages back to back, each answered, with tensors large enough to
   // go through more than one staging slot.
   cases.push_back(
