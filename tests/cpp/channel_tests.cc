@@ -343,6 +343,15 @@ std::vector<Case> makeCases() {
     cases.push_back({"SendFromGpuToCpu",
                      [](Endpoint& ep) { sender(ep, true, std::vector<uint8_t>(1024, 0x42)); },
                      [](Endpoint& ep) { receiver(ep, false, std::vector<uint8_t>(1024, 0x42)); }});
+    // channel_test_cuda_xdtt.cc:145-195: the channel is never chosen for a pair of
+    // CPU endpoints, yet carries CPU memory both ways when asked to.
+    cases.push_back({"SendFromCpuToCpu",
+                     [](Endpoint& ep) { sender(ep, false, std::vector<uint8_t>(1024, 0x42)); },
+                     [](Endpoint& ep) { receiver(ep, false, std::vector<uint8_t>(1024, 0x42)); }});
+    // The same over several chunks, with a ragged end.
+    cases.push_back({"SendFromCpuToCpuSeveralChunks",
+                     [](Endpoint& ep) { sender(ep, false, iota(3 * 1024 * 1024 + 5)); },
+                     [](Endpoint& ep) { receiver(ep, false, iota(3 * 1024 * 1024 + 5)); }});
     // cuda_basic_test.cc:40-62: a pair of CPU endpoints is left to CPU channels.
     auto cpuToCpu = [](Endpoint&) {
       auto c = makeContext();
