@@ -512,6 +512,90 @@ std::vector<Case> makeCases() {
     cases.push_back({"ServerPingPongTwice", pingPong, pingPong});
   }
 
+  // context_test.cc:634-738 (MixedTensorMessage): two reads are posted before
+  // anything arrives; a message with payloads and tensors is followed by one
+  // with nothing in it at all.
+  cases.push_back(
+      {"MixedTensorMessage",
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         Pipe* pipe = e->pipe.get();
+         struct Got {
+           Descriptor descriptor;
+           Storage storage;
+         };
+         auto got = std::make_shared<std::vector<Got>>(2);
+         auto left = std::make_shared<std::atomic<int>>(2);
+         auto done = std::make_shared<std::promise<std::string>>();
+         auto fDone = done->get_future();
+         auto finish = [done](const std::string& what) {
+           try {
+             done->set_value(what);
+           } catch (const std::future_error&) {
+           }
+         };
+         for (int i = 0; i < 2; ++i) {
+           pipe->readDescriptor([pipe, got, left, finish, i](const Error& err, Descriptor d) {
+             if (err) {
+               finish("readDescriptor: " + err.what());
+               return;
+             }
+             Got& g = (*got)[i];
+             Allocation a;
+             for (auto& p : d.payloads) {
+               g.storage.payloads.emplace_back(p.length, 0);
+               Allocation::Payload ap;
+               ap.data = g.storage.payloads.back().data();
+               a.payloads.push_back(ap);
+             }
+             for (auto& t : d.tensors) {
+               g.storage.tensors.push_back(makeData(gHaveGpu && t.sourceDevice == kGpu, t.length));
+               Allocation::Tensor at;
+               at.buffer = g.storage.tensors.back()->buffer();
+               a.tensors.push_back(std::move(at));
+             }
+             g.descriptor = std::move(d);
+             pipe->read(std::move(a), [left, finish](const Error& err2) {
+               if (err2) {
+                 finish("read: " + err2.what());
+               } else if (left->fetch_sub(1) == 1) {
+                 finish("");
+               }
+             });
+           });
+         }
+         ep.barrier(); // both reads are posted; now the peer writes
+         EXPECT_EQ(waitFor(fDone, "two posted reads"), std::string());
+         const InlineMessage im = messageWith({{"tensor #1", "tensor metadata #1", kGpu, nullopt},
+                                               {"tensor #2", "tensor metadata #2", kCpu, nullopt}});
+         const Got& first = (*got)[0];
+         EXPECT_EQ(first.descriptor.metadata, im.metadata);
+         EXPECT_EQ(first.descriptor.payloads.size(), im.payloads.size());
+         EXPECT_EQ(first.descriptor.tensors.size(), im.tensors.size());
+         for (size_t k = 0; k < first.storage.payloads.size() && k < im.payloads.size(); ++k) {
+           EXPECT_EQ(std::string(first.storage.payloads[k].begin(), first.storage.payloads[k].end()),
+                     im.payloads[k].first);
+         }
+         for (size_t k = 0; k < first.storage.tensors.size() && k < im.tensors.size(); ++k) {
+           std::vector<uint8_t> b = first.storage.tensors[k]->bytes();
+           EXPECT_EQ(std::string(b.begin(), b.end()), im.tensors[k].data);
+         }
+         const Got& second = (*got)[1];
+         EXPECT_EQ(second.descriptor.metadata, std::string());
+         EXPECT_EQ(second.descriptor.payloads.size(), size_t(0));
+         EXPECT_EQ(second.descriptor.tensors.size(), size_t(0));
+         ep.barrier();
+       },
+       [](Endpoint& ep) {
+         auto e = openPipe(ep);
+         ep.barrier();
+         writeMessage(*e->pipe, messageWith({{"tensor #1", "tensor metadata #1", kGpu, nullopt},
+                                              {"tensor #2", "tensor metadata #2", kCpu, nullopt}}));
+         InlineMessage nothing;
+         writeMessage(*e->pipe, nothing);
+         ep.barrier();
+       }});
+
   // Several messages back to back, each answered, with tensors large enough to
   // go through more than one staging slot.
   cases.push_back(
