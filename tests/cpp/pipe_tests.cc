@@ -354,6 +354,112 @@ void exchangeMany(Pipe& pipe, uint32_t myRole, uint32_t count, uint32_t lane = 0
   }
 }
 
+// Posts one readDescriptor -> read chain per expected message before anything
+// has arrived (pipeReadWithFuture of pipe_test.h, several at once), then checks
+// what each of them received.
+void readPostedAhead(Pipe& pipe, const std::vector<InlineMessage>& expected,
+                     const std::vector<std::vector<Device>>& devices) {
+  struct Got {
+    Descriptor descriptor;
+    Storage storage;
+  };
+  const size_t n = expected.size();
+  auto got = std::make_shared<std::vector<Got>>(n);
+  auto left = std::make_shared<std::atomic<int>>(static_cast<int>(n));
+  auto done = std::make_shared<std::promise<std::string>>();
+  auto fDone = done->get_future();
+  auto finish = [done](const std::string& what) {
+    try {
+      done->set_value(what);
+    } catch (const std::future_error&) {
+    }
+  };
+  Pipe* p = &pipe;
+  for (size_t i = 0; i < n; ++i) {
+    const std::vector<Device> onto = devices[i];
+    p->readDescriptor([p, got, left, finish, i, onto](const Error& err, Descriptor d) {
+      if (err) {
+        finish("readDescriptor: " + err.what());
+        return;
+      }
+      if (d.tensors.size() != onto.size()) {
+        finish("message " + std::to_string(i) + " has " + std::to_string(d.tensors.size()) + " tensors");
+        return;
+      }
+      Got& g = (*got)[i];
+      Allocation a;
+      for (auto& pl : d.payloads) {
+        g.storage.payloads.emplace_back(pl.length, 0);
+        Allocation::Payload ap;
+        ap.data = g.storage.payloads.back().data();
+        a.payloads.push_back(ap);
+      }
+      for (size_t t = 0; t < d.tensors.size(); ++t) {
+        g.storage.tensors.push_back(makeData(gHaveGpu && onto[t] == kGpu, d.tensors[t].length));
+        Allocation::Tensor at;
+        at.buffer = g.storage.tensors.back()->buffer();
+        a.tensors.push_back(std::move(at));
+      }
+      g.descriptor = std::move(d);
+      p->read(std::move(a), [left, finish](const Error& err2) {
+        if (err2) {
+          finish("read: " + err2.what());
+        } else if (left->fetch_sub(1) == 1) {
+          finish("");
+        }
+      });
+    });
+  }
+  const std::string problem = waitFor(fDone, "reads posted ahead");
+  EXPECT_EQ(problem, std::string());
+  if (!problem.empty()) {
+    return;
+  }
+  for (size_t i = 0; i < n; ++i) {
+    const InlineMessage& im = expected[i];
+    const Got& g = (*got)[i];
+    EXPECT_EQ(g.descriptor.metadata, im.metadata);
+    EXPECT_EQ(g.descriptor.payloads.size(), im.payloads.size());
+    EXPECT_EQ(g.descriptor.tensors.size(), im.tensors.size());
+    for (size_t k = 0; k < g.storage.payloads.size() && k < im.payloads.size(); ++k) {
+      EXPECT_EQ(g.descriptor.payloads[k].metadata, im.payloads[k].second);
+      EXPECT_EQ(std::string(g.storage.payloads[k].begin(), g.storage.payloads[k].end()), im.payloads[k].first);
+    }
+    for (size_t k = 0; k < g.storage.tensors.size() && k < im.tensors.size(); ++k) {
+      std::vector<uint8_t> b = g.storage.tensors[k]->bytes();
+      EXPECT_EQ(std::string(b.begin(), b.end()), im.tensors[k].data);
+      EXPECT_EQ(g.descriptor.tensors[k].metadata, im.tensors[k].metadata);
+      EXPECT_TRUE(g.descriptor.tensors[k].sourceDevice == im.tensors[k].device);
+      EXPECT_EQ(g.descriptor.tensors[k].targetDevice.has_value(), im.tensors[k].target.has_value());
+    }
+  }
+}
+
+// The server writes both messages without waiting in between; the client has
+// both reads posted.
+Case twoInFlight(std::string name, InlineMessage im1, InlineMessage im2, std::vector<Device> onto1,
+                 std::vector<Device> onto2) {
+  return Case{std::move(name),
+              [im1, im2](Endpoint& ep) {
+                auto e = openPipe(ep);
+                Storage s1, s2;
+                auto p1 = std::make_shared<std::promise<Error>>();
+                auto p2 = std::make_shared<std::promise<Error>>();
+                auto f1 = p1->get_future();
+                auto f2 = p2->get_future();
+                e->pipe->write(buildMessage(im1, &s1), [p1](const Error& err) { p1->set_value(err); });
+                e->pipe->write(buildMessage(im2, &s2), [p2](const Error& err) { p2->set_value(err); });
+                EXPECT_OK(waitFor(f1, "first write"));
+                EXPECT_OK(waitFor(f2, "second write"));
+                ep.barrier();
+              },
+              [im1, im2, onto1, onto2](Endpoint& ep) {
+                auto e = openPipe(ep);
+                readPostedAhead(*e->pipe, {im1, im2}, {onto1, onto2});
+                ep.barrier();
+              }};
+}
+
 std::vector<Case> makeCases() {
   std::vector<Case> cases;
 
@@ -510,6 +616,24 @@ std::vector<Case> makeCases() {
       ep.barrier();
     };
     cases.push_back({"ServerPingPongTwice", pingPong, pingPong});
+  }
+
+  // pipe_test.cc:286-364 (MultipleWriteRead) and :366-446
+  // (MultipleWriteReadWithSomeTargetDevices), and the same with a GPU tensor.
+  {
+    InlineMessage m1, m2;
+    m1.metadata = m2.metadata = "message metadata";
+    m1.payloads = {{"payload #1.1", "payload metadata #1.1"}};
+    m2.payloads = {{"payload #2.1", "payload metadata #2.1"}};
+    m1.tensors = {{"tensor #1.1", "tensor metadata #1.1", kCpu, nullopt}};
+    m2.tensors = {{"tensor #2.1", "tensor metadata #2.1", kCpu, nullopt}};
+    cases.push_back(twoInFlight("MultipleWriteRead", m1, m2, {kCpu}, {kCpu}));
+    m2.tensors = {{"tensor #2.1", "tensor metadata #2.1", kCpu, kCpu}};
+    cases.push_back(twoInFlight("MultipleWriteReadWithSomeTargetDevices", m1, m2, {kCpu}, {kCpu}));
+    m1.tensors = {{"tensor #1.1", "tensor metadata #1.1", kGpu, nullopt}};
+    m2.tensors = {{"tensor #2.1", "tensor metadata #2.1", kGpu, kGpu},
+                  {"tensor #2.2", "tensor metadata #2.2", kCpu, nullopt}};
+    cases.push_back(twoInFlight("MultipleWriteReadWithGpuTensors", m1, m2, {kCpu}, {kGpu, kGpu}));
   }
 
   // context_test.cc:634-738 (MixedTensorMessage): two reads are posted before

@@ -78,6 +78,31 @@ def test_pointer_queries(lib):
     _native.check(lib.tphip_free(0, p))
 
 
+def test_pointer_queries_from_a_fresh_thread(lib):
+    # tensorpipe/test/common/cuda_test.cc:33-62 (DeviceForPointer), on the one device there is: a
+    # thread that has made no GPU call yet asks where a pointer of another thread lives
+    import threading
+
+    p = _malloc(lib, 1024)
+    seen = {}
+
+    def ask():
+        dev, is_host = ctypes.c_int(-5), ctypes.c_int(-5)
+        seen["rc"] = lib.tphip_device_for_ptr(vp(p.value + 100), ctypes.byref(dev), ctypes.byref(is_host))
+        seen["dev"], seen["is_host"] = dev.value, is_host.value
+        ident = ctypes.c_uint64()
+        seen["rc_id"] = lib.tphip_mem_buffer_id(p, ctypes.byref(ident))
+        seen["id"] = ident.value
+
+    t = threading.Thread(target=ask)
+    t.start()
+    t.join()
+    here = ctypes.c_uint64()
+    _native.check(lib.tphip_mem_buffer_id(p, ctypes.byref(here)))
+    assert seen == {"rc": 0, "dev": 0, "is_host": 0, "rc_id": 0, "id": here.value}
+    _native.check(lib.tphip_free(0, p))
+
+
 def test_pinned_host_slab_is_visible_to_both_sides(lib):
     n = 1 << 16
     host, devp = vp(), vp()
