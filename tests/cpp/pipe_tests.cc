@@ -463,6 +463,15 @@ Case twoInFlight(std::string name, InlineMessage im1, InlineMessage im2, std::ve
 std::vector<Case> makeCases() {
   std::vector<Case> cases;
 
+  // pipe_test.cc:20-70 (SimpleWriteRead; context_test.cc ClientPingSerial sends
+  // the same kind of message once): payloads and three CPU tensors.
+  cases.push_back(oneWay(
+      "SimpleWriteRead",
+      messageWith({{"tensor #1", "tensor metadata #1", kCpu, nullopt},
+                   {"tensor #2", "tensor metadata #2", kCpu, nullopt},
+                   {"tensor #3", "tensor metadata #3", kCpu, nullopt}}),
+      {kCpu, kCpu, kCpu}));
+
   // pipe_cuda_test.cc:13-81
   cases.push_back(oneWay(
       "SimpleWriteReadWithAllTargetDevices",
