@@ -81,7 +81,7 @@ void HipEventPoller::run() {
   using Clock = std::chrono::steady_clock;
   std::deque<Item> active;
   auto lastBusy = Clock::now();
-  const auto hot = std::chrono::microseconds(runsOnOneCpu() ? 0 : 300);
+  const auto hot = std::chrono::microseconds(runsOnFewCpus() ? 0 : 300);
   for (;;) {
     // Idle and hot: watch one flag, leave the mutex to the threads that post.
     if (active.empty() && !incomingPending_.load(std::memory_order_acquire) &&
@@ -141,7 +141,7 @@ void HipEventPoller::run() {
     if (!any) {
       // Leave the runtime's locks alone for a moment between rounds: the
       // threads that launch the next copies need them too.
-      if (runsOnOneCpu()) {
+      if (runsOnFewCpus()) {
         // The copy's launcher and the callbacks' consumers need this CPU.
         ::sched_yield();
         continue;

@@ -23,6 +23,7 @@
 
 #include <atomic>
 #include <condition_variable>
+#include <cstdlib>
 #include <deque>
 #include <functional>
 #include <mutex>
@@ -42,16 +43,23 @@ inline bool& thisIsLibraryThread() {
   return flag;
 }
 
-// Whether this process may run on one CPU only (affinity mask, cgroup-pinned
-// containers): there a thread that spins keeps the thread it waits for off
-// the CPU, so the loops that stay hot after an event go to sleep at once.
-inline bool runsOnOneCpu() {
-  static const bool one = [] {
+// Whether this process has fewer CPUs to run on (affinity mask, pinned
+// containers) than a pipe keeps busy at full tilt: the caller, the context's
+// loop and the two threads that stay hot after an event (transport reactor,
+// event poller). With fewer, a thread that spins keeps the thread it waits for
+// off the CPU, so those loops go to sleep at once instead. The threshold can be
+// moved with TP_SPIN_MIN_CPUS.
+inline bool runsOnFewCpus() {
+  static const bool few = [] {
+    int need = 4;
+    if (const char* e = std::getenv("TP_SPIN_MIN_CPUS")) {
+      need = std::atoi(e);
+    }
     cpu_set_t set;
     CPU_ZERO(&set);
-    return ::sched_getaffinity(0, sizeof(set), &set) == 0 && CPU_COUNT(&set) < 2;
+    return ::sched_getaffinity(0, sizeof(set), &set) == 0 && CPU_COUNT(&set) < need;
   }();
-  return one;
+  return few;
 }
 
 class OnDemandLoop {

@@ -75,9 +75,9 @@ int spinMicros() {
     if (e != nullptr) {
       return std::atoi(e);
     }
-    // With one CPU to run on, a spinning reactor only keeps the thread it
+    // With too few CPUs to run on, a spinning reactor only keeps the thread it
     // waits for off that CPU (4 KiB round trip: 870 us spinning, 46 sleeping).
-    return runsOnOneCpu() ? 0 : 200;
+    return runsOnFewCpus() ? 0 : 200;
   }();
   return v;
 }
