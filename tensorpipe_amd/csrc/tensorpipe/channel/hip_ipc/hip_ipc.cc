@@ -640,18 +640,31 @@ class ChannelImpl final : public ChannelImplBase {
       return;
     }
     recvOps_.push_back(op);
-    readNextUnit(op);
+    pumpUnits();
   }
 
-  // The number of units of an op is only known once its first unit has been
-  // seen (a direct unit says how many tensors it covers), so units are read
-  // one at a time until every tensor of the op is accounted for.
-  void readNextUnit(const std::shared_ptr<RecvOp>& op) {
-    descriptorConnection_->read(onReadMessage([this, op](std::vector<uint8_t> bytes) {
-      if (error_) {
+  // One reader per channel. The transport serves reads in the order they were
+  // posted, and how many units an op takes is only known as they arrive (a
+  // direct unit says how many tensors it covers, a staged tensor takes one
+  // unit per chunk): a read posted for a later op while an earlier one still
+  // expects units would be handed that earlier op's next unit. So a single
+  // read is outstanding at any time and every unit goes to the oldest op that
+  // is still missing some, as the reference gates its descriptor reads per
+  // operation in sequence
+  // (tensorpipe/channel/cuda_ipc/channel_impl.cc:319-347,349-399).
+  void pumpUnits() {
+    if (unitReadPosted_ || recvOps_.empty() || error_) {
+      return;
+    }
+    unitReadPosted_ = true;
+    descriptorConnection_->read(onReadMessage([this](std::vector<uint8_t> bytes) {
+      unitReadPosted_ = false;
+      if (error_ || recvOps_.empty()) {
         return;
       }
+      auto op = recvOps_.front();
       onUnit(op, bytes);
+      pumpUnits();
     }));
   }
 
@@ -866,8 +879,6 @@ class ChannelImpl final : public ChannelImplBase {
       // Every copy of the op is enqueued: that is what the recv callback means.
       removeRecv(op);
       finishRecv(op);
-    } else {
-      readNextUnit(op);
     }
   }
 
@@ -988,7 +999,8 @@ class ChannelImpl final : public ChannelImplBase {
   std::shared_ptr<transport::Connection> descriptorConnection_;
   std::shared_ptr<transport::Connection> replyConnection_;
   std::deque<std::shared_ptr<SendOp>> sendOps_;
-  std::deque<std::shared_ptr<RecvOp>> recvOps_;
+  std::deque<std::shared_ptr<RecvOp>> recvOps_; // oldest first; the front one takes the next unit
+  bool unitReadPosted_{false};
   std::deque<std::shared_ptr<WireUnit>> wireQueue_;
   std::deque<std::shared_ptr<ReplyUnit>> replyQueue_;
   bool identitySent_{false};

@@ -1,4 +1,8 @@
+#include <atomic>
 #include <cstring>
+#include <iterator>
+#include <map>
+#include <mutex>
 #include <sstream>
 
 #include <tensorpipe/common/error.h>
@@ -56,17 +60,87 @@ int hipDeviceCountNoThrow() {
   return count;
 }
 
-int hipDeviceForPointer(const void* ptr) {
-  // With a single visible GPU every device pointer belongs to device 0: skip
-  // the driver query, which would otherwise run several times per tensor.
-  static const int count = hipDeviceCountNoThrow();
-  if (count == 1 && ptr != nullptr) {
-    return 0;
+namespace {
+
+// Address ranges the runtime has vouched for, so that the per-tensor question
+// "which device owns this pointer" costs a map lookup instead of driver calls
+// (the reference asks the driver every time,
+// tensorpipe/common/cuda.h:141-166). A range is entered after the runtime has
+// named its device and its extent; a pointer outside every known range goes
+// to the runtime, and one the runtime does not know (plain host memory) is
+// reported as such. A range stays until the table is cleared for size, so an
+// address freed and handed out again by the runtime keeps its answer: on one
+// device that answer is still right.
+class PointerRanges {
+ public:
+  int lookup(const void* ptr) {
+    const uintptr_t p = reinterpret_cast<uintptr_t>(ptr);
+    struct Last {
+      uintptr_t begin{0}, end{0};
+      int device{-1};
+      uint64_t generation{0};
+    };
+    thread_local Last last;
+    const uint64_t gen = generation_.load(std::memory_order_acquire);
+    if (last.generation == gen && p >= last.begin && p < last.end) {
+      return last.device;
+    }
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      auto it = ranges_.upper_bound(p);
+      if (it != ranges_.begin()) {
+        --it;
+        if (p < it->second.end) {
+          last = Last{it->first, it->second.end, it->second.device, gen};
+          return it->second.device;
+        }
+      }
+    }
+    int dev = -1;
+    int isHost = 0;
+    TP_HIP_CHECK(tphip_device_for_ptr(ptr, &dev, &isHost));
+    if (dev < 0) {
+      return -1; // memory the runtime has never seen: not something a kernel may touch
+    }
+    void* base = nullptr;
+    size_t size = 0;
+    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr || size == 0) {
+      return dev; // known to the runtime, extent unknown: answer, do not remember
+    }
+    const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (ranges_.size() >= 4096) {
+      ranges_.clear();
+      generation_.fetch_add(1, std::memory_order_acq_rel);
+    }
+    // whatever overlapped the new range has been freed since
+    auto it = ranges_.lower_bound(b);
+    if (it != ranges_.begin() && std::prev(it)->second.end > b) {
+      --it;
+    }
+    while (it != ranges_.end() && it->first < b + size) {
+      it = ranges_.erase(it);
+      generation_.fetch_add(1, std::memory_order_acq_rel);
+    }
+    ranges_[b] = Range{b + size, dev};
+    return dev;
   }
-  int dev = -1;
-  int isHost = 0;
-  TP_HIP_CHECK(tphip_device_for_ptr(ptr, &dev, &isHost));
-  return isHost ? -1 : dev;
+
+ private:
+  struct Range {
+    uintptr_t end;
+    int device;
+  };
+  std::mutex mutex_;
+  std::map<uintptr_t, Range> ranges_;
+  std::atomic<uint64_t> generation_{1};
+};
+
+} // namespace
+
+int hipDeviceForPointer(const void* ptr) {
+  static PointerRanges* ranges = new PointerRanges();
+  return ranges->lookup(ptr);
 }
 
 Device HipBuffer::getDevice() const {

@@ -28,9 +28,11 @@ TP_AMD_NAMESPACE_BEGIN
 // Number of usable GPUs; 0 when the runtime reports none or fails to load.
 int hipDeviceCountNoThrow();
 
-// Device index owning the device pointer ptr (tensorpipe/common/cuda.h:141-166).
-// Callers pass pointers taken from a HipBuffer, i.e. device memory; on a
-// multi-GPU machine a host pointer yields -1.
+// Device index owning ptr (tensorpipe/common/cuda.h:141-166): device memory and
+// pinned host memory yield their device, memory the runtime does not know
+// (plain host memory, null) yields -1, which callers turn into an exception as
+// the reference's driver check does. Answers are remembered per allocation, so
+// the runtime is asked once per allocation and not once per tensor.
 int hipDeviceForPointer(const void* ptr);
 
 class HipEvent {

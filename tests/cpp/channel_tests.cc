@@ -199,6 +199,50 @@ std::vector<Case> makeCases() {
          ep.barrier();
        }});
 
+  // Several receives posted ahead of tensors that take several wire units each
+  // (3.5 MiB against the 1 MiB staging slots of the chunking suites), every
+  // tensor with bytes of its own: a unit handed to the wrong operation shows.
+  {
+    auto pattern = [](int k) {
+      std::vector<uint8_t> v(3 * 1024 * 1024 + 512 * 1024 + 17);
+      for (size_t j = 0; j < v.size(); ++j) {
+        v[j] = static_cast<uint8_t>((j * 7 + static_cast<size_t>(k) * 37 + (j >> 12)) % 251);
+      }
+      return v;
+    };
+    cases.push_back(
+        {"SeveralChunkedTensorsPostedAhead",
+         [pattern](Endpoint& ep) {
+           auto o = open(ep);
+           std::vector<std::unique_ptr<Data>> ds;
+           std::vector<std::future<Error>> fs;
+           for (int k = 0; k < 4; ++k) {
+             ds.push_back(makeData(gGpu, pattern(k)));
+             fs.push_back(sendF(*o->ch, ds.back()->buffer(), ds.back()->size()));
+           }
+           for (auto& f : fs) {
+             EXPECT_OK(waitFor(f, "send"));
+           }
+           ep.barrier();
+         },
+         [pattern](Endpoint& ep) {
+           auto o = open(ep);
+           std::vector<std::unique_ptr<Data>> ds;
+           std::vector<std::future<Error>> fs;
+           for (int k = 0; k < 4; ++k) {
+             ds.push_back(makeData(gGpu, pattern(k).size()));
+             fs.push_back(recvF(*o->ch, ds.back()->buffer(), ds.back()->size()));
+           }
+           for (auto& f : fs) {
+             EXPECT_OK(waitFor(f, "recv"));
+           }
+           for (int k = 0; k < 4; ++k) {
+             expectBytes(*ds[k], pattern(k), "tensor");
+           }
+           ep.barrier();
+         }});
+  }
+
   // channel_test.cc:191-259: one send and one recv in flight on each side.
   auto bothWays = [](Endpoint& ep) {
     auto o = open(ep);

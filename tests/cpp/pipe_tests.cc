@@ -645,6 +645,43 @@ std::vector<Case> makeCases() {
     cases.push_back(twoInFlight("MultipleWriteReadWithGpuTensors", m1, m2, {kCpu}, {kGpu, kGpu}));
   }
 
+  // Two messages in flight whose GPU tensors each take several wire units in
+  // the cross-process channel (outbox route, 1 MiB slots): the second read is
+  // posted while the first tensor's chunks are still arriving.
+  if (gHaveGpu) {
+    auto big = [](int k) {
+      std::string v(3 * 1024 * 1024 + 300 * 1024 + 5, '\0');
+      for (size_t j = 0; j < v.size(); ++j) {
+        v[j] = static_cast<char>((j * 13 + static_cast<size_t>(k) * 101 + (j >> 11)) % 253);
+      }
+      return v;
+    };
+    InlineMessage m1, m2;
+    m1.metadata = m2.metadata = "message metadata";
+    m1.tensors = {{big(1), "tensor metadata #1.1", kGpu, kGpu}, {big(2), "tensor metadata #1.2", kGpu, kGpu}};
+    m2.tensors = {{big(3), "tensor metadata #2.1", kGpu, kGpu}};
+    Case inner = twoInFlight("ChunkedGpuTensorsTwoInFlight", m1, m2, {kGpu, kGpu}, {kGpu});
+    auto staged = [](std::function<void(Endpoint&)> fn) {
+      return [fn](Endpoint& ep) {
+        ::setenv("TP_HIP_IPC_MODE", "outbox", 1);
+        ::setenv("TP_HIP_IPC_SLOT_BYTES", "1048576", 1);
+        ::setenv("TP_HIP_IPC_NUM_SLOTS", "3", 1);
+        try {
+          fn(ep);
+        } catch (...) {
+          ::unsetenv("TP_HIP_IPC_MODE");
+          ::unsetenv("TP_HIP_IPC_SLOT_BYTES");
+          ::unsetenv("TP_HIP_IPC_NUM_SLOTS");
+          throw;
+        }
+        ::unsetenv("TP_HIP_IPC_MODE");
+        ::unsetenv("TP_HIP_IPC_SLOT_BYTES");
+        ::unsetenv("TP_HIP_IPC_NUM_SLOTS");
+      };
+    };
+    cases.push_back({inner.name, staged(inner.server), staged(inner.client)});
+  }
+
   // context_test.cc:634-738 (MixedTensorMessage): two reads are posted before
   // anything arrives; a message with payloads and tensors is followed by one
   // with nothing in it at all.

@@ -30,6 +30,8 @@
 #include <signal.h>
 #include <unistd.h>
 
+#include <tphip.h>
+
 #include <tensorpipe/common/buffer.h>
 #include <tensorpipe/common/cpu_buffer.h>
 #include <tensorpipe/common/device.h>
@@ -39,7 +41,7 @@
 #include <tensorpipe/common/wire.h>
 #include <tensorpipe/channel/error.h>
 #include <tensorpipe/tensorpipe.h>
-#include <tensorpipe/tensorpipe_cuda.h>
+#include <tensorpipe/tensorpipe_hip.h>
 #include <tensorpipe/transport/connection.h>
 #include <tensorpipe/transport/listener.h>
 
@@ -162,15 +164,6 @@ static int runBasics() {
   WireReader bad(lying, sizeof(lying));
   CHECK(bad.str().empty() && !bad.ok());
 
-  // The reference's names resolve to the HIP side (tensorpipe/tensorpipe_cuda.h).
-  CudaBuffer cb{reinterpret_cast<void*>(0x3000), nullptr};
-  Buffer viaAlias = cb;
-  CHECK(viaAlias.unwrap<HipBuffer>().ptr == reinterpret_cast<void*>(0x3000));
-  std::shared_ptr<channel::Context> (*makeXth)() = &channel::cuda_xth::create;
-  std::shared_ptr<channel::Context> (*makeIpc)() = &channel::cuda_ipc::create;
-  std::shared_ptr<channel::Context> (*makeBasic)(std::shared_ptr<channel::Context>) =
-      &channel::cuda_basic::create;
-  CHECK(makeXth != nullptr && makeIpc != nullptr && makeBasic != nullptr);
   CHECK(kCudaDeviceType == "cuda");
 
   if (failed == 0) {
@@ -353,6 +346,46 @@ static int runGarbage(int argc, char** argv) {
   return rc;
 }
 
+// What a HipBuffer may wrap: device memory and pinned host memory name their
+// device; plain host memory is refused with std::runtime_error, as the
+// reference's driver query does (tensorpipe/common/cuda.h:141-166,
+// tensorpipe/common/cuda_buffer.cc:16-28). Needs a GPU.
+static int runPointers() {
+  int failed = 0;
+  void* dev = nullptr;
+  CHECK(tphip_malloc(0, 1 << 20, &dev) == 0);
+  void* pinned = nullptr;
+  void* pinnedDev = nullptr;
+  CHECK(tphip_host_alloc(0, 1 << 16, &pinned, &pinnedDev) == 0);
+  std::vector<uint8_t> heap(4096);
+  uint8_t onStack[64];
+  for (int round = 0; round < 3; ++round) { // the second and third answers come from the range table
+    CHECK((HipBuffer{dev, nullptr}.getDevice() == Device{kHipDeviceType, 0}));
+    CHECK((HipBuffer{static_cast<uint8_t*>(dev) + (1 << 20) - 1, nullptr}.getDevice().index == 0));
+    CHECK((HipBuffer{pinned, nullptr}.getDevice().index == 0));
+    for (void* bad : {static_cast<void*>(heap.data()), static_cast<void*>(onStack), static_cast<void*>(nullptr)}) {
+      bool threw = false;
+      try {
+        (void)(HipBuffer{bad, nullptr}.getDevice());
+      } catch (const std::runtime_error&) {
+        threw = true;
+      }
+      CHECK(threw);
+    }
+  }
+  // an address that is freed keeps no stale answer once something else lives there
+  CHECK(tphip_free(0, dev) == 0);
+  void* again = nullptr;
+  CHECK(tphip_malloc(0, 1 << 12, &again) == 0);
+  CHECK((HipBuffer{again, nullptr}.getDevice().index == 0));
+  CHECK(tphip_free(0, again) == 0);
+  CHECK(tphip_host_free(pinned) == 0);
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
 // A crash names its stack before the process dies.
 static void onFatalSignal(int sig) {
   void* frames[48];
@@ -379,6 +412,9 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "departed_peer") == 0) {
     return runDepartedPeer();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | garbage <seed> <n>\n", argv[0]);
+  if (argc == 2 && std::strcmp(argv[1], "pointers") == 0) {
+    return runPointers();
+  }
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n>\n", argv[0]);
   return 2;
 }

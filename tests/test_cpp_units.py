@@ -67,6 +67,12 @@ def test_messages_of_a_departed_peer_are_delivered():
     assert rc == 0 and out.strip() == "OK", out
 
 
+@pytest.mark.gpu
+def test_host_pointer_in_a_hip_buffer_is_refused():
+    rc, out = run("pointers")
+    assert rc == 0 and out.strip() == "OK", out
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_garbage_on_new_connections(seed):
     # random bytes where the first packets of a pipe belong: the listening context survives them
