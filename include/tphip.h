@@ -163,6 +163,26 @@ int tphip_batched_copy(int dev, const tphip_copy_desc* table, uint32_t n, void* 
 int tphip_batched_copy_signal(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                               void* event, int unroll, uint32_t blocks, int nontemporal);
 
+/* tphip_batched_copy for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no
+ * counterpart in the reference. tphip_batched_copy keeps the plans of larger
+ * tables in rings of pinned and device memory that it allocates on first use;
+ * this variant calls no hipMalloc, hipHostMalloc, hipFree or other allocating
+ * routine, ever: its plan is written, by small kernels that carry it in their
+ * arguments, into a device array that is part of the library image
+ * (45 KiB per GPU the library runs on, held until the process ends), and the
+ * same table kernel then reads it from there. Same table semantics and results
+ * as tphip_batched_copy. Limits: n <= TPHIP_NOALLOC_MAX_BATCH, and the table's
+ * 16-byte vectors must fit one launch (just under 64 GiB); beyond either the
+ * call returns TPHIP_ERR_TOO_LARGE and enqueues nothing. All calls on one GPU
+ * share that GPU's array: calls on one stream are ordered by the stream, calls
+ * that may overlap on different streams of one GPU race and must be ordered
+ * by the caller. Under capture every replay rewrites the array with the
+ * captured plan before copying, so the same rule holds between a replay and
+ * any other call. */
+#define TPHIP_NOALLOC_MAX_BATCH 1024u
+int tphip_batched_copy_noalloc(int dev, const tphip_copy_desc* table, uint32_t n, void* stream);
+
 /* Single-copy convenience wrapper over the same kernel (n == 1, descriptor
  * travels in the kernel arguments). */
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream);

@@ -109,6 +109,7 @@ def tphip():
         lib.tphip_ipc_event_open.argtypes = [i32, ctypes.c_char_p, P(vp)]
         lib.tphip_batched_copy.argtypes = [i32, P(CopyDesc), u32, vp]
         lib.tphip_batched_copy_signal.argtypes = [i32, P(CopyDesc), u32, vp, vp, i32, u32, i32]
+        lib.tphip_batched_copy_noalloc.argtypes = [i32, P(CopyDesc), u32, vp]
         lib.tphip_copy.argtypes = [i32, vp, vp, u64, vp]
         lib.tphip_batched_copy_tuned.argtypes = [i32, P(CopyDesc), u32, vp, i32, u32, i32]
         lib.tphip_profile_start.argtypes = [i32, u32]

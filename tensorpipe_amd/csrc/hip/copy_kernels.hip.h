@@ -398,6 +398,26 @@ __global__ __launch_bounds__(kBlockThreads) void stage_plan_kernel(
   }
 }
 
+// A piece of a plan carried in the kernel arguments, written to device memory
+// at `byteOffset` of `dst` by one workgroup. Lets a caller that may not touch
+// pinned host memory or the copy engines put a plan of any size into device
+// memory with nothing but kernel launches.
+constexpr uint32_t kPlanPieceWords = 896;
+struct PlanPiece {
+  uint32_t words; // used entries of data[]
+  uint32_t byteOffset; // multiple of 4
+  uint32_t data[kPlanPieceWords];
+};
+static_assert(sizeof(PlanPiece) <= 3600, "kernel argument budget");
+
+__global__ __launch_bounds__(kBlockThreads) void write_plan_piece_kernel(
+    const PlanPiece piece, char* __restrict__ dst) {
+  uint32_t* out = reinterpret_cast<uint32_t*>(dst + piece.byteOffset);
+  for (uint32_t i = threadIdx.x; i < piece.words; i += kBlockThreads) {
+    out[i] = piece.data[i];
+  }
+}
+
 __global__ __launch_bounds__(kBlockThreads) void fill_kernel(
     unsigned char* __restrict__ p, unsigned char value, uint64_t n) {
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kBlockThreads;

@@ -319,15 +319,14 @@ int launchInline(int unroll, uint32_t blocks, hipStream_t stream, const InlinePl
 
 // Workgroups for `units` work units of one workgroup-iteration each: enough to
 // give every unit a workgroup, capped at blocksPerCu * CUs (or `blocks`).
-uint32_t pickBlocks(const DeviceState& st, uint64_t units, uint32_t minBlocks, uint32_t blocks,
-                    bool table) {
+uint32_t pickBlocks(int numCus, uint64_t units, uint32_t minBlocks, uint32_t blocks, bool table) {
   uint64_t want = units > minBlocks ? units : minBlocks;
   if (want == 0) {
     want = 1;
   }
   const uint64_t cap = blocks != 0
       ? blocks
-      : static_cast<uint64_t>(st.numCus > 0 ? st.numCus : 256) * defaultBlocksPerCu(table);
+      : static_cast<uint64_t>(numCus > 0 ? numCus : 256) * defaultBlocksPerCu(table);
   return static_cast<uint32_t>(want < cap ? want : cap);
 }
 
@@ -347,7 +346,7 @@ int copySingle(DeviceState& st, const tphip_copy_desc& d, hipStream_t stream, in
   }
   const uint64_t nvec = d.bytes >> 4;
   const uint64_t perBlock = uint64_t(kBlockThreads) * unroll;
-  const uint32_t grid = pickBlocks(st, (nvec + perBlock - 1) / perBlock, 1, blocks, false);
+  const uint32_t grid = pickBlocks(st.numCus, (nvec + perBlock - 1) / perBlock, 1, blocks, false);
   const char* src = static_cast<const char*>(d.src);
   char* dst = static_cast<char*>(d.dst);
   ProfileScope prof(st, stream, d.bytes);
@@ -399,7 +398,7 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     plan.n = n;
     plan.nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
     const uint32_t edgeBlocks = (n + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
-    const uint32_t grid = pickBlocks(st, plan.nchunks, edgeBlocks, blocks, true);
+    const uint32_t grid = pickBlocks(st.numCus, plan.nchunks, edgeBlocks, blocks, true);
     ProfileScope prof(st, stream, payloadBytes);
     switch (nt & 3) {
       case 0:
@@ -479,7 +478,7 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     const uint32_t nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
     // one wave per kEdgeGroup entries for the heads and tails
     const uint32_t edgeBlocks = (n + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
-    const uint32_t grid = pickBlocks(st, nchunks, edgeBlocks, blocks, true);
+    const uint32_t grid = pickBlocks(st.numCus, nchunks, edgeBlocks, blocks, true);
     const size_t lds = prefixBytes + (n <= kLdsBodies ? bodyBytes : 0);
     const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
     const CopyBody* dBodies = reinterpret_cast<const CopyBody*>(devp + prefixBytes);
@@ -634,6 +633,155 @@ int batchedCopyImpl(int dev, const tphip_copy_desc* table, uint32_t n, void* str
   return 0;
 }
 
+// ---- the entry point that allocates nothing ---------------------------------
+//
+// Its plan lives in a device array of the library image instead of the plan
+// ring (which is allocated on first use). Each GPU holds its own copy of the
+// array at its own address; the name below is only the host-side handle that
+// hipGetSymbolAddress turns into that address, once per device.
+constexpr size_t kNoAllocPrefixBytes =
+    ((TPHIP_NOALLOC_MAX_BATCH + 1) * sizeof(uint32_t) + 15) / 16 * 16;
+constexpr size_t kNoAllocPlanBytes =
+    kNoAllocPrefixBytes + TPHIP_NOALLOC_MAX_BATCH * (sizeof(CopyBody) + sizeof(tphip_copy_desc));
+constexpr size_t kNoAllocScratchBytes = (kNoAllocPlanBytes + 255) / 256 * 256;
+
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+struct NoAllocDevice {
+  std::once_flag once;
+  int initError{0};
+  int numCus{0};
+  char* scratchPtr{nullptr}; // this device's copy of `scratch`
+};
+NoAllocDevice gNoAlloc[kMaxDevices];
+
+// Call with `dev` current.
+int getNoAllocDevice(int dev, NoAllocDevice** out) {
+  NoAllocDevice& st = gNoAlloc[dev];
+  std::call_once(st.once, [&] {
+    hipError_t e = hipDeviceGetAttribute(&st.numCus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      st.scratchPtr = static_cast<char*>(p);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+    }
+    st.initError = static_cast<int>(e);
+  });
+  if (st.initError != 0) {
+    return st.initError;
+  }
+  if (st.scratchPtr == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  *out = &st;
+  return 0;
+}
+
+int noAllocCopy(int dev, const tphip_copy_desc* table, uint32_t n, hipStream_t stream) {
+  if (table == nullptr && n != 0) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  if (n > TPHIP_NOALLOC_MAX_BATCH) {
+    return TPHIP_ERR_TOO_LARGE;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  for (uint32_t i = 0; i < n; ++i) {
+    if (table[i].bytes != 0 && (table[i].src == nullptr || table[i].dst == nullptr)) {
+      return TPHIP_ERR_INVALID_ARG;
+    }
+  }
+  TPHIP_ON_DEVICE(dev);
+  NoAllocDevice* st = nullptr;
+  int rc = getNoAllocDevice(dev, &st);
+  if (rc != 0) {
+    return rc;
+  }
+
+  // The plan, built on the stack: prefix | bodies | descriptors of the
+  // non-empty entries (the layout batched_copy_kernel reads).
+  alignas(16) unsigned char plan[kNoAllocPlanBytes];
+  uint32_t m = 0;
+  for (uint32_t i = 0; i < n; ++i) {
+    m += table[i].bytes != 0 ? 1 : 0;
+  }
+  if (m == 0) {
+    return 0;
+  }
+  const size_t prefixBytes = ((size_t(m) + 1) * sizeof(uint32_t) + 15) / 16 * 16;
+  const size_t bodyBytes = size_t(m) * sizeof(CopyBody);
+  const size_t planBytes = prefixBytes + bodyBytes + size_t(m) * sizeof(tphip_copy_desc);
+  memset(plan, 0, prefixBytes);
+  uint32_t* prefix = reinterpret_cast<uint32_t*>(plan);
+  CopyBody* bodies = reinterpret_cast<CopyBody*>(plan + prefixBytes);
+  tphip_copy_desc* descs = reinterpret_cast<tphip_copy_desc*>(plan + prefixBytes + bodyBytes);
+  uint64_t total = 0;
+  uint64_t payloadBytes = 0;
+  uint32_t k = 0;
+  for (uint32_t i = 0; i < n; ++i) {
+    const uint64_t bytes = table[i].bytes;
+    if (bytes == 0) {
+      continue;
+    }
+    uint64_t head = (0 - reinterpret_cast<uintptr_t>(table[i].dst)) & 15u;
+    if (head > bytes) {
+      head = bytes;
+    }
+    prefix[k] = static_cast<uint32_t>(total);
+    bodies[k].src = static_cast<const char*>(table[i].src) + head;
+    bodies[k].dst = static_cast<char*>(table[i].dst) + head;
+    descs[k] = table[i];
+    total += (bytes - head) >> 4;
+    payloadBytes += bytes;
+    ++k;
+    if (total > kMaxTableVectors) {
+      return TPHIP_ERR_TOO_LARGE; // beyond what one launch can index
+    }
+  }
+  prefix[m] = static_cast<uint32_t>(total);
+
+  // Plan -> this device's scratch array, a kernel-argument load at a time.
+  for (size_t off = 0; off < planBytes; off += kPlanPieceWords * 4) {
+    PlanPiece piece;
+    const size_t bytes = planBytes - off < kPlanPieceWords * 4 ? planBytes - off : kPlanPieceWords * 4;
+    piece.words = static_cast<uint32_t>((bytes + 3) / 4);
+    piece.byteOffset = static_cast<uint32_t>(off);
+    memcpy(piece.data, plan + off, bytes);
+    rc = launchKernel(write_plan_piece_kernel, dim3(1), dim3(kBlockThreads), 0, stream, piece,
+                      st->scratchPtr);
+    if (rc != 0) {
+      return rc;
+    }
+  }
+
+  const int unroll = defaultUnroll(true);
+  const int nt = defaultNontemporal(payloadBytes);
+  const uint64_t chunk = uint64_t(kBlockThreads) * unroll;
+  const uint32_t nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
+  const uint32_t edgeBlocks = (m + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
+  const uint32_t grid = pickBlocks(st->numCus, nchunks, edgeBlocks, 0, true);
+  const size_t lds = prefixBytes + bodyBytes; // m <= kLdsBodies
+  const char* devp = st->scratchPtr;
+  const uint32_t* dPrefix = reinterpret_cast<const uint32_t*>(devp);
+  const CopyBody* dBodies = reinterpret_cast<const CopyBody*>(devp + prefixBytes);
+  const tphip_copy_desc* dDescs =
+      reinterpret_cast<const tphip_copy_desc*>(devp + prefixBytes + bodyBytes);
+  switch (nt & 3) {
+    case 0:
+      return launchTable<0>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, m, nchunks);
+    case 1:
+      return launchTable<1>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, m, nchunks);
+    case 2:
+      return launchTable<2>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, m, nchunks);
+    default:
+      return launchTable<3>(unroll, grid, lds, stream, dPrefix, dBodies, dDescs, m, nchunks);
+  }
+}
+
 struct HostFnThunk {
   tphip_host_fn fn;
   void* arg;
@@ -656,7 +804,7 @@ const char* tphip_strerror(int err) {
     case TPHIP_ERR_INVALID_ARG:
       return "tphip: invalid argument";
     case TPHIP_ERR_TOO_LARGE:
-      return "tphip: table larger than TPHIP_MAX_BATCH";
+      return "tphip: table larger than this entry point takes in one call";
     case TPHIP_ERR_NO_DEVICE:
       return "tphip: no usable GPU";
     case TPHIP_ERR_CAPTURING:
@@ -946,6 +1094,10 @@ int tphip_batched_copy_signal(int dev, const tphip_copy_desc* table, uint32_t n,
   }
   return batchedCopyImpl(dev, table, n, stream, unroll, blocks,
                          nontemporal < 0 ? -1 : (nontemporal & 3), static_cast<hipEvent_t>(event));
+}
+
+int tphip_batched_copy_noalloc(int dev, const tphip_copy_desc* table, uint32_t n, void* stream) {
+  return noAllocCopy(dev, table, n, static_cast<hipStream_t>(stream));
 }
 
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {
