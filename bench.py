@@ -28,6 +28,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+TRAFFIC_PROFILE = "profiles/single_copy_kernel_d2d_64MiB_pmc_fetch_write.txt"
 HBM_PEAK_GBPS = 8000.0
 PCIE_PEAK_GBPS = 63.0
 MIB = 1 << 20
@@ -50,6 +51,33 @@ def profiled(fn, max_launches):
     _native.check(lib.tphip_profile_stop(0, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(nbytes)),
                   "profile_stop")
     return out, n.value, ms.value, nbytes.value
+
+
+def traffic_from_profile(path, kernel):
+    """HBM-side bytes per launch of `kernel` from a committed rocprofv3 --pmc summary under
+    profiles/: average FETCH_SIZE and WRITE_SIZE per dispatch (KiB), each times the calibration
+    factor the summary's header states for it. None when the file or the rows are not there."""
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, path)).read()
+    except OSError:
+        return None
+    factors, values = {}, {}
+    for line in text.splitlines():
+        m = re.match(r"#\s*(FETCH_SIZE|WRITE_SIZE):.*", line)
+        if m:
+            current = m.group(1)
+        f = re.search(r"-> factor ([0-9.]+)", line)
+        if f and line.startswith("#") and "current" in locals():
+            factors[current] = float(f.group(1))
+        cols = line.split()
+        if kernel in line and not line.startswith("#") and len(cols) >= 5 and cols[-5] in ("FETCH_SIZE", "WRITE_SIZE"):
+            values[cols[-5]] = float(cols[-3])
+    if set(values) != {"FETCH_SIZE", "WRITE_SIZE"} or set(factors) != {"FETCH_SIZE", "WRITE_SIZE"}:
+        return None
+    kib = values["FETCH_SIZE"] * factors["FETCH_SIZE"] + values["WRITE_SIZE"] * factors["WRITE_SIZE"]
+    return int(kib * 1024)
 
 
 def make_pair(channels):
@@ -139,10 +167,10 @@ def bench_d2d(steps, warmup):
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            # HBM bytes per launch from the two rocprofv3 --pmc passes over this command (FETCH_SIZE x 2.000
-            # + WRITE_SIZE x 1.000, in KiB; see the profile named below): 1.0003 x the algorithmic bytes.
-            "traffic": int(131111.6 * 1024),
-            "traffic_source": "profiles/single_copy_kernel_d2d_64MiB_pmc_fetch_write.txt",
+            # HBM-side bytes per launch from the two rocprofv3 --pmc passes over this command
+            # (FETCH_SIZE and WRITE_SIZE, scaled as the named summary says), read from that file
+            "traffic": traffic_from_profile(TRAFFIC_PROFILE, "tphip::single_copy_kernel<4, 0>"),
+            "traffic_source": TRAFFIC_PROFILE,
             "kernel": "tphip::single_copy_kernel<4, 0>", "kernel_avg_us": kernel_us,
             "algorithmic_bytes_per_launch": 2 * nbytes,
         },
@@ -323,9 +351,10 @@ def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
     try:
         size = 4096
         while size <= max_bytes:
-            sample = min(size, 16 * MIB)  # seeded values in the first 16 MiB, repeated beyond
-            host = datagen.normal(datagen.SEED_BASE + 3, sample // 4, "f32").view(np.uint8)
-            src = torch.from_numpy(host).cuda().repeat(size // sample)
+            # seeded N(0,1) over the whole tensor, no two 16 MiB blocks alike
+            host = datagen.normal_large(datagen.SEED_BASE + 3, size // 4, "f32").view(np.uint8)
+            src = torch.from_numpy(host).cuda()
+            del host
             dst = torch.zeros(size, dtype=torch.uint8, device="cuda")
             st = [tp.make_tensor(src, target=(tp.HIP, 0))]
             rt = [tp.make_tensor(dst)]
@@ -370,9 +399,10 @@ def bench_staged(iters=50, warmup=3, nbytes=256 * MIB):
     from tensorpipe_amd import pipe as tp
 
     out = {}
-    sample = 16 * MIB
-    host = datagen.normal(datagen.SEED_BASE + 4, sample // 2, "bf16").view(np.uint8)
-    src = torch.from_numpy(host).cuda().repeat(nbytes // sample)
+    # seeded N(0,1) in bf16 over the whole tensor, no two 8 MiB blocks alike
+    host = datagen.normal_large(datagen.SEED_BASE + 4, nbytes // 2, "bf16").view(np.uint8)
+    src = torch.from_numpy(host).cuda()
+    del host
     dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
     for chunk in (1 * MIB, 4 * MIB):
         env = {"TP_HIP_BASIC_SLOT_BYTES": str(chunk), "TP_HIP_BASIC_NUM_SLOTS": "4"}
@@ -551,12 +581,24 @@ LEGS = {
 
 
 def run_leg(name, timeout_s=600, env=None):
-    proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--leg", name],
-                          stdout=subprocess.PIPE, timeout=timeout_s,
-                          env=dict(os.environ, **(env or {})))
+    """One configuration in a process (group) of its own; whatever happens, nothing of it is
+    left running afterwards."""
+    import signal
+
+    proc = subprocess.Popen([sys.executable, os.path.abspath(__file__), "--leg", name],
+                            stdout=subprocess.PIPE, env=dict(os.environ, **(env or {})),
+                            start_new_session=True)
+    try:
+        out, _ = proc.communicate(timeout=timeout_s)
+    finally:
+        try:
+            os.killpg(proc.pid, signal.SIGKILL)  # the leg's peer process too, should it still be there
+        except ProcessLookupError:
+            pass
+        proc.wait()
     if proc.returncode != 0:
         raise RuntimeError(f"bench leg {name} failed with exit code {proc.returncode}")
-    return json.loads(proc.stdout.decode().strip().splitlines()[-1])
+    return json.loads(out.decode().strip().splitlines()[-1])
 
 
 def extra_leg(name, env=None):

@@ -33,6 +33,7 @@ extern "C" {
 /* (-3 is not in use) */
 #define TPHIP_ERR_NO_DEVICE (-4)
 #define TPHIP_ERR_CAPTURING (-5)
+#define TPHIP_ERR_BUSY (-6)
 
 /* One entry of the copy table: `bytes` bytes from `src` to `dst`. Any
  * alignment, any length (including 0). Ranges of different entries must not
@@ -135,13 +136,13 @@ int tphip_ipc_event_open(int dev, const uint8_t handle[TPHIP_IPC_HANDLE_BYTES], 
 
 /* The hot path. Enqueue on `stream` ONE copy kernel that performs every copy
  * of `table[0..n)`; `table` is host memory and may be reused as soon as the
- * call returns. Tables of up to 64 entries travel in the kernel arguments (one
+ * call returns. Tables of up to 256 entries travel in the kernel arguments (one
  * launch in all); larger ones are written to a pinned plan ring and moved to
  * device memory by a small staging kernel enqueued ahead of the copy kernel. Any mix of device, mapped-pinned-host and peer-mapped (IPC)
  * addresses is accepted as long as the device can address them. n == 0 or an
  * all-empty table enqueues nothing. n > TPHIP_MAX_BATCH returns
  * TPHIP_ERR_TOO_LARGE. A call whose plan travels in the kernel arguments (up
- * to 64 non-empty entries; tphip_copy always) may be captured into a HIP
+ * to 256 non-empty entries; tphip_copy always) may be captured into a HIP
  * graph: every replay copies between the same addresses. A larger table on a
  * capturing stream returns TPHIP_ERR_CAPTURING and enqueues nothing, because
  * the plan ring is rewritten by later calls. Replaces one cudaMemcpyAsync per tensor at the three
@@ -182,6 +183,56 @@ int tphip_batched_copy_signal(int dev, const tphip_copy_desc* table, uint32_t n,
  * any other call. */
 #define TPHIP_NOALLOC_MAX_BATCH 1024u
 int tphip_batched_copy_noalloc(int dev, const tphip_copy_desc* table, uint32_t n, void* stream);
+
+/* ---- signal words and the resident copy agent ------------------------------ */
+
+/* Raises the 64-bit word at `word` (an address kernels can write: device
+ * memory, mapped pinned host memory, a peer's page mapped through an IPC
+ * handle) to `value` in stream order, behind everything enqueued on `stream`
+ * so far. The word is then seen by kernels and CPUs of every process that has
+ * the memory mapped. Stands in for cudaEventRecord on an inter-process event,
+ * tensorpipe/channel/cuda_ipc/channel_impl.cc:238-252 (exporting a HIP event
+ * to another process is refused where this library was built). */
+int tphip_stream_signal(int dev, void* stream, void* word, uint64_t value);
+
+/* tphip_batched_copy_signal behind a gate: a one-wavefront kernel enqueued
+ * ahead of the copies waits, on the GPU, until the 64-bit word at `gate_word`
+ * (readable by kernels of this device) has reached `gate_value`; the copy
+ * kernels start when it has ended. The receiving half of tphip_stream_signal,
+ * standing in for cudaStreamWaitEvent on an inter-process event,
+ * tensorpipe/channel/cuda_ipc/channel_impl.cc:453-457. The wait is bounded:
+ * if the word is not there after `max_wait_us` the gate raises the word at
+ * `expired_word` (which the caller has zeroed; writable by kernels, readable
+ * by the caller) to 1 and the copy kernels of the call do nothing, so the
+ * stream always drains. Once `event` has completed the caller reads
+ * *expired_word: non-zero means nothing was copied and the call must be
+ * repeated. Up to 256 gated calls may be in flight per GPU. */
+int tphip_batched_copy_gated(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
+                             void* event, const void* gate_word, uint64_t gate_value,
+                             uint32_t max_wait_us, void* expired_word);
+
+/* The resident copy agent: one workgroup that, once started, watches a ring
+ * of commands in pinned host memory and performs small copies a few
+ * microseconds after the host posted them -- no launch per copy. It starts
+ * with the first submission, leaves by itself when nothing has come for
+ * TPHIP_AGENT_IDLE_US (default 50) or after TPHIP_AGENT_LIFE_US (default
+ * 1000) and is started again on demand; tphip_agent_destroy stops it and
+ * waits for it. Copies are NOT ordered with any stream: the caller submits
+ * only what is ready to be read and free to be written. The reference has no
+ * counterpart (every one of its copies is a cudaMemcpyAsync). */
+int tphip_agent_create(int dev, void** agent);
+int tphip_agent_destroy(void* agent);
+/* Posts the non-empty entries of table[0..n) (n <= 32) in order; *ticket
+ * names the last one. After it has been copied, and made visible to every
+ * process, `notify` (may be NULL; same kinds of address as for
+ * tphip_stream_signal) is raised to `notify_value` (< 2^48). Returns
+ * TPHIP_ERR_BUSY, posting nothing, when the ring cannot take the table now. */
+int tphip_agent_submit(void* agent, const tphip_copy_desc* table, uint32_t n, void* notify,
+                       uint64_t notify_value, uint64_t* ticket);
+/* *done = 1 once the command named by `ticket` (and all before it) has been
+ * served. Call it until then: it also restarts an agent that left before it
+ * saw the command. */
+int tphip_agent_done(void* agent, uint64_t ticket, int* done);
 
 /* Single-copy convenience wrapper over the same kernel (n == 1, descriptor
  * travels in the kernel arguments). */

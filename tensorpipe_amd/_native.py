@@ -111,6 +111,12 @@ def tphip():
         lib.tphip_batched_copy_signal.argtypes = [i32, P(CopyDesc), u32, vp, vp, i32, u32, i32]
         lib.tphip_batched_copy_noalloc.argtypes = [i32, P(CopyDesc), u32, vp]
         lib.tphip_copy.argtypes = [i32, vp, vp, u64, vp]
+        lib.tphip_stream_signal.argtypes = [i32, vp, vp, u64]
+        lib.tphip_batched_copy_gated.argtypes = [i32, P(CopyDesc), u32, vp, vp, vp, u64, u32, vp]
+        lib.tphip_agent_create.argtypes = [i32, P(vp)]
+        lib.tphip_agent_destroy.argtypes = [vp]
+        lib.tphip_agent_submit.argtypes = [vp, P(CopyDesc), u32, vp, u64, P(u64)]
+        lib.tphip_agent_done.argtypes = [vp, u64, P(i32)]
         lib.tphip_batched_copy_tuned.argtypes = [i32, P(CopyDesc), u32, vp, i32, u32, i32]
         lib.tphip_profile_start.argtypes = [i32, u32]
         lib.tphip_profile_stop.argtypes = [i32, P(u32), P(ctypes.c_double), P(u64)]

@@ -463,6 +463,7 @@ struct TransferChain : std::enable_shared_from_this<TransferChain> {
     if (round >= warmup && perIterUs != nullptr) {
       perIterUs[round - warmup] = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
     }
+    TP_MARK("harness: step over");
     ++round;
     step();
   }

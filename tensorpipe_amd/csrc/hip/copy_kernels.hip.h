@@ -27,6 +27,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "tphip.h"
@@ -71,6 +72,71 @@ __device__ __forceinline__ uint64_t shfl64(uint64_t v, int srcLane) {
   return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
+// ---- signal words -----------------------------------------------------------
+//
+// 64-bit words in pinned host memory that both ends of a channel have mapped
+// (their own page and, through an IPC handle, the peer's). A word is raised to
+// a value once -- by a kernel in stream order, by a copy when it has finished,
+// or by a CPU -- and read by kernels and CPUs of either process. They stand in
+// for the inter-process events of the reference
+// (tensorpipe/channel/cuda_ipc/channel_impl.cc:238-252,453-463): the GPU orders
+// producer, copy and consumer by itself and the hosts only watch memory.
+
+__device__ __forceinline__ uint64_t read_signal(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Everything this thread wrote before is visible to whoever sees the value.
+__device__ __forceinline__ void raise_signal(uint64_t* p, uint64_t value) {
+  __hip_atomic_store(p, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// A copy may be told to wait for a signal word before it touches its sources:
+// the sender raises the word in stream order behind the work that produces the
+// tensor (tphip_stream_signal) and announces the tensor at once; the receiver
+// enqueues a gate kernel and, behind it on the same stream, the copy. The gate
+// kernel is one wavefront that watches the word; the copy kernel is not
+// resident meanwhile (256 workgroups polling a word in host memory while the
+// producer still runs cost the producer two thirds of its bandwidth), it
+// starts when the gate kernel has ended and first looks at the verdict the
+// gate left in device memory. The wait is bounded: after `maxTicks` of the
+// 100 MHz wall clock the gate gives up, says so in *expired (for the host) and
+// in *state (for the copy, which then does nothing), and the host enqueues the
+// pair again.
+constexpr uint64_t kGateOpen = 1;
+constexpr uint64_t kGateExpired = 2;
+
+__global__ void gate_kernel(
+    const uint64_t* word, uint64_t value, uint64_t maxTicks, uint64_t* expired, uint64_t* state) {
+  if (threadIdx.x != 0) {
+    return;
+  }
+  uint64_t verdict = kGateOpen;
+  const uint64_t t0 = wall_clock64();
+  while (read_signal(word) < value) {
+    if (wall_clock64() - t0 > maxTicks) {
+      verdict = kGateExpired;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(4);
+  }
+  if (verdict == kGateExpired) {
+    raise_signal(expired, 1);
+  }
+  __hip_atomic_store(state, verdict, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct Gate {
+  const uint64_t* state; // nullptr: no gate; else the verdict of the gate kernel ahead on the stream
+};
+
+__device__ __forceinline__ bool pass_gate(const Gate& g) {
+  if (g.state == nullptr) {
+    return true;
+  }
+  return __hip_atomic_load(g.state, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == kGateOpen;
+}
+
 // Entries whose heads and tails one wavefront moves. The gather below is a
 // chain of dependent byte loads and stores (about one memory latency per 64
 // bytes), so a group is kept small and the groups spread over many waves: 64
@@ -80,14 +146,13 @@ constexpr uint32_t kEdgeGroup = 8;
 
 // One wavefront moves the heads and tails of entries
 // [kEdgeGroup*group, kEdgeGroup*(group+1)); all 64 lanes share the byte copies.
-__device__ __forceinline__ void copy_edges(
-    const tphip_copy_desc* __restrict__ descs, uint32_t n, uint32_t group, uint32_t lane) {
+// `entry(t, &src, &dst, &bytes)` yields entry t as the caller gave it.
+template <typename Entry>
+__device__ __forceinline__ void copy_edges(Entry entry, uint32_t n, uint32_t group, uint32_t lane) {
   uint32_t t = group * kEdgeGroup + lane;
   uint64_t src = 0, dst = 0, bytes = 0;
   if (lane < kEdgeGroup && t < n) {
-    src = reinterpret_cast<uint64_t>(descs[t].src);
-    dst = reinterpret_cast<uint64_t>(descs[t].dst);
-    bytes = descs[t].bytes;
+    entry(t, &src, &dst, &bytes);
   }
   uint32_t head = head_bytes(reinterpret_cast<const void*>(dst), bytes);
   uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
@@ -152,11 +217,11 @@ constexpr uint32_t kLdsBodies = 1024;
 // part of a microsecond.
 // The work of a table copy once the plan is where the workgroup can read it
 // cheaply: sPrefix (and normally body) in LDS, descs wherever they are.
-template <int U, int NT>
+template <int U, int NT, typename Entry>
 __device__ __forceinline__ void table_copy(
     const uint32_t* sPrefix,
     const CopyBody* body,
-    const tphip_copy_desc* descs,
+    Entry entry,
     uint32_t n,
     uint32_t nchunks) {
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -291,7 +356,7 @@ __device__ __forceinline__ void table_copy(
   // out of chunks first): the byte-wise gather is latency-bound and would
   // otherwise delay the chunks of the workgroup that does it.
   for (uint32_t g = nwaves - 1 - wave; g * kEdgeGroup < n; g += nwaves) {
-    copy_edges(descs, n, g, lane);
+    copy_edges(entry, n, g, lane);
   }
 }
 
@@ -301,8 +366,12 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
     const CopyBody* __restrict__ bodies,
     const tphip_copy_desc* __restrict__ descs,
     uint32_t n,
-    uint32_t nchunks) {
+    uint32_t nchunks,
+    const Gate gate) {
   extern __shared__ __align__(16) uint32_t sPrefix[];
+  if (!pass_gate(gate)) {
+    return;
+  }
   const bool cached = n <= kLdsBodies;
   CopyBody* sBodies = reinterpret_cast<CopyBody*>(sPrefix + ((n + 1 + 3) & ~3u));
   for (uint32_t i = threadIdx.x; i <= n; i += kBlockThreads) {
@@ -314,34 +383,78 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
     }
   }
   __syncthreads();
-  table_copy<U, NT>(sPrefix, cached ? sBodies : bodies, descs, n, nchunks);
+  table_copy<U, NT>(
+      sPrefix,
+      cached ? sBodies : bodies,
+      [descs](uint32_t t, uint64_t* src, uint64_t* dst, uint64_t* bytes) {
+        *src = reinterpret_cast<uint64_t>(descs[t].src);
+        *dst = reinterpret_cast<uint64_t>(descs[t].dst);
+        *bytes = descs[t].bytes;
+      },
+      n,
+      nchunks);
 }
 
 // Small tables travel in the kernel arguments: no plan upload, no staging
-// kernel, nothing to recycle afterwards -- one launch is the whole cost. The
-// struct is a plain array of 32-bit words so that every lane can fetch its
-// share with one indexed load.
-constexpr uint32_t kInlineEntries = 64;
+// kernel, nothing to recycle afterwards -- one launch is the whole cost (the
+// runtime writes kernel arguments into device memory, 5.4 KiB of them for 256
+// entries cost about a microsecond more per launch call than a few bytes).
+// What travels is what the workgroups keep in LDS anyway: the prefix sums, the
+// bodies, and one byte per entry holding how many bytes precede and follow the
+// body (4 bits each), from which the wave that moves heads and tails rebuilds
+// the entry as the caller gave it. Two sizes, so that a two-tensor message
+// does not pay for 256 entries.
+constexpr uint32_t kInlineEntries = 256;
+constexpr uint32_t kInlineEntriesSmall = 64;
 
-struct InlinePlan {
+template <uint32_t N>
+struct InlinePlanT {
   uint32_t n;
   uint32_t nchunks;
-  uint32_t prefix[kInlineEntries + 2]; // n+1 used; padded to keep 8-byte alignment below
-  CopyBody bodies[kInlineEntries];
-  tphip_copy_desc descs[kInlineEntries];
+  uint32_t prefix[N + 2]; // n+1 used; padded to keep 8-byte alignment below
+  CopyBody bodies[N];
+  uint8_t edges[N]; // head << 4 | tail
 };
-static_assert(sizeof(InlinePlan) % 4 == 0 && sizeof(InlinePlan) <= 3072, "kernel argument budget");
+static_assert(sizeof(InlinePlanT<kInlineEntries>) % 4 == 0, "copied word by word");
+static_assert(sizeof(InlinePlanT<kInlineEntriesSmall>) % 4 == 0, "copied word by word");
+static_assert(sizeof(InlinePlanT<kInlineEntries>) <= 6144, "kernel argument budget");
 
-template <int U, int NT>
-__global__ __launch_bounds__(kBlockThreads) void inline_copy_kernel(const InlinePlan plan) {
-  __shared__ __align__(16) InlinePlan sPlan;
+template <int U, int NT, uint32_t N>
+__global__ __launch_bounds__(kBlockThreads) void inline_copy_kernel(
+    const InlinePlanT<N> plan, const Gate gate) {
+  __shared__ __align__(16) InlinePlanT<N> sPlan;
+  if (!pass_gate(gate)) {
+    return;
+  }
+  // Only what n entries use: header + prefix, bodies, edge bytes.
+  const uint32_t n = plan.n;
   const uint32_t* in = reinterpret_cast<const uint32_t*>(&plan);
   uint32_t* out = reinterpret_cast<uint32_t*>(&sPlan);
-  for (uint32_t i = threadIdx.x; i < sizeof(InlinePlan) / 4; i += kBlockThreads) {
+  constexpr uint32_t kBodiesAt = offsetof(InlinePlanT<N>, bodies) / 4;
+  constexpr uint32_t kEdgesAt = offsetof(InlinePlanT<N>, edges) / 4;
+  for (uint32_t i = threadIdx.x; i < 2 + n + 1; i += kBlockThreads) {
     out[i] = in[i];
   }
+  for (uint32_t i = threadIdx.x; i < n * 4; i += kBlockThreads) {
+    out[kBodiesAt + i] = in[kBodiesAt + i];
+  }
+  for (uint32_t i = threadIdx.x; i < (n + 3) / 4; i += kBlockThreads) {
+    out[kEdgesAt + i] = in[kEdgesAt + i];
+  }
   __syncthreads();
-  table_copy<U, NT>(sPlan.prefix, sPlan.bodies, sPlan.descs, sPlan.n, sPlan.nchunks);
+  const InlinePlanT<N>* p = &sPlan;
+  table_copy<U, NT>(
+      sPlan.prefix,
+      sPlan.bodies,
+      [p](uint32_t t, uint64_t* src, uint64_t* dst, uint64_t* bytes) {
+        const uint32_t head = p->edges[t] >> 4;
+        const uint32_t tail = p->edges[t] & 15u;
+        *src = reinterpret_cast<uint64_t>(p->bodies[t].src) - head;
+        *dst = reinterpret_cast<uint64_t>(p->bodies[t].dst) - head;
+        *bytes = head + (static_cast<uint64_t>(p->prefix[t + 1] - p->prefix[t]) << 4) + tail;
+      },
+      n,
+      sPlan.nchunks);
 }
 
 // Single-entry variant: the descriptor travels in the kernel arguments, no
@@ -350,7 +463,10 @@ __global__ __launch_bounds__(kBlockThreads) void inline_copy_kernel(const Inline
 // one contiguous G*U*16-byte window per iteration.
 template <int U, int NT>
 __global__ __launch_bounds__(kBlockThreads) void single_copy_kernel(
-    const char* __restrict__ src, char* __restrict__ dst, uint64_t bytes) {
+    const char* __restrict__ src, char* __restrict__ dst, uint64_t bytes, const Gate gate) {
+  if (!pass_gate(gate)) {
+    return;
+  }
   const uint64_t g = static_cast<uint64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
   const uint64_t G = static_cast<uint64_t>(gridDim.x) * kBlockThreads;
   const uint32_t head = head_bytes(dst, bytes);
@@ -395,6 +511,150 @@ __global__ __launch_bounds__(kBlockThreads) void stage_plan_kernel(
   for (uint32_t i = blockIdx.x * kBlockThreads + threadIdx.x; i < nvec;
        i += gridDim.x * kBlockThreads) {
     devPlan[i] = hostPlan[i];
+  }
+}
+
+// Raises a word in stream order: enqueued behind the work that produces a
+// tensor, it tells the peer's copy that the bytes are there.
+__global__ void raise_signal_kernel(uint64_t* word, uint64_t value) {
+  if (threadIdx.x == 0) {
+    raise_signal(word, value);
+  }
+}
+
+// One workgroup copies `bytes` bytes, any alignment: the same head / body /
+// tail split as the grid-wide kernels, four vectors in flight per lane.
+__device__ __forceinline__ void workgroup_copy(const char* src, char* dst, uint64_t bytes) {
+  const uint32_t tid = threadIdx.x;
+  const uint32_t head = head_bytes(dst, bytes);
+  const uint64_t nvec = (bytes - head) >> 4;
+  const uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
+  if (tid < head) {
+    dst[tid] = src[tid];
+  } else if (tid >= 16 && tid - 16 < tail) {
+    const uint64_t o = bytes - tail + (tid - 16);
+    dst[o] = src[o];
+  }
+  const char* s = src + head;
+  char* d = dst + head;
+  constexpr uint64_t kStep = 4ull * kBlockThreads;
+  const uint64_t full = nvec / kStep * kStep;
+#pragma clang loop unroll(disable)
+  for (uint64_t base = 0; base < full; base += kStep) {
+    u32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = load16<0>(s + (base + j * kBlockThreads + tid) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      store16<0>(d + (base + j * kBlockThreads + tid) * 16, v[j]);
+    }
+  }
+  for (uint64_t i = full + tid; i < nvec; i += kBlockThreads) {
+    store16<0>(d + i * 16, load16<0>(s + i * 16));
+  }
+}
+
+// ---- resident copy agent ------------------------------------------------------
+//
+// A launch costs about 7 us from the call to the host seeing the end of a
+// 4 KiB copy; a workgroup that is already running and watches a command ring
+// in pinned host memory does the same copy 2.5-3.5 us after the host wrote the
+// command. The agent is that workgroup: started when small transfers arrive,
+// it serves them while they keep coming and leaves by itself when nothing has
+// come for `idleTicks` of the 100 MHz wall clock, when `lifeTicks` have passed
+// since it started (so that no queue it may share with other work is held for
+// long), or on a stop command. The host starts it again when needed.
+//
+// A command is one 64-byte line written by the host: word 0 is its ticket
+// (tickets count up from 1), words 1-5 carry 48 bits of payload each under the
+// low 16 bits of the ticket as a tag in the top bits. The line may reach the
+// GPU in pieces, so a command counts as arrived only when ticket and all tags
+// agree -- no second round trip over the host link to re-read it.
+struct AgentCommand {
+  uint64_t w[8]; // ticket, src, dst, bytes, notify address, notify value, -, -
+};
+constexpr uint64_t kAgentPayloadMask = (1ull << 48) - 1;
+constexpr uint64_t kAgentStopBytes = kAgentPayloadMask; // "bytes" of the stop command
+
+struct AgentControl {
+  uint64_t done; // last ticket served (raised by the agent)
+  uint64_t exited; // epoch of the last agent that has left (raised by the agent)
+  uint64_t pad[6];
+};
+
+__global__ __launch_bounds__(kBlockThreads) void agent_kernel(
+    const AgentCommand* __restrict__ ring,
+    uint32_t ringMask,
+    AgentControl* __restrict__ ctl,
+    uint64_t ticket,
+    uint64_t epoch,
+    uint64_t idleTicks,
+    uint64_t lifeTicks) {
+  __shared__ uint64_t sCmd[5];
+  __shared__ int sLeave;
+  const uint64_t born = wall_clock64();
+  uint64_t lastWork = born;
+  for (;;) {
+    if (threadIdx.x < kWave) {
+      const uint32_t lane = threadIdx.x;
+      const AgentCommand* slot = ring + (ticket & ringMask);
+      const uint64_t tag = ticket & 0xffffu;
+      int leave = 0;
+      for (;;) {
+        uint64_t w = 0;
+        if (lane < 6) {
+          w = read_signal(&slot->w[lane]);
+        }
+        const bool ok = lane == 0 ? w == ticket : (lane < 6 ? (w >> 48) == tag : true);
+        if (__ballot(ok) == ~0ull) {
+          if (lane >= 1 && lane < 6) {
+            sCmd[lane - 1] = w & kAgentPayloadMask;
+          }
+          break;
+        }
+        const uint64_t now = wall_clock64();
+        if (now - lastWork > idleTicks || now - born > lifeTicks) {
+          leave = 1;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if (lane == 0) {
+        sLeave = leave;
+      }
+    }
+    __syncthreads();
+    if (sLeave != 0) {
+      break;
+    }
+    const uint64_t bytes = sCmd[2];
+    const bool stop = bytes == kAgentStopBytes;
+    if (!stop) {
+      // What other kernels (of this or the peer process) wrote since the last
+      // command must not be served from this workgroup's caches.
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+      workgroup_copy(reinterpret_cast<const char*>(sCmd[0]), reinterpret_cast<char*>(sCmd[1]), bytes);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+    }
+    const uint64_t notify = sCmd[3];
+    const uint64_t notifyValue = sCmd[4];
+    __syncthreads(); // every wave's stores are out; sCmd may be rewritten
+    if (threadIdx.x == 0) {
+      if (notify != 0) {
+        raise_signal(reinterpret_cast<uint64_t*>(notify), notifyValue);
+      }
+      raise_signal(&ctl->done, ticket);
+    }
+    if (stop) {
+      break;
+    }
+    ++ticket;
+    lastWork = wall_clock64();
+  }
+  if (threadIdx.x == 0) {
+    raise_signal(&ctl->exited, epoch);
   }
 }
 

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -51,7 +52,8 @@ struct DeviceState {
   hipEvent_t slotDone[kPlanSlots]{};
   bool slotUsed[kPlanSlots]{};
   uint32_t nextSlot{0};
-  std::mutex mutex;
+  std::mutex mutex; // nextSlot
+  std::mutex slotMutex[kPlanSlots]; // a slot from the wait for its last user to the record behind its next
   // Launch profiling (tphip_profile_start/stop).
   std::mutex profMutex;
   bool profiling{false};
@@ -68,6 +70,8 @@ thread_local hipEvent_t tlsProfStop = nullptr;
 // Event to attach to the next copy-kernel launch of this thread as its
 // completion signal (instead of a marker of its own behind the kernel).
 thread_local hipEvent_t tlsSignal = nullptr;
+// Gate for the copy launches of this thread's current call (tphip_batched_copy_gated).
+thread_local Gate tlsGate = {nullptr};
 
 class ProfileScope {
  public:
@@ -270,16 +274,16 @@ int launchSingle(int unroll, uint32_t blocks, hipStream_t stream, const char* sr
   switch (unroll) {
     case 1:
       return launchKernel(single_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
-                          dst, bytes);
+                          dst, bytes, tlsGate);
     case 2:
       return launchKernel(single_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
-                          dst, bytes);
+                          dst, bytes, tlsGate);
     case 8:
       return launchKernel(single_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
-                          dst, bytes);
+                          dst, bytes, tlsGate);
     default:
       return launchKernel(single_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, src,
-                          dst, bytes);
+                          dst, bytes, tlsGate);
   }
 }
 
@@ -290,30 +294,34 @@ int launchTable(int unroll, uint32_t blocks, size_t lds, hipStream_t stream,
   switch (unroll) {
     case 1:
       return launchKernel(batched_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, bodies, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks, tlsGate);
     case 2:
       return launchKernel(batched_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, bodies, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks, tlsGate);
     case 8:
       return launchKernel(batched_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, bodies, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks, tlsGate);
     default:
       return launchKernel(batched_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), lds, stream,
-                          prefix, bodies, descs, n, nchunks);
+                          prefix, bodies, descs, n, nchunks, tlsGate);
   }
 }
 
-template <int NT>
-int launchInline(int unroll, uint32_t blocks, hipStream_t stream, const InlinePlan& plan) {
+template <int NT, uint32_t N>
+int launchInline(int unroll, uint32_t blocks, hipStream_t stream, const InlinePlanT<N>& plan) {
   switch (unroll) {
     case 1:
-      return launchKernel(inline_copy_kernel<1, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+      return launchKernel(inline_copy_kernel<1, NT, N>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan,
+                          tlsGate);
     case 2:
-      return launchKernel(inline_copy_kernel<2, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+      return launchKernel(inline_copy_kernel<2, NT, N>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan,
+                          tlsGate);
     case 8:
-      return launchKernel(inline_copy_kernel<8, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+      return launchKernel(inline_copy_kernel<8, NT, N>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan,
+                          tlsGate);
     default:
-      return launchKernel(inline_copy_kernel<4, NT>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan);
+      return launchKernel(inline_copy_kernel<4, NT, N>, dim3(blocks), dim3(kBlockThreads), 0, stream, plan,
+                          tlsGate);
   }
 }
 
@@ -362,6 +370,48 @@ int copySingle(DeviceState& st, const tphip_copy_desc& d, hipStream_t stream, in
   }
 }
 
+// A table of at most N entries, plan in the kernel arguments.
+template <uint32_t N>
+int copyInline(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStream_t stream,
+               int unroll, uint32_t blocks, int nt, uint64_t payloadBytes) {
+  InlinePlanT<N> plan;
+  plan.n = n;
+  uint64_t total = 0;
+  for (uint32_t i = 0; i < n; ++i) {
+    plan.prefix[i] = static_cast<uint32_t>(total);
+    const uint64_t bytes = table[i].bytes;
+    uint64_t head = (0 - reinterpret_cast<uintptr_t>(table[i].dst)) & 15u;
+    if (head > bytes) {
+      head = bytes;
+    }
+    plan.bodies[i].src = static_cast<const char*>(table[i].src) + head;
+    plan.bodies[i].dst = static_cast<char*>(table[i].dst) + head;
+    plan.edges[i] = static_cast<uint8_t>((head << 4) | ((bytes - head) & 15u));
+    total += (bytes - head) >> 4;
+  }
+  for (uint32_t i = n; i < N + 2; ++i) {
+    plan.prefix[i] = static_cast<uint32_t>(total); // prefix[n] = total; the rest is never read
+  }
+  for (uint32_t i = n; i < N; ++i) {
+    plan.edges[i] = 0;
+  }
+  const uint64_t chunk = uint64_t(kBlockThreads) * unroll;
+  plan.nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
+  const uint32_t edgeBlocks = (n + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
+  const uint32_t grid = pickBlocks(st.numCus, plan.nchunks, edgeBlocks, blocks, true);
+  ProfileScope prof(st, stream, payloadBytes);
+  switch (nt & 3) {
+    case 0:
+      return launchInline<0>(unroll, grid, stream, plan);
+    case 1:
+      return launchInline<1>(unroll, grid, stream, plan);
+    case 2:
+      return launchInline<2>(unroll, grid, stream, plan);
+    default:
+      return launchInline<3>(unroll, grid, stream, plan);
+  }
+}
+
 // Launch one table kernel over table[0..n) whose body vector total fits 32 bits.
 int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStream_t stream,
               int unroll, uint32_t blocks, int nt) {
@@ -378,38 +428,9 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
 
   if (n <= kInlineEntries && inlinePlansEnabled()) {
     // The whole plan fits the kernel arguments.
-    InlinePlan plan;
-    memset(&plan, 0, sizeof(plan));
-    uint64_t total = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-      plan.prefix[i] = static_cast<uint32_t>(total);
-      const uint64_t bytes = table[i].bytes;
-      uint64_t head = (0 - reinterpret_cast<uintptr_t>(table[i].dst)) & 15u;
-      if (head > bytes) {
-        head = bytes;
-      }
-      plan.bodies[i].src = static_cast<const char*>(table[i].src) + head;
-      plan.bodies[i].dst = static_cast<char*>(table[i].dst) + head;
-      plan.descs[i] = table[i];
-      total += (bytes - head) >> 4;
-    }
-    plan.prefix[n] = static_cast<uint32_t>(total);
-    const uint64_t chunk = uint64_t(kBlockThreads) * unroll;
-    plan.n = n;
-    plan.nchunks = static_cast<uint32_t>((total + chunk - 1) / chunk);
-    const uint32_t edgeBlocks = (n + kEdgeGroup * kWavesPerBlock - 1) / (kEdgeGroup * kWavesPerBlock);
-    const uint32_t grid = pickBlocks(st.numCus, plan.nchunks, edgeBlocks, blocks, true);
-    ProfileScope prof(st, stream, payloadBytes);
-    switch (nt & 3) {
-      case 0:
-        return launchInline<0>(unroll, grid, stream, plan);
-      case 1:
-        return launchInline<1>(unroll, grid, stream, plan);
-      case 2:
-        return launchInline<2>(unroll, grid, stream, plan);
-      default:
-        return launchInline<3>(unroll, grid, stream, plan);
-    }
+    return n <= kInlineEntriesSmall
+        ? copyInline<kInlineEntriesSmall>(st, table, n, stream, unroll, blocks, nt, payloadBytes)
+        : copyInline<kInlineEntries>(st, table, n, stream, unroll, blocks, nt, payloadBytes);
   }
 
   // The plan ring is rewritten by later calls: a graph that captured this
@@ -432,6 +453,11 @@ int copyTable(DeviceState& st, const tphip_copy_desc* table, uint32_t n, hipStre
     std::lock_guard<std::mutex> lock(st.mutex);
     slot = st.nextSlot;
     st.nextSlot = (st.nextSlot + 1) % kPlanSlots;
+  }
+  {
+    // Only this slot is held while its last user is waited for: a slow stream
+    // there does not hold up table launches that take other slots.
+    std::lock_guard<std::mutex> lock(st.slotMutex[slot]);
     if (st.slotUsed[slot]) {
       // The launch that last used this slot must have consumed its plan.
       TPHIP_TRY(hipEventSynchronize(st.slotDone[slot]));
@@ -782,6 +808,59 @@ int noAllocCopy(int dev, const tphip_copy_desc* table, uint32_t n, hipStream_t s
   }
 }
 
+// ---- gates ------------------------------------------------------------------
+//
+// Verdicts of gate kernels, one word per gated call in flight, in a device
+// array of the library image (each GPU has its own copy; the host-side name is
+// turned into that GPU's address once).
+constexpr uint32_t kGateStates = 256;
+static __device__ __align__(256) uint64_t gateStates[kGateStates];
+
+struct GateDevice {
+  std::once_flag once;
+  int initError{0};
+  int wallClockKhz{0};
+  uint64_t* states{nullptr};
+  std::atomic<uint64_t> next{0};
+};
+GateDevice gGateDevices[kMaxDevices];
+
+// ---- resident copy agent ------------------------------------------------------
+
+constexpr uint32_t kAgentRing = 64; // commands the host may have posted ahead
+
+struct Agent {
+  int dev{0};
+  hipStream_t stream{nullptr};
+  AgentCommand* ring{nullptr}; // pinned host memory, as the host sees it
+  AgentCommand* ringDev{nullptr}; // and as kernels see it
+  AgentControl* ctl{nullptr};
+  AgentControl* ctlDev{nullptr};
+  uint64_t idleTicks{0};
+  uint64_t lifeTicks{0};
+  std::mutex mutex;
+  uint64_t nextTicket{1}; // under mutex
+  std::atomic<uint64_t> epoch{0}; // of the last launch
+  bool stopped{false}; // under mutex
+};
+
+uint64_t loadWord(const uint64_t* p) {
+  return __atomic_load_n(p, __ATOMIC_ACQUIRE);
+}
+
+// With the mutex held: starts an agent unless one is (still) running.
+int agentEnsureRunning(Agent& a) {
+  const uint64_t epoch = a.epoch.load(std::memory_order_relaxed);
+  if (epoch != 0 && loadWord(&a.ctl->exited) != epoch) {
+    return 0;
+  }
+  // The previous agent has left: what it served is final.
+  const uint64_t first = loadWord(&a.ctl->done) + 1;
+  a.epoch.store(epoch + 1, std::memory_order_release);
+  return launchKernel(agent_kernel, dim3(1), dim3(kBlockThreads), 0, a.stream, a.ringDev,
+                      kAgentRing - 1, a.ctlDev, first, epoch + 1, a.idleTicks, a.lifeTicks);
+}
+
 struct HostFnThunk {
   tphip_host_fn fn;
   void* arg;
@@ -807,8 +886,10 @@ const char* tphip_strerror(int err) {
       return "tphip: table larger than this entry point takes in one call";
     case TPHIP_ERR_NO_DEVICE:
       return "tphip: no usable GPU";
+    case TPHIP_ERR_BUSY:
+      return "tphip: the copy agent's command ring is full";
     case TPHIP_ERR_CAPTURING:
-      return "tphip: a table of more than 64 entries cannot be captured into a graph";
+      return "tphip: a table of more than 256 entries cannot be captured into a graph";
     default:
       return hipGetErrorString(static_cast<hipError_t>(err));
   }
@@ -1098,6 +1179,210 @@ int tphip_batched_copy_signal(int dev, const tphip_copy_desc* table, uint32_t n,
 
 int tphip_batched_copy_noalloc(int dev, const tphip_copy_desc* table, uint32_t n, void* stream) {
   return noAllocCopy(dev, table, n, static_cast<hipStream_t>(stream));
+}
+
+int tphip_stream_signal(int dev, void* stream, void* word, uint64_t value) {
+  if (word == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
+  return launchKernel(raise_signal_kernel, dim3(1), dim3(kWave), 0, static_cast<hipStream_t>(stream),
+                      static_cast<uint64_t*>(word), value);
+}
+
+int tphip_agent_create(int dev, void** agent) {
+  if (agent == nullptr || dev < 0 || dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
+  auto a = std::make_unique<Agent>();
+  a->dev = dev;
+  int khz = 0;
+  TPHIP_TRY(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+  if (khz <= 0) {
+    khz = 100000;
+  }
+  const int idleUs = envInt("TPHIP_AGENT_IDLE_US", 50);
+  const int lifeUs = envInt("TPHIP_AGENT_LIFE_US", 1000);
+  a->idleTicks = static_cast<uint64_t>(idleUs > 0 ? idleUs : 1) * khz / 1000;
+  a->lifeTicks = static_cast<uint64_t>(lifeUs > 0 ? lifeUs : 1) * khz / 1000;
+  void* host = nullptr;
+  const size_t bytes = sizeof(AgentCommand) * kAgentRing + sizeof(AgentControl);
+  TPHIP_TRY(hipHostMalloc(&host, bytes, hipHostMallocMapped | hipHostMallocPortable));
+  memset(host, 0, bytes);
+  void* devp = nullptr;
+  hipError_t e = hipHostGetDevicePointer(&devp, host, 0);
+  if (e == hipSuccess) {
+    e = hipStreamCreateWithFlags(&a->stream, hipStreamNonBlocking);
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipHostFree(host);
+    return static_cast<int>(e);
+  }
+  a->ring = static_cast<AgentCommand*>(host);
+  a->ringDev = static_cast<AgentCommand*>(devp);
+  a->ctl = reinterpret_cast<AgentControl*>(a->ring + kAgentRing);
+  a->ctlDev = reinterpret_cast<AgentControl*>(a->ringDev + kAgentRing);
+  *agent = a.release();
+  return 0;
+}
+
+int tphip_agent_submit(void* agent, const tphip_copy_desc* table, uint32_t n, void* notify,
+                       uint64_t notify_value, uint64_t* ticket) {
+  Agent* a = static_cast<Agent*>(agent);
+  if (a == nullptr || table == nullptr || n == 0 || n > kAgentRing / 2 || ticket == nullptr ||
+      notify_value > kAgentPayloadMask || reinterpret_cast<uintptr_t>(notify) > kAgentPayloadMask) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  uint32_t live = 0;
+  for (uint32_t i = 0; i < n; ++i) {
+    if (table[i].bytes == 0) {
+      continue;
+    }
+    if (table[i].src == nullptr || table[i].dst == nullptr || table[i].bytes >= kAgentStopBytes ||
+        reinterpret_cast<uintptr_t>(table[i].src) > kAgentPayloadMask ||
+        reinterpret_cast<uintptr_t>(table[i].dst) > kAgentPayloadMask) {
+      return TPHIP_ERR_INVALID_ARG;
+    }
+    ++live;
+  }
+  if (live == 0) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  std::lock_guard<std::mutex> lock(a->mutex);
+  if (a->stopped) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  if (a->nextTicket + live - 1 - loadWord(&a->ctl->done) > kAgentRing) {
+    return TPHIP_ERR_BUSY;
+  }
+  uint32_t k = 0;
+  for (uint32_t i = 0; i < n; ++i) {
+    if (table[i].bytes == 0) {
+      continue;
+    }
+    ++k;
+    const uint64_t t = a->nextTicket++;
+    const uint64_t tag = (t & 0xffffu) << 48;
+    AgentCommand& c = a->ring[t & (kAgentRing - 1)];
+    const bool last = k == live;
+    c.w[1] = reinterpret_cast<uintptr_t>(table[i].src) | tag;
+    c.w[2] = reinterpret_cast<uintptr_t>(table[i].dst) | tag;
+    c.w[3] = table[i].bytes | tag;
+    c.w[4] = (last ? reinterpret_cast<uintptr_t>(notify) : 0) | tag;
+    c.w[5] = (last ? notify_value : 0) | tag;
+    __atomic_store_n(&c.w[0], t, __ATOMIC_RELEASE);
+    *ticket = t;
+  }
+  TPHIP_ON_DEVICE(a->dev);
+  return agentEnsureRunning(*a);
+}
+
+int tphip_agent_done(void* agent, uint64_t ticket, int* done) {
+  Agent* a = static_cast<Agent*>(agent);
+  if (a == nullptr || done == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  if (loadWord(&a->ctl->done) >= ticket) {
+    *done = 1;
+    return 0;
+  }
+  *done = 0;
+  // An agent that left (idle, or its time was up) just before the command
+  // was posted has not seen it: start the next one.
+  const uint64_t epoch = a->epoch.load(std::memory_order_acquire);
+  if (epoch != 0 && loadWord(&a->ctl->exited) == epoch) {
+    std::lock_guard<std::mutex> lock(a->mutex);
+    if (!a->stopped && loadWord(&a->ctl->done) < a->nextTicket - 1) {
+      TPHIP_ON_DEVICE(a->dev);
+      return agentEnsureRunning(*a);
+    }
+  }
+  return 0;
+}
+
+int tphip_agent_destroy(void* agent) {
+  Agent* a = static_cast<Agent*>(agent);
+  if (a == nullptr) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  {
+    std::lock_guard<std::mutex> lock(a->mutex);
+    a->stopped = true;
+    const uint64_t epoch = a->epoch.load(std::memory_order_relaxed);
+    if (epoch != 0 && loadWord(&a->ctl->exited) != epoch) {
+      // A running agent leaves at this command (after everything posted before it).
+      const uint64_t t = a->nextTicket++;
+      const uint64_t tag = (t & 0xffffu) << 48;
+      AgentCommand& c = a->ring[t & (kAgentRing - 1)];
+      c.w[1] = tag;
+      c.w[2] = tag;
+      c.w[3] = kAgentStopBytes | tag;
+      c.w[4] = tag;
+      c.w[5] = tag;
+      __atomic_store_n(&c.w[0], t, __ATOMIC_RELEASE);
+    }
+  }
+  int rc = 0;
+  {
+    DeviceScope scope(a->dev);
+    hipError_t e = hipStreamSynchronize(a->stream);
+    if (e == hipSuccess) {
+      e = hipStreamDestroy(a->stream);
+    }
+    if (e == hipSuccess) {
+      e = hipHostFree(a->ring);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      rc = static_cast<int>(e);
+    }
+  }
+  delete a;
+  return rc;
+}
+
+int tphip_batched_copy_gated(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
+                             void* event, const void* gate_word, uint64_t gate_value,
+                             uint32_t max_wait_us, void* expired_word) {
+  if (event == nullptr || gate_word == nullptr || expired_word == nullptr || dev < 0 ||
+      dev >= kMaxDevices) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
+  GateDevice& gd = gGateDevices[dev];
+  std::call_once(gd.once, [&] {
+    hipError_t e = hipDeviceGetAttribute(&gd.wallClockKhz, hipDeviceAttributeWallClockRate, dev);
+    if (e == hipSuccess) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(gateStates));
+      gd.states = static_cast<uint64_t*>(p);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+    }
+    gd.initError = static_cast<int>(e);
+  });
+  if (gd.initError != 0) {
+    return gd.initError;
+  }
+  const int khz = gd.wallClockKhz > 0 ? gd.wallClockKhz : 100000;
+  uint64_t* state = gd.states + gd.next.fetch_add(1, std::memory_order_relaxed) % kGateStates;
+  int rc = launchKernel(gate_kernel, dim3(1), dim3(kWave), 0, static_cast<hipStream_t>(stream),
+                        static_cast<const uint64_t*>(gate_word), gate_value,
+                        static_cast<uint64_t>(max_wait_us) * khz / 1000,
+                        static_cast<uint64_t*>(expired_word), state);
+  if (rc != 0) {
+    return rc;
+  }
+  struct Disarm {
+    ~Disarm() {
+      tlsGate = Gate{nullptr};
+    }
+  } disarm;
+  tlsGate = Gate{state};
+  return batchedCopyImpl(dev, table, n, stream, 0, 0, -1, static_cast<hipEvent_t>(event));
 }
 
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {

@@ -45,7 +45,16 @@ HipEventPoller::~HipEventPoller() {
 void HipEventPoller::watch(std::unique_ptr<HipEvent> event, HipEventPool* pool, TCallback fn) {
   {
     std::lock_guard<std::mutex> lock(mutex_);
-    incoming_.push_back(Item{std::move(event), pool, std::move(fn)});
+    incoming_.push_back(Item{std::move(event), nullptr, pool, std::move(fn)});
+    incomingPending_.store(true, std::memory_order_release);
+  }
+  cv_.notify_one();
+}
+
+void HipEventPoller::watchCondition(TCheck check, TCallback fn) {
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    incoming_.push_back(Item{nullptr, std::move(check), nullptr, std::move(fn)});
     incomingPending_.store(true, std::memory_order_release);
   }
   cv_.notify_one();
@@ -118,17 +127,24 @@ void HipEventPoller::run() {
     bool any = false;
     for (auto it = active.begin(); it != active.end();) {
       int done = 0;
-      int rc = tphip_event_query(it->event->device(), it->event->raw(), &done);
+      int rc = 0;
+      if (it->event) {
+        rc = tphip_event_query(it->event->device(), it->event->raw(), &done);
+      } else {
+        bool happened = false;
+        rc = it->check(&happened);
+        done = happened ? 1 : 0;
+      }
       if (rc != 0 || done) {
         Item item = std::move(*it);
         it = active.erase(it);
         any = true;
         if (rc != 0) {
-          item.fn(TP_CREATE_ERROR(HipError, "tphip_event_query", rc));
+          item.fn(TP_CREATE_ERROR(HipError, item.event ? "tphip_event_query" : "completion check", rc));
         } else {
           item.fn(Error::kSuccess);
         }
-        if (item.pool != nullptr) {
+        if (item.pool != nullptr && item.event) {
           item.pool->put(std::move(item.event));
         }
       } else {

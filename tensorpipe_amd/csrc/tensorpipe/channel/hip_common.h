@@ -47,11 +47,19 @@ class HipEventPoller {
   // until the callback has run, then back to `pool` (if given).
   void watch(std::unique_ptr<HipEvent> event, HipEventPool* pool, TCallback fn);
 
+  // The same for anything else the host can only find out by looking: a
+  // signal word in shared pinned memory, a ticket of the copy agent. `check`
+  // sets *done once the awaited thing has happened and returns 0, or returns a
+  // tphip error code; it runs on the poller thread, again and again.
+  using TCheck = std::function<int(bool* done)>;
+  void watchCondition(TCheck check, TCallback fn);
+
   void join();
 
  private:
   struct Item {
-    std::unique_ptr<HipEvent> event;
+    std::unique_ptr<HipEvent> event; // or
+    TCheck check;
     HipEventPool* pool;
     TCallback fn;
   };

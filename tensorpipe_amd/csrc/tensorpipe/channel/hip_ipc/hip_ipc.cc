@@ -22,23 +22,52 @@
 //          writes per byte. Used when an allocation cannot be exported, or
 //          for everything when TP_HIP_IPC_MODE=outbox.
 //
-// Synchronisation between the two processes goes through the host: the sender
-// announces a tensor (or chunk) once a HIP event recorded behind the producing
-// work has completed, and the receiver replies once an event recorded behind
-// its copy has completed. Inter-process HIP events would let both sides skip
-// the host, as the reference does with CUDA IPC events, but exporting an event
-// fails on the deployment this was built for, so they are not used.
+// Synchronisation between the two processes. Exporting a HIP event to another
+// process fails on the deployment this was built for, so the inter-process
+// events of the reference (tensorpipe/channel/cuda_ipc/channel_impl.cc:238-252,
+// 453-463) are replaced by signal words: every channel end owns a few 64-bit
+// words in a pinned host page of its context, exported once; the peer maps the
+// page for its GPU (a peer's CPUs cannot reach a mapped page, only the owner's
+// can). For a unit small enough for the receiver's copy agent, the receiving
+// GPU raises acks[unit % 64] in the SENDER's page once the copy has finished
+// -- the agent does it as part of the command -- and the sender's host watches
+// that word of its own page: no reply message, no event polled for it. Other
+// units, and ends that have no page (TP_HIP_IPC_SIGNALS=0, or the export
+// failed), are acknowledged with a message on the reply connection; each unit
+// says which of the two its sender expects.
+//
+// A tensor whose producing work is still running on the sender's stream is
+// announced at once all the same: the sender raises ready[k % 64] of its page
+// in stream order behind that work (tphip_stream_signal) and names the word in
+// the unit; the receiver launches its copy gated on the word
+// (tphip_batched_copy_gated), so the copy starts on the GPU the moment the
+// bytes are there instead of an event poll, a message and a launch later. The
+// gate's wait is bounded and the launch repeated if it ran out, so no kernel
+// ever waits for good on something queued behind it; the recv callback of such
+// a unit fires when its copy has finished. This is switched on with
+// TP_HIP_IPC_GATES=1; by default, and without words on both ends, the sender
+// polls an event behind the producing work before it announces (see
+// gatesEnabled for the measurement behind that default).
+//
+// Small tensors whose source and destination streams have nothing pending are
+// copied by the context's resident copy agent (tphip_agent_*): no launch, the
+// bytes land about 3 us after the descriptor arrived. Everything else is one
+// batched copy launch on the caller's stream per unit.
 //
 // The recv callback fires when the copy has been enqueued on the caller's
-// stream (as in the reference); the send callback fires when the source may be
-// reused: after the receiver's reply (direct) or after the last chunk has been
-// staged (outbox).
+// stream (as in the reference), or, for a copy the agent does, when the bytes
+// have landed; callbacks fire in the order of the recv calls. The send
+// callback fires when the source may be reused: after the receiver's
+// acknowledgement (direct) or after the last chunk has been staged (outbox).
 
 #include <tensorpipe/channel/hip_ipc/factory.h>
 
 #include <algorithm>
 #include <array>
+#include <atomic>
+#include <chrono>
 #include <cstdlib>
+#include <cstring>
 #include <deque>
 #include <map>
 #include <mutex>
@@ -48,6 +77,7 @@
 #include <tensorpipe/channel/hip_common.h>
 #include <tensorpipe/common/hip_buffer.h>
 #include <tensorpipe/common/slot_allocator.h>
+#include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
 
 TP_AMD_NAMESPACE_BEGIN
@@ -153,11 +183,15 @@ class ExportRegistry {
         static_cast<const uint8_t*>(ptr) - static_cast<const uint8_t*>(base));
     std::lock_guard<std::mutex> lock(mutex_);
     auto it = exports_.find(base);
-    if (it != exports_.end() && it->second.size == size && it->second.bufferId == bufferId) {
+    if (bufferId != 0 && it != exports_.end() && it->second.size == size &&
+        it->second.bufferId == bufferId) {
       *out = it->second;
       return true;
     }
-    // New allocation, or the address was freed and handed out again.
+    // New allocation, or the address was freed and handed out again -- or the
+    // runtime cannot tell the two apart (no identifier): then every send
+    // exports afresh under a new identifier and nothing is remembered, rather
+    // than risk the peer reading a stale mapping of freed memory.
     ExportedAllocation e;
     if (tphip_ipc_mem_export(device, base, e.handle.data()) != 0) {
       return false;
@@ -166,9 +200,11 @@ class ExportRegistry {
     e.base = reinterpret_cast<uint64_t>(base);
     e.size = size;
     e.bufferId = bufferId;
-    exports_[base] = e;
     *out = e;
-    forgetFreedAllocations();
+    if (bufferId != 0) {
+      exports_[base] = e;
+      forgetFreedAllocations();
+    }
     return true;
   }
 
@@ -208,10 +244,134 @@ struct Outbox {
   const uint64_t id{nextExportId()};
 };
 
+// Signal words of one channel end (see the top of the file), all about the
+// units this end SENDS. Read and written by the owner's CPUs and by the GPU
+// on behalf of either process.
+constexpr size_t kWordSlots = 64;
+struct ChannelWords {
+  uint64_t acks[kWordSlots]; // acks[u % 64] == u + 1: the peer has copied unit u (raised by the peer's copy)
+  uint64_t ready[kWordSlots]; // ready[k % 64] > k: the sources of the k-th gated unit are ready (raised by the owner's stream)
+  uint64_t expired[kWordSlots]; // this end's own gated copies report here that they gave up waiting
+};
+constexpr size_t kChannelsPerSlab = 256;
+
+// Pinned page holding the words of up to kChannelsPerSlab channel ends of a
+// context, exported once.
+class SignalSlab {
+ public:
+  explicit SignalSlab(int device)
+      : slab_(device, sizeof(ChannelWords) * kChannelsPerSlab), device_(device) {
+    std::memset(slab_.host(), 0, slab_.size());
+    TP_HIP_CHECK(tphip_ipc_mem_export(device, slab_.host(), handle_.data()));
+    for (uint32_t i = 0; i < kChannelsPerSlab; ++i) {
+      free_.push_back(kChannelsPerSlab - 1 - i);
+    }
+  }
+  int acquire() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (free_.empty()) {
+      return -1;
+    }
+    const uint32_t i = free_.back();
+    free_.pop_back();
+    return static_cast<int>(i);
+  }
+  void release(int index) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    std::memset(hostWords(index), 0, sizeof(ChannelWords));
+    free_.push_back(static_cast<uint32_t>(index));
+  }
+  ChannelWords* hostWords(int index) const {
+    return reinterpret_cast<ChannelWords*>(slab_.host()) + index;
+  }
+  ChannelWords* devWords(int index) const {
+    return reinterpret_cast<ChannelWords*>(slab_.dev()) + index;
+  }
+  const HandleBytes& handle() const {
+    return handle_;
+  }
+  uint64_t id() const {
+    return id_;
+  }
+  uint64_t base() const {
+    return reinterpret_cast<uint64_t>(slab_.host());
+  }
+  uint64_t size() const {
+    return slab_.size();
+  }
+  int device() const {
+    return device_;
+  }
+
+ private:
+  HipPinnedSlab slab_;
+  int device_;
+  HandleBytes handle_;
+  const uint64_t id_{nextExportId()};
+  std::mutex mutex_;
+  std::vector<uint32_t> free_;
+};
+
+bool envFlag(const char* name, bool fallback) {
+  const char* e = std::getenv(name);
+  return e == nullptr || *e == 0 ? fallback : std::atoi(e) != 0;
+}
+
 class IpcContextCore final : public ContextCore {
  public:
   HipEventPool events;
   HipEventPoller poller;
+  // Signal words for the channels of this context; null when switched off
+  // (TP_HIP_IPC_SIGNALS=0) or when pinned memory cannot be exported here.
+  std::unique_ptr<SignalSlab> signals;
+  // Tensors of a unit adding up to at most this many bytes go to the copy
+  // agent when their streams are idle (TP_HIP_IPC_AGENT=0 switches it off,
+  // TP_HIP_IPC_AGENT_MAX_BYTES moves the limit).
+  const bool agentEnabled{envFlag("TP_HIP_IPC_AGENT", true)};
+  const size_t agentMaxBytes{envSize("TP_HIP_IPC_AGENT_MAX_BYTES", 64 * 1024)};
+  // How long the thread that posted a copy to the agent looks for its end
+  // itself before leaving that to the poller thread (TP_HIP_IPC_AGENT_SPIN_US).
+  const long agentSpinUs{static_cast<long>(envSize("TP_HIP_IPC_AGENT_SPIN_US", 8))};
+  // Gated copies are there, tested and switched off: TP_HIP_IPC_GATES=1 lets a
+  // sender whose stream is still producing announce at once and the receiver's
+  // GPU wait for its word. Measured against the host hand-off (event polled,
+  // then announced) in the ping-pong it is no faster on this stack -- the
+  // signal kernel behind the producer and the gate kernel ahead of the copy
+  // each cost a kernel-to-kernel gap of 3-4 us, which is what the host path
+  // costs too: 1 MiB 45.0 against 41.3 us per round trip, 64 MiB 76.0 against
+  // 74.9. A gate gives up after TP_HIP_IPC_GATE_WAIT_US (doubling up to 64
+  // times that on every further try).
+  const bool gatesEnabled{envFlag("TP_HIP_IPC_GATES", false)};
+  const uint32_t gateWaitUs{static_cast<uint32_t>(envSize("TP_HIP_IPC_GATE_WAIT_US", 2000))};
+
+  IpcContextCore() {
+    if (envFlag("TP_HIP_IPC_SIGNALS", true)) {
+      try {
+        signals = std::make_unique<SignalSlab>(0);
+      } catch (const std::exception& ex) {
+        TP_LOG_WARNING() << "hip_ipc: no signal words (" << ex.what()
+                         << "); acknowledging with messages";
+      }
+    }
+  }
+
+  // Loop only. The agent of `device`, created on first use; null if it cannot be.
+  void* agent(int device) {
+    if (!agentEnabled) {
+      return nullptr;
+    }
+    if (device >= static_cast<int>(agents_.size())) {
+      agents_.resize(device + 1, nullptr);
+    }
+    if (agents_[device] == nullptr && !agentFailed_) {
+      if (tphip_agent_create(device, &agents_[device]) != 0) {
+        agents_[device] = nullptr;
+        agentFailed_ = true;
+      }
+    }
+    return agents_[device];
+  }
+
   StreamIdleProbe idleProbe; // loop only
   StreamMarkers markers;
   const bool forceOutbox{outboxForcedByEnv()};
@@ -249,14 +409,22 @@ class IpcContextCore final : public ContextCore {
   }
 
   void joinImpl() override {
-    poller.join();
+    poller.join(); // nothing asks the agents about tickets any more
+    for (void*& a : agents_) {
+      if (a != nullptr) {
+        tphip_agent_destroy(a);
+        a = nullptr;
+      }
+    }
   }
 
  private:
   std::vector<std::unique_ptr<Outbox>> outboxes_;
+  std::vector<void*> agents_;
+  bool agentFailed_{false};
 };
 
-enum MsgKind : uint8_t { kDirect = 1, kChunk = 2 };
+enum MsgKind : uint8_t { kDirect = 1, kChunk = 2, kHello = 3 };
 
 class ChannelImpl final : public ChannelImplBase {
  public:
@@ -270,14 +438,18 @@ class ChannelImpl final : public ChannelImplBase {
         descriptorConnection_(std::move(descriptorConnection)),
         replyConnection_(std::move(replyConnection)) {}
 
-  // Every copy out of a mapped peer allocation is followed by an event whose
-  // watcher keeps this object alive, so nothing reads the mappings any more.
+  // Every copy out of a mapped peer allocation is followed by an event or an
+  // agent ticket whose watcher keeps this object alive, so nothing reads the
+  // mappings any more.
   ~ChannelImpl() override {
     for (auto& i : imports_) {
       HipIpcImports::get().release(i.device, i.peer, i.id);
     }
     for (auto& kv : remoteAllocations_) {
       HipIpcImports::get().release(kv.second.device, peerIdentity_, kv.first);
+    }
+    if (wordsIndex_ >= 0) {
+      ictx_->signals->release(wordsIndex_);
     }
   }
 
@@ -306,6 +478,39 @@ class ChannelImpl final : public ChannelImplBase {
   }
 
  protected:
+  // Both ends open with a hello: who they are and where their signal words
+  // live. It is the first message on the descriptor connection each way, so
+  // it is always there before the first unit.
+  void initFromLoop() override {
+    if (ictx_->signals) {
+      wordsIndex_ = ictx_->signals->acquire();
+    }
+    WireWriter w;
+    w.u8(kHello);
+    w.str(processIdentity());
+    w.u8(wordsIndex_ >= 0 ? 1 : 0);
+    if (wordsIndex_ >= 0) {
+      const SignalSlab& slab = *ictx_->signals;
+      w.u64(slab.id());
+      w.raw(slab.handle().data(), slab.handle().size());
+      w.u64(slab.base());
+      w.u64(slab.size());
+      w.u32(static_cast<uint32_t>(wordsIndex_ * sizeof(ChannelWords)));
+    }
+    // what this end's copy agent takes in one unit (0: it has none)
+    w.u64(ictx_->agentEnabled ? ictx_->agentMaxBytes : 0);
+    writeMessage(*descriptorConnection_, std::move(w.bytes()));
+    helloPending_ = true;
+    descriptorConnection_->read(onReadMessage([this](std::vector<uint8_t> bytes) {
+      helloPending_ = false;
+      if (error_) {
+        return;
+      }
+      onHello(bytes);
+      pumpUnits();
+    }));
+  }
+
   void sendFromLoop(uint64_t seq, Buffer buffer, size_t length, TSendCallback cb) override {
     std::vector<BatchEntry> entries;
     entries.push_back({std::move(buffer), length});
@@ -319,6 +524,14 @@ class ChannelImpl final : public ChannelImplBase {
   }
 
   void handleError() override {
+    cancel_->store(true, std::memory_order_release); // watchers of acknowledgement words give up
+    if (wordsIndex_ >= 0) {
+      // Copies of the peer that wait for a word of ours need not wait it out.
+      ChannelWords* mine = ictx_->signals->hostWords(wordsIndex_);
+      for (size_t k = 0; k < kWordSlots; ++k) {
+        __atomic_store_n(&mine->ready[k], ~uint64_t(0), __ATOMIC_RELEASE);
+      }
+    }
     descriptorConnection_->close();
     replyConnection_->close();
     // Slot requests still queued fail with AllocatorClosedError, as in
@@ -335,7 +548,10 @@ class ChannelImpl final : public ChannelImplBase {
     auto recvs = std::move(recvOps_);
     recvOps_.clear();
     for (auto& op : recvs) {
-      finishRecv(op);
+      // A buffer the agent is still writing is handed back when it has finished.
+      if (op->landing == 0) {
+        finishRecv(op);
+      }
     }
     wireQueue_.clear();
     replyQueue_.clear();
@@ -351,12 +567,27 @@ class ChannelImpl final : public ChannelImplBase {
   };
 
   // A unit that goes on the descriptor connection: a whole direct batch or one
-  // staged chunk. Units are written strictly in creation order.
+  // staged chunk. Units are written strictly in creation order. Every unit
+  // starts with {kind u8, acknowledgement mode u8, unit number u64}; the last
+  // two are filled in when the unit is written.
   struct WireUnit {
     std::vector<uint8_t> bytes;
     bool ready{false};
-    std::function<void()> onReply; // runs when the matching reply arrives
+    // Direct units: bytes and tensors in all, for the sender's guess whether
+    // the peer's copy agent will take the unit (0 tensors: a staged chunk).
+    uint64_t totalBytes{0};
+    uint32_t tensors{0};
+    std::function<void()> onReply; // runs when the unit has been acknowledged
   };
+  static constexpr size_t kUnitHeaderBytes = 10;
+  static constexpr uint32_t kAgentMaxTensors = 16;
+  enum AckMode : uint8_t { kAckByMessage = 0, kAckByWord = 1 };
+
+  static void unitHeader(WireWriter& w, MsgKind kind) {
+    w.u8(kind);
+    w.u8(kAckByMessage);
+    w.u64(0);
+  }
 
   struct SendOp {
     uint64_t seq;
@@ -371,6 +602,8 @@ class ChannelImpl final : public ChannelImplBase {
     std::vector<BatchEntry> entries;
     size_t unitsExpected{0};
     size_t unitsSeen{0};
+    bool allSeen{false}; // every unit of the op has arrived and its copy is enqueued or posted
+    size_t landing{0}; // units handed to the copy agent whose bytes have not landed yet
     bool done{false};
   };
 
@@ -382,6 +615,48 @@ class ChannelImpl final : public ChannelImplBase {
 
   size_t numChunks(size_t length) const {
     return (length + ictx_->slotBytes - 1) / ictx_->slotBytes;
+  }
+
+  void onHello(const std::vector<uint8_t>& bytes) {
+    WireReader r(bytes.data(), bytes.size());
+    if (r.u8() != kHello) {
+      failProtocol();
+      return;
+    }
+    peerIdentity_ = r.str();
+    const bool hasWords = r.u8() != 0;
+    if (!r.ok() || peerIdentity_.empty()) {
+      failProtocol();
+      return;
+    }
+    if (!hasWords) {
+      peerAgentMaxBytes_ = r.u64();
+      if (!r.ok()) {
+        failProtocol();
+      }
+      return;
+    }
+    const uint64_t id = r.u64();
+    HandleBytes h;
+    r.raw(h.data(), h.size());
+    const uint64_t base = r.u64();
+    const uint64_t size = r.u64();
+    const uint32_t offset = r.u32();
+    peerAgentMaxBytes_ = r.u64();
+    peerGates_ = true; // an end with words of its own can run gated copies
+    if (!r.ok() || size < sizeof(ChannelWords) || offset > size - sizeof(ChannelWords) ||
+        offset % alignof(ChannelWords) != 0) {
+      failProtocol();
+      return;
+    }
+    void* mapped = nullptr;
+    const int rc = HipIpcImports::get().acquire(0, peerIdentity_, id, h, base, size, &mapped);
+    if (rc != 0) {
+      setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open (signal words)", rc));
+      return;
+    }
+    imports_.push_back(Import{0, peerIdentity_, id});
+    peerWords_ = reinterpret_cast<ChannelWords*>(static_cast<uint8_t*>(mapped) + offset);
   }
 
   // ---- send -----------------------------------------------------------------
@@ -397,6 +672,7 @@ class ChannelImpl final : public ChannelImplBase {
       cb(error_); // zero length: tensorpipe/channel/cuda_ipc/channel_impl.cc:112-115
       return;
     }
+    TP_MARK("ipc: send");
     auto op = std::make_shared<SendOp>();
     op->seq = seq;
     op->cb = std::move(cb);
@@ -455,12 +731,14 @@ class ChannelImpl final : public ChannelImplBase {
         }
         WireWriter w;
         w.reserve(64 + 96 * allocs.size() + 24 * direct.size());
-        w.u8(kDirect);
-        w.u8(identitySent_ ? 0 : 1);
-        if (!identitySent_) {
-          w.str(processIdentity());
-          identitySent_ = true;
-        }
+        unitHeader(w, kDirect);
+        // gate: {used u8, word u32, value u64}, filled in below if one is used
+        const size_t gateAt = w.bytes().size();
+        uint32_t gateSlot = 0;
+        uint64_t gateValue = 0;
+        w.u8(0);
+        w.u32(0);
+        w.u64(0);
         w.u32(static_cast<uint32_t>(allocs.size()));
         for (const ExportedAllocation* a : allocs) {
           w.u64(a->id);
@@ -477,6 +755,10 @@ class ChannelImpl final : public ChannelImplBase {
         }
         auto unit = std::make_shared<WireUnit>();
         unit->bytes = std::move(w.bytes());
+        unit->tensors = static_cast<uint32_t>(direct.size());
+        for (auto& d : direct) {
+          unit->totalBytes += d.length;
+        }
         // The source may be reused once the receiver has copied it.
         ++op->pending;
         unit->onReply = [this, op] { sendStepDone(op); };
@@ -488,6 +770,26 @@ class ChannelImpl final : public ChannelImplBase {
           if (!ictx_->idleProbe.idle(s.device, s.stream)) {
             busy.push_back(s);
           }
+        }
+        if (busy.size() == 1 && wordsIndex_ >= 0 && peerGates_ && ictx_->gatesEnabled) {
+          // One stream still producing: its last kernel is followed by a word
+          // the receiver's copy waits for on the GPU.
+          const uint64_t k = nextGate_++;
+          gateSlot = static_cast<uint32_t>(k % kWordSlots);
+          gateValue = k + 1;
+          TP_HIP_CHECK(tphip_stream_signal(
+              busy[0].device,
+              busy[0].stream,
+              &ictx_->signals->devWords(wordsIndex_)->ready[gateSlot],
+              gateValue));
+          // a marker, so that the runtime knows when the stream has drained
+          auto marker = ictx_->events.get(busy[0].device);
+          marker->record(busy[0].stream);
+          ictx_->events.put(std::move(marker));
+          unit->bytes[gateAt] = 1;
+          std::memcpy(unit->bytes.data() + gateAt + 1, &gateSlot, sizeof(gateSlot));
+          std::memcpy(unit->bytes.data() + gateAt + 5, &gateValue, sizeof(gateValue));
+          busy.clear();
         }
         if (busy.empty()) {
           unit->ready = true;
@@ -529,7 +831,7 @@ class ChannelImpl final : public ChannelImplBase {
 
   // Outbox path, one chunk: wait for a slot, copy source -> slot on the
   // caller's stream, announce the slot when the copy is done, free the slot
-  // when the receiver has replied.
+  // when the receiver has acknowledged it.
   void stageChunk(
       const std::shared_ptr<SendOp>& op,
       const std::shared_ptr<WireUnit>& unit,
@@ -571,7 +873,7 @@ class ChannelImpl final : public ChannelImplBase {
         return;
       }
       WireWriter w;
-      w.u8(kChunk);
+      unitHeader(w, kChunk);
       w.u32(index);
       w.u32(static_cast<uint32_t>(device));
       const bool announce = !outboxAnnounced_[device];
@@ -590,7 +892,7 @@ class ChannelImpl final : public ChannelImplBase {
       w.u64(offset);
       w.u64(len);
       unit->bytes = std::move(w.bytes());
-      unit->onReply = [slot]() mutable { slot.reset(); }; // reply frees the slot
+      unit->onReply = [slot]() mutable { slot.reset(); }; // the acknowledgement frees the slot
       watchCopy(std::move(ev), device, hb.stream, onKernel, [this, op, unit] {
         unit->ready = true;
         flushWire();
@@ -607,26 +909,61 @@ class ChannelImpl final : public ChannelImplBase {
     finishSend(op);
   }
 
-  // Write every unit at the head of the queue whose data is ready, and post
-  // the read for its reply.
+  // Write every unit at the head of the queue whose data is ready, and start
+  // waiting for its acknowledgement: this end's acks word for the unit when
+  // the peer's copy agent is likely to take it (small enough; the word not
+  // still owed to an older unit), a message on the reply connection
+  // otherwise.
   void flushWire() {
     while (!wireQueue_.empty() && wireQueue_.front()->ready && !error_) {
       auto unit = wireQueue_.front();
       wireQueue_.pop_front();
-      TP_VLOG(6) << "Channel " << id_ << " is writing a descriptor";
+      const uint64_t seq = nextUnitOut_++;
+      const size_t slot = seq % kWordSlots;
+      const bool byWord = wordsIndex_ >= 0 && unit->tensors > 0 &&
+          unit->tensors <= kAgentMaxTensors && unit->totalBytes <= peerAgentMaxBytes_ &&
+          !ackSlotBusy_[slot];
+      unit->bytes[1] = byWord ? kAckByWord : kAckByMessage;
+      std::memcpy(unit->bytes.data() + 2, &seq, sizeof(seq));
+      TP_VLOG(6) << "Channel " << id_ << " is writing descriptor #" << seq;
       writeMessage(*descriptorConnection_, std::move(unit->bytes));
-      replyConnection_->read(nullptr, 0, onRead([this, unit] {
+      TP_MARK("ipc: unit written");
+      auto acknowledged = [this, unit] {
         if (!error_ && unit->onReply) {
           unit->onReply();
         }
         unit->onReply = nullptr;
-      }));
+      };
+      if (byWord) {
+        ackSlotBusy_[slot] = true;
+        const uint64_t* word = &ictx_->signals->hostWords(wordsIndex_)->acks[slot];
+        const uint64_t value = seq + 1;
+        auto cancel = cancel_;
+        auto self = shared_from_this();
+        ictx_->poller.watchCondition(
+            [word, value, cancel](bool* done) {
+              *done = __atomic_load_n(word, __ATOMIC_ACQUIRE) == value ||
+                  cancel->load(std::memory_order_acquire);
+              return 0;
+            },
+            [this, self, slot, acknowledged](const Error& error) {
+              TP_MARK("ipc: ack word seen");
+              ctx_->defer([this, self, slot, acknowledged, error] {
+                setError(error);
+                ackSlotBusy_[slot] = false;
+                acknowledged();
+              });
+            });
+      } else {
+        replyConnection_->read(nullptr, 0, onRead(acknowledged));
+      }
     }
   }
 
   // ---- recv -----------------------------------------------------------------
 
   void recvEntries(uint64_t seq, std::vector<BatchEntry> entries, TRecvCallback cb) {
+    TP_MARK("ipc: recv");
     auto op = std::make_shared<RecvOp>();
     op->seq = seq;
     op->cb = std::move(cb);
@@ -636,10 +973,10 @@ class ChannelImpl final : public ChannelImplBase {
       }
     }
     if (op->entries.empty()) {
-      op->cb(error_);
-      return;
+      op->allSeen = true; // nothing travels; the callback keeps its place in the order
     }
     recvOps_.push_back(op);
+    flushRecvCallbacks();
     pumpUnits();
   }
 
@@ -652,37 +989,93 @@ class ChannelImpl final : public ChannelImplBase {
   // is still missing some, as the reference gates its descriptor reads per
   // operation in sequence
   // (tensorpipe/channel/cuda_ipc/channel_impl.cc:319-347,349-399).
+  std::shared_ptr<RecvOp> opAwaitingUnits() const {
+    for (auto& op : recvOps_) {
+      if (!op->allSeen) {
+        return op;
+      }
+    }
+    return nullptr;
+  }
+
   void pumpUnits() {
-    if (unitReadPosted_ || recvOps_.empty() || error_) {
+    if (unitReadPosted_ || helloPending_ || error_ || opAwaitingUnits() == nullptr) {
       return;
     }
     unitReadPosted_ = true;
     descriptorConnection_->read(onReadMessage([this](std::vector<uint8_t> bytes) {
       unitReadPosted_ = false;
-      if (error_ || recvOps_.empty()) {
+      if (error_) {
         return;
       }
-      auto op = recvOps_.front();
+      auto op = opAwaitingUnits();
+      if (op == nullptr) {
+        return;
+      }
       onUnit(op, bytes);
       pumpUnits();
     }));
   }
 
+  // What has to happen once the copies of a received unit have finished.
+  struct UnitCompletion {
+    std::shared_ptr<ReplyUnit> reply; // owed when the peer waits for a message
+    bool byWord{false};
+    uint64_t unitSeq{0};
+    std::vector<uint64_t> inUse; // peer allocations the copies read from
+  };
+
+  void unitCopiesFinished(const UnitCompletion& c) {
+    for (uint64_t id : c.inUse) {
+      auto it = remoteAllocations_.find(id);
+      if (it != remoteAllocations_.end() && it->second.inFlight > 0) {
+        --it->second.inFlight;
+      }
+    }
+    dropLeastRecentlyUsedMappings();
+    if (c.reply) { // a unit acknowledged by word had its word raised by the GPU behind the copy
+      c.reply->ready = true;
+      flushReplies();
+    }
+  }
+
   void onUnit(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
+    TP_MARK("ipc: unit arrived");
     WireReader r(bytes.data(), bytes.size());
     const uint8_t kind = r.u8();
-    TP_VLOG(6) << "Channel " << id_ << " got a descriptor of kind " << int(kind) << " (#"
-               << op->seq << ")";
-    auto reply = std::make_shared<ReplyUnit>();
-    replyQueue_.push_back(reply);
+    const uint8_t ackMode = r.u8();
+    const uint64_t unitSeq = r.u64();
+    TP_VLOG(6) << "Channel " << id_ << " got descriptor #" << unitSeq << " of kind " << int(kind)
+               << " (recv #" << op->seq << ")";
+    if (!r.ok() || unitSeq != nextUnitIn_ || ackMode > kAckByWord ||
+        (ackMode == kAckByWord && peerWords_ == nullptr)) {
+      failProtocol();
+      return;
+    }
+    ++nextUnitIn_;
+    UnitCompletion completion;
+    completion.byWord = ackMode == kAckByWord;
+    completion.unitSeq = unitSeq;
+    if (!completion.byWord) {
+      completion.reply = std::make_shared<ReplyUnit>();
+      replyQueue_.push_back(completion.reply);
+    }
     std::vector<std::unique_ptr<HipEvent>> launched; // one event per copy launch
-    std::vector<uint64_t> inUse; // peer allocations the copies of this unit read from
+    std::vector<StreamRef> launchedOn;
     bool chunkOnKernel = false; // a staged chunk whose event is the kernel's own signal
     StreamRef chunkStream{nullptr, 0};
+    bool viaAgent = false;
+    bool gatedLaunched = false;
+    uint64_t agentTicket = 0;
+    void* agent = nullptr;
     try {
       if (kind == kDirect) {
-        if (r.u8() != 0) {
-          peerIdentity_ = r.str();
+        const bool gated = r.u8() != 0;
+        const uint32_t gateSlot = r.u32();
+        const uint64_t gateValue = r.u64();
+        if (gated && (peerWords_ == nullptr || wordsIndex_ < 0 || gateSlot >= kWordSlots)) {
+          failProtocol();
+          return;
         }
         const uint32_t nAllocs = r.u32();
         // every allocation takes 88 bytes on the wire
@@ -714,6 +1107,7 @@ class ChannelImpl final : public ChannelImplBase {
         };
         std::vector<Group> groups;
         std::vector<RemoteAllocation*> mappedOf(nAllocs, nullptr);
+        uint64_t totalBytes = 0;
         for (uint32_t k = 0; k < n; ++k) {
           const uint32_t index = r.u32();
           const uint32_t allocIdx = r.u32();
@@ -727,12 +1121,6 @@ class ChannelImpl final : public ChannelImplBase {
           const int device = hipDeviceForPointer(hb.ptr);
           TP_THROW_ASSERT_IF(device < 0);
           const Announced& a = announced[allocIdx];
-          // The range must lie inside the allocation the peer announced: the
-          // copy kernel would fault on anything else.
-          if (length != op->entries[index].length || offset > a.size || length > a.size - offset) {
-            failProtocol();
-            return;
-          }
           if (mappedOf[allocIdx] == nullptr) {
             auto it = remoteAllocations_.find(a.id);
             if (it == remoteAllocations_.end()) {
@@ -743,14 +1131,29 @@ class ChannelImpl final : public ChannelImplBase {
                 setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
                 return;
               }
-              it = remoteAllocations_.emplace(a.id, RemoteAllocation{mapped, a.size, device, 0, 0}).first;
+              // What the runtime says about the mapping bounds the ranges the
+              // peer may name; what the peer said about its size does not.
+              uint64_t realSize = a.size;
+              void* realBase = nullptr;
+              size_t queried = 0;
+              if (tphip_mem_base(mapped, &realBase, &queried) == 0 && realBase == mapped && queried > 0) {
+                realSize = std::min<uint64_t>(realSize, queried);
+              }
+              it = remoteAllocations_.emplace(a.id, RemoteAllocation{mapped, realSize, a.size, device, 0, 0}).first;
               mappedBytes_ += a.size;
-            } else if (it->second.size != a.size) {
+            } else if (it->second.announcedSize != a.size) {
               failProtocol(); // one identifier, one allocation
               return;
             }
             it->second.lastUse = ++useCounter_;
             mappedOf[allocIdx] = &it->second;
+          }
+          // The range must lie inside the mapped allocation: the copy kernel
+          // would fault on anything else.
+          const uint64_t limit = mappedOf[allocIdx]->size;
+          if (length != op->entries[index].length || offset > limit || length > limit - offset) {
+            failProtocol();
+            return;
           }
           StreamRef ref{hb.stream, device};
           Group* g = nullptr;
@@ -765,19 +1168,86 @@ class ChannelImpl final : public ChannelImplBase {
           }
           g->table.push_back(tphip_copy_desc{
               static_cast<const uint8_t*>(mappedOf[allocIdx]->ptr) + offset, hb.ptr, length});
+          totalBytes += length;
           ++op->unitsSeen;
         }
         // From here until the copies have finished the mappings must stay.
         for (uint32_t a = 0; a < nAllocs; ++a) {
           if (mappedOf[a] != nullptr) {
             ++mappedOf[a]->inFlight;
-            inUse.push_back(announced[a].id);
+            completion.inUse.push_back(announced[a].id);
           }
         }
-        for (auto& g : groups) {
-          auto ev = ictx_->events.get(g.dst.device);
-          hipBatchedCopy(g.dst.device, g.dst.stream, g.table, *ev, /*signalOnKernel=*/false);
-          launched.push_back(std::move(ev));
+        // Small and nothing pending on the streams the bytes go to: the copy
+        // agent, no launch. (The sender announced the unit only once its
+        // sources were ready.)
+        if (gated) {
+          // Launched now, started by the GPU when the sender's word is there.
+          auto pending = std::make_shared<GatedUnit>();
+          pending->completion = completion;
+          pending->op = op;
+          pending->word = &peerWords_->ready[gateSlot];
+          pending->value = gateValue;
+          pending->waitUs = ictx_->gateWaitUs;
+          for (auto& g : groups) {
+            pending->groups.push_back(GatedGroup{g.dst, std::move(g.table), 0});
+          }
+          pending->remaining = pending->groups.size();
+          ++op->landing;
+          gatedLaunched = true;
+          for (size_t k = 0; k < pending->groups.size(); ++k) {
+            try {
+              launchGated(pending, k);
+            } catch (const std::exception& ex) {
+              TP_LOG_WARNING() << "Channel " << id_ << " gated copy failed: " << ex.what();
+              setError(TP_CREATE_ERROR(HipError, "hip_ipc gated copy", TPHIP_ERR_INVALID_ARG));
+              for (size_t j = k; j < pending->groups.size(); ++j) {
+                gatedGroupFinished(pending); // this one and those never launched
+              }
+              break;
+            }
+          }
+          if (error_) {
+            return;
+          }
+        } else if (ictx_->agentEnabled && totalBytes <= ictx_->agentMaxBytes && n <= kAgentMaxTensors) {
+          const int device = groups.front().dst.device;
+          bool quiet = true;
+          for (auto& g : groups) {
+            quiet = quiet && g.dst.device == device && ictx_->idleProbe.idle(g.dst.device, g.dst.stream);
+          }
+          agent = quiet ? ictx_->agent(device) : nullptr;
+          if (agent != nullptr) {
+            std::vector<tphip_copy_desc> all;
+            for (auto& g : groups) {
+              all.insert(all.end(), g.table.begin(), g.table.end());
+            }
+            void* notify = completion.byWord ? &peerWords_->acks[unitSeq % kWordSlots] : nullptr;
+            const int rc = tphip_agent_submit(
+                agent, all.data(), static_cast<uint32_t>(all.size()), notify, unitSeq + 1, &agentTicket);
+            viaAgent = rc == 0; // a full ring or an address it cannot carry: launch as usual
+            TP_MARK("ipc: posted to the agent");
+          }
+        }
+        if (!viaAgent && !gatedLaunched) {
+          for (auto& g : groups) {
+            auto ev = ictx_->events.get(g.dst.device);
+            hipBatchedCopy(g.dst.device, g.dst.stream, g.table, *ev, /*signalOnKernel=*/false);
+            launched.push_back(std::move(ev));
+            launchedOn.push_back(g.dst);
+          }
+          if (completion.byWord) {
+            // The sender watches its word: raise it from the GPU behind the
+            // copies, on the first stream once it has waited for the others.
+            for (size_t k = 1; k < launched.size(); ++k) {
+              launched[k]->wait(launchedOn[0].stream, launchedOn[0].device);
+            }
+            TP_HIP_CHECK(tphip_stream_signal(
+                launchedOn[0].device,
+                launchedOn[0].stream,
+                &peerWords_->acks[unitSeq % kWordSlots],
+                unitSeq + 1));
+          }
         }
         op->unitsExpected += n;
       } else if (kind == kChunk) {
@@ -813,15 +1283,24 @@ class ChannelImpl final : public ChannelImplBase {
             setError(TP_CREATE_ERROR(HipError, "tphip_ipc_mem_open", rc));
             return;
           }
-          remoteOutboxes_[srcDevice] = RemoteOutbox{mapped, remoteSlotBytes, remoteNumSlots};
           imports_.push_back(Import{device, peer, outboxId});
+          // The slots must fit what was really mapped.
+          void* realBase = nullptr;
+          size_t queried = 0;
+          if (tphip_mem_base(mapped, &realBase, &queried) == 0 && realBase == mapped && queried > 0 &&
+              remoteSlotBytes > queried / remoteNumSlots) {
+            failProtocol();
+            return;
+          }
+          remoteOutboxes_[srcDevice] = RemoteOutbox{mapped, remoteSlotBytes, remoteNumSlots};
         }
         const uint32_t slotIdx = r.u32();
         const uint64_t offset = r.u64();
         const uint64_t len = r.u64();
         auto it = remoteOutboxes_.find(srcDevice);
+        const uint64_t tensorLength = op->entries[index].length;
         if (!r.ok() || it == remoteOutboxes_.end() || slotIdx >= it->second.numSlots ||
-            len > it->second.slotBytes || offset + len > op->entries[index].length) {
+            len > it->second.slotBytes || offset > tensorLength || len > tensorLength - offset) {
           failProtocol();
           return;
         }
@@ -834,13 +1313,13 @@ class ChannelImpl final : public ChannelImplBase {
                 static_cast<uint8_t*>(hb.ptr) + offset,
                 len}},
             *ev,
-            /*signalOnKernel=*/(op->entries[index].length + it->second.slotBytes - 1) /
-                    it->second.slotBytes >=
+            /*signalOnKernel=*/(tensorLength + it->second.slotBytes - 1) / it->second.slotBytes >=
                 kChunksForKernelSignals);
         chunkStream = StreamRef{hb.stream, device};
         launched.push_back(std::move(ev));
+        launchedOn.push_back(chunkStream);
         // A staged tensor counts as seen when its last chunk arrived.
-        if (offset + len == op->entries[index].length) {
+        if (offset + len == tensorLength) {
           ++op->unitsSeen;
         }
         if (offset == 0) {
@@ -852,32 +1331,172 @@ class ChannelImpl final : public ChannelImplBase {
       }
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " recv failed: " << ex.what();
+      // Copies already enqueued for this unit read the peer's memory; they are
+      // followed by no watcher now, so wait for them here before the error
+      // lets the mappings go.
+      for (auto& s : launchedOn) {
+        tphip_stream_sync(s.device, s.stream);
+      }
       setError(TP_CREATE_ERROR(HipError, "hip_ipc recv", TPHIP_ERR_INVALID_ARG));
       return;
     }
 
-    TP_VLOG(6) << "Channel " << id_ << " enqueued the copies (#" << op->seq << ")";
-    // Reply once the copies of this unit have finished.
-    auto remaining = std::make_shared<size_t>(launched.size());
-    for (auto& ev : launched) {
-      watchCopy(std::move(ev), chunkStream.device, chunkStream.stream, chunkOnKernel, [this, reply, remaining, inUse] {
-        if (--*remaining == 0) {
-          for (uint64_t id : inUse) {
-            auto it = remoteAllocations_.find(id);
-            if (it != remoteAllocations_.end() && it->second.inFlight > 0) {
-              --it->second.inFlight;
-            }
-          }
-          dropLeastRecentlyUsedMappings();
-          reply->ready = true;
-          flushReplies();
+    TP_VLOG(6) << "Channel " << id_ << " enqueued the copies (recv #" << op->seq << ")";
+    if (viaAgent) {
+      // The agent lands a small copy about 3 us after it was posted: less than
+      // handing the wait to the poller thread and coming back costs. Look for
+      // it right here for a few microseconds first.
+      const auto giveUp = std::chrono::steady_clock::now() + std::chrono::microseconds(ictx_->agentSpinUs);
+      bool landed = false;
+      do {
+        int d = 0;
+        if (tphip_agent_done(agent, agentTicket, &d) != 0) {
+          break;
         }
-      });
+        landed = d != 0;
+      } while (!landed && std::chrono::steady_clock::now() < giveUp);
+      if (landed) {
+        TP_MARK("ipc: agent done seen (inline)");
+        viaAgent = false;
+        unitCopiesFinished(completion);
+      }
+    }
+    if (viaAgent) {
+      // The recv callback waits for the bytes: nothing on the caller's stream
+      // orders later work behind the agent's copy.
+      ++op->landing;
+      auto self = shared_from_this();
+      ictx_->poller.watchCondition(
+          [agent, agentTicket](bool* done) {
+            int d = 0;
+            const int rc = tphip_agent_done(agent, agentTicket, &d);
+            *done = d != 0;
+            return rc;
+          },
+          [this, self, op, completion](const Error& error) {
+            TP_MARK("ipc: agent done seen");
+            ctx_->defer([this, self, op, completion, error] {
+              setError(error);
+              unitCopiesFinished(completion);
+              --op->landing;
+              if (error_) {
+                if (op->landing == 0) {
+                  finishRecv(op); // held back by handleError until now
+                }
+              } else {
+                flushRecvCallbacks();
+              }
+            });
+          });
+    } else if (!gatedLaunched) {
+      // Acknowledge once the copies of this unit have finished.
+      auto remaining = std::make_shared<size_t>(launched.size());
+      for (auto& ev : launched) {
+        watchCopy(std::move(ev), chunkStream.device, chunkStream.stream, chunkOnKernel, [this, remaining, completion] {
+          if (--*remaining == 0) {
+            unitCopiesFinished(completion);
+          }
+        });
+      }
     }
 
     if (op->unitsSeen == op->entries.size()) {
-      // Every copy of the op is enqueued: that is what the recv callback means.
-      removeRecv(op);
+      // Every copy of the op is enqueued (or posted to the agent).
+      op->allSeen = true;
+      flushRecvCallbacks();
+    }
+  }
+
+  // A received unit whose copies wait for the sender's word on the GPU.
+  struct GatedGroup {
+    StreamRef dst;
+    std::vector<tphip_copy_desc> table;
+    uint32_t expiredSlot;
+  };
+  struct GatedUnit {
+    UnitCompletion completion;
+    std::shared_ptr<RecvOp> op;
+    const uint64_t* word{nullptr};
+    uint64_t value{0};
+    uint32_t waitUs{0};
+    std::vector<GatedGroup> groups;
+    size_t remaining{0};
+    bool acked{false};
+  };
+
+  // Launch (again) the copies of group k behind the gate and look at how they
+  // ended once they have.
+  void launchGated(const std::shared_ptr<GatedUnit>& u, size_t k) {
+    GatedGroup& g = u->groups[k];
+    g.expiredSlot = static_cast<uint32_t>(nextExpired_++ % kWordSlots);
+    ChannelWords* mine = ictx_->signals->hostWords(wordsIndex_);
+    __atomic_store_n(&mine->expired[g.expiredSlot], uint64_t(0), __ATOMIC_RELEASE);
+    auto ev = ictx_->events.get(g.dst.device);
+    TP_HIP_CHECK(tphip_batched_copy_gated(
+        g.dst.device,
+        g.table.data(),
+        static_cast<uint32_t>(g.table.size()),
+        g.dst.stream,
+        ev->raw(),
+        u->word,
+        u->value,
+        u->waitUs,
+        &ictx_->signals->devWords(wordsIndex_)->expired[g.expiredSlot]));
+    auto self = shared_from_this();
+    ictx_->poller.watch(std::move(ev), &ictx_->events, [this, self, u, k](const Error& error) {
+      ctx_->defer([this, self, u, k, error] {
+        setError(error);
+        const ChannelWords* words = ictx_->signals->hostWords(wordsIndex_);
+        const bool gaveUp =
+            __atomic_load_n(&words->expired[u->groups[k].expiredSlot], __ATOMIC_ACQUIRE) != 0;
+        if (gaveUp && !error_) {
+          // The producer is not done yet: wait again, longer.
+          u->waitUs = std::min<uint32_t>(u->waitUs * 2, ictx_->gateWaitUs * 64);
+          try {
+            launchGated(u, k);
+            return;
+          } catch (const std::exception& ex) {
+            TP_LOG_WARNING() << "Channel " << id_ << " gated copy failed: " << ex.what();
+            setError(TP_CREATE_ERROR(HipError, "hip_ipc gated copy", TPHIP_ERR_INVALID_ARG));
+          }
+        }
+        gatedGroupFinished(u);
+      });
+    });
+  }
+
+  // One group of a gated unit will not be launched again; the last one
+  // acknowledges the unit and lets the recv callback go.
+  void gatedGroupFinished(const std::shared_ptr<GatedUnit>& u) {
+    if (--u->remaining > 0) {
+      return;
+    }
+    if (!error_ && u->completion.byWord) {
+      // the sender watches its word: raise it from the GPU, behind the copies
+      const StreamRef& first = u->groups[0].dst;
+      tphip_stream_signal(
+          first.device,
+          first.stream,
+          &peerWords_->acks[u->completion.unitSeq % kWordSlots],
+          u->completion.unitSeq + 1);
+    }
+    unitCopiesFinished(u->completion);
+    --u->op->landing;
+    if (error_) {
+      if (u->op->landing == 0) {
+        finishRecv(u->op);
+      }
+    } else {
+      flushRecvCallbacks();
+    }
+  }
+
+  // Recv callbacks fire in the order of the recv calls: an op whose copies are
+  // all enqueued waits for an older one whose bytes the agent has yet to land.
+  void flushRecvCallbacks() {
+    while (!recvOps_.empty() && recvOps_.front()->allSeen && recvOps_.front()->landing == 0) {
+      auto op = recvOps_.front();
+      recvOps_.pop_front();
       finishRecv(op);
     }
   }
@@ -899,7 +1518,7 @@ class ChannelImpl final : public ChannelImplBase {
       }
       TP_VLOG(5) << "Channel " << id_ << " drops its mapping of peer allocation #" << victim->first;
       HipIpcImports::get().release(victim->second.device, peerIdentity_, victim->first);
-      mappedBytes_ -= victim->second.size;
+      mappedBytes_ -= victim->second.announcedSize;
       remoteAllocations_.erase(victim);
     }
   }
@@ -968,15 +1587,6 @@ class ChannelImpl final : public ChannelImplBase {
     }
   }
 
-  void removeRecv(const std::shared_ptr<RecvOp>& op) {
-    for (auto it = recvOps_.begin(); it != recvOps_.end(); ++it) {
-      if (*it == op) {
-        recvOps_.erase(it);
-        return;
-      }
-    }
-  }
-
   void finishSend(const std::shared_ptr<SendOp>& op) {
     if (op->done) {
       return;
@@ -992,6 +1602,7 @@ class ChannelImpl final : public ChannelImplBase {
     }
     op->done = true;
     auto cb = std::move(op->cb);
+    TP_MARK("ipc: recv callback");
     cb(error_);
   }
 
@@ -999,22 +1610,36 @@ class ChannelImpl final : public ChannelImplBase {
   std::shared_ptr<transport::Connection> descriptorConnection_;
   std::shared_ptr<transport::Connection> replyConnection_;
   std::deque<std::shared_ptr<SendOp>> sendOps_;
-  std::deque<std::shared_ptr<RecvOp>> recvOps_; // oldest first; the front one takes the next unit
+  std::deque<std::shared_ptr<RecvOp>> recvOps_; // oldest first; callbacks fire from the front
   bool unitReadPosted_{false};
+  bool helloPending_{false};
   std::deque<std::shared_ptr<WireUnit>> wireQueue_;
   std::deque<std::shared_ptr<ReplyUnit>> replyQueue_;
-  bool identitySent_{false};
   std::map<int, bool> outboxAnnounced_;
+  // Signal words: this end's slot in the context's page, and the peer's words
+  // as mapped here for the GPU (null until its hello has arrived, or when it
+  // has none).
+  int wordsIndex_{-1};
+  ChannelWords* peerWords_{nullptr}; // a device address: kernels only, never this process's CPUs
+  uint64_t peerAgentMaxBytes_{0};
+  bool peerGates_{false};
+  uint64_t nextGate_{0};
+  uint64_t nextExpired_{0};
+  uint64_t nextUnitOut_{0};
+  uint64_t nextUnitIn_{0};
+  std::array<bool, kWordSlots> ackSlotBusy_{};
+  std::shared_ptr<std::atomic<bool>> cancel_{std::make_shared<std::atomic<bool>>(false)};
   // Peer allocations this channel keeps mapped (direct route), by export id.
   struct RemoteAllocation {
     void* ptr;
-    uint64_t size;
+    uint64_t size; // what a range inside it is checked against
+    uint64_t announcedSize;
     int device;
     uint64_t lastUse;
     uint32_t inFlight; // units whose copies may still read from it
   };
   std::map<uint64_t, RemoteAllocation> remoteAllocations_;
-  std::string peerIdentity_; // the peer's processIdentity(), from its first direct unit
+  std::string peerIdentity_; // the peer's processIdentity(), from its hello
   uint64_t mappedBytes_{0};
   uint64_t useCounter_{0};
   struct RemoteOutbox {
@@ -1023,7 +1648,8 @@ class ChannelImpl final : public ChannelImplBase {
     uint32_t numSlots;
   };
   std::map<int, RemoteOutbox> remoteOutboxes_;
-  // The peer's outboxes this channel holds in the process-wide import table.
+  // The peer's slabs (outboxes, signal page) this channel holds in the
+  // process-wide import table.
   struct Import {
     int device;
     std::string peer;

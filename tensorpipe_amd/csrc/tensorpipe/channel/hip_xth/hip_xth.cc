@@ -157,6 +157,7 @@ class ChannelImpl final : public ChannelImplBase {
       cb(error_);
       return;
     }
+    TP_MARK("xth: send");
     auto op = std::make_shared<SendOp>();
     op->seq = seq;
     op->cb = std::move(cb);
@@ -187,15 +188,18 @@ class ChannelImpl final : public ChannelImplBase {
     sendOps_.push_back(op);
     TP_VLOG(6) << "Channel " << id_ << " is writing descriptor (#" << seq << ")";
     writeMessage(*descriptorConnection_, std::move(w.bytes()));
+    TP_MARK("xth: descriptor written");
     TP_VLOG(6) << "Channel " << id_ << " is reading completion (#" << seq << ")";
     completionConnection_->read(nullptr, 0, onRead([this, op] {
       TP_VLOG(6) << "Channel " << id_ << " done reading completion (#" << op->seq << ")";
+      TP_MARK("xth: completion arrived (send callback)");
       removeSend(op);
       finishSend(op);
     }));
   }
 
   void recvEntries(uint64_t seq, std::vector<BatchEntry> entries, TRecvCallback cb) {
+    TP_MARK("xth: recv");
     auto op = std::make_shared<RecvOp>();
     op->seq = seq;
     op->cb = std::move(cb);
@@ -213,6 +217,7 @@ class ChannelImpl final : public ChannelImplBase {
     descriptorConnection_->read(onReadMessage([this, op](std::vector<uint8_t> bytes) {
       TP_VLOG(6) << "Channel " << id_ << " done reading descriptor (#" << op->seq << ")";
       if (!error_) {
+        TP_MARK("xth: descriptor arrived");
         copyFromDescriptor(op, bytes);
       }
     }));
@@ -290,6 +295,7 @@ class ChannelImpl final : public ChannelImplBase {
           launch = xctx_->markers.launched(g.src.device, g.src.stream, xctx_->events);
         }
         TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
+        TP_MARK("xth: copy launched");
         auto self = shared_from_this();
         // Counted per launch: if a later launch of this op fails, the error
         // path still waits for exactly the copies that are running.
@@ -297,6 +303,7 @@ class ChannelImpl final : public ChannelImplBase {
         const StreamRef src = g.src;
         xctx_->poller.watch(std::move(done), &xctx_->events, [this, self, op, src, onKernel, launch](
                                                                  const Error& error) {
+          TP_MARK("xth: copy seen finished");
           if (onKernel) {
             // before anybody hears of the completion: the stream is still the sender's to keep
             xctx_->markers.finished(src.device, src.stream, launch, xctx_->events);
@@ -312,6 +319,7 @@ class ChannelImpl final : public ChannelImplBase {
             }
             TP_VLOG(6) << "Channel " << id_ << " done copying payload (#" << op->seq << ")";
             op->copied = true;
+            TP_MARK("xth: recv callback due");
             flushRecvs();
           });
         });

@@ -155,6 +155,10 @@ TP_AMD_NAMESPACE_END
 
 #include <cstdio>
 #include <cstdlib>
+#include <memory>
+
+#include <pthread.h>
+#include <unistd.h>
 
 TP_AMD_NAMESPACE_BEGIN
 
@@ -200,6 +204,67 @@ StageTable& stageTable() {
 }
 
 } // namespace
+
+namespace {
+
+struct Timeline {
+  struct Mark {
+    const char* what;
+    uint64_t nanos;
+    uint64_t thread;
+  };
+  size_t capacity{0};
+  std::unique_ptr<Mark[]> marks;
+  std::atomic<uint64_t> next{0};
+  Timeline() {
+    const char* e = std::getenv("TP_TIMELINE");
+    capacity = e != nullptr ? static_cast<size_t>(std::atol(e)) : 0;
+    if (capacity > 0) {
+      marks.reset(new Mark[capacity]());
+    }
+  }
+  ~Timeline() {
+    if (capacity == 0) {
+      return;
+    }
+    const uint64_t end = next.load();
+    const uint64_t begin = end > capacity ? end - capacity : 0;
+    uint64_t prev = 0;
+    for (uint64_t i = begin; i < end; ++i) {
+      const Mark& m = marks[i % capacity];
+      if (m.what == nullptr) {
+        continue;
+      }
+      std::fprintf(
+          stderr, "[timeline %d] %12.2f us  +%8.2f  thread %04llx  %s\n", static_cast<int>(::getpid()),
+          m.nanos / 1e3, prev == 0 ? 0.0 : (static_cast<double>(m.nanos) - static_cast<double>(prev)) / 1e3,
+          static_cast<unsigned long long>(m.thread & 0xffff), m.what);
+      prev = m.nanos;
+    }
+  }
+};
+
+Timeline& timeline() {
+  static Timeline t;
+  return t;
+}
+
+} // namespace
+
+bool timelineEnabled() {
+  return timeline().capacity != 0;
+}
+
+void timelineMark(const char* what) {
+  Timeline& t = timeline();
+  const uint64_t i = t.next.fetch_add(1, std::memory_order_relaxed);
+  Timeline::Mark& m = t.marks[i % t.capacity];
+  m.nanos = static_cast<uint64_t>(std::chrono::duration_cast<std::chrono::nanoseconds>(
+                                      std::chrono::steady_clock::now().time_since_epoch())
+                                      .count());
+  m.thread = static_cast<uint64_t>(reinterpret_cast<uintptr_t>(pthread_self()) >> 12);
+  m.what = what;
+}
 
 bool stageStatsEnabled() {
   return stageTable().enabled;

@@ -52,4 +52,17 @@ class StageScope {
   std::chrono::steady_clock::time_point t0_;
 };
 
+// A timeline of named moments, for finding where the microseconds of a small
+// transfer go: TP_TIMELINE=<n> keeps the last n marks of the process (any
+// thread) and prints them at exit with their distance from the mark before.
+// Costs one relaxed load when switched off.
+bool timelineEnabled();
+void timelineMark(const char* what);
+#define TP_MARK(what)                          \
+  do {                                         \
+    if (::tensorpipe::timelineEnabled()) {     \
+      ::tensorpipe::timelineMark(what);        \
+    }                                          \
+  } while (0)
+
 TP_AMD_NAMESPACE_END

@@ -829,6 +829,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     const uint8_t type = r.u8();
     TP_VLOG(9) << "Pipe " << id_ << " got a packet of type " << int(type);
     if (type == kDescriptor) {
+      TP_MARK("pipe: descriptor packet arrived");
       StageScope timer(Stage::kPipeParseDescriptor);
       auto op = std::make_shared<ReadOp>();
       op->seq = nextReadSeq_++;
@@ -960,6 +961,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
                  << ")";
       // The op keeps shapes, devices and payload lengths; the descriptor
       // itself goes to the user without another copy.
+      TP_MARK("pipe: readDescriptor callback");
       fn(Error::kSuccess, std::move(next->descriptor));
     }
   }
@@ -970,6 +972,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       return;
     }
     TP_VLOG(9) << "Pipe " << id_ << " received a read request";
+    TP_MARK("pipe: read()");
     StageScope timer(Stage::kPipeReadRequest);
     std::shared_ptr<ReadOp> op;
     for (auto& o : readOps_) {
@@ -1105,6 +1108,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       readOps_.pop_front();
       if (op->fn) {
         TP_VLOG(3) << "Pipe " << id_ << " is calling a read callback (#" << op->seq << ")";
+        TP_MARK("pipe: read callback");
         auto fn = std::move(op->fn);
         fn(error_);
       }
@@ -1121,6 +1125,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     auto op = std::make_shared<WriteOp>();
     op->seq = nextWriteSeq_++;
     TP_VLOG(9) << "Pipe " << id_ << " received a write request (#" << op->seq << ")";
+    TP_MARK("pipe: write()");
     op->message = std::move(message);
     op->fn = std::move(fn);
     for (auto& t : op->message.tensors) {
@@ -1339,6 +1344,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       auto done = writeOps_.front();
       writeOps_.pop_front();
       TP_VLOG(3) << "Pipe " << id_ << " is calling a write callback (#" << done->seq << ")";
+      TP_MARK("pipe: write callback");
       auto fn = std::move(done->fn);
       fn(error_);
     }

@@ -2,7 +2,7 @@
 // plugin surface itself: channel::Context::createChannel over raw transport
 // connections, then Channel::send / recv with Buffer{HipBuffer|CpuBuffer}.
 //
-//   channel_tests --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_basic|basic|xth [--case SUBSTRING] [--list]
+//   channel_tests --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_ipc_gated|hip_ipc_messages|hip_basic|basic|xth [--case SUBSTRING] [--list]
 //
 // hip_xth and xth run both endpoints as two threads of this process; hip_ipc,
 // hip_basic and basic run them as two processes. The CPU channels (basic, xth)
@@ -25,12 +25,14 @@ std::string gSuite;
 bool gGpu = true; // whether the suite's tensors live on the GPU
 
 bool knownSuite(const std::string& s) {
-  return s == "hip_xth" || s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_basic" ||
+  return s == "hip_xth" || s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_ipc_gated" ||
+      s == "hip_ipc_messages" || s == "hip_basic" ||
       s == "basic" || s == "xth";
 }
 
 bool twoProcessSuite(const std::string& s) {
-  return s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_basic" || s == "basic";
+  return s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_ipc_gated" || s == "hip_ipc_messages" ||
+      s == "hip_basic" || s == "basic";
 }
 
 Buffer nullBuffer() {
@@ -44,7 +46,8 @@ std::shared_ptr<channel::Context> makeContext() {
   if (gSuite == "hip_xth") {
     return channel::hip_xth::create();
   }
-  if (gSuite == "hip_ipc" || gSuite == "hip_ipc_outbox") {
+  if (gSuite == "hip_ipc" || gSuite == "hip_ipc_outbox" || gSuite == "hip_ipc_gated" ||
+      gSuite == "hip_ipc_messages") {
     return channel::hip_ipc::create();
   }
   if (gSuite == "hip_basic") {
@@ -415,7 +418,8 @@ std::vector<Case> makeCases() {
     cases.push_back({"CannotCommunicateCpuToCpu", cpuToCpu, cpuToCpu});
   }
 
-  if (gSuite == "hip_ipc" || gSuite == "hip_ipc_outbox") {
+  if (gSuite == "hip_ipc" || gSuite == "hip_ipc_outbox" || gSuite == "hip_ipc_gated" ||
+      gSuite == "hip_ipc_messages") {
     // cuda_ipc_test.cc:37-57: two contexts of one process must not pick IPC.
     auto sameProcess = [](Endpoint&) {
       auto c1 = makeContext();
@@ -681,7 +685,7 @@ int main(int argc, char** argv) {
   Args args = parseArgs(argc, argv);
   if (!knownSuite(args.suite)) {
     std::fprintf(
-        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_basic|basic|xth [--case S] [--list]\n",
+        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_ipc_gated|hip_ipc_messages|hip_basic|basic|xth [--case S] [--list]\n",
         argv[0]);
     return 2;
   }
@@ -693,6 +697,17 @@ int main(int argc, char** argv) {
     ::setenv("TP_HIP_IPC_MODE", "outbox", 1);
     ::setenv("TP_HIP_IPC_SLOT_BYTES", "1048576", 1);
     ::setenv("TP_HIP_IPC_NUM_SLOTS", "3", 1);
+  }
+  if (gSuite == "hip_ipc_gated") {
+    // Senders whose stream is still producing announce at once; the receiver's
+    // GPU waits for their word (short waits, so that the retry path runs too).
+    ::setenv("TP_HIP_IPC_GATES", "1", 1);
+    ::setenv("TP_HIP_IPC_GATE_WAIT_US", "200", 1);
+  }
+  if (gSuite == "hip_ipc_messages") {
+    // No signal words, no copy agent: every unit acknowledged by a message.
+    ::setenv("TP_HIP_IPC_SIGNALS", "0", 1);
+    ::setenv("TP_HIP_IPC_AGENT", "0", 1);
   }
   std::vector<Case> cases = makeCases();
   if (args.list) {

@@ -122,16 +122,17 @@ def test_launch_shapes(oracle, unroll, nt):
 
 
 def test_plan_ring_reuse(oracle):
-    # more launches than plan slots on one stream, all checked; 70 entries each, so that the
-    # plans go through the ring (tables of up to 64 entries travel in the kernel arguments)
+    # more launches than plan slots on one stream, all checked; 270 entries each, so that the
+    # plans go through the ring (tables of up to 256 entries travel in the kernel arguments)
     for k in range(70):
-        sizes = [1000 + k, 17, 4096 + k] + [64 + (i * 37 + k) % 900 for i in range(67)]
+        sizes = [1000 + k, 17, 4096 + k] + [64 + (i * 37 + k) % 900 for i in range(267)]
         _run_case(oracle, _pack(sizes, lambda i: (i + k) % 16, lambda i: (i * 3 + k) % 16), seed=k)
 
 
-@pytest.mark.parametrize("n", [2, 3, 31, 63, 64, 65, 66, 130])
+@pytest.mark.parametrize("n", [2, 3, 31, 63, 64, 65, 66, 130, 255, 256, 257, 300])
 def test_inline_plan_boundary(oracle, n):
-    # either side of the largest table that travels in the kernel arguments, default and tuned launches
+    # either side of the two sizes of table that travel in the kernel arguments (64 and 256
+    # entries), default and tuned launches
     rng = np.random.default_rng(1000 + n)
     sizes = [int(x) for x in rng.integers(0, 70000, n)]
     sizes[0] = (2 << 20) + 3
@@ -332,7 +333,7 @@ def test_graph_capture_and_replay(oracle):
     big_src = torch.zeros(one + 16, dtype=torch.uint8, device="cuda")
     big_dst = torch.zeros(one + 16, dtype=torch.uint8, device="cuda")
     entries = [(src.data_ptr() + s, dst.data_ptr() + d, n) for s, d, n in layout]
-    many = [(src.data_ptr() + i, dst.data_ptr() + i, 1) for i in range(70)]
+    many = [(src.data_ptr() + i, dst.data_ptr() + i, 1) for i in range(270)]
     many_table, many_n = hip.make_table(many)
     torch.cuda.synchronize()
 
@@ -361,11 +362,11 @@ def test_graph_capture_and_replay(oracle):
         assert (got[3:3 + one] == host_big[1:1 + one]).all(), f"replay {replay}: single copy differs"
         assert (got[:3] == FILL).all() and (got[3 + one:] == FILL).all()
         # eager launches between replays, through the plan ring as well
-        _run_case(oracle, _pack([100 + replay] * 70), seed=replay)
+        _run_case(oracle, _pack([100 + replay] * 270), seed=replay)
     # outside capture the large table goes through as before
     _native.check(lib.tphip_batched_copy(0, many_table, many_n, None))
     torch.cuda.synchronize()
-    assert torch.equal(dst[:70], src[:70])
+    assert torch.equal(dst[:270], src[:270])
 
 
 def test_full_size_roundtrip_property():

@@ -575,3 +575,57 @@ def test_ipc_one_message_out_of_many_allocations(ipc_peer):
     finally:
         while held:
             lib.tphip_free(0, held.pop())
+
+
+# ---------------------------------------------------------------------------
+# The benchmark's own shapes at full size: same channels, geometries and tensor sizes as
+# bench.py's cross-process legs. The source is seeded over its whole length with no two blocks
+# alike (a chunk delivered from the wrong offset cannot compare equal); at these sizes the echo
+# is compared with the source on the device, and a 1 MiB sample at each end and in the middle
+# with the CPU oracle's result for the same chunking.
+# ---------------------------------------------------------------------------
+
+def _full_size_echo(oracle, peer, nbytes, dtype, kind, slot, num_slots):
+    import torch
+
+    elem = 4 if dtype == "f32" else 2
+    host = datagen.normal_large(datagen.SEED_BASE + (3 if kind == "ipc" else 4), nbytes // elem, dtype).view(np.uint8)
+    src = _gpu(host)
+    outs, _ = peer.echo([tp.make_tensor(src, nbytes=nbytes, target=(tp.HIP, 0))], "gpu")
+    out = outs[0]
+    assert bool(torch.equal(out[32:32 + nbytes], src)), "echoed bytes differ from the source"
+    assert bool((out[:32] == FILL).all()) and bool((out[32 + nbytes:] == FILL).all())
+    # oracle on three windows of whole chunks
+    win = max(slot, 1 << 20)
+    for lo in (0, (nbytes // 2) // slot * slot, nbytes - win):
+        ref = np.full(win, FILL, np.uint8)
+        piece = host[lo:lo + win]
+        if kind == "ipc":
+            oracle.ipc_tensor(piece, ref, win, slot=slot, num_slots=num_slots, in_flight=num_slots)
+        else:
+            oracle.staged_tensor(piece, ref, win, slot=slot, num_slots=num_slots)
+        got = out[32 + lo:32 + lo + win].cpu().numpy()
+        assert (got == ref).all(), f"window at {lo} differs from the oracle"
+    del src, out, outs
+
+
+@pytest.mark.parametrize("nbytes", [256 << 20, 1 << 30])
+def test_ipc_bench_shapes_full_size(oracle, ipc_peer, nbytes):
+    # configs[2]'s two largest points: fp32 N(0,1), 256 MiB and 1 GiB through hip_ipc
+    _full_size_echo(oracle, ipc_peer, nbytes, "f32", "ipc", 8 << 20, 4)
+
+
+@pytest.mark.parametrize("slot_mib", [1, 4])
+def test_staged_bench_shapes_full_size(oracle, slot_mib):
+    # configs[3]: 256 MiB bf16 N(0,1) through hip_basic with a 4-deep ring of 1 MiB and of 4 MiB slots
+    env = {"TP_HIP_BASIC_SLOT_BYTES": str(slot_mib << 20), "TP_HIP_BASIC_NUM_SLOTS": "4"}
+    os.environ.update(env)
+    try:
+        peer = Peer("basic:0,hip_basic:10", env=env)
+    finally:
+        for k in env:
+            del os.environ[k]
+    try:
+        _full_size_echo(oracle, peer, 256 << 20, "bf16", "staged", slot_mib << 20, 4)
+    finally:
+        peer.close()

@@ -17,6 +17,7 @@ BIN = os.path.join(ROOT, "tests", "cpp", "bin")
 CPU_SUITES = [("channel_tests", "basic"), ("channel_tests", "xth"),
               ("pipe_tests", "cpu_same_process"), ("pipe_tests", "cpu_two_process")]
 GPU_SUITES = [("channel_tests", "hip_xth"), ("channel_tests", "hip_ipc"), ("channel_tests", "hip_ipc_outbox"),
+              ("channel_tests", "hip_ipc_gated"), ("channel_tests", "hip_ipc_messages"),
               ("channel_tests", "hip_basic"),
               ("pipe_tests", "same_process"), ("pipe_tests", "two_process")]
 
@@ -60,7 +61,8 @@ def check_case(program, suite, case):
     assert case in per_case, f"no result for {case}; exit code {rc}\n{out}\n{err}"
     bad = [line for _, ok, line in per_case[case] if not ok]
     assert not bad, "\n".join(bad) + "\n" + err
-    two_process = suite in ("basic", "hip_ipc", "hip_ipc_outbox", "hip_basic", "two_process", "cpu_two_process")
+    two_process = suite in ("basic", "hip_ipc", "hip_ipc_outbox", "hip_ipc_gated", "hip_ipc_messages", "hip_basic",
+                            "two_process", "cpu_two_process")
     assert len(per_case[case]) == (2 if two_process else 1), per_case[case]
 
 
