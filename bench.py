@@ -338,7 +338,7 @@ class PeerRun:
             destroy([self.pipe, self.listener, self.ctx])
 
 
-def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
+def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30, min_bytes=4096):
     """configs[2]: hip_ipc, one fp32 tensor, 4 KiB * 4^k up to 1 GiB, ping-pong with a peer process."""
     import numpy as np
     import torch
@@ -349,7 +349,7 @@ def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
     peer = PeerRun("basic:0,hip_ipc:11")
     out = {"sizes": {}}
     try:
-        size = 4096
+        size = min_bytes
         while size <= max_bytes:
             # seeded N(0,1) over the whole tensor, no two 16 MiB blocks alike
             host = datagen.normal_large(datagen.SEED_BASE + 3, size // 4, "f32").view(np.uint8)
@@ -384,7 +384,8 @@ def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30):
             log(f"  ipc {size:>11d} B  rtt p50 {p50:10.1f} us  payload {gbps:8.1f} GB/s  exact={ok}")
             del src, dst
             size *= 4
-        out["rtt_4KiB_p50_us"] = out["sizes"]["4096"]["rtt_p50_us"]
+        if "4096" in out["sizes"]:
+            out["rtt_4KiB_p50_us"] = out["sizes"]["4096"]["rtt_p50_us"]
     finally:
         peer.close()
     return out
@@ -456,32 +457,87 @@ def bench_cpu_path():
     return out
 
 
-def bench_cold_copy(nbytes=64 * MIB):
+def bench_cold_copy():
     """The headline loop sends the same source every step, and 64 MiB stays resident in the
-    256 MiB Infinity Cache between steps. The same kernel over ten rotating 64 MiB
-    source/destination pairs (1.25 GiB working set) shows what it does when every byte comes
-    from HBM."""
+    256 MiB Infinity Cache between steps. The same kernel over rotating source/destination pairs
+    (working set 1.25 GiB and more) shows what it does when every byte comes from HBM: the
+    headline's 64 MiB, and 256 MiB and 1 GiB as in the cross-process sweep."""
     import torch
 
     from tensorpipe_amd import hip
 
-    pairs = [(torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(),
-              torch.empty(nbytes, dtype=torch.uint8, device="cuda")) for _ in range(10)]
-    torch.cuda.synchronize()
-
-    def rotate():
-        for _ in range(4):
-            for a, b in pairs:
-                hip.copy(b, a, nbytes)
+    out = {}
+    for name, nbytes, npairs, rounds in (("64MiB", 64 * MIB, 10, 4), ("256MiB", 256 * MIB, 4, 4),
+                                         ("1GiB", 1 << 30, 2, 4)):
+        pairs = [(torch.empty(nbytes // 8, dtype=torch.int64, device="cuda").random_().view(torch.uint8),
+                  torch.empty(nbytes, dtype=torch.uint8, device="cuda")) for _ in range(npairs)]
         torch.cuda.synchronize()
 
-    rotate()
-    _, cold_n, cold_ms, _ = profiled(rotate, 64)
-    cold_us = cold_ms / max(cold_n, 1) * 1e3
-    ok = all(bool(torch.equal(a, b)) for a, b in pairs[:2])
-    gbps = 2.0 * nbytes / (cold_us * 1e-6) / 1e9
-    return {"kernel_avg_us": cold_us, "hbm_GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBPS,
-            "working_set_bytes": 20 * nbytes, "byte_exact": ok}
+        def rotate():
+            for _ in range(rounds):
+                for a, b in pairs:
+                    hip.copy(b, a, nbytes)
+            torch.cuda.synchronize()
+
+        rotate()
+        _, cold_n, cold_ms, _ = profiled(rotate, 64)
+        cold_us = cold_ms / max(cold_n, 1) * 1e3
+        ok = all(bool(torch.equal(a, b)) for a, b in pairs[:2])
+        gbps = 2.0 * nbytes / (cold_us * 1e-6) / 1e9
+        out[name] = {"kernel_avg_us": cold_us, "hbm_GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBPS,
+                     "working_set_bytes": 2 * npairs * nbytes, "byte_exact": ok}
+        del pairs
+        torch.cuda.empty_cache()
+    # the figures of the 64 MiB case at the top level, where they have always been
+    out.update(out["64MiB"])
+    return out
+
+
+def bench_link_duplex(nbytes=256 * MIB):
+    """What the one host link of the one GPU gives when both directions run at once, which is
+    what a staged transfer between two processes on one GPU does all the time (the sender's
+    device-to-host chunks and the receiver's host-to-device chunks cross the same link): the copy
+    kernel towards pinned host memory on one stream and from it on another, as one launch each
+    and as back-to-back launches of 1 MiB and 4 MiB like the channel's chunks."""
+    import ctypes
+    import time
+
+    import torch
+
+    from tensorpipe_amd import _native, hip
+
+    lib = _native.tphip()
+    dsrc = torch.empty(nbytes // 8, dtype=torch.int64, device="cuda").random_().view(torch.uint8)
+    ddst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    up = torch.empty(nbytes, dtype=torch.uint8).pin_memory()
+    down = torch.empty(nbytes // 8, dtype=torch.int64).random_().view(torch.uint8).pin_memory()
+    s_up, s_down = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    out = {}
+    for name, chunk in (("one_launch", nbytes), ("chunks_4MiB", 4 * MIB), ("chunks_1MiB", 1 * MIB)):
+        n = nbytes // chunk
+        tables = []
+        for k in range(n):
+            tables.append((hip.make_table([(dsrc.data_ptr() + k * chunk, up.data_ptr() + k * chunk, chunk)])[0],
+                           hip.make_table([(down.data_ptr() + k * chunk, ddst.data_ptr() + k * chunk, chunk)])[0]))
+        for mode in ("d2h_alone", "h2d_alone", "both"):
+            best = 0.0
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for t_up, t_down in tables:
+                    if mode != "h2d_alone":
+                        _native.check(lib.tphip_batched_copy_tuned(0, t_up, 1, s_up.cuda_stream, 4, 32, 3))
+                    if mode != "d2h_alone":
+                        _native.check(lib.tphip_batched_copy_tuned(0, t_down, 1, s_down.cuda_stream, 4, 32, 3))
+                torch.cuda.synchronize()
+                best = max(best, nbytes / (time.perf_counter() - t0) / 1e9)
+            out[f"{name}_{mode}_GBps"] = best
+    ok = bool(torch.equal(up.cuda(), dsrc)) and bool(torch.equal(down.cuda(), ddst))
+    out["byte_exact"] = ok
+    out["duplex_ceiling_GBps"] = max(out["one_launch_both_GBps"], out["chunks_4MiB_both_GBps"],
+                                     out["chunks_1MiB_both_GBps"])
+    return out
 
 
 def bench_link_ceiling(nbytes=256 * MIB):
@@ -575,6 +631,9 @@ LEGS = {
     "staged": bench_staged,
     "staged_short": lambda: bench_staged(iters=20),
     "host_link": bench_link_ceiling,
+    "host_link_duplex": bench_link_duplex,
+    "ipc_rtt": lambda: bench_ipc(iters=300, warmup=30, max_bytes=4096),
+    "ipc_large": lambda: bench_ipc(iters=40, warmup=3, min_bytes=256 * MIB),
     "cpu_path": bench_cpu_path,
     "cold_copy": bench_cold_copy,
 }
@@ -658,6 +717,29 @@ def main():
         # the same transfers with the runtime's hipMemcpyAsync instead of the copy kernel
         extra["staged_hipMemcpyAsync"] = extra_leg("staged_short", env={"TP_HIP_BASIC_ENGINE": "sdma"})
         extra["host_link"] = extra_leg("host_link")
+        # both directions of the one host link at once: what bounds a staged transfer on one GPU
+        duplex = extra_leg("host_link_duplex")
+        extra["host_link_duplex"] = duplex
+        if "duplex_ceiling_GBps" in duplex and "error" not in extra["staged"]:
+            for name, leg in extra["staged"].items():
+                if isinstance(leg, dict) and "payload_GBps" in leg:
+                    # against the link with both directions busy: as one launch per direction, and
+                    # as back-to-back launches of this leg's chunk size
+                    leg["frac_of_duplex_one_launch"] = leg["payload_GBps"] / duplex["one_launch_both_GBps"]
+                    same = duplex.get("chunks_" + name.split("_", 1)[1] + "_both_GBps")
+                    if same:
+                        leg["frac_of_duplex_same_chunks"] = leg["payload_GBps"] / same
+        # the 4 KiB round trip in three more pairs of processes: it moves by a third from one
+        # pair of processes to the next on the same box (where the hypervisor puts the threads)
+        rtts = [extra["ipc"].get("rtt_4KiB_p50_us")] if "error" not in extra["ipc"] else []
+        for _ in range(3):
+            again = extra_leg("ipc_rtt")
+            if "rtt_4KiB_p50_us" in again:
+                rtts.append(again["rtt_4KiB_p50_us"])
+        rtts = sorted(r for r in rtts if r is not None)
+        if rtts:
+            extra["ipc_rtt_4KiB"] = {"p50_us_per_process_pair": rtts,
+                                     "median_us": rtts[len(rtts) // 2], "best_us": rtts[0]}
         # the headline's tensor with four transfers in flight instead of one
         extra["d2d_in_flight"] = extra_leg("d2d_in_flight")
         extra["d2d_cold_source"] = extra_leg("cold_copy")
@@ -666,6 +748,18 @@ def main():
     log("[bench] CPU baseline (port of shm + basic)")
     cpu = cpu_baseline()
     extra["bench_wall_s"] = time.time() - t_start
+
+    roofline = d2d["roofline"]
+    # Next to the kernel's own figure (achieved / frac, from the launches' begin and end): the
+    # same bytes over the whole timed step, host time included, and what the kernel does when
+    # nothing can come from the Infinity Cache.
+    roofline["step_frac"] = 2.0 * 64 * MIB / (d2d["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBPS
+    cold = extra.get("d2d_cold_source", {})
+    if "hbm_frac" in cold:
+        roofline["hbm_only_frac"] = cold["hbm_frac"]
+    roofline["note"] = ("achieved/frac: one launch of the copy kernel, source resident in the 256 MiB Infinity "
+                        "Cache as in any loop that re-sends a 64 MiB tensor; step_frac: the whole write/read "
+                        "step; hbm_only_frac: the same kernel over rotating buffers, every byte from HBM")
 
     line = {
         "metric": "payload GB/s, same-process D2D channel (fraction of HBM roofline under roofline.frac; "
@@ -683,7 +777,7 @@ def main():
         "data": "synthetic (seeded uniform bytes)",
         "config": {"workload": "configs[1]: hip_xth same-process D2D, 1 x 64 MiB uint8 tensor, "
                                "two connected pipes in one process, write/read per step, byte-exact"},
-        "roofline": d2d["roofline"],
+        "roofline": roofline,
         "cpu_baseline": cpu,
         "extra": extra,
     }

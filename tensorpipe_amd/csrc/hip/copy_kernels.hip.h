@@ -522,10 +522,11 @@ __global__ void raise_signal_kernel(uint64_t* word, uint64_t value) {
   }
 }
 
-// One workgroup copies `bytes` bytes, any alignment: the same head / body /
-// tail split as the grid-wide kernels, four vectors in flight per lane.
-__device__ __forceinline__ void workgroup_copy(const char* src, char* dst, uint64_t bytes) {
-  const uint32_t tid = threadIdx.x;
+// THREADS lanes (a workgroup, or one wavefront of it) copy `bytes` bytes, any
+// alignment: the same head / body / tail split as the grid-wide kernels, four
+// vectors in flight per lane.
+template <uint32_t THREADS>
+__device__ __forceinline__ void team_copy(const char* src, char* dst, uint64_t bytes, uint32_t tid) {
   const uint32_t head = head_bytes(dst, bytes);
   const uint64_t nvec = (bytes - head) >> 4;
   const uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
@@ -537,21 +538,21 @@ __device__ __forceinline__ void workgroup_copy(const char* src, char* dst, uint6
   }
   const char* s = src + head;
   char* d = dst + head;
-  constexpr uint64_t kStep = 4ull * kBlockThreads;
+  constexpr uint64_t kStep = 4ull * THREADS;
   const uint64_t full = nvec / kStep * kStep;
 #pragma clang loop unroll(disable)
   for (uint64_t base = 0; base < full; base += kStep) {
     u32x4 v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      v[j] = load16<0>(s + (base + j * kBlockThreads + tid) * 16);
+      v[j] = load16<0>(s + (base + j * THREADS + tid) * 16);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      store16<0>(d + (base + j * kBlockThreads + tid) * 16, v[j]);
+      store16<0>(d + (base + j * THREADS + tid) * 16, v[j]);
     }
   }
-  for (uint64_t i = full + tid; i < nvec; i += kBlockThreads) {
+  for (uint64_t i = full + tid; i < nvec; i += THREADS) {
     store16<0>(d + i * 16, load16<0>(s + i * 16));
   }
 }
@@ -584,7 +585,7 @@ struct AgentControl {
   uint64_t pad[6];
 };
 
-__global__ __launch_bounds__(kBlockThreads) void agent_kernel(
+__global__ __launch_bounds__(kWave) void agent_kernel(
     const AgentCommand* __restrict__ ring,
     uint32_t ringMask,
     AgentControl* __restrict__ ctl,
@@ -592,56 +593,49 @@ __global__ __launch_bounds__(kBlockThreads) void agent_kernel(
     uint64_t epoch,
     uint64_t idleTicks,
     uint64_t lifeTicks) {
-  __shared__ uint64_t sCmd[5];
-  __shared__ int sLeave;
+  // One wavefront: nothing to synchronise between finding a command, copying
+  // and reporting, and 64 lanes move the few KiB a command carries in a
+  // microsecond.
+  const uint32_t lane = threadIdx.x;
   const uint64_t born = wall_clock64();
   uint64_t lastWork = born;
   for (;;) {
-    if (threadIdx.x < kWave) {
-      const uint32_t lane = threadIdx.x;
-      const AgentCommand* slot = ring + (ticket & ringMask);
-      const uint64_t tag = ticket & 0xffffu;
-      int leave = 0;
-      for (;;) {
-        uint64_t w = 0;
-        if (lane < 6) {
-          w = read_signal(&slot->w[lane]);
-        }
-        const bool ok = lane == 0 ? w == ticket : (lane < 6 ? (w >> 48) == tag : true);
-        if (__ballot(ok) == ~0ull) {
-          if (lane >= 1 && lane < 6) {
-            sCmd[lane - 1] = w & kAgentPayloadMask;
-          }
-          break;
-        }
-        const uint64_t now = wall_clock64();
-        if (now - lastWork > idleTicks || now - born > lifeTicks) {
-          leave = 1;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(1);
+    const AgentCommand* slot = ring + (ticket & ringMask);
+    const uint64_t tag = ticket & 0xffffu;
+    uint64_t w = 0;
+    bool leave = false;
+    for (;;) {
+      if (lane < 6) {
+        w = read_signal(&slot->w[lane]);
       }
-      if (lane == 0) {
-        sLeave = leave;
+      const bool ok = lane == 0 ? w == ticket : (lane < 6 ? (w >> 48) == tag : true);
+      if (__ballot(ok) == ~0ull) {
+        break;
       }
+      const uint64_t now = wall_clock64();
+      if (now - lastWork > idleTicks || now - born > lifeTicks) {
+        leave = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
     }
-    __syncthreads();
-    if (sLeave != 0) {
+    if (leave) {
       break;
     }
-    const uint64_t bytes = sCmd[2];
+    const uint64_t src = shfl64(w, 1) & kAgentPayloadMask;
+    const uint64_t dst = shfl64(w, 2) & kAgentPayloadMask;
+    const uint64_t bytes = shfl64(w, 3) & kAgentPayloadMask;
+    const uint64_t notify = shfl64(w, 4) & kAgentPayloadMask;
+    const uint64_t notifyValue = shfl64(w, 5) & kAgentPayloadMask;
     const bool stop = bytes == kAgentStopBytes;
     if (!stop) {
       // What other kernels (of this or the peer process) wrote since the last
-      // command must not be served from this workgroup's caches.
+      // command must not be served from this CU's caches.
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-      workgroup_copy(reinterpret_cast<const char*>(sCmd[0]), reinterpret_cast<char*>(sCmd[1]), bytes);
+      team_copy<kWave>(reinterpret_cast<const char*>(src), reinterpret_cast<char*>(dst), bytes, lane);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
     }
-    const uint64_t notify = sCmd[3];
-    const uint64_t notifyValue = sCmd[4];
-    __syncthreads(); // every wave's stores are out; sCmd may be rewritten
-    if (threadIdx.x == 0) {
+    if (lane == 0) {
       if (notify != 0) {
         raise_signal(reinterpret_cast<uint64_t*>(notify), notifyValue);
       }
@@ -653,7 +647,7 @@ __global__ __launch_bounds__(kBlockThreads) void agent_kernel(
     ++ticket;
     lastWork = wall_clock64();
   }
-  if (threadIdx.x == 0) {
+  if (lane == 0) {
     raise_signal(&ctl->exited, epoch);
   }
 }

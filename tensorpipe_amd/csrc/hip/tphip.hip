@@ -131,26 +131,28 @@ int defaultBlocksPerCu(bool table) {
   return table ? multi : single;
 }
 
-// Cache policy mask (bit 0 = nontemporal loads, bit 1 = nontemporal stores).
-// Stores always stream: the consumer runs later. Loads stream only for copies
-// too large for any of the source to still sit in the Infinity Cache; below
-// that, a source that was produced just before the copy is partly resident
-// and cached loads pick it up (7.2 vs 6.5 TB/s at 256 MiB, and the reverse,
-// 5.9 vs 6.3 TB/s, at 1 GiB).
+// Cache policy mask (bit 0 = nontemporal loads, bit 1 = nontemporal stores),
+// by the bytes of the launch. Up to 64 MiB everything may stay in the caches
+// (256 MiB Infinity Cache): the bytes were usually just produced and will be
+// consumed next, and a copy that reads what another copy has just written runs
+// 15 % faster when that one's stores were cached (64 MiB ping-pong between two
+// processes: 86 % of the HBM roofline against 75 % with streaming loads and
+// stores). Up to 128 MiB -- source and destination together still fit that
+// cache -- the stores stream and the loads do not: a source that is sent again
+// or was just produced is found there (the 112 MiB many-tensor message: 39 us
+// against 44 with streaming loads). Beyond that nothing of the kind survives
+// until it is needed and both stream past the caches: 256 MiB 79-80 % against
+// 76 % with cached loads and 74 % with everything cached, in the same
+// ping-pong and over rotating buffers alike; 1 GiB 74-78 % against 72 %.
 int defaultNontemporal(uint64_t totalBytes) {
   static const int forced = envInt("TPHIP_COPY_NT", -1);
   if (forced >= 0) {
     return forced & 3;
   }
-  // Up to 64 MiB everything may stay in the caches (256 MiB Infinity Cache): the
-  // bytes were usually just produced and will be consumed next, and a copy
-  // that reads what another copy has just written runs 15 % faster when that
-  // one's stores were cached. Up to 512 MiB stores stream past the cache while
-  // loads still find parts of a fresh source there; beyond, both stream.
   if (totalBytes <= (64ull << 20)) {
     return 0;
   }
-  return totalBytes <= (512ull << 20) ? 2 : 3;
+  return totalBytes <= (128ull << 20) ? 2 : 3;
 }
 
 int planViaKernel() {
@@ -857,7 +859,7 @@ int agentEnsureRunning(Agent& a) {
   // The previous agent has left: what it served is final.
   const uint64_t first = loadWord(&a.ctl->done) + 1;
   a.epoch.store(epoch + 1, std::memory_order_release);
-  return launchKernel(agent_kernel, dim3(1), dim3(kBlockThreads), 0, a.stream, a.ringDev,
+  return launchKernel(agent_kernel, dim3(1), dim3(kWave), 0, a.stream, a.ringDev,
                       kAgentRing - 1, a.ctlDev, first, epoch + 1, a.idleTicks, a.lifeTicks);
 }
 

@@ -332,6 +332,12 @@ class IpcContextCore final : public ContextCore {
   // How long the thread that posted a copy to the agent looks for its end
   // itself before leaving that to the poller thread (TP_HIP_IPC_AGENT_SPIN_US).
   const long agentSpinUs{static_cast<long>(envSize("TP_HIP_IPC_AGENT_SPIN_US", 8))};
+  // A channel with nothing else in flight looks for the acknowledgement of a
+  // small unit itself for this long after writing it, before leaving it to
+  // the poller thread: it comes about 5 us later, and whatever the send
+  // callback starts then runs on the thread that has the pipe's state in its
+  // caches (TP_HIP_IPC_ACK_SPIN_US; 1 switches it off).
+  const long ackSpinUs{static_cast<long>(envSize("TP_HIP_IPC_ACK_SPIN_US", 8))};
   // Gated copies are there, tested and switched off: TP_HIP_IPC_GATES=1 lets a
   // sender whose stream is still producing announce at once and the receiver's
   // GPU wait for its word. Measured against the host hand-off (event polled,
@@ -555,6 +561,7 @@ class ChannelImpl final : public ChannelImplBase {
     }
     wireQueue_.clear();
     replyQueue_.clear();
+    pendingAcks_.clear(); // their watchers give up (cancel_); the send ops were finished above
   }
 
  private:
@@ -673,6 +680,7 @@ class ChannelImpl final : public ChannelImplBase {
       return;
     }
     TP_MARK("ipc: send");
+    reapAcks();
     auto op = std::make_shared<SendOp>();
     op->seq = seq;
     op->cb = std::move(cb);
@@ -715,6 +723,7 @@ class ChannelImpl final : public ChannelImplBase {
         }
       }
 
+      TP_MARK("ipc: sources looked up");
       if (!direct.empty()) {
         // The distinct allocations of the unit, then the tensors by reference.
         std::vector<const ExportedAllocation*> allocs;
@@ -771,6 +780,7 @@ class ChannelImpl final : public ChannelImplBase {
             busy.push_back(s);
           }
         }
+        TP_MARK("ipc: source streams probed");
         if (busy.size() == 1 && wordsIndex_ >= 0 && peerGates_ && ictx_->gatesEnabled) {
           // One stream still producing: its last kernel is followed by a word
           // the receiver's copy waits for on the GPU.
@@ -936,26 +946,86 @@ class ChannelImpl final : public ChannelImplBase {
       };
       if (byWord) {
         ackSlotBusy_[slot] = true;
-        const uint64_t* word = &ictx_->signals->hostWords(wordsIndex_)->acks[slot];
-        const uint64_t value = seq + 1;
+        auto ack = std::make_shared<PendingAck>();
+        ack->word = &ictx_->signals->hostWords(wordsIndex_)->acks[slot];
+        ack->value = seq + 1;
+        ack->slot = slot;
+        ack->done = acknowledged;
+        pendingAcks_.push_back(ack);
+        // The poller thread watches the word; whoever runs on the loop for
+        // this channel meanwhile looks at it in passing (reapAcks).
         auto cancel = cancel_;
         auto self = shared_from_this();
         ictx_->poller.watchCondition(
-            [word, value, cancel](bool* done) {
-              *done = __atomic_load_n(word, __ATOMIC_ACQUIRE) == value ||
-                  cancel->load(std::memory_order_acquire);
+            [ack, cancel](bool* done) {
+              *done = ack->reaped.load(std::memory_order_acquire) ||
+                  cancel->load(std::memory_order_acquire) ||
+                  __atomic_load_n(ack->word, __ATOMIC_ACQUIRE) == ack->value;
               return 0;
             },
-            [this, self, slot, acknowledged](const Error& error) {
+            [this, self, ack](const Error& error) {
+              if (ack->reaped.load(std::memory_order_acquire)) {
+                return; // the loop got there first
+              }
               TP_MARK("ipc: ack word seen");
-              ctx_->defer([this, self, slot, acknowledged, error] {
+              ctx_->defer([this, self, ack, error] {
                 setError(error);
-                ackSlotBusy_[slot] = false;
-                acknowledged();
+                reap(ack);
               });
             });
       } else {
         replyConnection_->read(nullptr, 0, onRead(acknowledged));
+      }
+    }
+    // Alone on the channel: wait for the word right here for a moment.
+    if (!error_ && pendingAcks_.size() == 1 && sendOps_.size() == 1 && recvOps_.empty() &&
+        wireQueue_.empty() && ictx_->ackSpinUs > 1) {
+      auto ack = pendingAcks_.front();
+      const auto giveUp = std::chrono::steady_clock::now() + std::chrono::microseconds(ictx_->ackSpinUs);
+      do {
+        if (__atomic_load_n(ack->word, __ATOMIC_ACQUIRE) == ack->value) {
+          TP_MARK("ipc: ack word seen (inline)");
+          reap(ack);
+          break;
+        }
+      } while (std::chrono::steady_clock::now() < giveUp);
+    }
+  }
+
+  // An acknowledgement word this end waits for. Loop only, except `reaped`.
+  struct PendingAck {
+    const uint64_t* word{nullptr};
+    uint64_t value{0};
+    size_t slot{0};
+    std::function<void()> done;
+    std::atomic<bool> reaped{false};
+  };
+
+  void reap(const std::shared_ptr<PendingAck>& ack) {
+    if (ack->reaped.exchange(true)) {
+      return;
+    }
+    for (auto it = pendingAcks_.begin(); it != pendingAcks_.end(); ++it) {
+      if (*it == ack) {
+        pendingAcks_.erase(it);
+        break;
+      }
+    }
+    ackSlotBusy_[ack->slot] = false;
+    ack->done();
+    flushWire(); // a unit may have been waiting for this word to come free
+  }
+
+  // Whoever runs on the loop on behalf of this channel looks at the words it
+  // is waiting for while it is there.
+  void reapAcks() {
+    for (size_t i = 0; i < pendingAcks_.size();) {
+      auto ack = pendingAcks_[i];
+      if (__atomic_load_n(ack->word, __ATOMIC_ACQUIRE) == ack->value) {
+        TP_MARK("ipc: ack word reaped in passing");
+        reap(ack); // erases it
+      } else {
+        ++i;
       }
     }
   }
@@ -964,6 +1034,7 @@ class ChannelImpl final : public ChannelImplBase {
 
   void recvEntries(uint64_t seq, std::vector<BatchEntry> entries, TRecvCallback cb) {
     TP_MARK("ipc: recv");
+    reapAcks();
     auto op = std::make_shared<RecvOp>();
     op->seq = seq;
     op->cb = std::move(cb);
@@ -1041,6 +1112,7 @@ class ChannelImpl final : public ChannelImplBase {
 
   void onUnit(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
     TP_MARK("ipc: unit arrived");
+    reapAcks();
     WireReader r(bytes.data(), bytes.size());
     const uint8_t kind = r.u8();
     const uint8_t ackMode = r.u8();
@@ -1171,6 +1243,7 @@ class ChannelImpl final : public ChannelImplBase {
           totalBytes += length;
           ++op->unitsSeen;
         }
+        TP_MARK("ipc: unit parsed and mapped");
         // From here until the copies have finished the mappings must stay.
         for (uint32_t a = 0; a < nAllocs; ++a) {
           if (mappedOf[a] != nullptr) {
@@ -1216,6 +1289,7 @@ class ChannelImpl final : public ChannelImplBase {
           for (auto& g : groups) {
             quiet = quiet && g.dst.device == device && ictx_->idleProbe.idle(g.dst.device, g.dst.stream);
           }
+          TP_MARK("ipc: destination streams probed");
           agent = quiet ? ictx_->agent(device) : nullptr;
           if (agent != nullptr) {
             std::vector<tphip_copy_desc> all;
@@ -1628,6 +1702,7 @@ class ChannelImpl final : public ChannelImplBase {
   uint64_t nextUnitOut_{0};
   uint64_t nextUnitIn_{0};
   std::array<bool, kWordSlots> ackSlotBusy_{};
+  std::deque<std::shared_ptr<PendingAck>> pendingAcks_;
   std::shared_ptr<std::atomic<bool>> cancel_{std::make_shared<std::atomic<bool>>(false)};
   // Peer allocations this channel keeps mapped (direct route), by export id.
   struct RemoteAllocation {
