@@ -57,6 +57,7 @@ HOST_SOURCES = [
     "tensorpipe/channel/hip_basic/hip_basic.cc",
     "tensorpipe/core/core.cc",
     "capi/tensorpipe_c.cc",
+    "bridge/bridge_amd.cc",
 ]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread"]
 
@@ -96,11 +97,52 @@ def build_cpp_tests():
              "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib"])
 
 
+def stock_tensorpipe():
+    """(include dir, lib dir) of the TensorPipe that PyTorch ships prebuilt, or None."""
+    try:
+        import importlib.util
+
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        return None
+    if spec is None or not spec.origin:
+        return None
+    root = os.path.dirname(spec.origin)
+    inc, lib = os.path.join(root, "include"), os.path.join(root, "lib")
+    if os.path.exists(os.path.join(inc, "tensorpipe", "tensorpipe.h")) and \
+            os.path.exists(os.path.join(lib, "libtorch_cpu.so")):
+        return inc, lib
+    return None
+
+
+def build_stock_conformance():
+    """tests/cpp/bin/stock_conformance: this library's channels registered in the unmodified
+    TensorPipe inside libtorch_cpu.so. The adapter is compiled against the STOCK headers (listed
+    first, so that <tensorpipe/...> means theirs) and reaches this library through
+    csrc/bridge/bridge.h only. Skipped where PyTorch's headers are not installed."""
+    found = stock_tensorpipe()
+    if found is None:
+        print("stock TensorPipe headers not found: skipping tests/cpp/bin/stock_conformance", flush=True)
+        return False
+    inc, lib = found
+    src_dir = os.path.join(ROOT, "tests", "cpp")
+    bin_dir = os.path.join(src_dir, "bin")
+    os.makedirs(bin_dir, exist_ok=True)
+    run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
+         f"-I{inc}", f"-I{INCLUDE}", f"-I{CSRC}",
+         os.path.join(CSRC, "bridge", "stock_adapter.cc"), os.path.join(src_dir, "stock_conformance.cc"),
+         "-o", os.path.join(bin_dir, "stock_conformance"),
+         f"-L{LIB}", "-ltensorpipe_amd", "-ltphip", f"-L{lib}", "-ltorch_cpu", "-lc10",
+         "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib", f"-Wl,-rpath,{lib}"])
+    return True
+
+
 def build_all():
     build_tphip()
     build_datagen()
     build_host()
     build_cpp_tests()
+    build_stock_conformance()
 
 
 if __name__ == "__main__":

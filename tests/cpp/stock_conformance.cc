@@ -1,0 +1,330 @@
+// This library's channels registered in an UNMODIFIED TensorPipe: the build
+// that PyTorch ships inside libtorch_cpu.so, driven through its public headers
+// (torch/include/tensorpipe). Its Context, Listener, Pipe, shm transport and
+// basic channel are the stock ones; the only thing added is
+// tensorpipe_amd_bridge::createChannelContext(...) handed to
+// Context::registerChannel, as tensorpipe/test/core/pipe_test.h:300-316 does
+// with the CUDA channels. A message with a payload, a CPU tensor and GPU
+// tensors then travels between two stock contexts and every byte is checked.
+//
+//   stock_conformance same_process   hip_xth between two contexts of this process
+//   stock_conformance two_process    hip_ipc and hip_basic between this process and a child
+//
+// Prints "RESULT <case> OK" or "RESULT <case> FAIL <why>" per case.
+#include <tensorpipe/tensorpipe.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <future>
+#include <string>
+#include <vector>
+
+#include <sys/wait.h>
+#include <unistd.h>
+
+#include <tphip.h>
+
+#include <bridge/stock_adapter.h>
+
+using namespace tensorpipe;
+using tensorpipe_amd_bridge::HipBuffer;
+
+#define CHECK_HIP(x)                                                           \
+  do {                                                                         \
+    int rc_ = (x);                                                             \
+    if (rc_ != 0) {                                                            \
+      std::fprintf(stderr, "%s failed: %s\n", #x, tphip_strerror(rc_));        \
+      std::exit(3);                                                            \
+    }                                                                          \
+  } while (0)
+
+static std::shared_ptr<Context> makeContext(const char* name, const std::vector<std::string>& channels) {
+  auto ctx = std::make_shared<Context>(ContextOptions().name(name));
+  ctx->registerTransport(0, "shm", transport::shm::create());
+  ctx->registerChannel(0, "basic", channel::basic::create());
+  int priority = 10;
+  for (auto& c : channels) {
+    auto cc = tensorpipe_amd_bridge::createChannelContext(c);
+    if (!cc || !cc->isViable()) {
+      std::fprintf(stderr, "channel %s is not viable here\n", c.c_str());
+      std::exit(3);
+    }
+    ctx->registerChannel(priority++, c, std::move(cc));
+  }
+  return ctx;
+}
+
+static uint8_t pattern(size_t i, int salt) {
+  return static_cast<uint8_t>((i * 7 + (i >> 9) * 13 + static_cast<size_t>(salt) * 101) % 251);
+}
+
+struct GpuTensor {
+  void* dev{nullptr};
+  size_t bytes{0};
+  void* stream{nullptr};
+  void fill(int salt) {
+    std::vector<uint8_t> host(bytes);
+    for (size_t i = 0; i < bytes; ++i) {
+      host[i] = pattern(i, salt);
+    }
+    void* pinned = nullptr;
+    void* pinnedDev = nullptr;
+    CHECK_HIP(tphip_host_alloc(0, bytes, &pinned, &pinnedDev));
+    std::memcpy(pinned, host.data(), bytes);
+    CHECK_HIP(tphip_copy(0, dev, pinnedDev, bytes, stream));
+    CHECK_HIP(tphip_stream_sync(0, stream));
+    CHECK_HIP(tphip_host_free(pinned));
+  }
+  std::string check(int salt) {
+    void* pinned = nullptr;
+    void* pinnedDev = nullptr;
+    CHECK_HIP(tphip_host_alloc(0, bytes, &pinned, &pinnedDev));
+    CHECK_HIP(tphip_stream_sync(0, stream));
+    CHECK_HIP(tphip_copy(0, pinnedDev, dev, bytes, stream));
+    CHECK_HIP(tphip_stream_sync(0, stream));
+    std::string bad;
+    const uint8_t* got = static_cast<const uint8_t*>(pinned);
+    for (size_t i = 0; i < bytes; ++i) {
+      if (got[i] != pattern(i, salt)) {
+        bad = "byte " + std::to_string(i) + " of a GPU tensor differs";
+        break;
+      }
+    }
+    CHECK_HIP(tphip_host_free(pinned));
+    return bad;
+  }
+};
+
+static GpuTensor makeGpu(size_t bytes) {
+  GpuTensor t;
+  t.bytes = bytes;
+  CHECK_HIP(tphip_malloc(0, bytes, &t.dev));
+  CHECK_HIP(tphip_stream_create(0, &t.stream));
+  CHECK_HIP(tphip_fill(0, t.dev, 0xEE, bytes, t.stream));
+  CHECK_HIP(tphip_stream_sync(0, t.stream));
+  return t;
+}
+
+static const std::vector<size_t> kGpuSizes = {4096, (3u << 20) + 17, 256};
+static const size_t kCpuBytes = 70001;
+static const std::string kPayload = "payload #1";
+
+// Sends the test message on `pipe` and waits for the write callback.
+static std::string sendMessage(Pipe& pipe, int salt) {
+  std::vector<GpuTensor> gpus;
+  std::vector<uint8_t> cpu(kCpuBytes);
+  for (size_t i = 0; i < cpu.size(); ++i) {
+    cpu[i] = pattern(i, salt + 50);
+  }
+  Message m;
+  m.metadata = "conformance";
+  Message::Payload p;
+  std::string payload = kPayload;
+  p.data = payload.data();
+  p.length = payload.size();
+  m.payloads.push_back(std::move(p));
+  for (size_t k = 0; k < kGpuSizes.size(); ++k) {
+    gpus.push_back(makeGpu(kGpuSizes[k]));
+    gpus.back().fill(salt + static_cast<int>(k));
+    Message::Tensor t;
+    t.buffer = HipBuffer{gpus.back().dev, gpus.back().stream, 0};
+    t.length = gpus.back().bytes;
+    t.targetDevice = Device{"cuda", 0};
+    m.tensors.push_back(std::move(t));
+  }
+  Message::Tensor ct;
+  ct.buffer = CpuBuffer{cpu.data()};
+  ct.length = cpu.size();
+  m.tensors.push_back(std::move(ct));
+  std::promise<std::string> done;
+  pipe.write(std::move(m), [&done](const Error& e) { done.set_value(e ? e.what() : std::string()); });
+  auto f = done.get_future();
+  if (f.wait_for(std::chrono::seconds(60)) != std::future_status::ready) {
+    return "write never completed";
+  }
+  return f.get();
+}
+
+static std::string recvMessage(Pipe& pipe, int salt) {
+  std::promise<std::string> done;
+  std::vector<GpuTensor> gpus;
+  std::vector<uint8_t> cpu;
+  std::string payload;
+  pipe.readDescriptor([&](const Error& e, Descriptor d) {
+    if (e) {
+      done.set_value("readDescriptor: " + e.what());
+      return;
+    }
+    if (d.metadata != "conformance" || d.payloads.size() != 1 || d.tensors.size() != kGpuSizes.size() + 1) {
+      done.set_value("unexpected descriptor");
+      return;
+    }
+    Allocation a;
+    payload.resize(d.payloads[0].length);
+    a.payloads.resize(1);
+    a.payloads[0].data = &payload[0];
+    a.tensors.resize(d.tensors.size());
+    for (size_t k = 0; k < kGpuSizes.size(); ++k) {
+      if (d.tensors[k].length != kGpuSizes[k] || d.tensors[k].sourceDevice.type != "cuda") {
+        done.set_value("unexpected GPU tensor in the descriptor");
+        return;
+      }
+      gpus.push_back(makeGpu(kGpuSizes[k]));
+      a.tensors[k].buffer = HipBuffer{gpus.back().dev, gpus.back().stream, 0};
+    }
+    cpu.assign(d.tensors.back().length, 0);
+    a.tensors.back().buffer = CpuBuffer{cpu.data()};
+    pipe.read(std::move(a), [&done](const Error& e2) { done.set_value(e2 ? "read: " + e2.what() : std::string()); });
+  });
+  auto f = done.get_future();
+  if (f.wait_for(std::chrono::seconds(60)) != std::future_status::ready) {
+    return "read never completed";
+  }
+  std::string err = f.get();
+  if (!err.empty()) {
+    return err;
+  }
+  if (payload != kPayload) {
+    return "payload differs";
+  }
+  for (size_t k = 0; k < gpus.size(); ++k) {
+    std::string bad = gpus[k].check(salt + static_cast<int>(k));
+    if (!bad.empty()) {
+      return bad;
+    }
+  }
+  if (cpu.size() != kCpuBytes) {
+    return "CPU tensor has the wrong length";
+  }
+  for (size_t i = 0; i < cpu.size(); ++i) {
+    if (cpu[i] != pattern(i, salt + 50)) {
+      return "byte " + std::to_string(i) + " of the CPU tensor differs";
+    }
+  }
+  return "";
+}
+
+static void report(const std::string& name, const std::string& problem) {
+  if (problem.empty()) {
+    std::printf("RESULT %s OK\n", name.c_str());
+  } else {
+    std::printf("RESULT %s FAIL %s\n", name.c_str(), problem.c_str());
+  }
+  std::fflush(stdout);
+}
+
+static std::shared_ptr<Pipe> acceptOne(Listener& listener) {
+  std::promise<std::shared_ptr<Pipe>> pp;
+  listener.accept([&pp](const Error& e, std::shared_ptr<Pipe> pipe) {
+    if (e) {
+      std::fprintf(stderr, "accept: %s\n", e.what().c_str());
+    }
+    pp.set_value(std::move(pipe));
+  });
+  return pp.get_future().get();
+}
+
+static int sameProcess() {
+  const std::string addr = "shm://tpamd_conf_" + std::to_string(::getpid());
+  auto server = makeContext("server", {"hip_xth"});
+  auto client = makeContext("client", {"hip_xth"});
+  auto listener = server->listen({addr});
+  auto cpipe = client->connect(listener->url("shm"));
+  auto spipe = acceptOne(*listener);
+  std::string problem;
+  for (int round = 0; round < 3 && problem.empty(); ++round) {
+    auto sent = std::async(std::launch::async, [&] { return sendMessage(*cpipe, 10 * round); });
+    problem = recvMessage(*spipe, 10 * round);
+    const std::string w = sent.get();
+    if (problem.empty()) {
+      problem = w;
+    }
+    // and back
+    if (problem.empty()) {
+      auto sent2 = std::async(std::launch::async, [&] { return sendMessage(*spipe, 10 * round + 5); });
+      problem = recvMessage(*cpipe, 10 * round + 5);
+      const std::string w2 = sent2.get();
+      if (problem.empty()) {
+        problem = w2;
+      }
+    }
+  }
+  if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() != 3 * 2 * 3 * 2) {
+    problem = "the GPU tensors did not all travel on this library's channel: " +
+        std::to_string(tensorpipe_amd_bridge::gpuOperationsServed()) + " operations served";
+  }
+  report("hip_xth_in_stock_context", problem);
+  cpipe.reset();
+  spipe.reset();
+  listener.reset();
+  client->join();
+  server->join();
+  return problem.empty() ? 0 : 1;
+}
+
+static int twoProcess(const std::string& channel) {
+  const std::string addr = "shm://tpamd_conf2_" + channel + "_" + std::to_string(::getpid());
+  int go[2];
+  if (::pipe(go) != 0) {
+    return 3;
+  }
+  pid_t pid = ::fork(); // before anything has touched the GPU
+  if (pid == 0) {
+    char byte = 0;
+    if (::read(go[0], &byte, 1) != 1) { // the parent is listening now
+      ::_exit(2);
+    }
+    auto ctx = makeContext("peer", {channel});
+    auto pipe = ctx->connect(addr);
+    std::string problem = recvMessage(*pipe, 1);
+    if (problem.empty()) {
+      problem = sendMessage(*pipe, 2);
+    }
+    if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() != 6) {
+      problem = "the GPU tensors did not all travel on this library's channel";
+    }
+    if (!problem.empty()) {
+      std::fprintf(stderr, "[peer] %s\n", problem.c_str());
+    }
+    pipe.reset();
+    ctx->join();
+    ::_exit(problem.empty() ? 0 : 1);
+  }
+  auto ctx = makeContext("main", {channel});
+  auto listener = ctx->listen({addr});
+  const char byte = 1;
+  if (::write(go[1], &byte, 1) != 1) {
+    return 3;
+  }
+  auto pipe = acceptOne(*listener);
+  std::string problem = pipe ? sendMessage(*pipe, 1) : std::string("accept failed");
+  if (problem.empty()) {
+    problem = recvMessage(*pipe, 2);
+  }
+  int status = 0;
+  ::waitpid(pid, &status, 0);
+  if (problem.empty() && !(WIFEXITED(status) && WEXITSTATUS(status) == 0)) {
+    problem = "the peer process reported a failure";
+  }
+  if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() != 6) {
+    problem = "the GPU tensors did not all travel on this library's channel: " +
+        std::to_string(tensorpipe_amd_bridge::gpuOperationsServed()) + " operations served";
+  }
+  report(channel + "_in_stock_context", problem);
+  pipe.reset();
+  listener.reset();
+  ctx->join();
+  return problem.empty() ? 0 : 1;
+}
+
+int main(int argc, char** argv) {
+  if (argc == 2 && std::strcmp(argv[1], "same_process") == 0) {
+    return sameProcess();
+  }
+  if (argc == 3 && std::strcmp(argv[1], "two_process") == 0) {
+    return twoProcess(argv[2]);
+  }
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic\n", argv[0]);
+  return 2;
+}

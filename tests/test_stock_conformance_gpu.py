@@ -1,0 +1,38 @@
+"""This library's device channels registered in an UNMODIFIED TensorPipe: the build that PyTorch
+ships inside libtorch_cpu.so (its own Context, Pipe, shm transport and basic channel), with
+hip_xth / hip_ipc / hip_basic added through Context::registerChannel exactly as the reference
+registers its CUDA channels (tensorpipe/core/context.h:67-70,
+tensorpipe/test/core/pipe_test.h:300-316). tests/cpp/stock_conformance.cc sends a message with a
+payload, three GPU tensors and one CPU tensor each way and checks every byte.
+
+The program only exists where PyTorch's TensorPipe headers were present at build time.
+"""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROGRAM = os.path.join(ROOT, "tests", "cpp", "bin", "stock_conformance")
+
+
+def _run(args):
+    if not os.path.exists(PROGRAM):
+        pytest.skip("tests/cpp/bin/stock_conformance is not built (no stock TensorPipe headers at build time)")
+    print("running stock_conformance", *args, flush=True)
+    proc = subprocess.run([PROGRAM, *args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    results = [line for line in proc.stdout.splitlines() if line.startswith("RESULT ")]
+    assert results, f"no result line; exit code {proc.returncode}\n{proc.stdout[-2000:]}\n{proc.stderr[-2000:]}"
+    bad = [line for line in results if line.split()[2] != "OK"]
+    assert not bad and proc.returncode == 0, "\n".join(bad) + f"\nexit code {proc.returncode}\n" + proc.stderr[-2000:]
+
+
+def test_hip_xth_in_a_stock_context_same_process():
+    _run(["same_process"])
+
+
+@pytest.mark.parametrize("channel", ["hip_ipc", "hip_basic"])
+def test_channel_in_stock_contexts_of_two_processes(channel):
+    _run(["two_process", channel])
