@@ -15,6 +15,13 @@
 
 #include <bridge/bridge.h>
 
+#ifdef TPAMD_BRIDGE_HOST_HAS_CHANNEL_HEADERS
+#include <tensorpipe/channel/channel.h>
+#include <tensorpipe/transport/connection.h>
+#else
+// A host that installs channel/context.h without these two abstract classes
+// (PyTorch does): their declaration, virtual functions in the order of
+// tensorpipe/transport/connection.h:21-69 and tensorpipe/channel/channel.h:52-72.
 namespace tensorpipe {
 
 class AbstractNopHolder; // only ever named, in two members this adapter does not call
@@ -50,6 +57,7 @@ class Channel {
 } // namespace channel
 
 } // namespace tensorpipe
+#endif
 
 namespace tensorpipe_amd_bridge {
 
