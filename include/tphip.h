@@ -242,7 +242,8 @@ int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream
  * `unroll` in {1,2,4,8} 16-byte vectors in flight per lane, `blocks` workgroups
  * of 256 threads (0 = default: one per CU), `nontemporal` a mask (bit 0 =
  * nontemporal loads, bit 1 = nontemporal stores; negative = the default, which
- * goes by the bytes of the launch: 0 up to 64 MiB, 2 up to 128 MiB, 3 above). */
+ * goes by the bytes of the launch: 0 up to 64 MiB, up to 128 MiB 2 for a single entry and 0
+ * for a table, 3 above). */
 int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
                              int unroll, uint32_t blocks, int nontemporal);
 

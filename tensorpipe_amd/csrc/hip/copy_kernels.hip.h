@@ -137,66 +137,66 @@ __device__ __forceinline__ bool pass_gate(const Gate& g) {
   return __hip_atomic_load(g.state, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == kGateOpen;
 }
 
-// Entries whose heads and tails one wavefront moves. The gather below is a
-// chain of dependent byte loads and stores (about one memory latency per 64
-// bytes), so a group is kept small and the groups spread over many waves: 64
-// entries per wave left one workgroup busy for microseconds after every other
-// one had finished.
-constexpr uint32_t kEdgeGroup = 8;
+// Entries whose heads and tails one wavefront moves: sixteen lanes per entry,
+// lane k of them owning byte k of the head and byte k of the tail (each at
+// most 15 bytes long). No lane needs to know about another entry, so the
+// wave spends a few LDS reads and two byte loads on it, nothing that depends
+// on a neighbour. (Gathering the bytes of more entries densely over the lanes
+// took a prefix scan and a search through cross-lane moves, about 1.5 us of
+// dependent latencies on the waves that did it, and those waves finished last.)
+constexpr uint32_t kEdgeGroup = kWave / 16;
+
+// In two halves, so that the latency of the byte loads hides behind the
+// wave's share of the bodies: edge_loads() before the chunk loop issues the
+// loads and keeps value and destination per lane, edge_stores() after it
+// writes them out. `entry(t, &src, &dst, &bytes)` yields entry t as the caller
+// gave it.
+struct EdgeBytes {
+  char* dst[2]; // head byte, tail byte; nullptr: none held
+  uint8_t val[2];
+};
+
+template <typename Entry>
+__device__ __forceinline__ void edge_loads(
+    Entry entry, uint32_t n, uint32_t group, uint32_t lane, EdgeBytes& held) {
+  held.dst[0] = held.dst[1] = nullptr;
+  held.val[0] = held.val[1] = 0;
+  const uint32_t t = group * kEdgeGroup + (lane >> 4);
+  const uint32_t k = lane & 15u;
+  if (t >= n) {
+    return;
+  }
+  uint64_t src = 0, dst = 0, bytes = 0;
+  entry(t, &src, &dst, &bytes);
+  const uint32_t head = head_bytes(reinterpret_cast<const void*>(dst), bytes);
+  const uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
+  if (k < head) {
+    held.val[0] = reinterpret_cast<const uint8_t*>(src)[k];
+    held.dst[0] = reinterpret_cast<char*>(dst) + k;
+  }
+  if (k < tail) {
+    const uint64_t off = bytes - tail + k;
+    held.val[1] = reinterpret_cast<const uint8_t*>(src)[off];
+    held.dst[1] = reinterpret_cast<char*>(dst) + off;
+  }
+}
+
+__device__ __forceinline__ void edge_stores(const EdgeBytes& held) {
+  if (held.dst[0] != nullptr) {
+    __builtin_nontemporal_store(static_cast<char>(held.val[0]), held.dst[0]);
+  }
+  if (held.dst[1] != nullptr) {
+    __builtin_nontemporal_store(static_cast<char>(held.val[1]), held.dst[1]);
+  }
+}
 
 // One wavefront moves the heads and tails of entries
-// [kEdgeGroup*group, kEdgeGroup*(group+1)); all 64 lanes share the byte copies.
-// `entry(t, &src, &dst, &bytes)` yields entry t as the caller gave it.
+// [kEdgeGroup*group, kEdgeGroup*(group+1)).
 template <typename Entry>
 __device__ __forceinline__ void copy_edges(Entry entry, uint32_t n, uint32_t group, uint32_t lane) {
-  uint32_t t = group * kEdgeGroup + lane;
-  uint64_t src = 0, dst = 0, bytes = 0;
-  if (lane < kEdgeGroup && t < n) {
-    entry(t, &src, &dst, &bytes);
-  }
-  uint32_t head = head_bytes(reinterpret_cast<const void*>(dst), bytes);
-  uint32_t tail = static_cast<uint32_t>((bytes - head) & 15u);
-  uint64_t tailOff = bytes - tail;
-  uint32_t cnt = head + tail;
-  if (__ballot(cnt != 0) == 0) {
-    return; // every entry of this group is vector-aligned at both ends
-  }
-  uint32_t incl = cnt;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    uint32_t o = __shfl_up(incl, d);
-    if (lane >= static_cast<uint32_t>(d)) {
-      incl += o;
-    }
-  }
-  uint32_t excl = incl - cnt;
-  uint32_t total = __shfl(incl, kWave - 1);
-  for (uint32_t base = 0; base < total; base += kWave) {
-    uint32_t b = base + lane;
-    bool active = b < total;
-    uint32_t bb = active ? b : total - 1;
-    // Largest lane whose exclusive prefix is <= bb owns byte bb.
-    int lo = 0, hi = kWave;
-#pragma unroll
-    for (int it = 0; it < 6; ++it) {
-      int mid = (lo + hi) >> 1;
-      uint32_t e = __shfl(excl, mid);
-      if (e <= bb) {
-        lo = mid;
-      } else {
-        hi = mid;
-      }
-    }
-    uint32_t k = bb - __shfl(excl, lo);
-    uint32_t oh = __shfl(head, lo);
-    uint64_t osrc = shfl64(src, lo);
-    uint64_t odst = shfl64(dst, lo);
-    uint64_t otail = shfl64(tailOff, lo);
-    uint64_t off = k < oh ? k : otail + (k - oh);
-    if (active) {
-      reinterpret_cast<char*>(odst)[off] = reinterpret_cast<const char*>(osrc)[off];
-    }
-  }
+  EdgeBytes held;
+  edge_loads(entry, n, group, lane, held);
+  edge_stores(held);
 }
 
 // Where the 16-byte aligned body of an entry starts (src + head, dst + head),
@@ -272,6 +272,18 @@ __device__ __forceinline__ void table_copy(
     w.d = body[w.t].dst + off;
     return w;
   };
+
+  // Heads and tails go to the waves at the far end of the grid, whose
+  // workgroups run out of chunks first. The byte-wise gather is a chain of
+  // dependent memory latencies: its loads are issued here, ahead of the wave's
+  // chunks, and its stores follow them.
+  const uint32_t edgeGroup = nwaves - 1 - wave;
+  const bool hasEdges = edgeGroup * kEdgeGroup < n;
+  EdgeBytes held;
+  if (hasEdges) {
+    edge_loads(entry, n, edgeGroup, lane, held);
+  }
+  bool edgesHeld = hasEdges;
 
   Where cur{};
   if (blockIdx.x < nchunks) {
@@ -350,13 +362,23 @@ __device__ __forceinline__ void table_copy(
       }
     }
     cur = nxt;
+    if (edgesHeld) {
+      // Right behind the wave's first chunk: the loads have long returned, and
+      // the partly written lines leave the L2 while the copy is still running
+      // rather than in the write-back at the end of the kernel.
+      edge_stores(held);
+      edgesHeld = false;
+    }
   }
 
-  // Heads and tails last, on the waves at the far end of the grid (they run
-  // out of chunks first): the byte-wise gather is latency-bound and would
-  // otherwise delay the chunks of the workgroup that does it.
-  for (uint32_t g = nwaves - 1 - wave; g * kEdgeGroup < n; g += nwaves) {
-    copy_edges(entry, n, g, lane);
+  if (hasEdges) {
+    if (edgesHeld) {
+      edge_stores(held);
+    }
+    // Tables with more groups than the grid has waves: the rest, one by one.
+    for (uint32_t g = edgeGroup + nwaves; g * kEdgeGroup < n; g += nwaves) {
+      copy_edges(entry, n, g, lane);
+    }
   }
 }
 
@@ -374,12 +396,42 @@ __global__ __launch_bounds__(kBlockThreads) void batched_copy_kernel(
   }
   const bool cached = n <= kLdsBodies;
   CopyBody* sBodies = reinterpret_cast<CopyBody*>(sPrefix + ((n + 1 + 3) & ~3u));
-  for (uint32_t i = threadIdx.x; i <= n; i += kBlockThreads) {
-    sPrefix[i] = prefix[i];
+  // Four loads per thread in flight before the first LDS write: a pass that
+  // waits for every load before issuing the next costs a memory latency per
+  // 256 entries, and every workgroup pays it before its first chunk.
+  constexpr int kBatch = 4;
+  for (uint32_t base = 0; base <= n; base += kBatch * kBlockThreads) {
+    uint32_t w[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const uint32_t i = base + k * kBlockThreads + threadIdx.x;
+      w[k] = i <= n ? prefix[i] : 0u;
+    }
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const uint32_t i = base + k * kBlockThreads + threadIdx.x;
+      if (i <= n) {
+        sPrefix[i] = w[k];
+      }
+    }
   }
   if (cached) {
-    for (uint32_t i = threadIdx.x; i < n; i += kBlockThreads) {
-      sBodies[i] = bodies[i];
+    const u32x4* in = reinterpret_cast<const u32x4*>(bodies);
+    u32x4* out = reinterpret_cast<u32x4*>(sBodies);
+    for (uint32_t base = 0; base < n; base += kBatch * kBlockThreads) {
+      u32x4 w[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const uint32_t i = base + k * kBlockThreads + threadIdx.x;
+        w[k] = in[i < n ? i : n - 1];
+      }
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const uint32_t i = base + k * kBlockThreads + threadIdx.x;
+        if (i < n) {
+          out[i] = w[k];
+        }
+      }
     }
   }
   __syncthreads();
@@ -426,20 +478,30 @@ __global__ __launch_bounds__(kBlockThreads) void inline_copy_kernel(
   if (!pass_gate(gate)) {
     return;
   }
-  // Only what n entries use: header + prefix, bodies, edge bytes.
+  // Only what n entries use: header + prefix, bodies, edge bytes. All loads
+  // of a thread are issued before its first LDS write, so the fill costs one
+  // memory latency, not one per pass.
   const uint32_t n = plan.n;
   const uint32_t* in = reinterpret_cast<const uint32_t*>(&plan);
   uint32_t* out = reinterpret_cast<uint32_t*>(&sPlan);
   constexpr uint32_t kBodiesAt = offsetof(InlinePlanT<N>, bodies) / 4;
   constexpr uint32_t kEdgesAt = offsetof(InlinePlanT<N>, edges) / 4;
-  for (uint32_t i = threadIdx.x; i < 2 + n + 1; i += kBlockThreads) {
-    out[i] = in[i];
+  constexpr uint32_t kWords = sizeof(InlinePlanT<N>) / 4;
+  constexpr int kPerThread = (kWords + kBlockThreads - 1) / kBlockThreads;
+  uint32_t word[kPerThread];
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const uint32_t i = k * kBlockThreads + threadIdx.x;
+    const bool used = i < 2 + n + 1 || (i >= kBodiesAt && i < kBodiesAt + n * 4) ||
+        (i >= kEdgesAt && i < kEdgesAt + (n + 3) / 4);
+    word[k] = used ? in[i] : 0u;
   }
-  for (uint32_t i = threadIdx.x; i < n * 4; i += kBlockThreads) {
-    out[kBodiesAt + i] = in[kBodiesAt + i];
-  }
-  for (uint32_t i = threadIdx.x; i < (n + 3) / 4; i += kBlockThreads) {
-    out[kEdgesAt + i] = in[kEdgesAt + i];
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const uint32_t i = k * kBlockThreads + threadIdx.x;
+    if (i < kWords) {
+      out[i] = word[k];
+    }
   }
   __syncthreads();
   const InlinePlanT<N>* p = &sPlan;
