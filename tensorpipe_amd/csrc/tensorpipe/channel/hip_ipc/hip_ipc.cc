@@ -249,7 +249,7 @@ struct Outbox {
 // on behalf of either process.
 constexpr size_t kWordSlots = 64;
 struct ChannelWords {
-  uint64_t acks[kWordSlots]; // acks[u % 64] == u + 1: the peer has copied unit u (raised by the peer's copy)
+  uint64_t acks[kWordSlots]; // acks[u % 64] == ackValue(generation, u): the peer has copied unit u (raised by the peer's copy)
   uint64_t ready[kWordSlots]; // ready[k % 64] > k: the sources of the k-th gated unit are ready (raised by the owner's stream)
   uint64_t expired[kWordSlots]; // this end's own gated copies report here that they gave up waiting
 };
@@ -267,13 +267,19 @@ class SignalSlab {
       free_.push_back(kChannelsPerSlab - 1 - i);
     }
   }
-  int acquire() {
+  // The index of a free set of words, or -1. `generation` tells this use of
+  // the words from earlier ones: a copy of a channel that is gone may still
+  // raise a word after the words have gone to the next channel, and must not
+  // be taken for the acknowledgement that one waits for.
+  int acquire(uint32_t* generation) {
     std::lock_guard<std::mutex> lock(mutex_);
     if (free_.empty()) {
       return -1;
     }
     const uint32_t i = free_.back();
     free_.pop_back();
+    nextGeneration_ = nextGeneration_ % 0xffffu + 1; // 1..65535
+    *generation = nextGeneration_;
     return static_cast<int>(i);
   }
   void release(int index) {
@@ -310,7 +316,15 @@ class SignalSlab {
   const uint64_t id_{nextExportId()};
   std::mutex mutex_;
   std::vector<uint32_t> free_;
+  uint32_t nextGeneration_{0};
 };
+
+// What acks[unit % 64] reads once the peer has copied `unit`: the unit's
+// number (+1, so that zeroed words mean nothing) under the generation of the
+// words' current user. Fits the 48 bits a copy agent command carries.
+uint64_t ackValue(uint32_t generation, uint64_t unitSeq) {
+  return (static_cast<uint64_t>(generation & 0xffffu) << 32) | ((unitSeq + 1) & 0xffffffffu);
+}
 
 bool envFlag(const char* name, bool fallback) {
   const char* e = std::getenv(name);
@@ -327,6 +341,7 @@ class IpcContextCore final : public ContextCore {
   // Tensors of a unit adding up to at most this many bytes go to the copy
   // agent when their streams are idle (TP_HIP_IPC_AGENT=0 switches it off,
   // TP_HIP_IPC_AGENT_MAX_BYTES moves the limit).
+  std::atomic<uint64_t> nextGateValue{0}; // what the gates of this context's channels wait for, ever growing
   const bool agentEnabled{envFlag("TP_HIP_IPC_AGENT", true)};
   const size_t agentMaxBytes{envSize("TP_HIP_IPC_AGENT_MAX_BYTES", 64 * 1024)};
   // How long the thread that posted a copy to the agent looks for its end
@@ -489,7 +504,7 @@ class ChannelImpl final : public ChannelImplBase {
   // it is always there before the first unit.
   void initFromLoop() override {
     if (ictx_->signals) {
-      wordsIndex_ = ictx_->signals->acquire();
+      wordsIndex_ = ictx_->signals->acquire(&wordsGeneration_);
     }
     WireWriter w;
     w.u8(kHello);
@@ -502,6 +517,7 @@ class ChannelImpl final : public ChannelImplBase {
       w.u64(slab.base());
       w.u64(slab.size());
       w.u32(static_cast<uint32_t>(wordsIndex_ * sizeof(ChannelWords)));
+      w.u32(wordsGeneration_);
     }
     // what this end's copy agent takes in one unit (0: it has none)
     w.u64(ictx_->agentEnabled ? ictx_->agentMaxBytes : 0);
@@ -649,6 +665,7 @@ class ChannelImpl final : public ChannelImplBase {
     const uint64_t base = r.u64();
     const uint64_t size = r.u64();
     const uint32_t offset = r.u32();
+    peerWordsGeneration_ = r.u32();
     peerAgentMaxBytes_ = r.u64();
     peerGates_ = true; // an end with words of its own can run gated copies
     if (!r.ok() || size < sizeof(ChannelWords) || offset > size - sizeof(ChannelWords) ||
@@ -784,9 +801,10 @@ class ChannelImpl final : public ChannelImplBase {
         if (busy.size() == 1 && wordsIndex_ >= 0 && peerGates_ && ictx_->gatesEnabled) {
           // One stream still producing: its last kernel is followed by a word
           // the receiver's copy waits for on the GPU.
-          const uint64_t k = nextGate_++;
-          gateSlot = static_cast<uint32_t>(k % kWordSlots);
-          gateValue = k + 1;
+          // Values grow over the whole context, so a word raised late for a
+          // channel that is gone can never open a gate of the words' next user.
+          gateSlot = static_cast<uint32_t>(nextGate_++ % kWordSlots);
+          gateValue = ictx_->nextGateValue.fetch_add(1, std::memory_order_relaxed) + 1;
           TP_HIP_CHECK(tphip_stream_signal(
               busy[0].device,
               busy[0].stream,
@@ -948,7 +966,7 @@ class ChannelImpl final : public ChannelImplBase {
         ackSlotBusy_[slot] = true;
         auto ack = std::make_shared<PendingAck>();
         ack->word = &ictx_->signals->hostWords(wordsIndex_)->acks[slot];
-        ack->value = seq + 1;
+        ack->value = ackValue(wordsGeneration_, seq);
         ack->slot = slot;
         ack->done = acknowledged;
         pendingAcks_.push_back(ack);
@@ -1298,7 +1316,8 @@ class ChannelImpl final : public ChannelImplBase {
             }
             void* notify = completion.byWord ? &peerWords_->acks[unitSeq % kWordSlots] : nullptr;
             const int rc = tphip_agent_submit(
-                agent, all.data(), static_cast<uint32_t>(all.size()), notify, unitSeq + 1, &agentTicket);
+                agent, all.data(), static_cast<uint32_t>(all.size()), notify,
+                ackValue(peerWordsGeneration_, unitSeq), &agentTicket);
             viaAgent = rc == 0; // a full ring or an address it cannot carry: launch as usual
             TP_MARK("ipc: posted to the agent");
           }
@@ -1320,7 +1339,7 @@ class ChannelImpl final : public ChannelImplBase {
                 launchedOn[0].device,
                 launchedOn[0].stream,
                 &peerWords_->acks[unitSeq % kWordSlots],
-                unitSeq + 1));
+                ackValue(peerWordsGeneration_, unitSeq)));
           }
         }
         op->unitsExpected += n;
@@ -1552,7 +1571,7 @@ class ChannelImpl final : public ChannelImplBase {
           first.device,
           first.stream,
           &peerWords_->acks[u->completion.unitSeq % kWordSlots],
-          u->completion.unitSeq + 1);
+          ackValue(peerWordsGeneration_, u->completion.unitSeq));
     }
     unitCopiesFinished(u->completion);
     --u->op->landing;
@@ -1697,6 +1716,8 @@ class ChannelImpl final : public ChannelImplBase {
   ChannelWords* peerWords_{nullptr}; // a device address: kernels only, never this process's CPUs
   uint64_t peerAgentMaxBytes_{0};
   bool peerGates_{false};
+  uint32_t wordsGeneration_{0}; // of this end's words, told to the peer in the hello
+  uint32_t peerWordsGeneration_{0};
   uint64_t nextGate_{0};
   uint64_t nextExpired_{0};
   uint64_t nextUnitOut_{0};
