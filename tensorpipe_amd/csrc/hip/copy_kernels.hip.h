@@ -584,9 +584,30 @@ __global__ void raise_signal_kernel(uint64_t* word, uint64_t value) {
   }
 }
 
+// K vectors per lane in flight over as many whole K * THREADS blocks as are
+// left from vector `done` on; returns the first vector not yet copied.
+template <uint32_t THREADS, int K>
+__device__ __forceinline__ uint64_t team_sweep(
+    const char* s, char* d, uint64_t done, uint64_t nvec, uint32_t tid) {
+  constexpr uint64_t kStep = static_cast<uint64_t>(K) * THREADS;
+  const uint64_t end = done + (nvec - done) / kStep * kStep;
+#pragma clang loop unroll(disable)
+  for (uint64_t base = done; base < end; base += kStep) {
+    u32x4 v[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      v[j] = load16<0>(s + (base + j * THREADS + tid) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      store16<0>(d + (base + j * THREADS + tid) * 16, v[j]);
+    }
+  }
+  return end;
+}
+
 // THREADS lanes (a workgroup, or one wavefront of it) copy `bytes` bytes, any
-// alignment: the same head / body / tail split as the grid-wide kernels, four
-// vectors in flight per lane.
+// alignment: the same head / body / tail split as the grid-wide kernels.
 template <uint32_t THREADS>
 __device__ __forceinline__ void team_copy(const char* src, char* dst, uint64_t bytes, uint32_t tid) {
   const uint32_t head = head_bytes(dst, bytes);
@@ -600,22 +621,14 @@ __device__ __forceinline__ void team_copy(const char* src, char* dst, uint64_t b
   }
   const char* s = src + head;
   char* d = dst + head;
-  constexpr uint64_t kStep = 4ull * THREADS;
-  const uint64_t full = nvec / kStep * kStep;
-#pragma clang loop unroll(disable)
-  for (uint64_t base = 0; base < full; base += kStep) {
-    u32x4 v[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      v[j] = load16<0>(s + (base + j * THREADS + tid) * 16);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      store16<0>(d + (base + j * THREADS + tid) * 16, v[j]);
-    }
-  }
-  for (uint64_t i = full + tid; i < nvec; i += THREADS) {
-    store16<0>(d + i * 16, load16<0>(s + i * 16));
+  // A team this small is bound by memory latency, not bandwidth: sixteen
+  // vectors per lane in flight while whole blocks of that size are left (one
+  // wavefront: 16 KiB per round trip to memory), then four, then one.
+  uint64_t done = team_sweep<THREADS, 16>(s, d, 0, nvec, tid);
+  done = team_sweep<THREADS, 4>(s, d, done, nvec, tid);
+  done = team_sweep<THREADS, 1>(s, d, done, nvec, tid);
+  if (done + tid < nvec) {
+    store16<0>(d + (done + tid) * 16, load16<0>(s + (done + tid) * 16));
   }
 }
 

@@ -343,7 +343,7 @@ class IpcContextCore final : public ContextCore {
   // TP_HIP_IPC_AGENT_MAX_BYTES moves the limit).
   std::atomic<uint64_t> nextGateValue{0}; // what the gates of this context's channels wait for, ever growing
   const bool agentEnabled{envFlag("TP_HIP_IPC_AGENT", true)};
-  const size_t agentMaxBytes{envSize("TP_HIP_IPC_AGENT_MAX_BYTES", 64 * 1024)};
+  const size_t agentMaxBytes{envSize("TP_HIP_IPC_AGENT_MAX_BYTES", 128 * 1024)};
   // How long the thread that posted a copy to the agent looks for its end
   // itself before leaving that to the poller thread (TP_HIP_IPC_AGENT_SPIN_US).
   const long agentSpinUs{static_cast<long>(envSize("TP_HIP_IPC_AGENT_SPIN_US", 8))};
