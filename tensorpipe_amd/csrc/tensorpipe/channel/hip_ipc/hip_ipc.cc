@@ -250,7 +250,7 @@ struct Outbox {
 constexpr size_t kWordSlots = 64;
 struct ChannelWords {
   uint64_t acks[kWordSlots]; // acks[u % 64] == ackValue(generation, u): the peer has copied unit u (raised by the peer's copy)
-  uint64_t ready[kWordSlots]; // ready[k % 64] > k: the sources of the k-th gated unit are ready (raised by the owner's stream)
+  uint64_t ready[kWordSlots]; // ready[k % 64] >= the value named in the k-th gated unit: its sources are ready (raised by the owner's stream)
   uint64_t expired[kWordSlots]; // this end's own gated copies report here that they gave up waiting
 };
 constexpr size_t kChannelsPerSlab = 256;
@@ -338,10 +338,12 @@ class IpcContextCore final : public ContextCore {
   // Signal words for the channels of this context; null when switched off
   // (TP_HIP_IPC_SIGNALS=0) or when pinned memory cannot be exported here.
   std::unique_ptr<SignalSlab> signals;
+  // What the gates of this context's channels wait for: ever growing, so that
+  // a word raised late for a channel that is gone opens nobody else's gate.
+  std::atomic<uint64_t> nextGateValue{0};
   // Tensors of a unit adding up to at most this many bytes go to the copy
   // agent when their streams are idle (TP_HIP_IPC_AGENT=0 switches it off,
   // TP_HIP_IPC_AGENT_MAX_BYTES moves the limit).
-  std::atomic<uint64_t> nextGateValue{0}; // what the gates of this context's channels wait for, ever growing
   const bool agentEnabled{envFlag("TP_HIP_IPC_AGENT", true)};
   const size_t agentMaxBytes{envSize("TP_HIP_IPC_AGENT_MAX_BYTES", 128 * 1024)};
   // How long the thread that posted a copy to the agent looks for its end
