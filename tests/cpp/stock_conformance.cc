@@ -318,6 +318,110 @@ static int twoProcess(const std::string& channel) {
   return problem.empty() ? 0 : 1;
 }
 
+// A message of one payload and one CPU tensor: what an endpoint with the HIP
+// channels registered can exchange with a peer that has none of them.
+static std::string sendCpuMessage(Pipe& pipe, int salt) {
+  std::vector<uint8_t> cpu(kCpuBytes);
+  for (size_t i = 0; i < cpu.size(); ++i) {
+    cpu[i] = pattern(i, salt);
+  }
+  Message m;
+  m.metadata = "cpu only";
+  Message::Payload p;
+  std::string payload = kPayload;
+  p.data = payload.data();
+  p.length = payload.size();
+  m.payloads.push_back(std::move(p));
+  Message::Tensor ct;
+  ct.buffer = CpuBuffer{cpu.data()};
+  ct.length = cpu.size();
+  m.tensors.push_back(std::move(ct));
+  std::promise<std::string> done;
+  pipe.write(std::move(m), [&done](const Error& e) { done.set_value(e ? e.what() : std::string()); });
+  auto f = done.get_future();
+  if (f.wait_for(std::chrono::seconds(60)) != std::future_status::ready) {
+    return "write never completed";
+  }
+  return f.get();
+}
+
+static std::string recvCpuMessage(Pipe& pipe, int salt) {
+  std::promise<std::string> done;
+  std::vector<uint8_t> cpu;
+  std::string payload;
+  pipe.readDescriptor([&](const Error& e, Descriptor d) {
+    if (e) {
+      done.set_value("readDescriptor: " + e.what());
+      return;
+    }
+    if (d.metadata != "cpu only" || d.payloads.size() != 1 || d.tensors.size() != 1) {
+      done.set_value("unexpected descriptor");
+      return;
+    }
+    Allocation a;
+    payload.resize(d.payloads[0].length);
+    a.payloads.resize(1);
+    a.payloads[0].data = &payload[0];
+    a.tensors.resize(1);
+    cpu.assign(d.tensors[0].length, 0);
+    a.tensors[0].buffer = CpuBuffer{cpu.data()};
+    pipe.read(std::move(a), [&done](const Error& e2) { done.set_value(e2 ? "read: " + e2.what() : std::string()); });
+  });
+  auto f = done.get_future();
+  if (f.wait_for(std::chrono::seconds(60)) != std::future_status::ready) {
+    return "read never completed";
+  }
+  std::string err = f.get();
+  if (!err.empty()) {
+    return err;
+  }
+  if (payload != kPayload || cpu.size() != kCpuBytes) {
+    return "payload or tensor length differs";
+  }
+  for (size_t i = 0; i < cpu.size(); ++i) {
+    if (cpu[i] != pattern(i, salt)) {
+      return "byte " + std::to_string(i) + " of the CPU tensor differs";
+    }
+  }
+  return "";
+}
+
+// One end has the three HIP channels registered next to the stock ones, the
+// other is an unmodified TensorPipe endpoint: channel selection must skip what
+// only one side offers and the two must still talk.
+static int unmodifiedPeer() {
+  const std::string addr = "shm://tpamd_conf3_" + std::to_string(::getpid());
+  auto server = makeContext("server", {"hip_xth", "hip_ipc", "hip_basic"});
+  auto client = makeContext("unmodified", {});
+  auto listener = server->listen({addr});
+  auto cpipe = client->connect(listener->url("shm"));
+  auto spipe = acceptOne(*listener);
+  std::string problem = spipe ? std::string() : std::string("accept failed");
+  for (int round = 0; round < 3 && problem.empty(); ++round) {
+    auto sent = std::async(std::launch::async, [&] { return sendCpuMessage(*spipe, 7 * round); });
+    problem = recvCpuMessage(*cpipe, 7 * round);
+    const std::string w = sent.get();
+    if (problem.empty()) {
+      problem = w;
+    }
+    if (problem.empty()) {
+      auto sent2 = std::async(std::launch::async, [&] { return sendCpuMessage(*cpipe, 7 * round + 3); });
+      problem = recvCpuMessage(*spipe, 7 * round + 3);
+      const std::string w2 = sent2.get();
+      if (problem.empty()) {
+        problem = w2;
+      }
+    }
+  }
+  report("hip_channels_registered_beside_an_unmodified_peer", problem);
+  cpipe.reset();
+  spipe.reset();
+  listener.reset();
+  client->join();
+  server->join();
+  return problem.empty() ? 0 : 1;
+}
+
 int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "same_process") == 0) {
     return sameProcess();
@@ -325,6 +429,9 @@ int main(int argc, char** argv) {
   if (argc == 3 && std::strcmp(argv[1], "two_process") == 0) {
     return twoProcess(argv[2]);
   }
-  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic\n", argv[0]);
+  if (argc == 2 && std::strcmp(argv[1], "unmodified_peer") == 0) {
+    return unmodifiedPeer();
+  }
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer\n", argv[0]);
   return 2;
 }

@@ -36,3 +36,9 @@ def test_hip_xth_in_a_stock_context_same_process():
 @pytest.mark.parametrize("channel", ["hip_ipc", "hip_basic"])
 def test_channel_in_stock_contexts_of_two_processes(channel):
     _run(["two_process", channel])
+
+
+def test_endpoint_with_hip_channels_talks_to_an_unmodified_peer():
+    """Registering the channels does not get in the way of a peer that has none of them: payloads
+    and CPU tensors still travel on the stock channels."""
+    _run(["unmodified_peer"])
