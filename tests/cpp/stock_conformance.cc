@@ -13,6 +13,8 @@
 // Prints "RESULT <case> OK" or "RESULT <case> FAIL <why>" per case.
 #include <tensorpipe/tensorpipe.h>
 
+#include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -422,6 +424,69 @@ static int unmodifiedPeer() {
   return problem.empty() ? 0 : 1;
 }
 
+// Timing, not a test: one GPU tensor of `bytes` bytes per message over hip_xth
+// between two stock contexts of this process, one message at a time, the next
+// write issued by the thread that saw both callbacks of the previous one.
+static int timeSameProcess(size_t bytes, int iters) {
+  const std::string addr = "shm://tpamd_conf4_" + std::to_string(::getpid());
+  auto server = makeContext("server", {"hip_xth"});
+  auto client = makeContext("client", {"hip_xth"});
+  auto listener = server->listen({addr});
+  auto cpipe = client->connect(listener->url("shm"));
+  auto spipe = acceptOne(*listener);
+  GpuTensor src = makeGpu(bytes);
+  GpuTensor dst = makeGpu(bytes);
+  src.fill(3);
+  std::vector<double> us;
+  std::string problem;
+  for (int it = 0; it < iters + 10 && problem.empty(); ++it) {
+    std::promise<std::string> wrote, read;
+    const auto t0 = std::chrono::steady_clock::now();
+    Message m;
+    Message::Tensor t;
+    t.buffer = HipBuffer{src.dev, src.stream, 0};
+    t.length = bytes;
+    t.targetDevice = Device{"cuda", 0};
+    m.tensors.push_back(std::move(t));
+    spipe->readDescriptor([&](const Error& e, Descriptor d) {
+      if (e || d.tensors.size() != 1) {
+        read.set_value("readDescriptor failed");
+        return;
+      }
+      Allocation a;
+      a.tensors.resize(1);
+      a.tensors[0].buffer = HipBuffer{dst.dev, dst.stream, 0};
+      spipe->read(std::move(a), [&read](const Error& e2) { read.set_value(e2 ? e2.what() : std::string()); });
+    });
+    cpipe->write(std::move(m), [&wrote](const Error& e) { wrote.set_value(e ? e.what() : std::string()); });
+    problem = read.get_future().get();
+    const std::string w = wrote.get_future().get();
+    if (problem.empty()) {
+      problem = w;
+    }
+    const auto t1 = std::chrono::steady_clock::now();
+    if (it >= 10) {
+      us.push_back(std::chrono::duration<double, std::micro>(t1 - t0).count());
+    }
+  }
+  if (problem.empty()) {
+    problem = dst.check(3);
+  }
+  std::sort(us.begin(), us.end());
+  if (problem.empty() && !us.empty()) {
+    const double p50 = us[us.size() / 2];
+    std::printf("TIMING hip_xth in stock contexts: %zu bytes, %d messages, p50 %.1f us per message, %.1f GB/s payload\n",
+                bytes, iters, p50, static_cast<double>(bytes) / p50 / 1e3);
+  }
+  report("timing_hip_xth_in_stock_context", problem);
+  cpipe.reset();
+  spipe.reset();
+  listener.reset();
+  client->join();
+  server->join();
+  return problem.empty() ? 0 : 1;
+}
+
 int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "same_process") == 0) {
     return sameProcess();
@@ -432,6 +497,9 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "unmodified_peer") == 0) {
     return unmodifiedPeer();
   }
-  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer\n", argv[0]);
+  if (argc == 4 && std::strcmp(argv[1], "time_same_process") == 0) {
+    return timeSameProcess(std::strtoull(argv[2], nullptr, 10), std::atoi(argv[3]));
+  }
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer | time_same_process <bytes> <messages>\n", argv[0]);
   return 2;
 }
