@@ -58,6 +58,8 @@ HOST_SOURCES = [
     "tensorpipe/core/core.cc",
     "capi/tensorpipe_c.cc",
     "bridge/bridge_amd.cc",
+    "nopwire/nop_wire.cc",
+    "nopwire/compat_pipe.cc",
 ]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread"]
 
@@ -132,6 +134,14 @@ def build_stock_conformance():
          f"-I{inc}", f"-I{INCLUDE}", f"-I{CSRC}",
          os.path.join(CSRC, "bridge", "stock_adapter.cc"), os.path.join(src_dir, "stock_conformance.cc"),
          "-o", os.path.join(bin_dir, "stock_conformance"),
+         f"-L{LIB}", "-ltensorpipe_amd", "-ltphip", f"-L{lib}", "-ltorch_cpu", "-lc10",
+         "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib", f"-Wl,-rpath,{lib}"])
+    # tests/cpp/bin/stock_wire_interop: the stock-protocol endpoint of csrc/nopwire against the same
+    # unmodified TensorPipe, over TCP (no GPU); `capture` mode wrote tests/golden/stock_wire_vectors.txt.
+    run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
+         f"-I{inc}", f"-I{CSRC}",
+         os.path.join(src_dir, "stock_wire_interop.cc"),
+         "-o", os.path.join(bin_dir, "stock_wire_interop"),
          f"-L{LIB}", "-ltensorpipe_amd", "-ltphip", f"-L{lib}", "-ltorch_cpu", "-lc10",
          "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib", f"-Wl,-rpath,{lib}"])
     return True

@@ -14,6 +14,13 @@
 //   unit_tests departed_peer
 //       a peer writes two messages and goes away before the reader posts its
 //       reads: both messages are handed over, the third read reports the end.
+//   unit_tests nop_wire <vectors file>
+//       the control frames an unmodified TensorPipe endpoint wrote (name, hex):
+//       each must decode, carry the fields the capturing program put in, and
+//       encode back to the same bytes; cut short anywhere, or with bytes
+//       flipped, a frame must be refused without reading out of bounds.
+//   unit_tests compat_pipe
+//       two ends of the stock-protocol endpoint talk to each other over TCP.
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -44,6 +51,9 @@
 #include <tensorpipe/tensorpipe_hip.h>
 #include <tensorpipe/transport/connection.h>
 #include <tensorpipe/transport/listener.h>
+
+#include <nopwire/compat_pipe.h>
+#include <nopwire/nop_wire.h>
 
 using namespace tensorpipe;
 
@@ -387,6 +397,230 @@ static int runPointers() {
 }
 
 // A crash names its stack before the process dies.
+static bool fromHex(const std::string& hex, tpnop::Bytes* out) {
+  if (hex.size() % 2 != 0) {
+    return false;
+  }
+  out->clear();
+  for (size_t i = 0; i < hex.size(); i += 2) {
+    unsigned v = 0;
+    if (std::sscanf(hex.c_str() + i, "%2x", &v) != 1) {
+      return false;
+    }
+    out->push_back(static_cast<uint8_t>(v));
+  }
+  return true;
+}
+
+// Decodes `bytes` as what `name` says it is and encodes it again.
+static bool roundTrip(const std::string& name, const tpnop::Bytes& bytes, tpnop::Bytes* again, std::string* facts) {
+  const uint8_t* p = bytes.data();
+  const size_t n = bytes.size();
+  if (name.find("spontaneous_connection") != std::string::npos || name.find("requested_connection") != std::string::npos) {
+    tpnop::Packet v;
+    if (!tpnop::decode(p, n, &v)) {
+      return false;
+    }
+    *again = tpnop::encode(v);
+    *facts = v.which == tpnop::Packet::kSpontaneous ? "name=" + v.spontaneous.contextName
+                                                    : "token=" + std::to_string(v.requested.registrationId);
+    return true;
+  }
+  if (name.find("brochure_answer") != std::string::npos) {
+    tpnop::BrochureAnswer v;
+    if (!tpnop::decode(p, n, &v)) {
+      return false;
+    }
+    *again = tpnop::encode(v);
+    *facts = "transport=" + v.transport + " domain=" + v.transportDomainDescriptor +
+        " ids=" + std::to_string(v.transportRegistrationIds.size()) +
+        " channels=" + std::to_string(v.channelRegistrationIds.size()) +
+        " pairs=" + std::to_string(v.channelForDevicePair.size());
+    if (!v.channelForDevicePair.empty()) {
+      *facts += " first_pair=" + v.channelForDevicePair[0].first.first.type + "," +
+          v.channelForDevicePair[0].first.second.type + "->" + v.channelForDevicePair[0].second;
+    }
+    return true;
+  }
+  if (name.find("brochure") != std::string::npos) {
+    tpnop::Brochure v;
+    if (!tpnop::decode(p, n, &v)) {
+      return false;
+    }
+    *again = tpnop::encode(v);
+    *facts = "transports=" + std::to_string(v.transportDomainDescriptors.size()) +
+        " channels=" + std::to_string(v.channelDeviceDescriptors.size());
+    if (!v.transportDomainDescriptors.empty()) {
+      *facts += " first=" + v.transportDomainDescriptors[0].first + ":" + v.transportDomainDescriptors[0].second;
+    }
+    return true;
+  }
+  if (name.find("descriptor_reply") != std::string::npos) {
+    tpnop::DescriptorReply v;
+    if (!tpnop::decode(p, n, &v)) {
+      return false;
+    }
+    *again = tpnop::encode(v);
+    *facts = "devices=" + std::to_string(v.targetDevices.size());
+    for (auto& d : v.targetDevices) {
+      *facts += " " + d.type + ":" + std::to_string(d.index);
+    }
+    return true;
+  }
+  if (name.find("descriptor") != std::string::npos) {
+    tpnop::Descriptor v;
+    if (!tpnop::decode(p, n, &v)) {
+      return false;
+    }
+    *again = tpnop::encode(v);
+    *facts = "metadata=" + v.metadata + " payloads=";
+    for (auto& pl : v.payloads) {
+      *facts += std::to_string(pl.length) + "[" + pl.metadata + "]";
+    }
+    *facts += " tensors=";
+    for (auto& t : v.tensors) {
+      *facts += std::to_string(t.length) + "@" + t.sourceDevice.type + (t.hasTargetDevice ? ">" + t.targetDevice.type : ">?") +
+          "[" + t.metadata + "]";
+    }
+    return true;
+  }
+  return false;
+}
+
+static int runNopWire(const char* file) {
+  FILE* f = std::fopen(file, "r");
+  if (f == nullptr) {
+    std::perror(file);
+    return 2;
+  }
+  int failures = 0, vectors = 0;
+  char* line = nullptr;
+  size_t cap = 0;
+  std::mt19937 rng(99);
+  while (::getline(&line, &cap, f) > 0) {
+    std::string l(line);
+    while (!l.empty() && (l.back() == '\n' || l.back() == '\r')) {
+      l.pop_back();
+    }
+    if (l.empty() || l[0] == '#') {
+      continue;
+    }
+    const size_t sp = l.find(' ');
+    const std::string name = l.substr(0, sp);
+    tpnop::Bytes bytes, again;
+    std::string facts;
+    if (sp == std::string::npos || !fromHex(l.substr(sp + 1), &bytes)) {
+      std::printf("FAIL %s: not a vector line\n", name.c_str());
+      ++failures;
+      continue;
+    }
+    ++vectors;
+    if (!roundTrip(name, bytes, &again, &facts)) {
+      std::printf("FAIL %s: does not decode\n", name.c_str());
+      ++failures;
+      continue;
+    }
+    if (again != bytes) {
+      std::printf("FAIL %s: encodes back to other bytes\n", name.c_str());
+      ++failures;
+    }
+    std::printf("VECTOR %s %s\n", name.c_str(), facts.c_str());
+    // Cut short anywhere it must be refused; with a byte changed it may decode
+    // or not, but must not read out of bounds (the copies are exactly sized,
+    // so a sanitizer build sees an overrun).
+    for (size_t cut = 0; cut < bytes.size(); ++cut) {
+      tpnop::Bytes part(bytes.begin(), bytes.begin() + cut), ignored;
+      std::string ignoredFacts;
+      if (roundTrip(name, part, &ignored, &ignoredFacts)) {
+        std::printf("FAIL %s: decodes when cut to %zu bytes\n", name.c_str(), cut);
+        ++failures;
+        break;
+      }
+    }
+    for (int k = 0; k < 200; ++k) {
+      tpnop::Bytes bent(bytes), ignored;
+      std::string ignoredFacts;
+      bent[rng() % bent.size()] = static_cast<uint8_t>(rng());
+      (void)roundTrip(name, bent, &ignored, &ignoredFacts);
+    }
+  }
+  std::free(line);
+  std::fclose(f);
+  // What the writer does with values the captured frames do not hold.
+  {
+    tpnop::Descriptor d;
+    d.metadata = std::string(300, 'm');
+    d.payloads.push_back({uint64_t(1) << 40, "big"});
+    d.tensors.push_back({0xffff, {"cuda", 3}, true, {"cuda", -1}, ""});
+    d.tensors.push_back({0x10000, {"cpu", 200}, false, {}, "x"});
+    tpnop::Descriptor back;
+    const tpnop::Bytes b = tpnop::encode(d);
+    if (!tpnop::decode(b.data(), b.size(), &back) || back.metadata != d.metadata || back.payloads[0].length != d.payloads[0].length ||
+        back.tensors[0].targetDevice.index != -1 || back.tensors[0].length != 0xffff || back.tensors[1].sourceDevice.index != 200 ||
+        back.tensors[1].hasTargetDevice || back.tensors[1].length != 0x10000) {
+      std::printf("FAIL a descriptor with large and negative values does not survive a round trip\n");
+      ++failures;
+    }
+    uint8_t header[tpnop::kFrameHeaderBytes];
+    tpnop::putFrameHeader(0x0102030405060708ull, header);
+    if (header[0] != 8 || header[7] != 1 || tpnop::getFrameHeader(header) != 0x0102030405060708ull) {
+      std::printf("FAIL frame header\n");
+      ++failures;
+    }
+  }
+  std::printf("%s %d vectors\n", failures == 0 ? "OK" : "FAILED", vectors);
+  return failures == 0 ? 0 : 1;
+}
+
+static int runCompatPipe() {
+  std::string error;
+  auto listener = tpnop::CompatListener::create(&error);
+  if (!listener) {
+    std::printf("FAIL listen: %s\n", error.c_str());
+    return 1;
+  }
+  std::string clientError;
+  auto connecting = std::async(std::launch::async, [&] {
+    return tpnop::CompatPipe::connect(listener->address(), "client end", &clientError);
+  });
+  auto server = listener->accept("server end", &error);
+  auto client = connecting.get();
+  if (!server || !client) {
+    std::printf("FAIL handshake: %s %s\n", error.c_str(), clientError.c_str());
+    return 1;
+  }
+  int failures = 0;
+  if (server->remoteName() != "client end") {
+    std::printf("FAIL the listening end heard the name %s\n", server->remoteName().c_str());
+    ++failures;
+  }
+  for (int round = 0; round < 4 && failures == 0; ++round) {
+    tpnop::CompatMessage m, got;
+    m.metadata = "round " + std::to_string(round);
+    m.payloads.push_back({std::string(1000 + round, 'p'), "payload metadata"});
+    m.payloads.push_back({"", ""});
+    m.tensors.push_back({std::string(100000 + round, 't'), "tensor", round % 2 == 0});
+    m.tensors.push_back({"", "empty", false});
+    tpnop::CompatPipe& from = round % 2 == 0 ? *client : *server;
+    tpnop::CompatPipe& to = round % 2 == 0 ? *server : *client;
+    std::string writeError;
+    auto writing = std::async(std::launch::async, [&] { return from.write(m, &writeError); });
+    const bool readOk = to.read(&got, &error);
+    if (!writing.get() || !readOk) {
+      std::printf("FAIL round %d: %s %s\n", round, writeError.c_str(), error.c_str());
+      ++failures;
+    } else if (got.metadata != m.metadata || got.payloads.size() != 2 || got.payloads[0].bytes != m.payloads[0].bytes ||
+               got.payloads[0].metadata != "payload metadata" || got.tensors.size() != 2 ||
+               got.tensors[0].bytes != m.tensors[0].bytes || got.tensors[0].nameTarget != m.tensors[0].nameTarget ||
+               !got.tensors[1].bytes.empty() || got.tensors[1].metadata != "empty") {
+      std::printf("FAIL round %d: the message arrived changed\n", round);
+      ++failures;
+    }
+  }
+  std::printf("%s\n", failures == 0 ? "OK" : "FAILED");
+  return failures == 0 ? 0 : 1;
+}
+
 static void onFatalSignal(int sig) {
   void* frames[48];
   const int n = backtrace(frames, 48);
@@ -415,6 +649,12 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "pointers") == 0) {
     return runPointers();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n>\n", argv[0]);
+  if (argc == 3 && std::strcmp(argv[1], "nop_wire") == 0) {
+    return runNopWire(argv[2]);
+  }
+  if (argc == 2 && std::strcmp(argv[1], "compat_pipe") == 0) {
+    return runCompatPipe();
+  }
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe\n", argv[0]);
   return 2;
 }

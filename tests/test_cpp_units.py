@@ -79,3 +79,34 @@ def test_garbage_on_new_connections(seed):
     # and still serves a proper pipe
     out = subprocess.run([BIN, "garbage", str(seed), "100"], stdout=subprocess.PIPE, text=True, timeout=120)
     assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
+
+
+def test_nop_wire_decodes_and_reproduces_the_frames_of_a_stock_endpoint():
+    """tests/golden/stock_wire_vectors.txt holds control frames written by the TensorPipe inside
+    PyTorch (tests/cpp/stock_wire_interop.cc capture made it): every one decodes to what the
+    capturing program sent and encodes back to the same bytes; cut or bent frames are refused."""
+    rc, out = run("nop_wire", os.path.join(ROOT, "tests", "golden", "stock_wire_vectors.txt"))
+    assert rc == 0, out
+    facts = {}
+    for line in out.splitlines():
+        if line.startswith("VECTOR "):
+            _, name, rest = line.split(" ", 2)
+            facts[name] = rest
+    assert out.strip().splitlines()[-1] == f"OK {len(facts)} vectors" and len(facts) >= 12
+    assert facts["stock_client.spontaneous_connection"] == "name=stock_client"
+    assert facts["stock_client.requested_connection_r"].startswith("token=")
+    assert facts["stock_client.brochure"] == "transports=1 channels=1 first=uv:uv:*"
+    assert facts["stock_server.brochure_answer"] == (
+        "transport=uv domain=uv:* ids=1 channels=1 pairs=1 first_pair=cpu,cpu->basic")
+    # the message of the capturing program: 300 B and empty payloads; 70001 B with the target named,
+    # 129 B without, an empty tensor
+    for who, salt in (("stock_client", 110), ("stock_server", 100)):
+        assert facts[f"{who}.descriptor_0"] == (
+            f"metadata=message metadata {salt} payloads=300[first payload]0[] "
+            "tensors=70001@cpu>cpu[named target]129@cpu>?[]0@cpu>cpu[empty]")
+        assert facts[f"{who}.descriptor_reply_0"] == "devices=1 cpu:0"
+
+
+def test_compat_pipe_talks_to_itself():
+    rc, out = run("compat_pipe")
+    assert rc == 0 and out.strip() == "OK", out
