@@ -58,6 +58,7 @@ HOST_SOURCES = [
     "tensorpipe/core/core.cc",
     "capi/tensorpipe_c.cc",
     "bridge/bridge_amd.cc",
+    "tensorpipe/transport/tcp/tcp.cc",
     "nopwire/nop_wire.cc",
     "nopwire/compat_pipe.cc",
 ]

@@ -21,6 +21,11 @@
 //       flipped, a frame must be refused without reading out of bounds.
 //   unit_tests compat_pipe
 //       two ends of the stock-protocol endpoint talk to each other over TCP.
+//   unit_tests tcp
+//       the TCP transport: messages of every size class both ways (empty, small,
+//       many MiB: partial reads and writes), exact-length reads, a peer that
+//       wrote and left, a frame written by hand with the reference's framing,
+//       and a pipe with payloads and CPU tensors over it.
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -51,6 +56,12 @@
 #include <tensorpipe/tensorpipe_hip.h>
 #include <tensorpipe/transport/connection.h>
 #include <tensorpipe/transport/listener.h>
+
+#include <tensorpipe/transport/tcp/factory.h>
+
+#include <arpa/inet.h>
+#include <netinet/in.h>
+#include <sys/socket.h>
 
 #include <nopwire/compat_pipe.h>
 #include <nopwire/nop_wire.h>
@@ -621,6 +632,222 @@ static int runCompatPipe() {
   return failures == 0 ? 0 : 1;
 }
 
+static int runTcp() {
+  int failed = 0;
+  auto serverSide = transport::tcp::create();
+  auto listener = serverSide->listen("127.0.0.1");
+  const std::string addr = listener->addr();
+  CHECK(addr.find("127.0.0.1:") == 0 && addr != "127.0.0.1:0");
+  CHECK(serverSide->domainDescriptor() == "uv:*");
+  std::promise<std::shared_ptr<transport::Connection>> acceptedP;
+  listener->accept([&](const Error& e, std::shared_ptr<transport::Connection> c) {
+    acceptedP.set_value(e ? nullptr : std::move(c));
+  });
+  auto clientSide = transport::tcp::create();
+  auto conn = clientSide->connect(addr);
+  auto accepted = acceptedP.get_future().get();
+  CHECK(accepted != nullptr);
+  if (!accepted) {
+    return 1;
+  }
+  // Messages of every size class, both ways, reads posted before and after the writes.
+  const std::vector<size_t> sizes = {0, 1, 7, 8, 9, 4096, 65537, 1 << 20, (24u << 20) + 3};
+  for (int direction = 0; direction < 2; ++direction) {
+    auto& from = direction == 0 ? conn : accepted;
+    auto& to = direction == 0 ? accepted : conn;
+    std::vector<std::vector<uint8_t>> sent;
+    for (size_t k = 0; k < sizes.size(); ++k) {
+      std::vector<uint8_t> m(sizes[k]);
+      for (size_t i = 0; i < m.size(); ++i) {
+        m[i] = static_cast<uint8_t>((i * 13 + k * 7 + direction) % 251);
+      }
+      sent.push_back(std::move(m));
+    }
+    std::vector<std::future<bool>> results;
+    std::vector<std::shared_ptr<std::vector<uint8_t>>> exactBuffers;
+    auto postRead = [&](size_t k) {
+      auto p = std::make_shared<std::promise<bool>>();
+      results.push_back(p->get_future());
+      const std::vector<uint8_t>* want = &sent[k];
+      if (k % 2 == 0) {
+        to->read([p, want](const Error& e, const void* ptr, size_t len) {
+          p->set_value(!e && len == want->size() && (len == 0 || std::memcmp(ptr, want->data(), len) == 0));
+        });
+      } else {
+        auto buf = std::make_shared<std::vector<uint8_t>>(want->size());
+        exactBuffers.push_back(buf);
+        to->read(buf->data(), buf->size(), [p, want, buf](const Error& e, const void*, size_t len) {
+          p->set_value(!e && len == want->size() && *buf == *want);
+        });
+      }
+    };
+    for (size_t k = 0; k < sizes.size() / 2; ++k) {
+      postRead(k); // these wait for their bytes
+    }
+    std::promise<void> wroteAll;
+    for (size_t k = 0; k < sizes.size(); ++k) {
+      const bool last = k + 1 == sizes.size();
+      from->write(sent[k].data(), sent[k].size(), [&wroteAll, last](const Error& e) {
+        if (last) {
+          wroteAll.set_value();
+        }
+        (void)e;
+      });
+    }
+    for (size_t k = sizes.size() / 2; k < sizes.size(); ++k) {
+      postRead(k); // these find their bytes already there, or on their way
+    }
+    for (auto& r : results) {
+      CHECK(r.wait_for(std::chrono::seconds(30)) == std::future_status::ready && r.get());
+    }
+    wroteAll.get_future().get();
+  }
+  // An exact-length read that meets a message of another length fails the connection.
+  {
+    auto other = clientSide->connect(addr);
+    std::promise<std::shared_ptr<transport::Connection>> p2;
+    listener->accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p2.set_value(e ? nullptr : std::move(c)); });
+    auto acc2 = p2.get_future().get();
+    CHECK(acc2 != nullptr);
+    const std::string msg = "five!";
+    other->write(msg.data(), msg.size(), [](const Error&) {});
+    char buf[4];
+    std::promise<bool> failedRead;
+    acc2->read(buf, sizeof(buf), [&](const Error& e, const void*, size_t) { failedRead.set_value(static_cast<bool>(e)); });
+    CHECK(failedRead.get_future().get());
+  }
+  // A frame written by hand, the way the reference frames a stream: 8-byte little-endian length, bytes.
+  {
+    std::promise<std::shared_ptr<transport::Connection>> p3;
+    listener->accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p3.set_value(e ? nullptr : std::move(c)); });
+    const int fd = ::socket(AF_INET, SOCK_STREAM, 0);
+    sockaddr_in sa{};
+    sa.sin_family = AF_INET;
+    sa.sin_port = htons(static_cast<uint16_t>(std::atoi(addr.c_str() + addr.rfind(':') + 1)));
+    ::inet_pton(AF_INET, "127.0.0.1", &sa.sin_addr);
+    CHECK(::connect(fd, reinterpret_cast<sockaddr*>(&sa), sizeof(sa)) == 0);
+    auto acc3 = p3.get_future().get();
+    CHECK(acc3 != nullptr);
+    const uint8_t frame[8 + 3] = {3, 0, 0, 0, 0, 0, 0, 0, 'a', 'b', 'c'};
+    CHECK(::write(fd, frame, 5) == 5); // in two pieces, cut inside the length
+    std::promise<std::string> got;
+    acc3->read([&](const Error& e, const void* ptr, size_t len) {
+      got.set_value(e ? "error" : std::string(static_cast<const char*>(ptr), len));
+    });
+    std::this_thread::sleep_for(std::chrono::milliseconds(50));
+    CHECK(::write(fd, frame + 5, sizeof(frame) - 5) == static_cast<ssize_t>(sizeof(frame) - 5));
+    CHECK(got.get_future().get() == "abc");
+    // and what this transport writes reads back the same way
+    const std::string reply = "reply";
+    acc3->write(reply.data(), reply.size(), [](const Error&) {});
+    uint8_t back[8 + 5];
+    size_t have = 0;
+    while (have < sizeof(back)) {
+      const ssize_t r = ::read(fd, back + have, sizeof(back) - have);
+      if (r <= 0) {
+        break;
+      }
+      have += static_cast<size_t>(r);
+    }
+    CHECK(have == sizeof(back) && back[0] == 5 && back[1] == 0 && back[7] == 0 && std::memcmp(back + 8, "reply", 5) == 0);
+    // the peer writes once more and leaves before anybody reads: the message, then the end
+    const uint8_t last[8 + 2] = {2, 0, 0, 0, 0, 0, 0, 0, 'o', 'k'};
+    CHECK(::write(fd, last, sizeof(last)) == static_cast<ssize_t>(sizeof(last)));
+    ::close(fd);
+    std::this_thread::sleep_for(std::chrono::milliseconds(100));
+    for (int i = 0; i < 2; ++i) {
+      std::promise<std::pair<bool, std::string>> gotP;
+      acc3->read([&](const Error& e, const void* ptr, size_t len) {
+        gotP.set_value({static_cast<bool>(e), e ? e.what() : std::string(static_cast<const char*>(ptr), len)});
+      });
+      auto g = gotP.get_future().get();
+      if (i == 0) {
+        CHECK(!g.first && g.second == "ok");
+      } else {
+        CHECK(g.first && g.second.find("eof") != std::string::npos);
+      }
+    }
+  }
+  // Closing this end fails what is pending on it.
+  {
+    std::promise<bool> pending;
+    accepted->read([&](const Error& e, const void*, size_t) { pending.set_value(static_cast<bool>(e)); });
+    accepted->close();
+    CHECK(pending.get_future().get());
+  }
+  conn.reset();
+  accepted.reset();
+  listener->close();
+  listener.reset();
+  clientSide->join();
+  serverSide->join();
+
+  // A pipe over it: payload and CPU tensors through the basic channel.
+  {
+    auto make = [](const char* name) {
+      auto ctx = std::make_shared<Context>(ContextOptions().name(name));
+      ctx->registerTransport(0, "uv", transport::tcp::create());
+      ctx->registerChannel(0, "basic", channel::basic::create());
+      return ctx;
+    };
+    auto server = make("tcp server");
+    auto client = make("tcp client");
+    auto plistener = server->listen({"uv://127.0.0.1"});
+    const std::string url = plistener->url("uv");
+    CHECK(url.find("uv://127.0.0.1:") == 0);
+    std::promise<std::shared_ptr<Pipe>> acceptedPipe;
+    plistener->accept([&](const Error& e, std::shared_ptr<Pipe> p) { acceptedPipe.set_value(e ? nullptr : std::move(p)); });
+    auto cpipe = client->connect(url);
+    auto spipe = acceptedPipe.get_future().get();
+    CHECK(spipe != nullptr);
+    if (spipe) {
+      std::vector<uint8_t> tensor(3 << 20), landed;
+      for (size_t i = 0; i < tensor.size(); ++i) {
+        tensor[i] = static_cast<uint8_t>(i * 31 % 253);
+      }
+      std::string payload = "payload over tcp", payloadLanded;
+      Message m;
+      m.metadata = "over tcp";
+      Message::Payload mp;
+      mp.data = &payload[0];
+      mp.length = payload.size();
+      m.payloads.push_back(std::move(mp));
+      Message::Tensor mt;
+      mt.buffer = CpuBuffer{tensor.data()};
+      mt.length = tensor.size();
+      m.tensors.push_back(std::move(mt));
+      std::promise<bool> wrote, readDone;
+      spipe->readDescriptor([&](const Error& e, Descriptor d) {
+        if (e || d.metadata != "over tcp" || d.payloads.size() != 1 || d.tensors.size() != 1) {
+          readDone.set_value(false);
+          return;
+        }
+        payloadLanded.resize(d.payloads[0].length);
+        landed.resize(d.tensors[0].length);
+        Allocation a;
+        a.payloads.resize(1);
+        a.payloads[0].data = &payloadLanded[0];
+        a.tensors.resize(1);
+        a.tensors[0].buffer = CpuBuffer{landed.data()};
+        spipe->read(std::move(a), [&](const Error& e2) { readDone.set_value(!e2); });
+      });
+      cpipe->write(std::move(m), [&](const Error& e) { wrote.set_value(!e); });
+      CHECK(readDone.get_future().get());
+      CHECK(wrote.get_future().get());
+      CHECK(payloadLanded == payload && landed == tensor);
+    }
+    cpipe.reset();
+    spipe.reset();
+    plistener.reset();
+    client->join();
+    server->join();
+  }
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
 static void onFatalSignal(int sig) {
   void* frames[48];
   const int n = backtrace(frames, 48);
@@ -655,6 +882,9 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "compat_pipe") == 0) {
     return runCompatPipe();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe\n", argv[0]);
+  if (argc == 2 && std::strcmp(argv[1], "tcp") == 0) {
+    return runTcp();
+  }
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp\n", argv[0]);
   return 2;
 }

@@ -110,3 +110,10 @@ def test_nop_wire_decodes_and_reproduces_the_frames_of_a_stock_endpoint():
 def test_compat_pipe_talks_to_itself():
     rc, out = run("compat_pipe")
     assert rc == 0 and out.strip() == "OK", out
+
+
+def test_tcp_transport():
+    """Messages of every size class both ways, exact-length reads, the reference's stream framing
+    written and read by hand, a peer that wrote and left, and a pipe over it."""
+    rc, out = run("tcp")
+    assert rc == 0 and out.strip() == "OK", out
