@@ -73,9 +73,15 @@ typedef struct tpc_descriptor {
 const char* tpc_last_error(void);
 
 /* Context: `transports` and `channels` are comma-separated lists of
- * "name:priority" with names from {shm} and {basic, xth, hip_xth, hip_ipc,
+ * "name:priority" with names from {shm, uv} and {basic, xth, hip_xth, hip_ipc,
  * hip_basic}; hip_basic wraps a fresh basic context. */
 tpc_context* tpc_context_create(const char* name, const char* transports, const char* channels);
+/* The same with two more things to say: "uv" among the transports is this
+ * library's TCP transport under the name a stock TensorPipe gives its own, and
+ * stock_wire chooses the encodings on the wire (1: the reference's own, so
+ * that the peer may be an unmodified TensorPipe; 0: this library's; -1: as
+ * TP_STOCK_WIRE in the environment says). */
+tpc_context* tpc_context_create_ex(const char* name, const char* transports, const char* channels, int stock_wire);
 void tpc_context_close(tpc_context* ctx);
 void tpc_context_destroy(tpc_context* ctx); /* join + free */
 /* 1 if the named channel was viable and got registered. */

@@ -140,7 +140,7 @@ def build_stock_conformance():
     # tests/cpp/bin/stock_wire_interop: the stock-protocol endpoint of csrc/nopwire against the same
     # unmodified TensorPipe, over TCP (no GPU); `capture` mode wrote tests/golden/stock_wire_vectors.txt.
     run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
-         f"-I{inc}", f"-I{CSRC}",
+         f"-I{inc}", f"-I{INCLUDE}", f"-I{CSRC}",
          os.path.join(src_dir, "stock_wire_interop.cc"),
          "-o", os.path.join(bin_dir, "stock_wire_interop"),
          f"-L{LIB}", "-ltensorpipe_amd", "-ltphip", f"-L{lib}", "-ltorch_cpu", "-lc10",

@@ -206,12 +206,20 @@ const char* tpc_last_error(void) {
 }
 
 tpc_context* tpc_context_create(const char* name, const char* transports, const char* channels) {
+  return tpc_context_create_ex(name, transports, channels, -1);
+}
+
+tpc_context* tpc_context_create_ex(const char* name, const char* transports, const char* channels, int stock_wire) {
   TPC_GUARD_BEGIN
   auto out = std::make_unique<tpc_context>();
-  out->ctx = std::make_shared<Context>(ContextOptions().name(name != nullptr ? name : ""));
+  out->ctx = stock_wire < 0
+      ? std::make_shared<Context>(ContextOptions().name(name != nullptr ? name : ""))
+      : std::make_shared<Context>(ContextOptions().name(name != nullptr ? name : "").stockWireFormat(stock_wire != 0));
   for (auto& t : parseList(transports)) {
     if (t.first == "shm") {
       out->ctx->registerTransport(t.second, "shm", transport::shm::create());
+    } else if (t.first == "uv") {
+      out->ctx->registerTransport(t.second, "uv", transport::tcp::create());
     } else {
       setLastError("unknown transport " + t.first);
       return nullptr;

@@ -22,8 +22,21 @@ class ContextOptions {
     return std::move(*this);
   }
 
+  // Not in the reference: the pipes of this context put the reference's own
+  // encodings on the wire (the libnop forms of tensorpipe/core/nop_types.h:26-80,
+  // descriptor replies on a connection of their own as in
+  // tensorpipe/core/pipe_impl.cc:262-345,987-1157) instead of this library's, so
+  // that the peer may be an unmodified TensorPipe. Both ends of a pipe must
+  // agree on the format. TP_STOCK_WIRE=1 in the environment switches it on
+  // for every context.
+  ContextOptions&& stockWireFormat(bool on = true) && {
+    stockWire_ = on ? 1 : 0;
+    return std::move(*this);
+  }
+
  private:
   std::string name_;
+  int stockWire_{-1}; // -1: as the environment says
   friend ContextImpl;
 };
 

@@ -30,6 +30,7 @@
 #include <tensorpipe/common/loop.h>
 #include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
+#include <nopwire/nop_wire.h>
 #include <tensorpipe/core/error.h>
 #include <tensorpipe/transport/connection.h>
 #include <tensorpipe/transport/listener.h>
@@ -101,13 +102,81 @@ bool splitUrl(const std::string& url, std::string* transport, std::string* addr)
 
 using DevicePairMap = std::unordered_map<std::pair<Device, Device>, std::string>;
 
+// ---- the reference's wire format (ContextOptions::stockWireFormat) ----------
+//
+// The pipe below speaks this library's packets. With the stock format on, what
+// goes out is translated at the last moment and what comes in is turned into
+// this library's packets before it is parsed, so that there is one pipe.
+
+tpnop::Device toNop(const Device& d) {
+  return tpnop::Device{d.type, d.index};
+}
+
+Device fromNop(const tpnop::Device& d) {
+  Device out;
+  out.type = d.type;
+  out.index = static_cast<int>(d.index);
+  return out;
+}
+
+std::vector<uint8_t> helloPacketFromStock(const std::string& name, const tpnop::Brochure& b) {
+  WireWriter w;
+  w.u8(kHelloSpontaneous);
+  w.str(name);
+  w.u32(static_cast<uint32_t>(b.transportDomainDescriptors.size()));
+  for (auto& t : b.transportDomainDescriptors) {
+    w.str(t.first);
+    w.str(t.second);
+  }
+  w.u32(static_cast<uint32_t>(b.channelDeviceDescriptors.size()));
+  for (auto& c : b.channelDeviceDescriptors) {
+    w.str(c.first);
+    w.u32(static_cast<uint32_t>(c.second.size()));
+    for (auto& d : c.second) {
+      putDevice(w, fromNop(d.first));
+      w.str(d.second);
+    }
+  }
+  return std::move(w.bytes());
+}
+
+std::vector<uint8_t> descriptorPacketFromStock(const tpnop::Descriptor& d) {
+  WireWriter w;
+  w.u8(kDescriptor);
+  w.str(d.metadata);
+  w.u32(static_cast<uint32_t>(d.payloads.size()));
+  for (auto& p : d.payloads) {
+    w.u64(p.length);
+    w.str(p.metadata);
+  }
+  w.u32(static_cast<uint32_t>(d.tensors.size()));
+  for (auto& t : d.tensors) {
+    w.u64(t.length);
+    w.u8(static_cast<uint8_t>((t.hasTargetDevice ? kTensorHasTarget : 0) | (t.metadata.empty() ? 0 : kTensorHasMetadata)));
+    putDevice(w, fromNop(t.sourceDevice));
+    if (t.hasTargetDevice) {
+      putDevice(w, fromNop(t.targetDevice));
+    }
+    if (!t.metadata.empty()) {
+      w.str(t.metadata);
+    }
+  }
+  return std::move(w.bytes());
+}
+
+bool stockWireFromEnv() {
+  const char* e = std::getenv("TP_STOCK_WIRE");
+  return e != nullptr && std::atoi(e) != 0;
+}
+
 } // namespace
 
 class PipeImpl;
 
 class ContextImpl final : public std::enable_shared_from_this<ContextImpl> {
  public:
-  explicit ContextImpl(ContextOptions opts) : name_(std::move(opts.name_)) {
+  explicit ContextImpl(ContextOptions opts)
+      : name_(std::move(opts.name_)), stockWire_(opts.stockWire_ < 0 ? stockWireFromEnv() : opts.stockWire_ != 0) {
     static std::atomic<uint64_t> counter{0};
     id_ = std::to_string(::getpid()) + ":c" + std::to_string(counter.fetch_add(1));
   }
@@ -205,6 +274,9 @@ class ContextImpl final : public std::enable_shared_from_this<ContextImpl> {
   const std::string& name() const {
     return name_;
   }
+  bool stockWire() const {
+    return stockWire_;
+  }
   const std::string& id() const {
     return id_;
   }
@@ -267,6 +339,7 @@ class ContextImpl final : public std::enable_shared_from_this<ContextImpl> {
 
  private:
   const std::string name_;
+  const bool stockWire_;
   std::string id_;
   OnDemandLoop loop_;
   std::mutex mutex_;
@@ -370,12 +443,14 @@ class ListenerImpl final : public std::enable_shared_from_this<ListenerImpl> {
               return;
             }
             self->armAccept(transport);
-            self->onConnection(std::move(conn));
+            self->onConnection(std::move(conn), transport);
           });
         });
   }
 
-  void onConnection(std::shared_ptr<transport::Connection> conn);
+  void onConnection(std::shared_ptr<transport::Connection> conn, const std::string& transport);
+  void onStockConnection(std::shared_ptr<transport::Connection> conn, const std::string& transport);
+  void serveRequested(uint64_t token, std::shared_ptr<transport::Connection> conn);
 
   void matchPipes() {
     while (!acceptors_.empty() && !readyPipes_.empty()) {
@@ -436,7 +511,8 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         remoteName_(std::move(remoteName)),
         transport_(std::move(transport)),
         addr_(std::move(addr)),
-        isClient_(true) {}
+        isClient_(true),
+        stock_(ctx_->stockWire()) {}
 
   // Server side: `hello` is the spontaneous-connection packet already read.
   PipeImpl(
@@ -444,13 +520,18 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       std::shared_ptr<ListenerImpl> listener,
       std::string id,
       std::shared_ptr<transport::Connection> conn,
-      std::vector<uint8_t> hello)
+      std::vector<uint8_t> hello,
+      std::string transport,
+      std::string remoteName)
       : ctx_(std::move(ctx)),
         listener_(std::move(listener)),
         id_(std::move(id)),
+        remoteName_(std::move(remoteName)), // known from the start: the pipe is handed out before it runs
+        transport_(std::move(transport)),
         connection_(std::move(conn)),
         hello_(std::move(hello)),
-        isClient_(false) {}
+        isClient_(false),
+        stock_(ctx_->stockWire()) {}
 
   void init() {
     auto self = shared_from_this();
@@ -551,6 +632,26 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
     connection_ = tctx->connect(addr_);
     connection_->setId(id_ + ".tr_" + transport_);
+    if (stock_) {
+      tpnop::Packet packet;
+      packet.which = tpnop::Packet::kSpontaneous;
+      packet.spontaneous.contextName = ctx_->name();
+      writeControl(tpnop::encode(packet));
+      tpnop::Brochure brochure;
+      for (auto& t : ctx_->transportDescriptors()) {
+        brochure.transportDomainDescriptors.emplace_back(t.first, t.second);
+      }
+      for (auto& c : ctx_->channels()) {
+        tpnop::WireMap<tpnop::Device, std::string> devices;
+        for (auto& d : c.context->deviceDescriptors()) {
+          devices.emplace_back(toNop(d.first), d.second);
+        }
+        brochure.channelDeviceDescriptors.emplace_back(c.name, std::move(devices));
+      }
+      writeControl(tpnop::encode(brochure));
+      readControl([this](std::vector<uint8_t> bytes) { onStockBrochureAnswer(std::move(bytes)); });
+      return;
+    }
     WireWriter w;
     w.u8(kHelloSpontaneous);
     w.str(ctx_->name());
@@ -573,6 +674,73 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
     writeControl(std::move(w.bytes()));
     readControl([this](std::vector<uint8_t> bytes) { onBrochureAnswer(std::move(bytes)); });
+  }
+
+  // The first thing a requested connection says: the token it was asked for.
+  void introduce(transport::Connection& conn, uint64_t token) {
+    std::shared_ptr<std::vector<uint8_t>> holder;
+    if (stock_) {
+      tpnop::Packet packet;
+      packet.which = tpnop::Packet::kRequested;
+      packet.requested.registrationId = token;
+      holder = std::make_shared<std::vector<uint8_t>>(tpnop::encode(packet));
+    } else {
+      WireWriter w;
+      w.u8(kHelloRequested);
+      w.u64(token);
+      holder = std::make_shared<std::vector<uint8_t>>(std::move(w.bytes()));
+    }
+    conn.write(holder->data(), holder->size(), [holder](const Error&) {});
+  }
+
+  // tensorpipe/core/pipe_impl.cc:1087-1157: the answer names the transport and
+  // where to reach it, a token for the descriptor reply connection, tokens per
+  // channel, and who serves which pair of devices.
+  void onStockBrochureAnswer(std::vector<uint8_t> bytes) {
+    if (error_) {
+      return;
+    }
+    tpnop::BrochureAnswer answer;
+    if (!tpnop::decode(bytes.data(), bytes.size(), &answer)) {
+      setError(TP_CREATE_ERROR(LogicError, "malformed brochure answer"));
+      return;
+    }
+    const uint64_t* replyToken = nullptr;
+    for (auto& kv : answer.transportRegistrationIds) {
+      if (kv.first == 1) {
+        replyToken = &kv.second;
+      }
+    }
+    if (answer.transport != transport_ || replyToken == nullptr) {
+      // A peer that wants another transport for the pipe's own connections
+      // would have to be followed there; this library has one per pipe.
+      setError(TP_CREATE_ERROR(LogicError, "the peer chose transport " + answer.transport));
+      return;
+    }
+    addr_ = answer.address; // where requested connections go
+    auto tctx = ctx_->transport(transport_);
+    replyConnection_ = tctx->connect(addr_);
+    replyConnection_->setId(id_ + ".r.tr_" + transport_);
+    introduce(*replyConnection_, *replyToken);
+    // From here on as with this library's own answer.
+    WireWriter w;
+    w.u8(kBrochureAnswer);
+    w.str(remoteName_);
+    w.u32(static_cast<uint32_t>(answer.channelRegistrationIds.size()));
+    for (auto& c : answer.channelRegistrationIds) {
+      w.str(c.first);
+      w.u32(static_cast<uint32_t>(c.second.size()));
+      for (uint64_t token : c.second) {
+        w.u64(token);
+      }
+    }
+    w.u32(static_cast<uint32_t>(answer.channelForDevicePair.size()));
+    for (auto& p : answer.channelForDevicePair) {
+      putDevice(w, fromNop(p.first.first));
+      putDevice(w, fromNop(p.first.second));
+      w.str(p.second);
+    }
+    onBrochureAnswer(std::move(w.bytes()));
   }
 
   void onBrochureAnswer(std::vector<uint8_t> bytes) {
@@ -599,11 +767,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         const uint64_t token = r.u64();
         auto conn = tctx->connect(addr_);
         conn->setId(id_ + ".ch_" + name + "_" + std::to_string(k));
-        WireWriter w;
-        w.u8(kHelloRequested);
-        w.u64(token);
-        auto holder = std::make_shared<std::vector<uint8_t>>(std::move(w.bytes()));
-        conn->write(holder->data(), holder->size(), [holder](const Error&) {});
+        introduce(*conn, token);
         conns.push_back(std::move(conn));
       }
       auto cctx = ctx_->channel(name);
@@ -684,6 +848,10 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       }
     }
 
+    if (stock_) {
+      writeStockBrochureAnswer(selected);
+      return;
+    }
     WireWriter w;
     w.u8(kBrochureAnswer);
     w.str(ctx_->name());
@@ -725,6 +893,65 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     pumpPackets();
   }
 
+  // tensorpipe/core/pipe_impl.cc:987-1042. The pipe's own connection keeps its
+  // transport, so only the descriptor reply connection is asked for besides
+  // those of the channels.
+  void writeStockBrochureAnswer(const std::vector<std::string>& selected) {
+    auto self = shared_from_this();
+    tpnop::BrochureAnswer answer;
+    answer.transport = transport_;
+    auto addrIt = listener_->addresses().find(transport_);
+    answer.address = addrIt != listener_->addresses().end() ? addrIt->second : std::string();
+    auto tctx = ctx_->transport(transport_);
+    answer.transportDomainDescriptor = tctx ? tctx->domainDescriptor() : std::string();
+    ++connectionsAwaited_;
+    const uint64_t replyToken = listener_->registerConnectionRequest(
+        [self](const Error& error, std::shared_ptr<transport::Connection> conn) {
+          if (self->error_) {
+            return;
+          }
+          if (error) {
+            self->setError(error);
+            return;
+          }
+          conn->setId(self->id_ + ".r.tr_" + self->transport_);
+          self->replyConnection_ = std::move(conn);
+          if (--self->connectionsAwaited_ == 0) {
+            self->createServerChannels();
+          }
+        });
+    tokens_.push_back(replyToken);
+    answer.transportRegistrationIds.emplace_back(1, replyToken);
+    for (auto& name : selected) {
+      auto cctx = ctx_->channel(name);
+      const size_t n = cctx->numConnectionsNeeded();
+      auto& slots = pendingChannelConns_[name];
+      slots.resize(n);
+      std::vector<uint64_t> channelTokens;
+      for (size_t k = 0; k < n; ++k) {
+        ++connectionsAwaited_;
+        const uint64_t token = listener_->registerConnectionRequest(
+            [self, name, k](const Error& error, std::shared_ptr<transport::Connection> conn) {
+              self->onRequestedConnection(name, k, error, std::move(conn));
+            });
+        tokens_.push_back(token);
+        channelTokens.push_back(token);
+      }
+      answer.channelRegistrationIds.emplace_back(name, std::move(channelTokens));
+      tpnop::WireMap<tpnop::Device, std::string> devices;
+      for (auto& d : cctx->deviceDescriptors()) {
+        devices.emplace_back(toNop(d.first), d.second);
+      }
+      answer.channelDeviceDescriptors.emplace_back(name, std::move(devices));
+    }
+    for (auto& p : channelForDevicePair_) {
+      answer.channelForDevicePair.emplace_back(std::make_pair(toNop(p.first.first), toNop(p.first.second)), p.second);
+    }
+    writeControl(tpnop::encode(answer));
+    awaitingChannelConnections_ = true;
+    pumpPackets();
+  }
+
   void onRequestedConnection(
       const std::string& name,
       size_t k,
@@ -762,11 +989,76 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     TP_VLOG(2) << "Pipe " << id_ << " is established with " << channels_.size() << " channel(s)";
     if (haveEarlyPacket_) {
       haveEarlyPacket_ = false;
-      onPacket(std::move(earlyPacket_));
+      onFrame(std::move(earlyPacket_));
       earlyPacket_.clear();
     }
     pumpPackets();
+    pumpReplies();
     advanceWrites();
+  }
+
+  // What arrives on the pipe's own connection once it is established: one of
+  // this library's packets, or (stock format) a descriptor and nothing else.
+  void onFrame(std::vector<uint8_t> bytes) {
+    if (!stock_) {
+      onPacket(std::move(bytes));
+      return;
+    }
+    tpnop::Descriptor d;
+    if (!tpnop::decode(bytes.data(), bytes.size(), &d)) {
+      setError(TP_CREATE_ERROR(LogicError, "malformed descriptor"));
+      return;
+    }
+    onPacket(descriptorPacketFromStock(d));
+  }
+
+  // Stock format: descriptor replies come on their own connection
+  // (tensorpipe/core/pipe_impl.cc:961-985) and name a device only for the
+  // tensors whose descriptor named none.
+  void pumpReplies() {
+    if (!stock_ || !replyConnection_ || error_) {
+      return;
+    }
+    auto self = shared_from_this();
+    replyConnection_->read([self](const Error& error, const void* ptr, size_t len) {
+      tpnop::DescriptorReply reply;
+      const bool ok = !error && tpnop::decode(static_cast<const uint8_t*>(ptr), len, &reply);
+      self->ctx_->defer([self, error, ok, reply{std::move(reply)}]() mutable {
+        if (self->error_) {
+          return;
+        }
+        if (error) {
+          self->setError(error);
+          return;
+        }
+        std::shared_ptr<WriteOp> waiting;
+        for (auto& op : self->writeOps_) {
+          if (op->needsReply && !op->haveReply) {
+            waiting = op;
+            break;
+          }
+        }
+        size_t missing = 0;
+        if (waiting) {
+          for (auto& t : waiting->message.tensors) {
+            missing += t.targetDevice.has_value() ? 0 : 1;
+          }
+        }
+        if (!ok || !waiting || reply.targetDevices.size() != missing) {
+          self->setError(TP_CREATE_ERROR(LogicError, "malformed descriptor reply"));
+          return;
+        }
+        WireWriter w;
+        w.u8(kDescriptorReply);
+        w.u32(static_cast<uint32_t>(waiting->message.tensors.size()));
+        size_t next = 0;
+        for (auto& t : waiting->message.tensors) {
+          putDevice(w, t.targetDevice.has_value() ? *t.targetDevice : fromNop(reply.targetDevices[next++]));
+        }
+        self->onPacket(std::move(w.bytes()));
+        self->pumpReplies();
+      });
+    });
   }
 
   // ---- control-connection plumbing ---------------------------------------
@@ -819,7 +1111,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         haveEarlyPacket_ = true;
         return;
       }
-      onPacket(std::move(bytes));
+      onFrame(std::move(bytes));
       pumpPackets();
     });
   }
@@ -909,7 +1201,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       }
       bool hasPayloadBytes = false;
       for (size_t len : op->payloadLengths) {
-        hasPayloadBytes |= len > 0;
+        hasPayloadBytes |= len > 0 || stock_; // the stock format frames empty payloads too
       }
       if (hasPayloadBytes) {
         payloadsUnclaimed_ = true;
@@ -1009,8 +1301,8 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     auto self = shared_from_this();
     bool claimed = false;
     for (size_t i = 0; i < op->payloadLengths.size(); ++i) {
-      if (op->payloadLengths[i] == 0) {
-        continue;
+      if (op->payloadLengths[i] == 0 && !stock_) {
+        continue; // nothing travels for an empty payload (the stock format sends an empty message)
       }
       claimed = true;
       ++op->pendingPayloads;
@@ -1031,7 +1323,22 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     }
 
     // Tell the sender where tensors without a target device ended up.
-    if (needsReply) {
+    if (needsReply && stock_) {
+      tpnop::DescriptorReply reply;
+      for (size_t i = 0; i < nT; ++i) {
+        if (shapes[i].target == kNoDevice) {
+          reply.targetDevices.push_back(toNop(targets[i]));
+        }
+      }
+      auto holder = std::make_shared<std::vector<uint8_t>>(tpnop::encode(reply));
+      if (replyConnection_) {
+        replyConnection_->write(holder->data(), holder->size(), [self, holder](const Error& error) {
+          if (error) {
+            self->ctx_->defer([self, error] { self->setError(error); });
+          }
+        });
+      }
+    } else if (needsReply) {
       WireWriter w;
       w.u8(kDescriptorReply);
       w.u32(static_cast<uint32_t>(targets.size()));
@@ -1064,7 +1371,8 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
           self->maybeFinishRead(op);
         });
       };
-      auto* batched = dynamic_cast<channel::BatchedChannel*>(ch.get());
+      // A stock pipe on the other end hands its channel one tensor at a time.
+      auto* batched = stock_ ? nullptr : dynamic_cast<channel::BatchedChannel*>(ch.get());
       if (batched != nullptr && g.second.size() > 1) {
         std::vector<channel::BatchEntry> entries;
         entries.reserve(g.second.size());
@@ -1221,6 +1529,26 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
         self->flushWrites();
       });
     };
+    if (stock_) {
+      // tensorpipe/core/pipe_impl.cc:70-99: the same facts as a Descriptor object
+      tpnop::Descriptor d;
+      d.metadata = m.metadata;
+      for (auto& p : m.payloads) {
+        d.payloads.push_back(tpnop::PayloadDescriptor{p.length, p.metadata});
+      }
+      for (auto& t : m.tensors) {
+        tpnop::TensorDescriptor td;
+        td.length = t.length;
+        td.sourceDevice = toNop(t.buffer.device());
+        td.hasTargetDevice = t.targetDevice.has_value();
+        if (td.hasTargetDevice) {
+          td.targetDevice = toNop(*t.targetDevice);
+        }
+        td.metadata = t.metadata;
+        d.tensors.push_back(std::move(td));
+      }
+      w.bytes() = tpnop::encode(d);
+    }
     auto holder = std::make_shared<std::vector<uint8_t>>(std::move(w.bytes()));
     ++op->pendingWrites;
     encodeTimer.reset();
@@ -1229,7 +1557,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     connection_->write(holder->data(), holder->size(), [holder, done](const Error& e) { done(e); });
     TP_VLOG(9) << "Pipe " << id_ << " wrote descriptor (#" << op->seq << ")";
     for (auto& p : m.payloads) {
-      if (p.length == 0) {
+      if (p.length == 0 && !stock_) {
         continue;
       }
       ++op->pendingWrites;
@@ -1266,7 +1594,8 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
           self->flushWrites();
         });
       };
-      auto* batched = dynamic_cast<channel::BatchedChannel*>(ch.get());
+      // A stock pipe on the other end hands its channel one tensor at a time.
+      auto* batched = stock_ ? nullptr : dynamic_cast<channel::BatchedChannel*>(ch.get());
       if (batched != nullptr && g.second.size() > 1) {
         std::vector<channel::BatchEntry> entries;
         entries.reserve(g.second.size());
@@ -1361,6 +1690,9 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     if (connection_) {
       connection_->close();
     }
+    if (replyConnection_) {
+      replyConnection_->close();
+    }
     for (auto& ch : channels_) {
       ch.second->close();
     }
@@ -1391,6 +1723,10 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   std::shared_ptr<transport::Connection> connection_;
   std::vector<uint8_t> hello_;
   const bool isClient_;
+  // The reference's encodings on the wire (ContextOptions::stockWireFormat);
+  // descriptor replies then have a connection of their own.
+  const bool stock_;
+  std::shared_ptr<transport::Connection> replyConnection_;
   uint64_t childKey_{0};
   Error error_;
   bool established_{false};
@@ -1417,37 +1753,81 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
 
 // ---------------------------------------------------------------------------
 
-void ListenerImpl::onConnection(std::shared_ptr<transport::Connection> conn) {
+void ListenerImpl::serveRequested(uint64_t token, std::shared_ptr<transport::Connection> conn) {
+  auto it = requests_.find(token);
+  if (it == requests_.end()) {
+    TP_VLOG(1) << "Listener got a connection for unknown token " << token;
+    return;
+  }
+  auto fn = std::move(it->second);
+  requests_.erase(it);
+  fn(Error::kSuccess, std::move(conn));
+}
+
+// The reference's opening (tensorpipe/core/listener_impl.cc:280-338,
+// pipe_impl.cc:262-345): a Packet that is either a requested connection, or a
+// spontaneous one which a Brochure follows.
+void ListenerImpl::onStockConnection(std::shared_ptr<transport::Connection> conn, const std::string& transport) {
+  auto self = shared_from_this();
+  auto* raw = conn.get();
+  raw->read([self, conn, transport](const Error& error, const void* ptr, size_t len) mutable {
+    tpnop::Packet packet;
+    const bool ok = !error && tpnop::decode(static_cast<const uint8_t*>(ptr), len, &packet);
+    self->ctx_->defer([self, conn, transport, ok, packet{std::move(packet)}]() mutable {
+      if (self->error_ || !ok) {
+        return;
+      }
+      if (packet.which == tpnop::Packet::kRequested) {
+        self->serveRequested(packet.requested.registrationId, std::move(conn));
+        return;
+      }
+      auto* raw2 = conn.get();
+      std::string name = std::move(packet.spontaneous.contextName);
+      raw2->read([self, conn, transport, name{std::move(name)}](const Error& error2, const void* ptr2, size_t len2) mutable {
+        tpnop::Brochure brochure;
+        const bool ok2 = !error2 && tpnop::decode(static_cast<const uint8_t*>(ptr2), len2, &brochure);
+        self->ctx_->defer([self, conn, transport, ok2, name{std::move(name)}, brochure{std::move(brochure)}]() mutable {
+          if (self->error_ || !ok2) {
+            return;
+          }
+          auto impl = std::make_shared<PipeImpl>(
+              self->ctx_, self, self->ctx_->nextPipeId(), std::move(conn), helloPacketFromStock(name, brochure), transport, name);
+          impl->init();
+          self->onPipeReady(std::make_shared<Pipe>(Pipe::ConstructorToken(), std::move(impl)));
+        });
+      });
+    });
+  });
+}
+
+void ListenerImpl::onConnection(std::shared_ptr<transport::Connection> conn, const std::string& transport) {
+  if (ctx_->stockWire()) {
+    onStockConnection(std::move(conn), transport);
+    return;
+  }
   auto self = shared_from_this();
   // The first packet says whether this is a new pipe or a connection a pipe
   // asked for (tensorpipe/core/listener_impl.cc, "hello" handling).
   auto* raw = conn.get();
-  raw->read([self, conn](const Error& error, const void* ptr, size_t len) mutable {
+  raw->read([self, conn, transport](const Error& error, const void* ptr, size_t len) mutable {
     std::vector<uint8_t> bytes;
     if (!error) {
       bytes.assign(static_cast<const uint8_t*>(ptr), static_cast<const uint8_t*>(ptr) + len);
     }
-    self->ctx_->defer([self, conn, error, bytes{std::move(bytes)}]() mutable {
+    self->ctx_->defer([self, conn, transport, error, bytes{std::move(bytes)}]() mutable {
       if (self->error_ || error || bytes.empty()) {
         return;
       }
       WireReader r(bytes.data(), bytes.size());
       const uint8_t type = r.u8();
       if (type == kHelloSpontaneous) {
+        std::string name = r.str();
         auto impl = std::make_shared<PipeImpl>(
-            self->ctx_, self, self->ctx_->nextPipeId(), std::move(conn), std::move(bytes));
+            self->ctx_, self, self->ctx_->nextPipeId(), std::move(conn), std::move(bytes), transport, std::move(name));
         impl->init();
         self->onPipeReady(std::make_shared<Pipe>(Pipe::ConstructorToken(), std::move(impl)));
       } else if (type == kHelloRequested) {
-        const uint64_t token = r.u64();
-        auto it = self->requests_.find(token);
-        if (it == self->requests_.end()) {
-          TP_VLOG(1) << "Listener got a connection for unknown token " << token;
-          return;
-        }
-        auto fn = std::move(it->second);
-        self->requests_.erase(it);
-        fn(Error::kSuccess, std::move(conn));
+        self->serveRequested(r.u64(), std::move(conn));
       }
     });
   });

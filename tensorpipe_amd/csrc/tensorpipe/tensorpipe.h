@@ -17,6 +17,7 @@
 #include <tensorpipe/transport/context.h>
 #include <tensorpipe/transport/error.h>
 #include <tensorpipe/transport/shm/factory.h>
+#include <tensorpipe/transport/tcp/factory.h>
 
 #include <tensorpipe/channel/context.h>
 #include <tensorpipe/channel/error.h>

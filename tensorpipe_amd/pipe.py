@@ -62,6 +62,8 @@ def lib():
         l.tpc_last_error.restype = ctypes.c_char_p
         l.tpc_context_create.restype = vp
         l.tpc_context_create.argtypes = [ctypes.c_char_p] * 3
+        l.tpc_context_create_ex.restype = vp
+        l.tpc_context_create_ex.argtypes = [ctypes.c_char_p] * 3 + [ctypes.c_int]
         l.tpc_context_close.argtypes = [vp]
         l.tpc_context_destroy.argtypes = [vp]
         l.tpc_context_has_channel.argtypes = [vp, ctypes.c_char_p]
@@ -231,8 +233,12 @@ class Listener:
 class Context:
     """transports / channels: e.g. "shm:0" and "basic:0,hip_xth:10"."""
 
-    def __init__(self, name="", transports="shm:0", channels="basic:0"):
-        self._h = lib().tpc_context_create(name.encode(), transports.encode(), channels.encode())
+    def __init__(self, name="", transports="shm:0", channels="basic:0", stock_wire=None):
+        """`transports` may name "uv" (TCP, framed like the reference's uv transport); `stock_wire`
+        True puts the reference's own encodings on the wire, so that the peer may be an unmodified
+        TensorPipe (None: as TP_STOCK_WIRE in the environment says)."""
+        self._h = lib().tpc_context_create_ex(name.encode(), transports.encode(), channels.encode(),
+                                              -1 if stock_wire is None else int(bool(stock_wire)))
         if not self._h:
             _fail("context")
 

@@ -28,6 +28,7 @@
 #include <tphip.h>
 
 #include <bridge/stock_adapter.h>
+#include <tensorpipe_c.h>
 
 using namespace tensorpipe;
 using tensorpipe_amd_bridge::HipBuffer;
@@ -41,9 +42,13 @@ using tensorpipe_amd_bridge::HipBuffer;
     }                                                                          \
   } while (0)
 
-static std::shared_ptr<Context> makeContext(const char* name, const std::vector<std::string>& channels) {
+static std::shared_ptr<Context> makeContext(const char* name, const std::vector<std::string>& channels, bool withUv = false) {
   auto ctx = std::make_shared<Context>(ContextOptions().name(name));
-  ctx->registerTransport(0, "shm", transport::shm::create());
+  if (withUv) {
+    ctx->registerTransport(0, "uv", transport::uv::create());
+  } else {
+    ctx->registerTransport(0, "shm", transport::shm::create());
+  }
   ctx->registerChannel(0, "basic", channel::basic::create());
   int priority = 10;
   for (auto& c : channels) {
@@ -487,6 +492,214 @@ static int timeSameProcess(size_t bytes, int iters) {
   return problem.empty() ? 0 : 1;
 }
 
+// ---- this library's own pipe as the peer -----------------------------------------
+//
+// One end is a context of this library in stock wire format (its pipe, its TCP
+// transport under the name "uv", its channels natively), driven through the C
+// harness API; the other end is the stock TensorPipe with the same channel
+// registered through the bridge. The two were built from different headers and
+// meet on the wire only.
+
+static std::string nativeSend(tpc_pipe* pipe, int salt) {
+  std::vector<GpuTensor> gpus;
+  std::vector<uint8_t> cpu(kCpuBytes);
+  for (size_t i = 0; i < cpu.size(); ++i) {
+    cpu[i] = pattern(i, salt + 50);
+  }
+  std::string payload = kPayload;
+  tpc_payload p{&payload[0], payload.size()};
+  std::vector<tpc_tensor> tensors;
+  for (size_t k = 0; k < kGpuSizes.size(); ++k) {
+    gpus.push_back(makeGpu(kGpuSizes[k]));
+    gpus.back().fill(salt + static_cast<int>(k));
+    tpc_tensor t{};
+    t.ptr = gpus.back().dev;
+    t.length = gpus.back().bytes;
+    t.device_type = TPC_DEVICE_HIP;
+    t.target_type = TPC_DEVICE_HIP;
+    t.target_index = 0;
+    t.stream = gpus.back().stream;
+    tensors.push_back(t);
+  }
+  tpc_tensor ct{};
+  ct.ptr = cpu.data();
+  ct.length = cpu.size();
+  ct.device_type = TPC_DEVICE_CPU;
+  ct.target_type = TPC_NO_TARGET;
+  tensors.push_back(ct);
+  tpc_op* op = tpc_write_async(pipe, "conformance", &p, 1, tensors.data(), static_cast<uint32_t>(tensors.size()));
+  if (op == nullptr || tpc_op_wait(op, 60000) != 0) {
+    return std::string("native write: ") + tpc_last_error();
+  }
+  return "";
+}
+
+static std::string nativeRecv(tpc_pipe* pipe, int salt) {
+  auto d = std::make_unique<tpc_descriptor>();
+  if (tpc_read_descriptor(pipe, d.get(), 60000) != 0) {
+    return std::string("native readDescriptor: ") + tpc_last_error();
+  }
+  if (std::string(d->metadata) != "conformance" || d->num_payloads != 1 || d->num_tensors != kGpuSizes.size() + 1) {
+    return "unexpected descriptor on the native end";
+  }
+  std::string payload(d->payload_lengths[0], '\0');
+  void* payloadPtr = &payload[0];
+  std::vector<GpuTensor> gpus;
+  std::vector<uint8_t> cpu(d->tensor_lengths[kGpuSizes.size()]);
+  std::vector<tpc_tensor> tensors;
+  for (size_t k = 0; k < kGpuSizes.size(); ++k) {
+    if (d->tensor_lengths[k] != kGpuSizes[k] || d->tensor_source_type[k] != TPC_DEVICE_HIP) {
+      return "unexpected GPU tensor in the descriptor on the native end";
+    }
+    gpus.push_back(makeGpu(kGpuSizes[k]));
+    tpc_tensor t{};
+    t.ptr = gpus.back().dev;
+    t.length = gpus.back().bytes;
+    t.device_type = TPC_DEVICE_HIP;
+    t.target_type = TPC_NO_TARGET;
+    t.stream = gpus.back().stream;
+    tensors.push_back(t);
+  }
+  tpc_tensor ct{};
+  ct.ptr = cpu.data();
+  ct.length = cpu.size();
+  ct.device_type = TPC_DEVICE_CPU;
+  ct.target_type = TPC_NO_TARGET;
+  tensors.push_back(ct);
+  tpc_op* op = tpc_read_async(pipe, &payloadPtr, 1, tensors.data(), static_cast<uint32_t>(tensors.size()));
+  if (op == nullptr || tpc_op_wait(op, 60000) != 0) {
+    return std::string("native read: ") + tpc_last_error();
+  }
+  if (payload != kPayload) {
+    return "payload differs on the native end";
+  }
+  for (size_t k = 0; k < gpus.size(); ++k) {
+    std::string bad = gpus[k].check(salt + static_cast<int>(k));
+    if (!bad.empty()) {
+      return bad + " (native end)";
+    }
+  }
+  if (cpu.size() != kCpuBytes) {
+    return "CPU tensor has the wrong length on the native end";
+  }
+  for (size_t i = 0; i < cpu.size(); ++i) {
+    if (cpu[i] != pattern(i, salt + 50)) {
+      return "byte " + std::to_string(i) + " of the CPU tensor differs on the native end";
+    }
+  }
+  return "";
+}
+
+// hip_xth needs both ends in one process: a native server and a stock client.
+static int nativePeerSameProcess() {
+  tpc_context* native = tpc_context_create_ex("native_server", "uv:0", "basic:0,hip_xth:12", 1);
+  tpc_listener* listener = native != nullptr ? tpc_listen(native, "uv://127.0.0.1") : nullptr;
+  char url[256] = {0};
+  if (listener == nullptr || tpc_listener_url(listener, "uv", url, sizeof(url)) != 0) {
+    report("native_hip_xth_with_stock_peer", std::string("native listen: ") + tpc_last_error());
+    return 1;
+  }
+  auto ctx = makeContext("stock_client", {"hip_xth"}, /*withUv=*/true);
+  auto stock = ctx->connect(url);
+  tpc_pipe* pipe = tpc_accept(listener, 30000);
+  std::string problem = pipe != nullptr ? std::string() : std::string("native accept: ") + tpc_last_error();
+  const unsigned long long before = tensorpipe_amd_bridge::gpuOperationsServed();
+  for (int round = 0; round < 3 && problem.empty(); ++round) {
+    auto sent = std::async(std::launch::async, [&] { return nativeSend(pipe, 20 * round); });
+    problem = recvMessage(*stock, 20 * round);
+    const std::string w = sent.get();
+    if (problem.empty()) {
+      problem = w;
+    }
+    if (problem.empty()) {
+      auto sent2 = std::async(std::launch::async, [&] { return sendMessage(*stock, 20 * round + 7); });
+      problem = nativeRecv(pipe, 20 * round + 7);
+      const std::string w2 = sent2.get();
+      if (problem.empty()) {
+        problem = w2;
+      }
+    }
+  }
+  if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() - before != 3 * 2 * 3) {
+    problem = "the GPU tensors did not all travel on this library's channel on the stock end";
+  }
+  report("native_hip_xth_with_stock_peer", problem);
+  stock.reset();
+  if (pipe != nullptr) {
+    tpc_pipe_destroy(pipe);
+  }
+  tpc_listener_destroy(listener);
+  tpc_context_destroy(native);
+  ctx->join();
+  return problem.empty() ? 0 : 1;
+}
+
+// hip_ipc / hip_basic: the native end in a child process, the stock end here.
+static int nativePeerTwoProcess(const std::string& channel) {
+  int toChild[2], toParent[2];
+  if (::pipe(toChild) != 0 || ::pipe(toParent) != 0) {
+    return 3;
+  }
+  pid_t pid = ::fork(); // before anything has touched the GPU
+  if (pid == 0) {
+    const std::string channels = "basic:0," + channel + ":10";
+    tpc_context* native = tpc_context_create_ex("native_peer", "uv:0", channels.c_str(), 1);
+    tpc_listener* listener = native != nullptr ? tpc_listen(native, "uv://127.0.0.1") : nullptr;
+    char url[256] = {0};
+    if (listener == nullptr || tpc_listener_url(listener, "uv", url, sizeof(url)) != 0) {
+      std::fprintf(stderr, "[native] listen: %s\n", tpc_last_error());
+      ::_exit(2);
+    }
+    if (::write(toParent[1], url, sizeof(url)) != static_cast<ssize_t>(sizeof(url))) {
+      ::_exit(2);
+    }
+    tpc_pipe* pipe = tpc_accept(listener, 30000);
+    std::string problem = pipe != nullptr ? std::string() : std::string("accept: ") + tpc_last_error();
+    if (problem.empty()) {
+      problem = nativeRecv(pipe, 1);
+    }
+    if (problem.empty()) {
+      problem = nativeSend(pipe, 2);
+    }
+    if (!problem.empty()) {
+      std::fprintf(stderr, "[native] %s\n", problem.c_str());
+    }
+    char byte = 0;
+    (void)!::read(toChild[0], &byte, 1); // the stock end has checked what it received
+    if (pipe != nullptr) {
+      tpc_pipe_destroy(pipe);
+    }
+    tpc_listener_destroy(listener);
+    tpc_context_destroy(native);
+    ::_exit(problem.empty() ? 0 : 1);
+  }
+  char url[256] = {0};
+  if (::read(toParent[0], url, sizeof(url)) != static_cast<ssize_t>(sizeof(url))) {
+    report("native_" + channel + "_with_stock_peer", "the native process did not come up");
+    return 1;
+  }
+  auto ctx = makeContext("stock_main", {channel}, /*withUv=*/true);
+  auto pipe = ctx->connect(url);
+  std::string problem = sendMessage(*pipe, 1);
+  if (problem.empty()) {
+    problem = recvMessage(*pipe, 2);
+  }
+  if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() != 6) {
+    problem = "the GPU tensors did not all travel on this library's channel on the stock end";
+  }
+  const char byte = 1;
+  (void)!::write(toChild[1], &byte, 1);
+  int status = 0;
+  ::waitpid(pid, &status, 0);
+  if (problem.empty() && !(WIFEXITED(status) && WEXITSTATUS(status) == 0)) {
+    problem = "the native process reported a failure";
+  }
+  report("native_" + channel + "_with_stock_peer", problem);
+  pipe.reset();
+  ctx->join();
+  return problem.empty() ? 0 : 1;
+}
+
 int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "same_process") == 0) {
     return sameProcess();
@@ -497,9 +710,12 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "unmodified_peer") == 0) {
     return unmodifiedPeer();
   }
+  if (argc == 3 && std::strcmp(argv[1], "native_peer") == 0) {
+    return std::strcmp(argv[2], "hip_xth") == 0 ? nativePeerSameProcess() : nativePeerTwoProcess(argv[2]);
+  }
   if (argc == 4 && std::strcmp(argv[1], "time_same_process") == 0) {
     return timeSameProcess(std::strtoull(argv[2], nullptr, 10), std::atoi(argv[3]));
   }
-  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer | time_same_process <bytes> <messages>\n", argv[0]);
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic | time_same_process <bytes> <messages>\n", argv[0]);
   return 2;
 }

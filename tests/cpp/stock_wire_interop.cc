@@ -10,6 +10,11 @@
 //   stock_wire_interop capture <file>      also writes the frames the STOCK end produced
 //                                          (name, hex) -- how tests/golden/stock_wire_vectors.txt was made
 //
+// The same two roles once more with this library's own asynchronous pipe on the
+// compat side: a context in stock wire format (ContextOptions::stockWireFormat)
+// over its TCP transport registered as "uv", driven through the C harness API
+// because its C++ headers share their names with the stock ones.
+//
 // No GPU involved.
 #include <tensorpipe/tensorpipe.h> // the stock headers: listed first on the include path
 
@@ -21,6 +26,7 @@
 #include <vector>
 
 #include <nopwire/compat_pipe.h>
+#include <tensorpipe_c.h>
 
 using namespace tensorpipe;
 
@@ -277,6 +283,198 @@ int stockConnectsToCompat() {
   return problem.empty() ? 0 : 1;
 }
 
+// ---- this library's pipe in stock wire format ---------------------------------
+
+// Writes `m` on the native pipe and waits for the callback.
+std::string nativeWrite(tpc_pipe* pipe, const tpnop::CompatMessage& m) {
+  std::vector<tpc_payload> payloads;
+  std::vector<tpc_tensor> tensors;
+  for (auto& p : m.payloads) {
+    payloads.push_back(tpc_payload{const_cast<char*>(p.bytes.data()), p.bytes.size()});
+  }
+  for (auto& t : m.tensors) {
+    tpc_tensor ct{};
+    ct.ptr = const_cast<char*>(t.bytes.data());
+    ct.length = t.bytes.size();
+    ct.device_type = TPC_DEVICE_CPU;
+    ct.target_type = t.nameTarget ? TPC_DEVICE_CPU : TPC_NO_TARGET;
+    ct.target_index = 0;
+    tensors.push_back(ct);
+  }
+  tpc_op* op = tpc_write_async(pipe, m.metadata.c_str(), payloads.data(), static_cast<uint32_t>(payloads.size()),
+                               tensors.data(), static_cast<uint32_t>(tensors.size()));
+  if (op == nullptr) {
+    return std::string("native write: ") + tpc_last_error();
+  }
+  return tpc_op_wait(op, 30000) == 0 ? "" : std::string("native write: ") + tpc_last_error();
+}
+
+// Reads one message on the native pipe (lengths and bytes; the C API does not
+// hand out per-item metadata).
+std::string nativeRead(tpc_pipe* pipe, tpnop::CompatMessage* got) {
+  auto d = std::make_unique<tpc_descriptor>();
+  if (tpc_read_descriptor(pipe, d.get(), 30000) != 0) {
+    return std::string("native readDescriptor: ") + tpc_last_error();
+  }
+  got->metadata = d->metadata;
+  got->payloads.resize(d->num_payloads);
+  got->tensors.resize(d->num_tensors);
+  std::vector<void*> payloadPtrs;
+  std::vector<tpc_tensor> tensors;
+  for (uint32_t i = 0; i < d->num_payloads; ++i) {
+    got->payloads[i].bytes.assign(d->payload_lengths[i], '\0');
+    payloadPtrs.push_back(&got->payloads[i].bytes[0]);
+  }
+  for (uint32_t i = 0; i < d->num_tensors; ++i) {
+    if (d->tensor_source_type[i] != TPC_DEVICE_CPU) {
+      return "a tensor announced on another device type";
+    }
+    got->tensors[i].bytes.assign(d->tensor_lengths[i], '\0');
+    got->tensors[i].nameTarget = d->tensor_target_type[i] != TPC_NO_TARGET;
+    tpc_tensor ct{};
+    ct.ptr = &got->tensors[i].bytes[0];
+    ct.length = d->tensor_lengths[i];
+    ct.device_type = TPC_DEVICE_CPU;
+    ct.target_type = TPC_NO_TARGET;
+    tensors.push_back(ct);
+  }
+  tpc_op* op = tpc_read_async(pipe, payloadPtrs.data(), d->num_payloads, tensors.data(), d->num_tensors);
+  if (op == nullptr) {
+    return std::string("native read: ") + tpc_last_error();
+  }
+  return tpc_op_wait(op, 30000) == 0 ? "" : std::string("native read: ") + tpc_last_error();
+}
+
+std::string compareBytes(const tpnop::CompatMessage& got, const tpnop::CompatMessage& want, bool itemMetadata) {
+  if (got.metadata != want.metadata || got.payloads.size() != want.payloads.size() ||
+      got.tensors.size() != want.tensors.size()) {
+    return "metadata or counts differ";
+  }
+  for (size_t i = 0; i < want.payloads.size(); ++i) {
+    if (got.payloads[i].bytes != want.payloads[i].bytes ||
+        (itemMetadata && got.payloads[i].metadata != want.payloads[i].metadata)) {
+      return "payload " + std::to_string(i) + " differs";
+    }
+  }
+  for (size_t i = 0; i < want.tensors.size(); ++i) {
+    if (got.tensors[i].bytes != want.tensors[i].bytes || got.tensors[i].nameTarget != want.tensors[i].nameTarget ||
+        (itemMetadata && got.tensors[i].metadata != want.tensors[i].metadata)) {
+      return "tensor " + std::to_string(i) + " differs";
+    }
+  }
+  return "";
+}
+
+// The C API sends no per-item metadata: the message without it.
+tpnop::CompatMessage plain(tpnop::CompatMessage m) {
+  for (auto& p : m.payloads) {
+    p.metadata.clear();
+  }
+  for (auto& t : m.tensors) {
+    t.metadata.clear();
+  }
+  return m;
+}
+
+std::string nativeExchange(tpc_pipe* native, Pipe& stock, int salt) {
+  for (int round = 0; round < 3; ++round) {
+    // native -> stock
+    const tpnop::CompatMessage sent = plain(testMessage(salt + round));
+    tpnop::CompatMessage got;
+    auto reading = std::async(std::launch::async, [&] { return stockRead(stock, &got); });
+    std::string problem = nativeWrite(native, sent);
+    const std::string r = reading.get();
+    if (problem.empty()) {
+      problem = r.empty() ? compareBytes(got, sent, true) : r;
+    }
+    if (!problem.empty()) {
+      return "native -> stock: " + problem;
+    }
+    // stock -> native
+    const tpnop::CompatMessage back = testMessage(salt + round + 50);
+    tpnop::CompatMessage got2;
+    auto writing = std::async(std::launch::async, [&] { return stockWrite(stock, back); });
+    problem = nativeRead(native, &got2);
+    const std::string w = writing.get();
+    if (problem.empty()) {
+      problem = w.empty() ? compareBytes(got2, back, false) : w;
+    }
+    if (!problem.empty()) {
+      return "stock -> native: " + problem;
+    }
+  }
+  return "";
+}
+
+int nativeConnectsToStock() {
+  auto ctx = stockContext("stock_server");
+  auto listener = ctx->listen({"uv://127.0.0.1"});
+  auto accepted = std::make_shared<std::promise<std::shared_ptr<Pipe>>>();
+  listener->accept([accepted](const Error& e, std::shared_ptr<Pipe> p) { accepted->set_value(e ? nullptr : p); });
+  tpc_context* native = tpc_context_create_ex("native_client", "uv:0", "basic:0", 1);
+  tpc_pipe* pipe = native != nullptr ? tpc_connect(native, listener->url("uv").c_str()) : nullptr;
+  std::string problem;
+  std::shared_ptr<Pipe> stock;
+  if (pipe == nullptr) {
+    problem = std::string("native connect: ") + tpc_last_error();
+  } else {
+    auto f = accepted->get_future();
+    if (f.wait_for(std::chrono::seconds(30)) != std::future_status::ready || !(stock = f.get())) {
+      problem = "the stock listener did not hand out a pipe";
+    }
+  }
+  if (problem.empty() && stock->getRemoteName() != "native_client") {
+    problem = "the stock end heard the name " + stock->getRemoteName();
+  }
+  if (problem.empty()) {
+    problem = nativeExchange(pipe, *stock, 200);
+  }
+  report("native_client_with_stock_server", problem);
+  stock.reset();
+  if (pipe != nullptr) {
+    tpc_pipe_destroy(pipe);
+  }
+  if (native != nullptr) {
+    tpc_context_destroy(native);
+  }
+  listener.reset();
+  ctx->join();
+  return problem.empty() ? 0 : 1;
+}
+
+int stockConnectsToNative() {
+  tpc_context* native = tpc_context_create_ex("native_server", "uv:0", "basic:0", 1);
+  tpc_listener* listener = native != nullptr ? tpc_listen(native, "uv://127.0.0.1") : nullptr;
+  char url[256] = {0};
+  std::string problem;
+  if (listener == nullptr || tpc_listener_url(listener, "uv", url, sizeof(url)) != 0) {
+    problem = std::string("native listen: ") + tpc_last_error();
+    report("stock_client_with_native_server", problem);
+    return 1;
+  }
+  auto ctx = stockContext("stock_client");
+  auto stock = ctx->connect(url);
+  tpc_pipe* pipe = tpc_accept(listener, 30000);
+  char name[256] = {0};
+  if (pipe == nullptr) {
+    problem = std::string("native accept: ") + tpc_last_error();
+  } else if (tpc_pipe_remote_name(pipe, name, sizeof(name)) != 0 || std::string(name) != "stock_client") {
+    problem = std::string("the native end heard the name ") + name;
+  }
+  if (problem.empty()) {
+    problem = nativeExchange(pipe, *stock, 300);
+  }
+  report("stock_client_with_native_server", problem);
+  stock.reset();
+  if (pipe != nullptr) {
+    tpc_pipe_destroy(pipe);
+  }
+  tpc_listener_destroy(listener);
+  tpc_context_destroy(native);
+  ctx->join();
+  return problem.empty() ? 0 : 1;
+}
+
 } // namespace
 
 int main(int argc, char** argv) {
@@ -287,6 +485,8 @@ int main(int argc, char** argv) {
   }
   int rc = compatConnectsToStock();
   rc |= stockConnectsToCompat();
+  rc |= nativeConnectsToStock();
+  rc |= stockConnectsToNative();
   if (std::strcmp(argv[1], "capture") == 0 && rc == 0) {
     FILE* f = std::fopen(argv[2], "w");
     if (f == nullptr) {

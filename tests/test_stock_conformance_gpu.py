@@ -42,3 +42,11 @@ def test_endpoint_with_hip_channels_talks_to_an_unmodified_peer():
     """Registering the channels does not get in the way of a peer that has none of them: payloads
     and CPU tensors still travel on the stock channels."""
     _run(["unmodified_peer"])
+
+
+@pytest.mark.parametrize("channel", ["hip_xth", "hip_ipc", "hip_basic"])
+def test_native_pipe_in_stock_wire_format_with_a_stock_peer(channel):
+    """One end is a context of this library with ContextOptions::stockWireFormat (its own pipe, its
+    TCP transport registered as "uv", the channel natively), the other the stock TensorPipe with the
+    same channel through the bridge: payload, GPU tensors and a CPU tensor both ways, byte for byte."""
+    _run(["native_peer", channel])

@@ -19,7 +19,9 @@ def test_compat_endpoint_and_stock_endpoint_understand_each_other():
         pytest.skip("tests/cpp/bin/stock_wire_interop is not built (no stock TensorPipe headers at build time)")
     proc = subprocess.run([PROGRAM, "run"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
     results = [line for line in proc.stdout.splitlines() if line.startswith("RESULT ")]
-    assert [r.split()[1] for r in results] == ["compat_client_with_stock_server", "stock_client_with_compat_server"], (
+    assert [r.split()[1] for r in results] == [
+        "compat_client_with_stock_server", "stock_client_with_compat_server",
+        "native_client_with_stock_server", "stock_client_with_native_server"], (
         proc.stdout[-2000:] + proc.stderr[-2000:])
     bad = [r for r in results if r.split()[2] != "OK"]
     assert not bad and proc.returncode == 0, "\n".join(bad) + proc.stderr[-2000:]
