@@ -39,13 +39,14 @@ def list_cases(program, suite):
     return out.stdout.split()
 
 
-def run_suite(program, suite):
+def run_suite(program, suite, stock_wire=False):
     """One run per suite and session; returns {case: [(role, ok, detail), ...]}."""
-    key = (program, suite)
+    key = (program, suite, stock_wire)
     if key not in _results:
-        print(f"running {program} --suite {suite}", flush=True)
+        print(f"running {program} --suite {suite}" + (" in stock wire format" if stock_wire else ""), flush=True)
+        env = dict(os.environ, TP_STOCK_WIRE="1") if stock_wire else None
         proc = subprocess.run([_binary(program), "--suite", suite], stdout=subprocess.PIPE,
-                              stderr=subprocess.PIPE, text=True, timeout=600)
+                              stderr=subprocess.PIPE, text=True, timeout=600, env=env)
         per_case = {}
         for line in proc.stdout.splitlines():
             parts = line.split(" ", 4)
@@ -56,8 +57,8 @@ def run_suite(program, suite):
     return _results[key]
 
 
-def check_case(program, suite, case):
-    rc, per_case, out, err = run_suite(program, suite)
+def check_case(program, suite, case, stock_wire=False):
+    rc, per_case, out, err = run_suite(program, suite, stock_wire)
     assert case in per_case, f"no result for {case}; exit code {rc}\n{out}\n{err}"
     bad = [line for _, ok, line in per_case[case] if not ok]
     assert not bad, "\n".join(bad) + "\n" + err
@@ -79,3 +80,17 @@ def test_cpu_suite(program, suite, case):
 @pytest.mark.parametrize("program,suite,case", _params(GPU_SUITES))
 def test_gpu_suite(program, suite, case):
     check_case(program, suite, case)
+
+
+# The pipe suites once more with the reference's encodings on the wire (TP_STOCK_WIRE=1: its
+# handshake, libnop descriptors, descriptor replies on their own connection, no batching across
+# the channel interface): the same cases must pass, both ends being this library's.
+@pytest.mark.parametrize("program,suite,case", _params([s for s in CPU_SUITES if s[0] == "pipe_tests"]))
+def test_cpu_suite_in_stock_wire_format(program, suite, case):
+    check_case(program, suite, case, stock_wire=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("program,suite,case", _params([s for s in GPU_SUITES if s[0] == "pipe_tests"]))
+def test_gpu_suite_in_stock_wire_format(program, suite, case):
+    check_case(program, suite, case, stock_wire=True)
