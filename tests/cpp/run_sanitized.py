@@ -18,8 +18,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 sys.path.insert(0, ROOT)
 from tensorpipe_amd import build as tp_build  # noqa: E402
 
-SUITES = [("channel_tests", "xth"), ("channel_tests", "basic"),
-          ("pipe_tests", "cpu_same_process"), ("pipe_tests", "cpu_two_process")]
+# (program, suite, stock wire format)
+SUITES = [("channel_tests", "xth", False), ("channel_tests", "basic", False),
+          ("pipe_tests", "cpu_same_process", False), ("pipe_tests", "cpu_two_process", False),
+          ("pipe_tests", "cpu_same_process", True), ("pipe_tests", "cpu_two_process", True)]
 
 
 def main():
@@ -39,18 +41,19 @@ def main():
     lib = os.path.join(out, "libtensorpipe_amd.so")
     subprocess.run(["g++", "-shared", f"-fsanitize={san}", "-pthread", "-o", lib, *objs, f"-L{tp_build.LIB}",
                     "-ltphip", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
-    for prog in sorted({p for p, _ in SUITES} | {"unit_tests"}):
+    for prog in sorted({p for p, _, _ in SUITES} | {"unit_tests"}):
         subprocess.run(["g++", *flags, os.path.join(ROOT, "tests", "cpp", prog + ".cc"), "-o",
                         os.path.join(out, prog), f"-L{out}", "-ltensorpipe_amd", f"-L{tp_build.LIB}", "-ltphip",
                         f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
     bad = 0
-    for prog, suite in SUITES:
+    for prog, suite, stock_wire in SUITES:
+        env = dict(os.environ, TP_STOCK_WIRE="1") if stock_wire else None
         proc = subprocess.run([os.path.join(out, prog), "--suite", suite], stdout=subprocess.PIPE,
-                              stderr=subprocess.STDOUT, text=True, timeout=1800)
+                              stderr=subprocess.STDOUT, text=True, timeout=1800, env=env)
         results = [l for l in proc.stdout.splitlines() if l.startswith("RESULT")]
         failed = [l for l in results if " OK" not in l]
         reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
-        print(f"{prog} --suite {suite}: {len(results)} results, {len(failed)} failed, {len(reports)} sanitizer reports")
+        print(f"{prog} --suite {suite}{' (stock wire format)' if stock_wire else ''}: {len(results)} results, {len(failed)} failed, {len(reports)} sanitizer reports")
         for l in failed + reports[:5]:
             print("   ", l[:200])
         bad += len(failed) + len(reports) + (0 if results else 1)

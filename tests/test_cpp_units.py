@@ -73,6 +73,14 @@ def test_host_pointer_in_a_hip_buffer_is_refused():
     assert rc == 0 and out.strip() == "OK", out
 
 
+@pytest.mark.parametrize("seed", [4, 5])
+def test_garbage_on_new_connections_in_stock_wire_format(seed):
+    # the same where the first packets are the reference's libnop objects
+    out = subprocess.run([BIN, "garbage", str(seed), "100"], stdout=subprocess.PIPE, text=True, timeout=120,
+                         env=dict(os.environ, TP_STOCK_WIRE="1"))
+    assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_garbage_on_new_connections(seed):
     # random bytes where the first packets of a pipe belong: the listening context survives them
