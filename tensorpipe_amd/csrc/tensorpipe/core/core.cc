@@ -5,12 +5,17 @@
 //
 // Differences from the reference that a user can observe:
 //  * the pipe stays on the transport it was opened on (no transport upgrade);
-//  * control messages use common/wire.h instead of libnop, so this Pipe does
-//    not interoperate with a stock TensorPipe peer;
-//  * all tensors of a message that map to one channel are handed to that
+//  * by default control messages use common/wire.h instead of libnop, and
+//    all tensors of a message that map to one channel are handed to that
 //    channel as ONE batch when it implements channel::BatchedChannel, so a
 //    message costs one control message and one kernel launch, not one per
-//    tensor (cf. the per-tensor loop at tensorpipe/core/pipe_impl.cc:884-915).
+//    tensor (cf. the per-tensor loop at tensorpipe/core/pipe_impl.cc:884-915);
+//  * with ContextOptions::stockWireFormat the bytes on the wire are the
+//    reference's own (nopwire/nop_wire.h: its packets as libnop objects, the
+//    descriptor-reply connection, a frame per payload, one tensor per channel
+//    call), so the peer may be an unmodified TensorPipe. The pipe itself keeps
+//    running on its own packets: what goes out is re-encoded at the last
+//    moment, what comes in is turned into a packet before it is parsed.
 
 #include <tensorpipe/core/context.h>
 #include <tensorpipe/core/listener.h>
