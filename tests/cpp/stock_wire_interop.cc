@@ -494,7 +494,7 @@ int main(int argc, char** argv) {
       return 3;
     }
     std::fprintf(f, "# Control frames written by an unmodified TensorPipe endpoint (the build inside PyTorch's\n");
-    std::fprintf(f, "# libtorch_cpu.so), as read off the TCP connections by tests/cpp/stock_wire_interop.cc capture:\n");
+    std::fprintf(f, "# libtorch_cpu.so), as read off the TCP connections by tests/cpp/stock_wire_interop.cc capture\n# (tests/golden/make_stock_wire_vectors.sh runs it):\n");
     std::fprintf(f, "# <who wrote it>.<what> <hex>. Ports and registration tokens are those of the capturing run.\n");
     for (auto& kv : captured) {
       std::fprintf(f, "%s ", kv.first.c_str());
