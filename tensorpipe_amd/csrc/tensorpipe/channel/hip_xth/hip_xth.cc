@@ -274,6 +274,7 @@ class ChannelImpl final : public ChannelImplBase {
         g->table.push_back(tphip_copy_desc{src, hb.ptr, len});
       }
       decodeTimer.reset();
+      TP_MARK("xth: descriptor decoded");
       for (auto& g : groups) {
         StageScope launchTimer(Stage::kXthLaunch);
         // The copy may only touch a destination once everything the receiver
@@ -287,9 +288,11 @@ class ChannelImpl final : public ChannelImplBase {
           }
         }
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
+        TP_MARK("xth: destination streams checked");
         auto done = xctx_->events.get(g.src.device);
         const bool onKernel =
             hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*signalOnKernel=*/true);
+        TP_MARK("xth: kernel launch call returned");
         StreamMarkers::Launch launch;
         if (onKernel) {
           launch = xctx_->markers.launched(g.src.device, g.src.stream, xctx_->events);
