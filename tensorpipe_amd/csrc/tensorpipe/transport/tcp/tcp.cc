@@ -47,7 +47,28 @@ class FdHandler {
   virtual ~FdHandler() = default;
 };
 
-bool parseAddr(const std::string& addr, sockaddr_in* out) {
+// "a.b.c.d:port", "a.b.c.d", "[v6 address]:port" or "[v6 address]", as the
+// reference's uv transport writes its addresses (tensorpipe/transport/uv/sockaddr.cc).
+bool parseAddr(const std::string& addr, sockaddr_storage* out, socklen_t* len) {
+  std::memset(out, 0, sizeof(*out));
+  if (!addr.empty() && addr[0] == '[') {
+    const size_t close = addr.find(']');
+    if (close == std::string::npos) {
+      return false;
+    }
+    int port = 0;
+    if (close + 1 < addr.size()) {
+      if (addr[close + 1] != ':') {
+        return false;
+      }
+      port = std::atoi(addr.c_str() + close + 2);
+    }
+    auto* sa = reinterpret_cast<sockaddr_in6*>(out);
+    sa->sin6_family = AF_INET6;
+    sa->sin6_port = htons(static_cast<uint16_t>(port));
+    *len = sizeof(sockaddr_in6);
+    return ::inet_pton(AF_INET6, addr.substr(1, close - 1).c_str(), &sa->sin6_addr) == 1;
+  }
   std::string host = addr;
   int port = 0;
   const size_t colon = addr.rfind(':');
@@ -55,10 +76,23 @@ bool parseAddr(const std::string& addr, sockaddr_in* out) {
     host = addr.substr(0, colon);
     port = std::atoi(addr.c_str() + colon + 1);
   }
-  std::memset(out, 0, sizeof(*out));
-  out->sin_family = AF_INET;
-  out->sin_port = htons(static_cast<uint16_t>(port));
-  return ::inet_pton(AF_INET, host.c_str(), &out->sin_addr) == 1;
+  auto* sa = reinterpret_cast<sockaddr_in*>(out);
+  sa->sin_family = AF_INET;
+  sa->sin_port = htons(static_cast<uint16_t>(port));
+  *len = sizeof(sockaddr_in);
+  return ::inet_pton(AF_INET, host.c_str(), &sa->sin_addr) == 1;
+}
+
+std::string formatAddr(const sockaddr_storage& ss) {
+  char host[INET6_ADDRSTRLEN] = {0};
+  if (ss.ss_family == AF_INET6) {
+    const auto* sa = reinterpret_cast<const sockaddr_in6*>(&ss);
+    ::inet_ntop(AF_INET6, &sa->sin6_addr, host, sizeof(host));
+    return "[" + std::string(host) + "]:" + std::to_string(ntohs(sa->sin6_port));
+  }
+  const auto* sa = reinterpret_cast<const sockaddr_in*>(&ss);
+  ::inet_ntop(AF_INET, &sa->sin_addr, host, sizeof(host));
+  return std::string(host) + ":" + std::to_string(ntohs(sa->sin_port));
 }
 
 class Reactor final : public std::enable_shared_from_this<Reactor> {
@@ -361,17 +395,18 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       return;
     }
     if (fd_ < 0) {
-      sockaddr_in sa;
-      if (!parseAddr(addr_, &sa)) {
+      sockaddr_storage sa;
+      socklen_t salen = 0;
+      if (!parseAddr(addr_, &sa, &salen)) {
         fail(TP_CREATE_ERROR(SystemError, "inet_pton", EINVAL));
         return;
       }
-      fd_ = ::socket(AF_INET, SOCK_STREAM | SOCK_NONBLOCK | SOCK_CLOEXEC, 0);
+      fd_ = ::socket(sa.ss_family, SOCK_STREAM | SOCK_NONBLOCK | SOCK_CLOEXEC, 0);
       if (fd_ < 0) {
         fail(TP_CREATE_ERROR(SystemError, "socket", errno));
         return;
       }
-      const int rc = ::connect(fd_, reinterpret_cast<sockaddr*>(&sa), sizeof(sa));
+      const int rc = ::connect(fd_, reinterpret_cast<sockaddr*>(&sa), salen);
       if (rc != 0 && errno != EINPROGRESS) {
         fail(TP_CREATE_ERROR(SystemError, "connect", errno));
         return;
@@ -631,13 +666,14 @@ class ListenerImpl final : public FdHandler, public std::enable_shared_from_this
 
   // Binds at once, so that the address is known when listen() returns.
   ListenerImpl(std::shared_ptr<Reactor> reactor, const std::string& addr) : reactor_(std::move(reactor)) {
-    sockaddr_in sa;
-    TP_THROW_ASSERT_IF(!parseAddr(addr, &sa));
-    fd_ = ::socket(AF_INET, SOCK_STREAM | SOCK_NONBLOCK | SOCK_CLOEXEC, 0);
+    sockaddr_storage sa;
+    socklen_t salen = 0;
+    TP_THROW_ASSERT_IF(!parseAddr(addr, &sa, &salen));
+    fd_ = ::socket(sa.ss_family, SOCK_STREAM | SOCK_NONBLOCK | SOCK_CLOEXEC, 0);
     TP_THROW_ASSERT_IF(fd_ < 0);
     int one = 1;
     ::setsockopt(fd_, SOL_SOCKET, SO_REUSEADDR, &one, sizeof(one));
-    if (::bind(fd_, reinterpret_cast<sockaddr*>(&sa), sizeof(sa)) != 0 || ::listen(fd_, 128) != 0) {
+    if (::bind(fd_, reinterpret_cast<sockaddr*>(&sa), salen) != 0 || ::listen(fd_, 128) != 0) {
       const int err = errno;
       ::close(fd_);
       fd_ = -1;
@@ -645,9 +681,7 @@ class ListenerImpl final : public FdHandler, public std::enable_shared_from_this
     }
     socklen_t len = sizeof(sa);
     ::getsockname(fd_, reinterpret_cast<sockaddr*>(&sa), &len);
-    char host[INET_ADDRSTRLEN];
-    ::inet_ntop(AF_INET, &sa.sin_addr, host, sizeof(host));
-    addr_ = std::string(host) + ":" + std::to_string(ntohs(sa.sin_port));
+    addr_ = formatAddr(sa);
   }
 
   ~ListenerImpl() override {

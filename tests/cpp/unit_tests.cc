@@ -782,6 +782,38 @@ static int runTcp() {
   clientSide->join();
   serverSide->join();
 
+  // IPv6 loopback, where the host has it.
+  {
+    auto v6 = transport::tcp::create();
+    std::shared_ptr<transport::Listener> l6;
+    try {
+      l6 = v6->listen("[::1]");
+    } catch (const std::exception&) {
+      // no IPv6 here
+    }
+    if (l6) {
+      CHECK(l6->addr().find("[::1]:") == 0);
+      std::promise<std::shared_ptr<transport::Connection>> p6;
+      l6->accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p6.set_value(e ? nullptr : std::move(c)); });
+      auto c6 = v6->connect(l6->addr());
+      auto a6 = p6.get_future().get();
+      CHECK(a6 != nullptr);
+      if (a6) {
+        const std::string hello = "over v6";
+        c6->write(hello.data(), hello.size(), [](const Error&) {});
+        std::promise<std::string> got6;
+        a6->read([&](const Error& e, const void* ptr, size_t len) {
+          got6.set_value(e ? "error" : std::string(static_cast<const char*>(ptr), len));
+        });
+        CHECK(got6.get_future().get() == hello);
+      }
+      c6.reset();
+      a6.reset();
+      l6.reset();
+    }
+    v6->join();
+  }
+
   // A pipe over it: payload and CPU tensors through the basic channel.
   {
     auto make = [](const char* name) {
