@@ -292,26 +292,27 @@ def bench_rpc_message(messages=500, warmup=20):
 class PeerRun:
     """A bench_peer child process connected through one pipe."""
 
-    def __init__(self, channels, env=None):
+    def __init__(self, channels, env=None, transport="shm"):
         from tensorpipe_amd import pipe as tp
 
         self.tp = tp
         saved = {k: os.environ.get(k) for k in (env or {})}
         os.environ.update(env or {})
         try:
-            self.ctx = tp.Context("bench_main", channels=channels)
+            self.ctx = tp.Context("bench_main", transports=transport + ":0", channels=channels)
         finally:
             for k, v in saved.items():
                 if v is None:
                     os.environ.pop(k, None)
                 else:
                     os.environ[k] = v
-        self.listener = self.ctx.listen()
+        self.listener = self.ctx.listen("uv://127.0.0.1" if transport == "uv" else "shm://")
+        self.transport = transport
         child_env = dict(os.environ)
         child_env.update(env or {})
         child_env["PYTHONPATH"] = ROOT + os.pathsep + child_env.get("PYTHONPATH", "")
         self.proc = subprocess.Popen(
-            [sys.executable, "-m", "tensorpipe_amd.bench_peer", self.listener.url(), channels],
+            [sys.executable, "-m", "tensorpipe_amd.bench_peer", self.listener.url(self.transport), channels],
             env=child_env, cwd=ROOT)
         self.pipe = self.listener.accept(180000)
 
@@ -429,16 +430,18 @@ def bench_staged(iters=50, warmup=3, nbytes=256 * MIB):
     return out
 
 
-def bench_cpu_path():
+def bench_cpu_path(stock_wire_tcp=False):
     """configs[0] on this library's own CPU side (Pipe + shm transport + basic channel, two
-    processes): the control plane the device channels ride on, next to the reference's."""
+    processes): the control plane the device channels ride on, next to the reference's. With
+    `stock_wire_tcp` the same over the TCP transport with the reference's encodings on the wire:
+    what the route to unmodified peers costs."""
     import numpy as np
 
     from tensorpipe_amd import datagen
     from tensorpipe_amd import pipe as tp
 
     out = {}
-    peer = PeerRun("basic:0")
+    peer = PeerRun("basic:0", env={"TP_STOCK_WIRE": "1"}, transport="uv") if stock_wire_tcp else PeerRun("basic:0")
     try:
         for name, n, iters in (("4KiB", 4096, 2000), ("1MiB", MIB, 1000), ("64MiB", 64 * MIB, 40)):
             src = datagen.uniform_u8(datagen.SEED_BASE + 1, n)
@@ -635,6 +638,7 @@ LEGS = {
     "ipc_rtt": lambda: bench_ipc(iters=300, warmup=30, max_bytes=4096),
     "ipc_large": lambda: bench_ipc(iters=40, warmup=3, min_bytes=256 * MIB),
     "cpu_path": bench_cpu_path,
+    "cpu_path_stock_wire_tcp": lambda: bench_cpu_path(stock_wire_tcp=True),
     "cold_copy": bench_cold_copy,
 }
 
@@ -745,6 +749,8 @@ def main():
         extra["d2d_cold_source"] = extra_leg("cold_copy")
         log("[bench] this library's CPU path (shm + basic)")
         extra["cpu_path"] = extra_leg("cpu_path")
+        log("[bench] the same over TCP in the reference's wire format")
+        extra["cpu_path_stock_wire_tcp"] = extra_leg("cpu_path_stock_wire_tcp")
     log("[bench] CPU baseline (port of shm + basic)")
     cpu = cpu_baseline()
     extra["bench_wall_s"] = time.time() - t_start

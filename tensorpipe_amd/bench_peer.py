@@ -30,7 +30,8 @@ def main(url, channels):
 
     from tensorpipe_amd import pipe as tp
 
-    ctx = tp.Context("bench_peer", channels=channels)
+    # the transport is the one the URL names ("uv" is this library's TCP transport)
+    ctx = tp.Context("bench_peer", transports=url.split("://", 1)[0] + ":0", channels=channels)
     p = ctx.connect(url)
     while True:
         d = p.read_descriptor(timeout_ms=600000)

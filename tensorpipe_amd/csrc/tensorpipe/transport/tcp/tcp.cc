@@ -17,8 +17,12 @@
 #include <sys/socket.h>
 #include <unistd.h>
 
+#include <sched.h>
+
 #include <atomic>
 #include <cerrno>
+#include <chrono>
+#include <cstdlib>
 #include <cstring>
 #include <deque>
 #include <mutex>
@@ -205,8 +209,28 @@ class Reactor final : public std::enable_shared_from_this<Reactor> {
  private:
   void run() {
     std::vector<epoll_event> events(64);
+    // After an event the loop keeps asking without sleeping for a short while:
+    // in a ping-pong the next message is a few microseconds away, and a wake-up
+    // from epoll costs more than that (TP_TCP_SPIN_US, 0 = always sleep; no
+    // spinning where the process has fewer than four CPUs to run on).
+    const long spinUs = [] {
+      const char* e = std::getenv("TP_TCP_SPIN_US");
+      long v = e != nullptr ? std::atol(e) : 100;
+      cpu_set_t set;
+      CPU_ZERO(&set);
+      if (::sched_getaffinity(0, sizeof(set), &set) == 0 && CPU_COUNT(&set) < 4) {
+        v = 0;
+      }
+      return v;
+    }();
+    auto lastEvent = std::chrono::steady_clock::now() - std::chrono::seconds(1);
     while (!stop_) {
-      const int n = ::epoll_wait(epollFd_, events.data(), static_cast<int>(events.size()), -1);
+      const bool spin = spinUs > 0 &&
+          std::chrono::steady_clock::now() - lastEvent < std::chrono::microseconds(spinUs);
+      const int n = ::epoll_wait(epollFd_, events.data(), static_cast<int>(events.size()), spin ? 0 : -1);
+      if (n > 0) {
+        lastEvent = std::chrono::steady_clock::now();
+      }
       for (int i = 0; i < n; ++i) {
         if (events[i].data.ptr == nullptr) {
           uint64_t v;
