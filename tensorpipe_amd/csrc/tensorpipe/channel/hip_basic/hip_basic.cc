@@ -44,6 +44,7 @@
 #include <tensorpipe/common/cpu_buffer.h>
 #include <tensorpipe/common/hip_buffer.h>
 #include <tensorpipe/common/slot_allocator.h>
+#include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
 
 TP_AMD_NAMESPACE_BEGIN
@@ -393,6 +394,7 @@ class ChannelImpl final : public ChannelImplBase {
       peerMappedOurRing_ = r.u8() != 0;
       gotHelloAck_ = true;
     } else if (kind == kAck) {
+      TP_MARK("basic: acknowledgement arrived");
       const uint32_t count = r.u32();
       for (uint32_t i = 0; i < count; ++i) {
         const uint32_t slot = r.u32();
@@ -557,7 +559,9 @@ class ChannelImpl final : public ChannelImplBase {
       if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/true, *ev)) {
         return;
       }
+      TP_MARK("basic: chunk staged towards the host (launched)");
       watch(std::move(ev), [this, chunks{std::move(chunks)}] {
+        TP_MARK("basic: staging seen finished");
         for (auto& c : chunks) {
           c->ready = true;
         }
@@ -653,6 +657,7 @@ class ChannelImpl final : public ChannelImplBase {
         w.u64(n.second);
       }
       writeMessage(*controlConnection_, std::move(w.bytes()));
+      TP_MARK("basic: notification written");
       notifies.clear();
     };
     while (!sendQueue_.empty() && sendQueue_.front()->ready && !error_) {
@@ -757,6 +762,7 @@ class ChannelImpl final : public ChannelImplBase {
     const uint8_t* remote = remoteRing_ + static_cast<size_t>(slot) * remoteSlotBytes_;
     TP_VLOG(7) << "Channel " << id_ << " got notification for slot " << slot << " (" << len
                << " B)";
+    TP_MARK("basic: notification arrived");
     if (!isCpu(op->buffer)) {
       const HipBuffer hb = op->buffer.unwrap<HipBuffer>();
       ringPending_.push_back(RingItem{
@@ -831,8 +837,12 @@ class ChannelImpl final : public ChannelImplBase {
       if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/false, *ev)) {
         return;
       }
+      TP_MARK("basic: chunk copied from the ring (launched)");
       // The slots go back to the sender when the copy has read them.
-      watch(std::move(ev), [this, slots{std::move(slots)}] { ackSlots(slots); });
+      watch(std::move(ev), [this, slots{std::move(slots)}] {
+        TP_MARK("basic: ring copy seen finished");
+        ackSlots(slots);
+      });
       for (auto& op : ops) {
         chunkLanded(op); // enqueued on the caller's stream
       }
@@ -855,6 +865,7 @@ class ChannelImpl final : public ChannelImplBase {
       w.u32(slot);
     }
     writeMessage(*controlConnection_, std::move(w.bytes()));
+    TP_MARK("basic: acknowledgement written");
   }
 
   void startInnerRecv(const std::shared_ptr<Op>& op) {
