@@ -8,6 +8,7 @@
 #include <sys/socket.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <cerrno>
 #include <cstring>
 
@@ -142,9 +143,16 @@ bool CompatPipe::readFrame(int fd, char which, Bytes* out, std::string* error) {
   if (size > (uint64_t(1) << 32)) {
     return fail(error, "frame too large");
   }
-  out->resize(static_cast<size_t>(size));
-  if (size > 0 && !readAll(fd, out->data(), out->size())) {
-    return fail(error, "a frame stopped short");
+  // The buffer grows with what arrives, not with what the header announces.
+  out->clear();
+  constexpr size_t kStep = 1 << 20;
+  for (size_t have = 0; have < size;) {
+    const size_t n = static_cast<size_t>(std::min<uint64_t>(size - have, kStep));
+    out->resize(have + n);
+    if (!readAll(fd, out->data() + have, n)) {
+      return fail(error, "a frame stopped short");
+    }
+    have += n;
   }
   frames_.push_back(Frame{'r', which, *out});
   return true;

@@ -19,6 +19,7 @@
 
 #include <sched.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cerrno>
 #include <chrono>
@@ -43,6 +44,7 @@ namespace tcp {
 namespace {
 
 constexpr size_t kHeader = 8;
+constexpr uint64_t kGrowBytes = 1 << 20; // step in which the buffer of an unsized read grows
 
 class FdHandler {
  public:
@@ -240,14 +242,11 @@ class Reactor final : public std::enable_shared_from_this<Reactor> {
         // A handler may be destroyed by an earlier event of this batch: only
         // those still enrolled are called.
         FdHandler* h = static_cast<FdHandler*>(events[i].data.ptr);
-        std::shared_ptr<FdHandler> keep;
-        for (auto& l : live_) {
-          if (l.get() == h) {
-            keep = l;
-            break;
-          }
-        }
-        if (keep) {
+        // (the set orders its members by address: an owner-less pointer to the
+        // same address finds the member)
+        const auto it = live_.find(std::shared_ptr<FdHandler>(std::shared_ptr<FdHandler>(), h));
+        if (it != live_.end()) {
+          std::shared_ptr<FdHandler> keep = *it;
           keep->onEvents(events[i].events);
         }
       }
@@ -382,6 +381,16 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       if (events & (EPOLLRDHUP | EPOLLHUP | EPOLLERR)) {
         peerClosed_ = true; // what it sent before leaving is still delivered
       }
+      if (events & (EPOLLHUP | EPOLLERR)) {
+        // epoll reports these two whatever was asked for, and keeps reporting
+        // them: the socket leaves the set, and from here on reads and writes
+        // find out what the socket holds when they are posted.
+        hungUp_ = true;
+        if (registered_) {
+          reactor_->forget(fd_);
+          registered_ = false;
+        }
+      }
       pumpReads(); // with nobody reading, the hang-up is remembered and no longer asked about
     }
     if (!error_ && (events & EPOLLOUT)) {
@@ -453,7 +462,7 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
   }
 
   void updateInterest() {
-    if (fd_ < 0 || error_) {
+    if (fd_ < 0 || error_ || hungUp_) {
       return;
     }
     uint32_t want = 0;
@@ -520,17 +529,27 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
             fail(TP_CREATE_ERROR(ShortReadError, -1, static_cast<ssize_t>(messageLength_)));
             return;
           }
-          scratch_.resize(static_cast<size_t>(messageLength_));
+          scratch_.clear();
         }
       }
-      uint8_t* dst = op.exact ? op.ptr : scratch_.data();
       while (payloadDone_ < messageLength_) {
-        const ssize_t r = ::recv(fd_, dst + payloadDone_, static_cast<size_t>(messageLength_ - payloadDone_), 0);
+        uint64_t room = messageLength_ - payloadDone_;
+        if (!op.exact) {
+          // The length is the peer's word: the buffer grows with the bytes
+          // that really arrive, not with the announcement.
+          room = std::min<uint64_t>(room, kGrowBytes);
+          if (scratch_.size() < payloadDone_ + room) {
+            scratch_.resize(static_cast<size_t>(payloadDone_ + room));
+          }
+        }
+        uint8_t* dst = op.exact ? op.ptr : scratch_.data();
+        const ssize_t r = ::recv(fd_, dst + payloadDone_, static_cast<size_t>(room), 0);
         if (!absorb(r)) {
           return;
         }
         payloadDone_ += static_cast<size_t>(r);
       }
+      uint8_t* dst = op.exact ? op.ptr : scratch_.data();
       ReadOp finished = std::move(op);
       reads_.pop_front();
       headerDone_ = 0;
@@ -583,6 +602,9 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
         }
         if (r < 0) {
           if (errno == EAGAIN || errno == EWOULDBLOCK) {
+            if (hungUp_) {
+              fail(TP_CREATE_ERROR(EOFError)); // nobody will ever say "writable" again
+            }
             return;
           }
           if (errno == EINTR) {
@@ -633,6 +655,7 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
   bool connected_{false};
   bool registered_{false};
   bool peerClosed_{false};
+  bool hungUp_{false}; // EPOLLHUP or EPOLLERR was seen; the socket is out of the epoll set
   uint32_t interest_{0};
   Error error_;
   std::deque<ReadOp> reads_;
@@ -769,7 +792,7 @@ class ListenerImpl final : public FdHandler, public std::enable_shared_from_this
 
   void drain() {
     while (!acceptors_.empty() && !error_) {
-      const int fd = ::accept4(fd_, nullptr, nullptr, SOCK_CLOEXEC);
+      const int fd = ::accept4(fd_, nullptr, nullptr, SOCK_CLOEXEC | SOCK_NONBLOCK);
       if (fd < 0) {
         if (errno == EAGAIN || errno == EWOULDBLOCK || errno == EINTR || errno == ECONNABORTED) {
           return;

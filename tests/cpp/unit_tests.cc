@@ -768,6 +768,60 @@ static int runTcp() {
       }
     }
   }
+  // A peer that announces half a terabyte, sends three bytes and leaves: the read ends with
+  // an error, and no buffer of the announced size was ever asked for.
+  // Then a peer that resets the connection while nobody reads: the reactor must not spin on
+  // the hang-up (epoll keeps reporting it), and the next read learns of it.
+  for (int scenario = 0; scenario < 2; ++scenario) {
+    std::promise<std::shared_ptr<transport::Connection>> p4;
+    listener->accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p4.set_value(e ? nullptr : std::move(c)); });
+    const int fd = ::socket(AF_INET, SOCK_STREAM, 0);
+    sockaddr_in sa{};
+    sa.sin_family = AF_INET;
+    sa.sin_port = htons(static_cast<uint16_t>(std::atoi(addr.c_str() + addr.rfind(':') + 1)));
+    ::inet_pton(AF_INET, "127.0.0.1", &sa.sin_addr);
+    CHECK(::connect(fd, reinterpret_cast<sockaddr*>(&sa), sizeof(sa)) == 0);
+    auto acc4 = p4.get_future().get();
+    CHECK(acc4 != nullptr);
+    if (!acc4) {
+      ::close(fd);
+      continue;
+    }
+    if (scenario == 0) {
+      const uint8_t lie[8 + 3] = {0, 0, 0, 0, 0x80, 0, 0, 0, 'x', 'y', 'z'};
+      CHECK(::write(fd, lie, sizeof(lie)) == static_cast<ssize_t>(sizeof(lie)));
+      ::close(fd);
+    } else {
+      // one message arrives first, so that the reset finds the connection set up and idle
+      const uint8_t hello[8 + 2] = {2, 0, 0, 0, 0, 0, 0, 0, 'h', 'i'};
+      CHECK(::write(fd, hello, sizeof(hello)) == static_cast<ssize_t>(sizeof(hello)));
+      std::promise<bool> first;
+      acc4->read([&](const Error& e, const void*, size_t len) { first.set_value(!e && len == 2); });
+      CHECK(first.get_future().get());
+      linger lg{1, 0};
+      ::setsockopt(fd, SOL_SOCKET, SO_LINGER, &lg, sizeof(lg));
+      ::close(fd); // sends a reset
+      timespec before{}, after{};
+      ::clock_gettime(CLOCK_PROCESS_CPUTIME_ID, &before);
+      std::this_thread::sleep_for(std::chrono::milliseconds(400));
+      ::clock_gettime(CLOCK_PROCESS_CPUTIME_ID, &after);
+      const double cpuMs = (after.tv_sec - before.tv_sec) * 1e3 + (after.tv_nsec - before.tv_nsec) / 1e6;
+      if (cpuMs > 200) {
+        std::printf("FAIL: %.0f ms of CPU time in 400 ms of idling after a reset\n", cpuMs);
+        ++failed;
+      }
+    }
+    std::promise<bool> ended;
+    acc4->read([&](const Error& e, const void*, size_t) { ended.set_value(static_cast<bool>(e)); });
+    auto f = ended.get_future();
+    CHECK(f.wait_for(std::chrono::seconds(20)) == std::future_status::ready && f.get());
+    // a write on the dead connection fails too, it does not wait for ever
+    std::promise<bool> wrote;
+    const char byte = 'b';
+    acc4->write(&byte, 1, [&](const Error& e) { wrote.set_value(static_cast<bool>(e)); });
+    auto fw = wrote.get_future();
+    CHECK(fw.wait_for(std::chrono::seconds(20)) == std::future_status::ready && fw.get());
+  }
   // Closing this end fails what is pending on it.
   {
     std::promise<bool> pending;
