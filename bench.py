@@ -460,6 +460,34 @@ def bench_cpu_path(stock_wire_tcp=False):
     return out
 
 
+def bench_torch_rpc():
+    """torch.distributed.rpc round trips (PyTorch's own TensorPipe agent) with GPU tensors on this
+    library's channels, next to CPU tensors on the agent's stock channels."""
+    import socket
+
+    from tensorpipe_amd import torch_rpc as tp_rpc
+
+    if not os.path.exists(tp_rpc.library_path()):
+        return {"error": "libtensorpipe_amd_torch_rpc.so is not built"}
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+    ranks = [subprocess.Popen([sys.executable, "-m", "tensorpipe_amd.bench_rpc_peer", str(r), str(port)],
+                              stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, cwd=ROOT)
+             for r in (1, 0)]
+    try:
+        out, _ = ranks[1].communicate(timeout=240)
+        ranks[0].communicate(timeout=60)
+    finally:
+        for p in ranks:
+            if p.poll() is None:
+                p.kill()
+                p.wait()
+    if ranks[1].returncode != 0:
+        raise RuntimeError(f"rank 0 of the RPC group ended with {ranks[1].returncode}")
+    return json.loads(out.decode().strip().splitlines()[-1])
+
+
 def bench_cold_copy():
     """The headline loop sends the same source every step, and 64 MiB stays resident in the
     256 MiB Infinity Cache between steps. The same kernel over rotating source/destination pairs
@@ -640,6 +668,7 @@ LEGS = {
     "cpu_path": bench_cpu_path,
     "cpu_path_stock_wire_tcp": lambda: bench_cpu_path(stock_wire_tcp=True),
     "cold_copy": bench_cold_copy,
+    "torch_rpc": bench_torch_rpc,
 }
 
 
@@ -751,6 +780,8 @@ def main():
         extra["cpu_path"] = extra_leg("cpu_path")
         log("[bench] the same over TCP in the reference's wire format")
         extra["cpu_path_stock_wire_tcp"] = extra_leg("cpu_path_stock_wire_tcp")
+        log("[bench] torch.distributed.rpc with GPU tensors on these channels")
+        extra["torch_rpc"] = extra_leg("torch_rpc")
     log("[bench] CPU baseline (port of shm + basic)")
     cpu = cpu_baseline()
     extra["bench_wall_s"] = time.time() - t_start

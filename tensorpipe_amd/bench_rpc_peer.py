@@ -1,0 +1,65 @@
+"""One rank of the torch.distributed.rpc measurement of bench.py (leg "torch_rpc"):
+
+    python -m tensorpipe_amd.bench_rpc_peer <rank> <port>
+
+Two processes on the one GPU, PyTorch's own TensorPipe agent, this library's channels registered
+with it (tensorpipe_amd.torch_rpc). Rank 0 times rpc_sync(echo) round trips -- the tensor goes to
+the other process and comes back -- for GPU tensors, and for CPU tensors of the same sizes on the
+agent's stock channels, and prints one JSON line."""
+import json
+import os
+import sys
+import time
+
+import torch
+import torch.distributed.rpc as rpc
+
+from tensorpipe_amd import torch_rpc as tp_rpc
+
+
+def echo(t):
+    return t
+
+
+def main():
+    rank, port = int(sys.argv[1]), int(sys.argv[2])
+    tp_rpc.load()
+    os.environ["MASTER_ADDR"] = "127.0.0.1"
+    os.environ["MASTER_PORT"] = str(port)
+    opts = rpc.TensorPipeRpcBackendOptions(num_worker_threads=8, rpc_timeout=120)
+    opts.set_device_map(f"w{1 - rank}", {0: 0})
+    rpc.init_rpc(f"w{rank}", rank=rank, world_size=2, rpc_backend_options=opts)
+    out = {}
+    if rank == 0:
+        g = torch.Generator(device="cpu")
+        g.manual_seed(5)
+        for device in ("cuda:0", "cpu"):
+            legs = {}
+            for nbytes, iters in ((4096, 300), (1 << 20, 200), (64 << 20, 30)):
+                x = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g).to(device)
+                for _ in range(5):
+                    y = rpc.rpc_sync("w1", echo, args=(x,))
+                times = []
+                for _ in range(iters):
+                    t0 = time.perf_counter()
+                    y = rpc.rpc_sync("w1", echo, args=(x,))
+                    if device != "cpu":
+                        torch.cuda.current_stream().synchronize()  # the result is usable on this stream
+                    times.append(time.perf_counter() - t0)
+                times.sort()
+                p50 = times[len(times) // 2]
+                legs[str(nbytes)] = {
+                    "rtt_p50_us": p50 * 1e6,
+                    "payload_GBps": 2 * nbytes / p50 / 1e9,
+                    "byte_exact": bool(torch.equal(x, y)),
+                    "iters": iters,
+                }
+            out["gpu_tensors_hip_channels" if device != "cpu" else "cpu_tensors_stock_channels"] = legs
+        out["gpu_buffers_by_channel"] = tp_rpc.gpu_operations_by_channel()
+    rpc.shutdown()
+    if rank == 0:
+        print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

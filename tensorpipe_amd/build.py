@@ -2,6 +2,8 @@
 
   libtphip.so       HIP kernels + C ABI (include/tphip.h)           hipcc, gfx950
   libtpdatagen.so   seeded payload generator (include/tp_datagen.h)  gcc
+  libtensorpipe_amd.so            channels, transports, pipe, C harness API        g++
+  libtensorpipe_amd_torch_rpc.so  the channels registered with PyTorch's RPC agent g++
 """
 import os
 import subprocess
@@ -148,12 +150,36 @@ def build_stock_conformance():
     return True
 
 
+def build_torch_rpc_plugin():
+    """lib/libtensorpipe_amd_torch_rpc.so: registers hip_xth / hip_ipc / hip_basic and a GPU tensor
+    converter with the TensorPipe agent of the installed PyTorch (torch.distributed.rpc), whose ROCm
+    builds come without GPU channels. g++ against PyTorch's own headers (its TensorPipe's listed
+    first); skipped where they are not installed."""
+    found = stock_tensorpipe()
+    if found is None or not os.path.exists(
+            os.path.join(found[0], "torch", "csrc", "distributed", "rpc", "tensorpipe_agent.h")):
+        print("PyTorch's RPC agent headers not found: skipping libtensorpipe_amd_torch_rpc.so", flush=True)
+        return False
+    inc, lib = found
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    run(["g++", "-O1", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread",
+         "-DUSE_TENSORPIPE", "-DUSE_ROCM", "-D__HIP_PLATFORM_AMD__", "-DUSE_DISTRIBUTED", "-DUSE_RPC",
+         f"-I{inc}", f"-I{inc}/torch/csrc/api/include", f"-I{rocm}/include", f"-I{INCLUDE}", f"-I{CSRC}",
+         os.path.join(CSRC, "bridge", "torch_rpc_plugin.cc"), os.path.join(CSRC, "bridge", "stock_adapter.cc"),
+         "-o", os.path.join(LIB, "libtensorpipe_amd_torch_rpc.so"),
+         f"-L{LIB}", "-ltensorpipe_amd", "-ltphip",
+         f"-L{lib}", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+         "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{lib}"])
+    return True
+
+
 def build_all():
     build_tphip()
     build_datagen()
     build_host()
     build_cpp_tests()
     build_stock_conformance()
+    build_torch_rpc_plugin()
 
 
 if __name__ == "__main__":

@@ -113,9 +113,21 @@ class ConnectionFace final : public tpbridge::Connection {
   std::shared_ptr<tp::transport::Connection> inner_;
 };
 
+// GPU buffers handed over so far: all, and per channel kind.
 std::atomic<unsigned long long> gpuOperations{0};
+constexpr const char* kChannelNames[] = {"hip_xth", "hip_ipc", "hip_basic"};
+std::atomic<unsigned long long> gpuOperationsOf[3];
 
-tpbridge::BufferRef toRef(const tp::Buffer& buffer) {
+int channelKind(const std::string& name) {
+  for (int k = 0; k < 3; ++k) {
+    if (name == kChannelNames[k]) {
+      return k;
+    }
+  }
+  return -1;
+}
+
+tpbridge::BufferRef toRef(const tp::Buffer& buffer, int kind) {
   tpbridge::BufferRef ref;
   if (buffer.device().type == tp::kCpuDeviceType) {
     ref.ptr = buffer.unwrap<tp::CpuBuffer>().ptr;
@@ -123,6 +135,9 @@ tpbridge::BufferRef toRef(const tp::Buffer& buffer) {
   }
   const HipBuffer& hb = buffer.unwrap<HipBuffer>(); // throws on any other kind, as Buffer::unwrap does
   gpuOperations.fetch_add(1, std::memory_order_relaxed);
+  if (kind >= 0) {
+    gpuOperationsOf[kind].fetch_add(1, std::memory_order_relaxed);
+  }
   ref.onGpu = true;
   ref.ptr = hb.ptr;
   ref.stream = hb.stream;
@@ -131,14 +146,14 @@ tpbridge::BufferRef toRef(const tp::Buffer& buffer) {
 
 class ChannelAdapter final : public tp::channel::Channel {
  public:
-  explicit ChannelAdapter(std::shared_ptr<tpbridge::Channel> impl) : impl_(std::move(impl)) {}
+  ChannelAdapter(std::shared_ptr<tpbridge::Channel> impl, int kind) : impl_(std::move(impl)), kind_(kind) {}
   void send(tp::Buffer buffer, size_t length, tp::channel::TSendCallback callback) override {
-    impl_->send(toRef(buffer), length, [callback{std::move(callback)}](const std::string& e) {
+    impl_->send(toRef(buffer, kind_), length, [callback{std::move(callback)}](const std::string& e) {
       callback(toError(e));
     });
   }
   void recv(tp::Buffer buffer, size_t length, tp::channel::TRecvCallback callback) override {
-    impl_->recv(toRef(buffer), length, [callback{std::move(callback)}](const std::string& e) {
+    impl_->recv(toRef(buffer, kind_), length, [callback{std::move(callback)}](const std::string& e) {
       callback(toError(e));
     });
   }
@@ -151,11 +166,12 @@ class ChannelAdapter final : public tp::channel::Channel {
 
  private:
   std::shared_ptr<tpbridge::Channel> impl_;
+  const int kind_;
 };
 
 class ContextAdapter final : public tp::channel::Context {
  public:
-  explicit ContextAdapter(std::shared_ptr<tpbridge::Context> impl) : impl_(std::move(impl)) {
+  ContextAdapter(std::shared_ptr<tpbridge::Context> impl, int kind) : impl_(std::move(impl)), kind_(kind) {
     for (auto& d : impl_->deviceDescriptors()) {
       descriptors_[tp::Device{d.deviceType, d.deviceIndex}] = d.descriptor;
     }
@@ -180,7 +196,7 @@ class ContextAdapter final : public tp::channel::Context {
       faces.push_back(std::make_shared<ConnectionFace>(std::move(c)));
     }
     return std::make_shared<ChannelAdapter>(
-        impl_->createChannel(std::move(faces), endpoint == tp::channel::Endpoint::kListen));
+        impl_->createChannel(std::move(faces), endpoint == tp::channel::Endpoint::kListen), kind_);
   }
   void setId(std::string id) override {
     impl_->setId(std::move(id));
@@ -194,6 +210,7 @@ class ContextAdapter final : public tp::channel::Context {
 
  private:
   std::shared_ptr<tpbridge::Context> impl_;
+  const int kind_;
   std::unordered_map<tp::Device, std::string> descriptors_;
 };
 
@@ -203,12 +220,17 @@ unsigned long long gpuOperationsServed() {
   return gpuOperations.load(std::memory_order_relaxed);
 }
 
+unsigned long long gpuOperationsServedBy(const std::string& channelName) {
+  const int kind = channelKind(channelName);
+  return kind < 0 ? 0 : gpuOperationsOf[kind].load(std::memory_order_relaxed);
+}
+
 std::shared_ptr<::tensorpipe::channel::Context> createChannelContext(const std::string& channelName) {
   auto impl = tpbridge::createContext(channelName);
   if (!impl) {
     return nullptr;
   }
-  return std::make_shared<ContextAdapter>(std::move(impl));
+  return std::make_shared<ContextAdapter>(std::move(impl), channelKind(channelName));
 }
 
 } // namespace tensorpipe_amd_bridge

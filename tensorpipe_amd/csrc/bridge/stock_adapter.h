@@ -31,6 +31,8 @@ struct HipBuffer {
 // adapter so far (sends plus receives): lets a test prove which channel a
 // tensor travelled on.
 unsigned long long gpuOperationsServed();
+// The same count for one kind of channel ("hip_xth", "hip_ipc", "hip_basic").
+unsigned long long gpuOperationsServedBy(const std::string& channelName);
 
 // channelName: "hip_xth", "hip_ipc" or "hip_basic".
 std::shared_ptr<::tensorpipe::channel::Context> createChannelContext(const std::string& channelName);

@@ -1,0 +1,53 @@
+"""torch.distributed.rpc with this library's module loaded, on a machine without a GPU: the hip_*
+channels report themselves not viable, the agent leaves them out, and CPU tensors travel as
+before. (The GPU cases are in test_torch_rpc_gpu.py.)"""
+import os
+import socket
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CASES = os.path.join(ROOT, "tests", "torch_rpc_cases.py")
+PLUGIN = os.path.join(ROOT, "tensorpipe_amd", "lib", "libtensorpipe_amd_torch_rpc.so")
+
+
+def free_port():
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        return s.getsockname()[1]
+
+
+def run_group(mode, timeout=240):
+    if not os.path.exists(PLUGIN):
+        pytest.skip("libtensorpipe_amd_torch_rpc.so is not built (no RPC agent headers at build time)")
+    port = free_port()
+    print(f"running torch_rpc_cases.py, mode {mode}, port {port}", flush=True)
+    ranks = [
+        subprocess.Popen([sys.executable, "-u", CASES, str(rank), str(port), mode],
+                         stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        for rank in range(2)
+    ]
+    outs = []
+    try:
+        for p in ranks:
+            outs.append(p.communicate(timeout=timeout))
+    finally:
+        for p in ranks:
+            if p.poll() is None:
+                p.kill()
+                p.communicate()
+    text = outs[0][0]
+    results = [line for line in text.splitlines() if line.startswith("RESULT ")]
+    tail = "\n".join(f"--- rank {i}\n{o[-1500:]}\n{e[-2500:]}" for i, (o, e) in enumerate(outs))
+    assert results, f"no result line\n{tail}"
+    bad = [line for line in results if line.split()[2] != "OK"]
+    assert not bad and all(p.returncode == 0 for p in ranks), "\n".join(bad) + "\n" + tail
+    return results, [o for o, _ in outs]
+
+
+def test_cpu_rpc_is_undisturbed_by_the_module():
+    results, _ = run_group("cpu")
+    names = {line.split()[1] for line in results}
+    assert {"echo_0", "echo_67108864", "mixed_echo", "in_flight_24", "callee_calls_back", "route"} <= names

@@ -1,0 +1,22 @@
+"""torch.distributed.rpc moving GPU tensors between two processes (and to oneself) on this
+library's channels, registered with PyTorch's own TensorPipe agent by
+tensorpipe_amd/csrc/bridge/torch_rpc_plugin.cc: the counterpart of the registration the reference's
+CUDA channels get in PyTorch's CUDA builds. Every tensor is compared bit for bit with what was sent,
+and the module's counter proves that GPU buffers went through the hip_* channels."""
+import pytest
+
+from tests.test_torch_rpc import run_group
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("mode", ["gpu", "staged"])
+def test_gpu_tensors_over_rpc(mode):
+    results, outs = run_group(mode)
+    names = {line.split()[1] for line in results}
+    assert {"echo_0", "echo_4097", "echo_67108864", "add_one", "checksum_at_callee", "mixed_devices_arrive_in_place",
+            "mixed_echo", "in_flight_24", "view", "rref_to_here", "to_self", "to_self_used_the_channels",
+            "channel_chosen", "callee_calls_back", "route"} <= names
+    for rank, out in enumerate(outs):
+        counts = [int(line.split()[3]) for line in out.splitlines() if line.startswith(f"RANK {rank} ")]
+        assert counts and counts[0] > 50, f"rank {rank}: {counts}"
