@@ -19,7 +19,7 @@ def free_port():
         return s.getsockname()[1]
 
 
-def run_group(mode, timeout=240):
+def run_group(mode, timeout=240, rank1_exit=0):
     if not os.path.exists(PLUGIN):
         pytest.skip("libtensorpipe_amd_torch_rpc.so is not built (no RPC agent headers at build time)")
     port = free_port()
@@ -43,7 +43,8 @@ def run_group(mode, timeout=240):
     tail = "\n".join(f"--- rank {i}\n{o[-1500:]}\n{e[-2500:]}" for i, (o, e) in enumerate(outs))
     assert results, f"no result line\n{tail}"
     bad = [line for line in results if line.split()[2] != "OK"]
-    assert not bad and all(p.returncode == 0 for p in ranks), "\n".join(bad) + "\n" + tail
+    codes = [p.returncode for p in ranks]
+    assert not bad and codes == [0, rank1_exit], "\n".join(bad) + f"\nexit codes {codes}\n" + tail
     return results, [o for o, _ in outs]
 
 
@@ -51,3 +52,8 @@ def test_cpu_rpc_is_undisturbed_by_the_module():
     results, _ = run_group("cpu")
     names = {line.split()[1] for line in results}
     assert {"echo_0", "echo_67108864", "mixed_echo", "in_flight_24", "callee_calls_back", "route"} <= names
+
+
+def test_cpu_calls_fail_when_the_peer_dies():
+    results, _ = run_group("cpu_peer_dies", timeout=120, rank1_exit=3)
+    assert {"before", "calls_fail_instead_of_hanging"} <= {line.split()[1] for line in results}

@@ -20,3 +20,10 @@ def test_gpu_tensors_over_rpc(mode):
     for rank, out in enumerate(outs):
         counts = [int(line.split()[3]) for line in out.splitlines() if line.startswith(f"RANK {rank} ")]
         assert counts and counts[0] > 50, f"rank {rank}: {counts}"
+
+
+def test_calls_with_gpu_tensors_fail_when_the_peer_dies():
+    """The other process ends abruptly with GPU tensors of several calls in flight on hip_ipc: every
+    pending call reports an error, nothing waits for ever."""
+    results, _ = run_group("peer_dies", timeout=120, rank1_exit=3)
+    assert {"before", "calls_fail_instead_of_hanging"} <= {line.split()[1] for line in results}

@@ -6,6 +6,9 @@ library's channels (tensorpipe_amd.torch_rpc). Started by tests/test_torch_rpc*.
 mode: "cpu"    no device map, CPU tensors only (the module loaded must not disturb the agent)
       "gpu"    device maps 0 -> 0 both ways and to oneself; all three channels registered
       "staged" as "gpu" with the agent's channel list cut to hip_basic + basic
+      "peer_dies" / "cpu_peer_dies"   rank 1 ends abruptly inside a call that brought it a (GPU)
+               tensor while more calls with tensors are on their way: rank 0's calls must fail,
+               none may hang
 
 Rank 0 drives the cases and prints "RESULT <case> OK|FAIL ..." lines; both ranks print how many GPU
 buffers went through the hip_* channels. What the reference's agent tests for its CUDA channels
@@ -51,6 +54,10 @@ def make_on_gpu(nbytes, seed):
     return seeded(nbytes, seed, "cuda:0")
 
 
+def leave_abruptly(t):
+    os._exit(3)
+
+
 def checksum(t):
     # computed where the tensor arrived, on the stream the agent made current
     return int(t.to(torch.int64).sum().item())
@@ -58,7 +65,7 @@ def checksum(t):
 
 def main():
     rank, port, mode = int(sys.argv[1]), int(sys.argv[2]), sys.argv[3]
-    gpu = mode in ("gpu", "staged")
+    gpu = mode in ("gpu", "staged", "peer_dies")
     tp_rpc.load()
     os.environ["MASTER_ADDR"] = "127.0.0.1"
     os.environ["MASTER_PORT"] = str(port)
@@ -77,6 +84,33 @@ def main():
         failures += 0 if ok else 1
         print(f"RESULT {name} {'OK' if ok else 'FAIL'} {note}", flush=True)
 
+    if mode.endswith("peer_dies"):
+        if rank == 0:
+            dev = "cuda:0" if gpu else "cpu"
+            x = seeded(3 << 20, 21, dev)
+            ok = rpc.rpc_sync("w1", checksum, args=(x,)) == int(x.to(torch.int64).sum().item())
+            result("before", ok)
+            futs = [rpc.rpc_async("w1", leave_abruptly if i == 2 else echo, args=(seeded((1 << 20) + i, 30 + i, dev),))
+                    for i in range(8)]
+            failed = 0
+            for f in futs:
+                try:
+                    f.wait()
+                except RuntimeError:
+                    failed += 1
+            # the calls behind the fatal one fail; those ahead of it may have been answered
+            result("calls_fail_instead_of_hanging", failed >= 6, f"{failed} of 8 failed")
+            print("RESULT route OK", flush=True)
+            sys.stdout.flush()
+            try:
+                rpc.shutdown(graceful=False)
+            finally:
+                os._exit(1 if failures else 0)
+        else:
+            import time
+
+            time.sleep(60)  # ended from inside leave_abruptly long before
+            os._exit(4)
     if rank == 0:
         dev = "cuda:0" if gpu else "cpu"
         # a tensor there and back, sizes from nothing to 64 MiB, odd ones among them
