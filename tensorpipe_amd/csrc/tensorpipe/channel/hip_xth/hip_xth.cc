@@ -11,6 +11,9 @@
 // made a dependency of the copy (event + stream wait); an idle one costs one
 // query. A poller thread watches an event recorded behind the copy; when it
 // has completed the recv callback fires and the completion message goes out.
+// Receives that become ready while a copy of the channel is still running
+// share the next launch (launchReady below): a caller that moves a message
+// tensor by tensor still gets few launches.
 //
 // Same wire protocol as tensorpipe/channel/cuda_xth/channel_impl.cc:30-36,
 // 96-315 (descriptor one way, empty completion back). Differences, all for
@@ -29,7 +32,6 @@
 #include <tensorpipe/channel/channel_base.h>
 #include <tensorpipe/channel/hip_common.h>
 #include <tensorpipe/common/hip_buffer.h>
-#include <tensorpipe/common/optional.h>
 #include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
 
@@ -119,6 +121,9 @@ class ChannelImpl final : public ChannelImplBase {
     for (auto& op : sends) {
       finishSend(op);
     }
+    toLaunch_.clear();
+    toLaunchBytes_ = 0;
+    decodedInQueue_ = 0;
     auto recvs = std::move(recvOps_);
     recvOps_.clear();
     for (auto& op : recvs) {
@@ -139,6 +144,14 @@ class ChannelImpl final : public ChannelImplBase {
     uint64_t seq;
     TRecvCallback cb;
     std::vector<BatchEntry> entries; // non-empty ones only
+    // From the descriptor: where each entry comes from, which streams are involved.
+    struct Piece {
+      StreamRef src;
+      StreamRef dst;
+      tphip_copy_desc copy;
+    };
+    std::vector<Piece> pieces;
+    uint64_t bytes{0};
     size_t copiesInFlight{0};
     bool copied{false}; // every copy of the op has completed
     bool done{false};
@@ -223,7 +236,8 @@ class ChannelImpl final : public ChannelImplBase {
     }));
   }
 
-  // One launch per source stream (normally one in total), on that stream.
+  // Reads where the op's tensors come from, then launches -- at once, or
+  // together with the ops behind it (see launchReady).
   void copyFromDescriptor(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
     WireReader r(bytes.data(), bytes.size());
     const uint32_t n = r.u32();
@@ -231,50 +245,97 @@ class ChannelImpl final : public ChannelImplBase {
       setError(TP_CREATE_ERROR(ShortReadError, static_cast<ssize_t>(op->entries.size()), n));
       return;
     }
+    {
+      StageScope decodeTimer(Stage::kXthDecode);
+      try {
+        op->pieces.reserve(n);
+        for (uint32_t i = 0; i < n; ++i) {
+          StreamRef srcRef;
+          srcRef.stream = reinterpret_cast<void*>(r.u64());
+          srcRef.device = static_cast<int>(r.u32());
+          const void* src = reinterpret_cast<const void*>(r.u64());
+          const uint64_t len = r.u64();
+          if (!r.ok() || len != op->entries[i].length) {
+            setError(TP_CREATE_ERROR(
+                ShortReadError, static_cast<ssize_t>(op->entries[i].length), static_cast<ssize_t>(len)));
+            return;
+          }
+          const HipBuffer& hb = op->entries[i].buffer.unwrap<HipBuffer>();
+          StreamRef dstRef{hb.stream, hipDeviceForPointer(hb.ptr)};
+          TP_THROW_ASSERT_IF(dstRef.device < 0);
+          op->pieces.push_back(RecvOp::Piece{srcRef, dstRef, tphip_copy_desc{src, hb.ptr, len}});
+          op->bytes += len;
+        }
+      } catch (const std::exception& ex) {
+        TP_LOG_WARNING() << "Channel " << id_ << " copy failed: " << ex.what();
+        setError(TP_CREATE_ERROR(HipError, "hip_xth copy", TPHIP_ERR_INVALID_ARG));
+        return;
+      }
+    }
+    TP_MARK("xth: descriptor decoded");
+    ++decodedInQueue_;
+    toLaunch_.push_back(op);
+    toLaunchBytes_ += op->bytes;
+    launchReady(/*copyFinished=*/false);
+  }
+
+  // Launches the ops whose descriptors are in, all of them in one kernel per
+  // source stream. A caller that hands over a message tensor by tensor (a
+  // stock pipe does: one send and one recv per tensor) would otherwise pay one
+  // launch, one event and one poll per tensor, 4-5 us of host time each, for
+  // copies that take the GPU a microsecond. So while a copy of this channel is
+  // still running and more receives are posted than descriptors have come in,
+  // small ops wait and ride together on the next launch, which goes out when
+  // the running copy ends, when every posted receive has its descriptor, or
+  // when enough has gathered. Nothing waits while the GPU has none of this
+  // channel's work, and large copies never wait: for them the launch is
+  // noise, and queueing them behind the running one keeps the GPU fed.
+  void launchReady(bool copyFinished) {
+    if (toLaunch_.empty() || error_) {
+      return;
+    }
+    const bool moreComing = recvOps_.size() > decodedInQueue_;
+    if (!copyFinished && launchesInFlight_ > 0 && moreComing && toLaunchBytes_ < kGatherBytes &&
+        toLaunch_.size() < kGatherOps) {
+      return;
+    }
     struct Group {
       StreamRef src;
       std::vector<StreamRef> dstStreams;
       std::vector<tphip_copy_desc> table;
+      std::vector<std::shared_ptr<RecvOp>> ops;
     };
     std::vector<Group> groups;
-    optional<StageScope> decodeTimer;
-    decodeTimer.emplace(Stage::kXthDecode);
-    try {
-      for (uint32_t i = 0; i < n; ++i) {
-        StreamRef srcRef;
-        srcRef.stream = reinterpret_cast<void*>(r.u64());
-        srcRef.device = static_cast<int>(r.u32());
-        const void* src = reinterpret_cast<const void*>(r.u64());
-        const uint64_t len = r.u64();
-        if (!r.ok() || len != op->entries[i].length) {
-          setError(TP_CREATE_ERROR(
-              ShortReadError, static_cast<ssize_t>(op->entries[i].length), static_cast<ssize_t>(len)));
-          return;
-        }
-        const HipBuffer& hb = op->entries[i].buffer.unwrap<HipBuffer>();
-        StreamRef dstRef{hb.stream, hipDeviceForPointer(hb.ptr)};
-        TP_THROW_ASSERT_IF(dstRef.device < 0);
+    auto ops = std::move(toLaunch_);
+    toLaunch_.clear();
+    toLaunchBytes_ = 0;
+    for (auto& op : ops) {
+      for (auto& piece : op->pieces) {
         Group* g = nullptr;
         for (auto& cand : groups) {
-          if (cand.src == srcRef) {
+          if (cand.src == piece.src) {
             g = &cand;
           }
         }
         if (g == nullptr) {
-          groups.push_back(Group{srcRef, {}, {}});
+          groups.push_back(Group{piece.src, {}, {}, {}});
           g = &groups.back();
         }
         bool known = false;
         for (auto& d : g->dstStreams) {
-          known |= d == dstRef;
+          known |= d == piece.dst;
         }
-        if (!known && !(dstRef == srcRef)) {
-          g->dstStreams.push_back(dstRef);
+        if (!known && !(piece.dst == piece.src)) {
+          g->dstStreams.push_back(piece.dst);
         }
-        g->table.push_back(tphip_copy_desc{src, hb.ptr, len});
+        g->table.push_back(piece.copy);
+        if (g->ops.empty() || g->ops.back() != op) {
+          g->ops.push_back(op);
+        }
       }
-      decodeTimer.reset();
-      TP_MARK("xth: descriptor decoded");
+      op->pieces.clear();
+    }
+    try {
       for (auto& g : groups) {
         StageScope launchTimer(Stage::kXthLaunch);
         // The copy may only touch a destination once everything the receiver
@@ -287,7 +348,8 @@ class ChannelImpl final : public ChannelImplBase {
             xctx_->events.put(std::move(ev)); // the wait captured the record
           }
         }
-        TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << op->seq << ")";
+        TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << g.ops.front()->seq << " to #"
+                   << g.ops.back()->seq << ")";
         TP_MARK("xth: destination streams checked");
         auto done = xctx_->events.get(g.src.device);
         const bool onKernel =
@@ -297,35 +359,44 @@ class ChannelImpl final : public ChannelImplBase {
         if (onKernel) {
           launch = xctx_->markers.launched(g.src.device, g.src.stream, xctx_->events);
         }
-        TP_VLOG(9) << "Channel " << id_ << " launched the copy (#" << op->seq << ")";
         TP_MARK("xth: copy launched");
         auto self = shared_from_this();
-        // Counted per launch: if a later launch of this op fails, the error
-        // path still waits for exactly the copies that are running.
-        ++op->copiesInFlight;
+        // Counted per launch: if a later launch fails, the error path still
+        // waits for exactly the copies that are running.
+        for (auto& op : g.ops) {
+          ++op->copiesInFlight;
+        }
+        ++launchesInFlight_;
         const StreamRef src = g.src;
-        xctx_->poller.watch(std::move(done), &xctx_->events, [this, self, op, src, onKernel, launch](
-                                                                 const Error& error) {
-          TP_MARK("xth: copy seen finished");
-          if (onKernel) {
-            // before anybody hears of the completion: the stream is still the sender's to keep
-            xctx_->markers.finished(src.device, src.stream, launch, xctx_->events);
-          }
-          ctx_->defer([this, self, op, error] {
-            setError(error);
-            if (--op->copiesInFlight > 0) {
-              return;
-            }
-            if (error_) {
-              finishRecv(op); // no longer in recvOps_: the error path left it to us
-              return;
-            }
-            TP_VLOG(6) << "Channel " << id_ << " done copying payload (#" << op->seq << ")";
-            op->copied = true;
-            TP_MARK("xth: recv callback due");
-            flushRecvs();
-          });
-        });
+        xctx_->poller.watch(
+            std::move(done), &xctx_->events,
+            [this, self, carried{std::move(g.ops)}, src, onKernel, launch](const Error& error) {
+              TP_MARK("xth: copy seen finished");
+              if (onKernel) {
+                // before anybody hears of the completion: the stream is still the sender's to keep
+                xctx_->markers.finished(src.device, src.stream, launch, xctx_->events);
+              }
+              ctx_->defer([this, self, carried, error] {
+                setError(error);
+                --launchesInFlight_;
+                for (auto& op : carried) {
+                  if (--op->copiesInFlight > 0) {
+                    continue;
+                  }
+                  if (error_) {
+                    finishRecv(op); // no longer in recvOps_: the error path left it to us
+                    continue;
+                  }
+                  TP_VLOG(6) << "Channel " << id_ << " done copying payload (#" << op->seq << ")";
+                  op->copied = true;
+                }
+                if (!error_) {
+                  TP_MARK("xth: recv callback due");
+                  launchReady(/*copyFinished=*/true); // what gathered meanwhile goes first: the GPU is idle
+                  flushRecvs();
+                }
+              });
+            });
       }
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " copy failed: " << ex.what();
@@ -344,6 +415,7 @@ class ChannelImpl final : public ChannelImplBase {
     while (!recvOps_.empty() && recvOps_.front()->copied && !error_) {
       auto op = recvOps_.front();
       recvOps_.pop_front();
+      --decodedInQueue_;
       // The receiver's callback first, the completion after it: the sender's
       // callback then is the last one of a transfer and runs on the sender's own
       // loop, where a caller that chains its next write from the callbacks
@@ -396,6 +468,13 @@ class ChannelImpl final : public ChannelImplBase {
   std::shared_ptr<transport::Connection> completionConnection_;
   std::deque<std::shared_ptr<SendOp>> sendOps_;
   std::deque<std::shared_ptr<RecvOp>> recvOps_;
+  // Decoded, not yet launched (a run at the tail of the decoded part of recvOps_).
+  std::vector<std::shared_ptr<RecvOp>> toLaunch_;
+  uint64_t toLaunchBytes_{0};
+  size_t launchesInFlight_{0};
+  size_t decodedInQueue_{0}; // members of recvOps_ whose descriptor has come in (they sit at its front)
+  static constexpr uint64_t kGatherBytes = 8u << 20;
+  static constexpr size_t kGatherOps = 256;
 };
 
 class XthChannel final : public ChannelHandle<ChannelImpl>, public BatchedChannel {

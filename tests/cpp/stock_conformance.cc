@@ -432,7 +432,7 @@ static int unmodifiedPeer() {
 // Timing, not a test: one GPU tensor of `bytes` bytes per message over hip_xth
 // between two stock contexts of this process, one message at a time, the next
 // write issued by the thread that saw both callbacks of the previous one.
-static int timeSameProcess(size_t bytes, int iters) {
+static int timeSameProcess(size_t bytes, int iters, size_t pieces) {
   const std::string addr = "shm://tpamd_conf4_" + std::to_string(::getpid());
   auto server = makeContext("server", {"hip_xth"});
   auto client = makeContext("client", {"hip_xth"});
@@ -447,20 +447,26 @@ static int timeSameProcess(size_t bytes, int iters) {
   for (int it = 0; it < iters + 10 && problem.empty(); ++it) {
     std::promise<std::string> wrote, read;
     const auto t0 = std::chrono::steady_clock::now();
+    // the bytes as `pieces` tensors of one message, cut at odd places
     Message m;
-    Message::Tensor t;
-    t.buffer = HipBuffer{src.dev, src.stream, 0};
-    t.length = bytes;
-    t.targetDevice = Device{"cuda", 0};
-    m.tensors.push_back(std::move(t));
+    const size_t each = bytes / pieces;
+    for (size_t k = 0; k < pieces; ++k) {
+      Message::Tensor t;
+      t.buffer = HipBuffer{static_cast<char*>(src.dev) + k * each, src.stream, 0};
+      t.length = k + 1 == pieces ? bytes - k * each : each;
+      t.targetDevice = Device{"cuda", 0};
+      m.tensors.push_back(std::move(t));
+    }
     spipe->readDescriptor([&](const Error& e, Descriptor d) {
-      if (e || d.tensors.size() != 1) {
+      if (e || d.tensors.size() != pieces) {
         read.set_value("readDescriptor failed");
         return;
       }
       Allocation a;
-      a.tensors.resize(1);
-      a.tensors[0].buffer = HipBuffer{dst.dev, dst.stream, 0};
+      a.tensors.resize(pieces);
+      for (size_t k = 0; k < pieces; ++k) {
+        a.tensors[k].buffer = HipBuffer{static_cast<char*>(dst.dev) + k * each, dst.stream, 0};
+      }
       spipe->read(std::move(a), [&read](const Error& e2) { read.set_value(e2 ? e2.what() : std::string()); });
     });
     cpipe->write(std::move(m), [&wrote](const Error& e) { wrote.set_value(e ? e.what() : std::string()); });
@@ -480,8 +486,8 @@ static int timeSameProcess(size_t bytes, int iters) {
   std::sort(us.begin(), us.end());
   if (problem.empty() && !us.empty()) {
     const double p50 = us[us.size() / 2];
-    std::printf("TIMING hip_xth in stock contexts: %zu bytes, %d messages, p50 %.1f us per message, %.1f GB/s payload\n",
-                bytes, iters, p50, static_cast<double>(bytes) / p50 / 1e3);
+    std::printf("TIMING hip_xth in stock contexts: %zu bytes in %zu tensors, %d messages, p50 %.1f us per message, %.1f GB/s payload\n",
+                bytes, pieces, iters, p50, static_cast<double>(bytes) / p50 / 1e3);
   }
   report("timing_hip_xth_in_stock_context", problem);
   cpipe.reset();
@@ -713,9 +719,15 @@ int main(int argc, char** argv) {
   if (argc == 3 && std::strcmp(argv[1], "native_peer") == 0) {
     return std::strcmp(argv[2], "hip_xth") == 0 ? nativePeerSameProcess() : nativePeerTwoProcess(argv[2]);
   }
-  if (argc == 4 && std::strcmp(argv[1], "time_same_process") == 0) {
-    return timeSameProcess(std::strtoull(argv[2], nullptr, 10), std::atoi(argv[3]));
+  if ((argc == 4 || argc == 5) && std::strcmp(argv[1], "time_same_process") == 0) {
+    const size_t pieces = argc == 5 ? std::strtoull(argv[4], nullptr, 10) : 1;
+    const size_t bytes = std::strtoull(argv[2], nullptr, 10);
+    if (pieces == 0 || bytes < pieces) {
+      std::fprintf(stderr, "need at least one byte per tensor\n");
+      return 2;
+    }
+    return timeSameProcess(bytes, std::atoi(argv[3]), pieces);
   }
-  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic | time_same_process <bytes> <messages>\n", argv[0]);
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic | time_same_process <bytes> <messages> [tensors per message]\n", argv[0]);
   return 2;
 }
