@@ -246,6 +246,56 @@ std::vector<Case> makeCases() {
          }});
   }
 
+  // Many small tensors of different sizes, each with bytes of its own, all
+  // posted before any is awaited: a channel that lets ready receives share a
+  // launch (or a unit) must still put every byte where it belongs.
+  {
+    auto sizeOf = [](int k) { return static_cast<size_t>(1 + (k * 7919) % 40000 + (k % 5 == 0 ? 70000 : 0)); };
+    auto pattern = [sizeOf](int k) {
+      std::vector<uint8_t> v(sizeOf(k));
+      for (size_t j = 0; j < v.size(); ++j) {
+        v[j] = static_cast<uint8_t>((j * 13 + static_cast<size_t>(k) * 101 + (j >> 9)) % 253);
+      }
+      return v;
+    };
+    constexpr int kTensors = 160;
+    cases.push_back(
+        {"ManySmallTensorsEachItsOwn",
+         [pattern](Endpoint& ep) {
+           auto o = open(ep);
+           std::vector<std::unique_ptr<Data>> ds;
+           std::vector<std::future<Error>> fs;
+           for (int k = 0; k < kTensors; ++k) {
+             ds.push_back(makeData(gGpu, pattern(k)));
+           }
+           for (int k = 0; k < kTensors; ++k) {
+             fs.push_back(sendF(*o->ch, ds[k]->buffer(), ds[k]->size()));
+           }
+           for (auto& f : fs) {
+             EXPECT_OK(waitFor(f, "send"));
+           }
+           ep.barrier();
+         },
+         [pattern, sizeOf](Endpoint& ep) {
+           auto o = open(ep);
+           std::vector<std::unique_ptr<Data>> ds;
+           std::vector<std::future<Error>> fs;
+           for (int k = 0; k < kTensors; ++k) {
+             ds.push_back(makeData(gGpu, sizeOf(k)));
+           }
+           for (int k = 0; k < kTensors; ++k) {
+             fs.push_back(recvF(*o->ch, ds[k]->buffer(), ds[k]->size()));
+           }
+           for (auto& f : fs) {
+             EXPECT_OK(waitFor(f, "recv"));
+           }
+           for (int k = 0; k < kTensors; ++k) {
+             expectBytes(*ds[k], pattern(k), "tensor");
+           }
+           ep.barrier();
+         }});
+  }
+
   // channel_test.cc:191-259: one send and one recv in flight on each side.
   auto bothWays = [](Endpoint& ep) {
     auto o = open(ep);
