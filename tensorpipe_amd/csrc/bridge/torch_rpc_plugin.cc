@@ -19,7 +19,6 @@
 // Compiled against the HOST's TensorPipe headers (the ones PyTorch installs),
 // never against this library's.
 #include <memory>
-#include <stdexcept>
 
 #include <ATen/hip/impl/HIPCachingAllocatorMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
@@ -90,16 +89,17 @@ std::unique_ptr<rpc::ChannelRegistration> makeHipBasic() {
   return makeChannel("hip_basic", 0);
 }
 
-// A build that already converts CUDA tensors (one with the reference's CUDA
+// A build that already converts GPU tensors (one with the reference's CUDA
 // channels compiled in) wraps them in its own buffer type, which these
-// channels do not take: loading this module there is a mistake worth a loud
-// error, not a silent replacement.
+// channels do not take. Its converter is left in place and the module reports
+// the conflict through tensorpipe_amd_torch_rpc_status(): an exception out of
+// a static initialiser would end the process inside dlopen.
+bool converterConflict = false;
 struct ConverterRegistration {
   ConverterRegistration() {
     if (rpc::getDeviceTypeConverter(c10::DeviceType::CUDA) != nullptr) {
-      throw std::runtime_error(
-          "tensorpipe_amd: this PyTorch already has a TensorPipe converter for GPU tensors; "
-          "the hip_* channels are meant for builds without one");
+      converterConflict = true;
+      return;
     }
     static rpc::TensorpipeDeviceTypeConverterRegistrar registrar(c10::DeviceType::CUDA, new GpuTensorConverter());
   }
@@ -116,6 +116,12 @@ C10_REGISTER_CREATOR(TensorPipeChannelRegistry, hip_xth, ::tensorpipe_amd_bridge
 C10_REGISTER_CREATOR(TensorPipeChannelRegistry, hip_ipc, ::tensorpipe_amd_bridge::makeHipIpc)
 C10_REGISTER_CREATOR(TensorPipeChannelRegistry, hip_basic, ::tensorpipe_amd_bridge::makeHipBasic)
 } // namespace torch::distributed::rpc
+
+// 0: channels and converter registered. 1: this PyTorch already had a converter
+// for GPU tensors; the module must not be used with it.
+extern "C" int tensorpipe_amd_torch_rpc_status() {
+  return tensorpipe_amd_bridge::converterConflict ? 1 : 0;
+}
 
 // For a caller that wants proof of the route taken: GPU buffers handed to
 // this library's channels by this process so far.

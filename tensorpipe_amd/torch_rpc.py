@@ -39,7 +39,12 @@ def load():
         import torch
 
         torch.ops.load_library(_LIB)
-        _loaded = ctypes.CDLL(_LIB)
+        lib = ctypes.CDLL(_LIB)
+        if lib.tensorpipe_amd_torch_rpc_status() != 0:
+            raise RuntimeError(
+                "this PyTorch already has a TensorPipe converter for GPU tensors (a build with its own GPU "
+                "channels); the hip_* channels are meant for builds without one")
+        _loaded = lib
         _loaded.tensorpipe_amd_torch_rpc_gpu_operations.restype = ctypes.c_ulonglong
         _loaded.tensorpipe_amd_torch_rpc_gpu_operations_of.restype = ctypes.c_ulonglong
         _loaded.tensorpipe_amd_torch_rpc_gpu_operations_of.argtypes = [ctypes.c_char_p]
