@@ -19,7 +19,7 @@ def free_port():
         return s.getsockname()[1]
 
 
-def run_group(mode, timeout=240, rank1_exit=0):
+def run_group(mode, timeout=240, rank1_exit=0, world=2):
     if not os.path.exists(PLUGIN):
         pytest.skip("libtensorpipe_amd_torch_rpc.so is not built (no RPC agent headers at build time)")
     port = free_port()
@@ -27,7 +27,7 @@ def run_group(mode, timeout=240, rank1_exit=0):
     ranks = [
         subprocess.Popen([sys.executable, "-u", CASES, str(rank), str(port), mode],
                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
-        for rank in range(2)
+        for rank in range(world)
     ]
     outs = []
     try:
@@ -44,7 +44,8 @@ def run_group(mode, timeout=240, rank1_exit=0):
     assert results, f"no result line\n{tail}"
     bad = [line for line in results if line.split()[2] != "OK"]
     codes = [p.returncode for p in ranks]
-    assert not bad and codes == [0, rank1_exit], "\n".join(bad) + f"\nexit codes {codes}\n" + tail
+    want = [0, rank1_exit] + [0] * (world - 2)
+    assert not bad and codes == want, "\n".join(bad) + f"\nexit codes {codes}\n" + tail
     return results, [o for o, _ in outs]
 
 

@@ -27,3 +27,10 @@ def test_calls_with_gpu_tensors_fail_when_the_peer_dies():
     pending call reports an error, nothing waits for ever."""
     results, _ = run_group("peer_dies", timeout=120, rank1_exit=3)
     assert {"before", "calls_fail_instead_of_hanging"} <= {line.split()[1] for line in results}
+
+
+def test_three_processes_share_the_gpu():
+    """Three RPC workers on the one GPU, every pair connected: calls to both peers at once, and a
+    call that the first peer relays to the second with the tensor on the GPU all the way."""
+    results, _ = run_group("gpu3", timeout=180, world=3)
+    assert {"both_peers", "relayed", "channel_chosen", "route"} <= {line.split()[1] for line in results}

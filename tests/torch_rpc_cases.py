@@ -6,6 +6,8 @@ library's channels (tensorpipe_amd.torch_rpc). Started by tests/test_torch_rpc*.
 mode: "cpu"    no device map, CPU tensors only (the module loaded must not disturb the agent)
       "gpu"    device maps 0 -> 0 both ways and to oneself; all three channels registered
       "staged" as "gpu" with the agent's channel list cut to hip_basic + basic
+      "gpu3"   three processes on the one GPU, device maps between all of them: calls to both
+               peers and a call that the first peer relays to the second
       "peer_dies" / "cpu_peer_dies"   rank 1 ends abruptly inside a call that brought it a (GPU)
                tensor while more calls with tensors are on their way: rank 0's calls must fail,
                none may hang
@@ -54,6 +56,11 @@ def make_on_gpu(nbytes, seed):
     return seeded(nbytes, seed, "cuda:0")
 
 
+def relay(name, t):
+    # the tensor goes on to a third process, comes back changed, and returns to the first
+    return rpc.rpc_sync(name, add_one, args=(t,))
+
+
 def leave_abruptly(t):
     os._exit(3)
 
@@ -65,7 +72,8 @@ def checksum(t):
 
 def main():
     rank, port, mode = int(sys.argv[1]), int(sys.argv[2]), sys.argv[3]
-    gpu = mode in ("gpu", "staged", "peer_dies")
+    gpu = mode in ("gpu", "staged", "peer_dies", "gpu3")
+    world = 3 if mode == "gpu3" else 2
     tp_rpc.load()
     os.environ["MASTER_ADDR"] = "127.0.0.1"
     os.environ["MASTER_PORT"] = str(port)
@@ -74,9 +82,9 @@ def main():
         kwargs["_channels"] = ["hip_basic", "basic"]
     opts = rpc.TensorPipeRpcBackendOptions(num_worker_threads=8, rpc_timeout=90, **kwargs)
     if gpu:
-        for peer in range(2):
+        for peer in range(world):
             opts.set_device_map(f"w{peer}", {0: 0})
-    rpc.init_rpc(f"w{rank}", rank=rank, world_size=2, rpc_backend_options=opts)
+    rpc.init_rpc(f"w{rank}", rank=rank, world_size=world, rpc_backend_options=opts)
     failures = 0
 
     def result(name, ok, note=""):
@@ -84,6 +92,23 @@ def main():
         failures += 0 if ok else 1
         print(f"RESULT {name} {'OK' if ok else 'FAIL'} {note}", flush=True)
 
+    if mode == "gpu3":
+        if rank == 0:
+            dev = "cuda:0"
+            xs = [seeded((1 << 20) + 17 * i, 400 + i, dev) for i in range(6)]
+            futs = [rpc.rpc_async(f"w{1 + i % 2}", echo, args=(x,)) for i, x in enumerate(xs)]
+            result("both_peers", all(torch.equal(x, f.wait()) for x, f in zip(xs, futs)))
+            x = seeded((2 << 20) + 3, 41, dev)
+            y = rpc.rpc_sync("w1", relay, args=("w2", x))
+            result("relayed", str(y.device) == dev and torch.equal(y, x + 1))
+            by = tp_rpc.gpu_operations_by_channel()
+            result("channel_chosen", by["hip_ipc"] >= 14 and by["hip_basic"] == 0, str(by))
+        rpc.shutdown()
+        print(f"RANK {rank} gpu_buffers_through_hip_channels {tp_rpc.gpu_operations()} {tp_rpc.gpu_operations_by_channel()}",
+              flush=True)
+        if rank == 0:
+            print("RESULT route OK" if tp_rpc.gpu_operations() else "RESULT route FAIL", flush=True)
+        sys.exit(1 if failures else 0)
     if mode.endswith("peer_dies"):
         if rank == 0:
             dev = "cuda:0" if gpu else "cpu"
