@@ -119,6 +119,17 @@ bool outboxForcedByEnv() {
 // context (TP_HIP_IPC_MAX_EXPORT_BYTES) where larger mappings are known to work.
 constexpr size_t kDefaultMaxExportBytes = size_t(2) << 30;
 
+// Allocations smaller than this are staged through the outbox as well. The
+// runtime carves small device allocations out of 2 MiB blocks, and the handle
+// of one such allocation stops working when ANOTHER exported allocation of the
+// same block is freed before the peer has opened it ("IPC Attach: Invalid IPC
+// handle", seen for allocations of 100 KB and 1 MiB, not for 2 MiB - 4 KiB and
+// more, nor for pinned host memory): a sender that frees tensors as their
+// sends complete would break the sends behind them. Allocators of frameworks
+// hand out tensors inside segments of 2 MiB and more, which are exported as
+// before. TP_HIP_IPC_MIN_EXPORT_BYTES overrides.
+constexpr size_t kDefaultMinExportBytes = size_t(2) << 20;
+
 // Peer allocations a channel keeps mapped: least recently used ones go once
 // their sizes add up to more than this, or there are more than this many.
 constexpr size_t kDefaultMaxMappedBytes = size_t(64) << 30;
@@ -149,6 +160,7 @@ class ExportRegistry {
   bool lookup(
       int device,
       const void* ptr,
+      size_t minExportBytes,
       size_t maxExportBytes,
       ExportedAllocation* out,
       uint64_t* offset) {
@@ -165,7 +177,7 @@ class ExportRegistry {
         const uint8_t* base = static_cast<const uint8_t*>(it->first);
         const uint8_t* p = static_cast<const uint8_t*>(ptr);
         if (p < base + it->second.size && it->second.bufferId == bufferId &&
-            it->second.size < maxExportBytes) {
+            it->second.size < maxExportBytes && it->second.size >= minExportBytes) {
           *out = it->second;
           *offset = static_cast<uint64_t>(p - base);
           return true;
@@ -174,7 +186,8 @@ class ExportRegistry {
     }
     void* base = nullptr;
     size_t size = 0;
-    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr || size >= maxExportBytes) {
+    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr || size >= maxExportBytes ||
+        size < minExportBytes) {
       return false;
     }
     uint64_t bufferId = 0;
@@ -200,6 +213,7 @@ class ExportRegistry {
     e.base = reinterpret_cast<uint64_t>(base);
     e.size = size;
     e.bufferId = bufferId;
+    TP_VLOG(5) << "IPC exports: #" << e.id << " is " << base << " + " << size << " (allocation " << bufferId << ")";
     *out = e;
     if (bufferId != 0) {
       exports_[base] = e;
@@ -235,7 +249,9 @@ class ExportRegistry {
 // Per-device staging slab of the outbox path, created on first use.
 struct Outbox {
   Outbox(int device, size_t slotBytes, size_t numSlots)
-      : slab(device, slotBytes * numSlots), allocator(slab.ptr(), numSlots, slotBytes) {
+      // (never below the size at which the runtime gives an allocation a block of its own)
+      : slab(device, std::max(slotBytes * numSlots, kDefaultMinExportBytes)),
+        allocator(slab.ptr(), numSlots, slotBytes) {
     TP_HIP_CHECK(tphip_ipc_mem_export(device, slab.ptr(), handle.data()));
   }
   HipDeviceSlab slab;
@@ -398,6 +414,7 @@ class IpcContextCore final : public ContextCore {
   StreamIdleProbe idleProbe; // loop only
   StreamMarkers markers;
   const bool forceOutbox{outboxForcedByEnv()};
+  const size_t minExportBytes{envSize("TP_HIP_IPC_MIN_EXPORT_BYTES", kDefaultMinExportBytes)};
   const size_t maxExportBytes{envSize("TP_HIP_IPC_MAX_EXPORT_BYTES", kDefaultMaxExportBytes)};
   const size_t maxMappedBytes{envSize("TP_HIP_IPC_MAX_MAPPED_BYTES", kDefaultMaxMappedBytes)};
   // 16-byte multiples keep every slot vector-aligned.
@@ -725,7 +742,7 @@ class ChannelImpl final : public ChannelImplBase {
         TP_THROW_ASSERT_IF(device < 0);
         DirectItem item;
         if (!ictx_->forceOutbox && ExportRegistry::get().lookup(
-                device, hb.ptr, ictx_->maxExportBytes, &item.alloc, &item.offset)) {
+                device, hb.ptr, ictx_->minExportBytes, ictx_->maxExportBytes, &item.alloc, &item.offset)) {
           item.length = live[i].length;
           item.index = i;
           direct.push_back(item);

@@ -296,6 +296,101 @@ std::vector<Case> makeCases() {
          }});
   }
 
+  // Traffic in both directions from one seeded schedule that both ends know:
+  // sizes from nothing to a few MiB, directions mixed, up to sixteen
+  // operations in flight on each end. Every tensor has bytes of its own.
+  {
+    struct Step {
+      bool fromServer;
+      size_t size;
+    };
+    auto schedule = [] {
+      std::vector<Step> steps;
+      uint64_t x = 0x9e3779b97f4a7c15ull; // splitmix64
+      auto next = [&x] {
+        x += 0x9e3779b97f4a7c15ull;
+        uint64_t z = x;
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        return z ^ (z >> 31);
+      };
+      for (int i = 0; i < 96; ++i) {
+        const uint64_t r = next();
+        size_t size;
+        switch (r % 8) {
+          case 0:
+            size = 0;
+            break;
+          case 1:
+          case 2:
+            size = 1 + (r >> 8) % 300;
+            break;
+          case 3:
+          case 4:
+          case 5:
+            size = 4000 + (r >> 8) % 200000;
+            break;
+          case 6:
+            size = (1u << 20) + (r >> 8) % 4096;
+            break;
+          default:
+            size = (2u << 20) + (1u << 19) + (r >> 8) % 77777;
+        }
+        steps.push_back(Step{((r >> 40) & 1) != 0, size});
+      }
+      return steps;
+    };
+    auto pattern = [](int k, size_t size) {
+      std::vector<uint8_t> v(size);
+      for (size_t j = 0; j < size; ++j) {
+        v[j] = static_cast<uint8_t>((j * 31 + static_cast<size_t>(k) * 59 + (j >> 10) * 7) % 251);
+      }
+      return v;
+    };
+    auto side = [schedule, pattern](Endpoint& ep) {
+      auto o = open(ep);
+      const auto steps = schedule();
+      std::vector<std::unique_ptr<Data>> ds(steps.size());
+      std::vector<std::future<Error>> fs(steps.size());
+      const size_t window = 16;
+      auto settle = [&](size_t k) {
+        const bool mine = steps[k].fromServer == ep.isServer();
+        EXPECT_OK(waitFor(fs[k], mine ? "send" : "recv"));
+        if (!mine) {
+          expectBytes(*ds[k], pattern(static_cast<int>(k), steps[k].size), "tensor");
+        }
+        ds[k].reset();
+      };
+      for (size_t k = 0; k < steps.size(); ++k) {
+        if (k >= window) {
+          settle(k - window);
+        }
+        const bool mine = steps[k].fromServer == ep.isServer();
+        if (mine) {
+          ds[k] = makeData(gGpu, pattern(static_cast<int>(k), steps[k].size));
+          fs[k] = sendF(*o->ch, ds[k]->buffer(), ds[k]->size());
+        } else {
+          ds[k] = makeData(gGpu, steps[k].size);
+          fs[k] = recvF(*o->ch, ds[k]->buffer(), ds[k]->size());
+        }
+      }
+      for (size_t k = steps.size() > window ? steps.size() - window : 0; k < steps.size(); ++k) {
+        settle(k);
+      }
+      ep.barrier();
+    };
+    cases.push_back({"SeededTrafficBothWays", side, side});
+    // The same with every tensor in a device allocation of exactly its size,
+    // allocated for the operation and freed when it completes: allocations
+    // that the runtime packs several to a block come and go while transfers
+    // of their neighbours are still under way.
+    auto exact = [side](Endpoint& ep) {
+      ExactGpuAllocations guard;
+      side(ep);
+    };
+    cases.push_back({"SeededTrafficSmallAllocations", exact, exact});
+  }
+
   // channel_test.cc:191-259: one send and one recv in flight on each side.
   auto bothWays = [](Endpoint& ep) {
     auto o = open(ep);
@@ -490,10 +585,11 @@ std::vector<Case> makeCases() {
 
   if (gSuite == "hip_ipc") {
     // An allocation at or above the export limit is not mapped by the peer but
-    // staged through the outbox. The two routes are told apart by when the send
-    // completes: a staged send once its bytes sit in the outbox, before the
-    // peer has posted its recv; a direct send only after the peer's copy.
-    const size_t big = 256 * 1024, small = 4096;
+    // staged through the outbox, and so is one below the size at which the
+    // runtime gives an allocation a block of its own. The two routes are told
+    // apart by when the send completes: a staged send once its bytes sit in
+    // the outbox, before the peer has posted its recv; a direct send only
+    // after the peer's copy.
     auto pattern = [](size_t n, uint8_t salt) {
       std::vector<uint8_t> v(n);
       for (size_t i = 0; i < n; ++i) {
@@ -501,13 +597,22 @@ std::vector<Case> makeCases() {
       }
       return v;
     };
-    auto sendSide = [=](Endpoint& ep) {
-      ::setenv("TP_HIP_IPC_MAX_EXPORT_BYTES", "65536", 1);
+    const size_t direct = 4096; // inside an allocation of 2 MiB, as all allocations of these tests
+    // staged: how many bytes, and whether the allocation is exactly that large
+    auto sendSide = [=](Endpoint& ep, size_t staged, bool exact) {
+      ::setenv("TP_HIP_IPC_MAX_EXPORT_BYTES", "3145728", 1);
       auto o = open(ep);
       ::unsetenv("TP_HIP_IPC_MAX_EXPORT_BYTES");
-      GpuData above(pattern(big, 1));
-      GpuData below(pattern(small, 2));
-      auto fa = sendF(*o->ch, above.buffer(), above.size());
+      std::unique_ptr<GpuData> other;
+      {
+        std::unique_ptr<ExactGpuAllocations> guard;
+        if (exact) {
+          guard = std::make_unique<ExactGpuAllocations>();
+        }
+        other = std::make_unique<GpuData>(pattern(staged, 1));
+      }
+      GpuData below(pattern(direct, 2));
+      auto fa = sendF(*o->ch, other->buffer(), other->size());
       EXPECT_OK(waitFor(fa, "staged send before the peer's recv"));
       auto fb = sendF(*o->ch, below.buffer(), below.size());
       EXPECT_TRUE(fb.wait_for(std::chrono::milliseconds(300)) == std::future_status::timeout);
@@ -515,19 +620,25 @@ std::vector<Case> makeCases() {
       EXPECT_OK(waitFor(fb, "direct send"));
       ep.barrier();
     };
-    auto recvSide = [=](Endpoint& ep) {
+    auto recvSide = [=](Endpoint& ep, size_t staged) {
       auto o = open(ep);
-      GpuData a(big), b(small);
+      GpuData a(staged), b(direct);
       ep.barrier();
       auto fa = recvF(*o->ch, a.buffer(), a.size());
       auto fb = recvF(*o->ch, b.buffer(), b.size());
       EXPECT_OK(waitFor(fa, "recv of the staged tensor"));
       EXPECT_OK(waitFor(fb, "recv of the direct tensor"));
-      expectBytes(a, pattern(big, 1), "staged tensor");
-      expectBytes(b, pattern(small, 2), "direct tensor");
+      expectBytes(a, pattern(staged, 1), "staged tensor");
+      expectBytes(b, pattern(direct, 2), "direct tensor");
       ep.barrier();
     };
-    cases.push_back({"AllocationsAboveExportLimitAreStaged", sendSide, recvSide});
+    const size_t big = 4 * 1024 * 1024, little = 256 * 1024;
+    cases.push_back({"AllocationsAboveExportLimitAreStaged",
+                     [=](Endpoint& ep) { sendSide(ep, big, false); },
+                     [=](Endpoint& ep) { recvSide(ep, big); }});
+    cases.push_back({"AllocationsBelowBlockSizeAreStaged",
+                     [=](Endpoint& ep) { sendSide(ep, little, true); },
+                     [=](Endpoint& ep) { recvSide(ep, little); }});
   }
 
   if (gSuite == "hip_ipc") {

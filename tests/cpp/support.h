@@ -13,6 +13,7 @@
 #include <sys/wait.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cstdint>
@@ -153,11 +154,31 @@ class CpuData final : public Data {
   std::vector<uint8_t> v_;
 };
 
+// Device allocations of the tests are at least this large, as the segments of
+// a framework's caching allocator are; a case that wants the exact size (the
+// runtime then carves the allocation out of a block it shares with others)
+// holds an ExactGpuAllocations while it allocates.
+inline std::atomic<int>& exactGpuAllocationHolders() {
+  static std::atomic<int> n{0};
+  return n;
+}
+inline size_t minGpuAllocation() {
+  return exactGpuAllocationHolders().load() > 0 ? size_t(1) : size_t(2) << 20;
+}
+struct ExactGpuAllocations {
+  ExactGpuAllocations() {
+    ++exactGpuAllocationHolders();
+  }
+  ~ExactGpuAllocations() {
+    --exactGpuAllocationHolders();
+  }
+};
+
 class GpuData final : public Data {
  public:
   // `offset` bytes of 0xff precede the payload inside the allocation.
   explicit GpuData(size_t n, size_t offset = 0) : n_(n), offset_(offset) {
-    HIP_OK(tphip_malloc(0, n + offset > 0 ? n + offset : 1, &base_));
+    HIP_OK(tphip_malloc(0, std::max(n + offset, minGpuAllocation()), &base_));
     HIP_OK(tphip_stream_create(0, &stream_));
     HIP_OK(tphip_fill(0, base_, 0xff, n + offset, stream_));
     HIP_OK(tphip_stream_sync(0, stream_));
