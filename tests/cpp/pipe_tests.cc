@@ -904,6 +904,23 @@ std::vector<Case> makeCases() {
                      ep.barrier();
                    }});
 
+  // The same with every GPU tensor in a device allocation of exactly its own
+  // size, freed when its message is done (the runtime packs such allocations
+  // several to a block).
+  cases.push_back({"ManyMessagesSmallAllocations",
+                   [](Endpoint& ep) {
+                     ExactGpuAllocations guard;
+                     auto e = openPipe(ep);
+                     exchangeMany(*e->pipe, 0, 60);
+                     ep.barrier();
+                   },
+                   [](Endpoint& ep) {
+                     ExactGpuAllocations guard;
+                     auto e = openPipe(ep);
+                     exchangeMany(*e->pipe, 1, 60);
+                     ep.barrier();
+                   }});
+
   // One message with more tensors than a copy table holds (4096): the channels
   // cut it into several launches, the pipe into nothing. 5000 tensors of 1 to
   // 200 bytes, carved at odd offsets out of one allocation on each side.
