@@ -436,15 +436,6 @@ class ChannelImpl final : public ChannelImplBase {
     }
   }
 
-  void removeRecv(const std::shared_ptr<RecvOp>& op) {
-    for (auto it = recvOps_.begin(); it != recvOps_.end(); ++it) {
-      if (*it == op) {
-        recvOps_.erase(it);
-        return;
-      }
-    }
-  }
-
   void finishSend(const std::shared_ptr<SendOp>& op) {
     if (op->done) {
       return;
