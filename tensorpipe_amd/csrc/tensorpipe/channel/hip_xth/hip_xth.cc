@@ -309,6 +309,10 @@ class ChannelImpl final : public ChannelImplBase {
     auto ops = std::move(toLaunch_);
     toLaunch_.clear();
     toLaunchBytes_ = 0;
+    size_t pieces = 0;
+    for (auto& op : ops) {
+      pieces += op->pieces.size();
+    }
     for (auto& op : ops) {
       for (auto& piece : op->pieces) {
         Group* g = nullptr;
@@ -320,6 +324,7 @@ class ChannelImpl final : public ChannelImplBase {
         if (g == nullptr) {
           groups.push_back(Group{piece.src, {}, {}, {}});
           g = &groups.back();
+          g->table.reserve(pieces); // normally the only group
         }
         bool known = false;
         for (auto& d : g->dstStreams) {
