@@ -19,29 +19,31 @@ def free_port():
         return s.getsockname()[1]
 
 
-def run_group(mode, timeout=240, rank1_exit=0, world=2):
+def run_group(mode, timeout=120, rank1_exit=0, world=2):
     if not os.path.exists(PLUGIN):
         pytest.skip("libtensorpipe_amd_torch_rpc.so is not built (no RPC agent headers at build time)")
     port = free_port()
     print(f"running torch_rpc_cases.py, mode {mode}, port {port}", flush=True)
+    # The ranks keep a short timeline of what the channels did last and print it when they end;
+    # a rank that stalls ends itself (torch_rpc_cases.py) well inside this function's time limit.
+    env = dict(os.environ, TP_TIMELINE=os.environ.get("TP_TIMELINE", "400"))
     ranks = [
         subprocess.Popen([sys.executable, "-u", CASES, str(rank), str(port), mode],
-                         stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+                         stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env)
         for rank in range(world)
     ]
     outs = []
-    try:
-        for p in ranks:
+    for p in ranks:
+        try:
             outs.append(p.communicate(timeout=timeout))
-    finally:
-        for p in ranks:
-            if p.poll() is None:
-                p.kill()
-                p.communicate()
+        except subprocess.TimeoutExpired:
+            p.kill()
+            outs.append(p.communicate())
     text = outs[0][0]
     results = [line for line in text.splitlines() if line.startswith("RESULT ")]
-    tail = "\n".join(f"--- rank {i}\n{o[-1500:]}\n{e[-2500:]}" for i, (o, e) in enumerate(outs))
+    tail = "\n".join(f"--- rank {i}\n{o[-2500:]}\n{e[-12000:]}" for i, (o, e) in enumerate(outs))
     assert results, f"no result line\n{tail}"
+    results += [line for o, _ in outs[1:] for line in o.splitlines() if line.startswith("RESULT stalled")]
     bad = [line for line in results if line.split()[2] != "OK"]
     codes = [p.returncode for p in ranks]
     want = [0, rank1_exit] + [0] * (world - 2)

@@ -17,8 +17,11 @@ buffers went through the hip_* channels. What the reference's agent tests for it
 (PyTorch's torch/testing/_internal/distributed/rpc/rpc_test.py: device maps, tensors in arguments and
 results, many calls in flight, RRefs) is the model for the cases.
 """
+import ctypes
+import faulthandler
 import os
 import sys
+import threading
 
 import torch
 import torch.distributed.rpc as rpc
@@ -72,6 +75,22 @@ def checksum(t):
 
 def main():
     rank, port, mode = int(sys.argv[1]), int(sys.argv[2]), sys.argv[3]
+    # A rank that is still here after this long says where every thread stands and ends, so that
+    # the test reports what was reached instead of running into the runner's own time limit.
+    limit = int(os.environ.get("TP_RPC_CASES_LIMIT_S", "90"))
+
+    def stalled():
+        print(f"RESULT stalled FAIL rank {rank} was still running after {limit} s", flush=True)
+        faulthandler.dump_traceback(all_threads=True)
+        sys.stderr.flush()
+        # exit() rather than _exit(): the library prints its timeline of recent events
+        # (TP_TIMELINE) when the process ends in the ordinary way
+        ctypes.CDLL(None).exit(3)
+
+    watchdog = threading.Timer(limit, stalled)
+    watchdog.daemon = True
+    watchdog.start()
+    faulthandler.dump_traceback_later(limit + 20, exit=True)  # should the ordinary exit not get through
     gpu = mode in ("gpu", "staged", "peer_dies", "gpu3")
     world = 3 if mode == "gpu3" else 2
     tp_rpc.load()
