@@ -391,6 +391,140 @@ std::vector<Case> makeCases() {
     cases.push_back({"SeededTrafficSmallAllocations", exact, exact});
   }
 
+  // Both ends of a channel on ONE context: a process that talks to itself (an
+  // RPC worker calling itself does). Tensors go both ways at once; the context
+  // shares its loop, its staging rings and its poller between the two ends.
+  if (gSuite != "hip_ipc" && gSuite.rfind("hip_ipc_", 0) != 0) {
+    auto sizeOf = [](int k) {
+      static const size_t sizes[] = {(1u << 20) + 1, (3u << 20) + 5, 100, 0, 65536, (2u << 20) + (1u << 19)};
+      return sizes[k % 6] + static_cast<size_t>(k / 6) * 4099;
+    };
+    auto pattern = [sizeOf](int k, int dir) {
+      std::vector<uint8_t> v(sizeOf(k));
+      for (size_t j = 0; j < v.size(); ++j) {
+        v[j] = static_cast<uint8_t>((j * 17 + static_cast<size_t>(k) * 29 + static_cast<size_t>(dir) * 7 + (j >> 11)) % 249);
+      }
+      return v;
+    };
+    auto oneContext = [sizeOf, pattern](Endpoint& ep) {
+      if (ep.isServer()) {
+        auto ctx = makeContext();
+        ctx->setId("talks_to_itself");
+        if (!ctx->isViable()) {
+          throw Fatal("context is not viable");
+        }
+        const size_t n = ctx->numConnectionsNeeded();
+        const std::string addr = ep.freshAddr() + "_self";
+        auto listener = ep.transport()->listen(addr);
+        std::vector<std::shared_ptr<transport::Connection>> connecting(n), accepted(n);
+        for (size_t i = 0; i < n; ++i) {
+          // one at a time, so that the i-th ends belong together
+          connecting[i] = ep.transport()->connect(addr);
+          accepted[i] = acceptOne(*listener);
+          writeByte(*connecting[i], static_cast<uint8_t>(i));
+          if (readByte(*accepted[i]) != i) {
+            throw Fatal("connections paired out of order");
+          }
+        }
+        listener->close();
+        {
+          auto a = ctx->createChannel(std::move(accepted), channel::Endpoint::kListen);
+          auto b = ctx->createChannel(std::move(connecting), channel::Endpoint::kConnect);
+          constexpr int kTensors = 18;
+          std::vector<std::unique_ptr<Data>> out[2], in[2];
+          std::vector<std::future<Error>> sends, recvs;
+          for (int k = 0; k < kTensors; ++k) {
+            for (int dir = 0; dir < 2; ++dir) {
+              out[dir].push_back(makeData(gGpu, pattern(k, dir)));
+              in[dir].push_back(makeData(gGpu, sizeOf(k)));
+            }
+          }
+          for (int k = 0; k < kTensors; ++k) {
+            // dir 0: a -> b, dir 1: b -> a; receives posted now and then ahead of the sends
+            if (k % 3 == 0) {
+              recvs.push_back(recvF(*b, in[0][k]->buffer(), in[0][k]->size()));
+              recvs.push_back(recvF(*a, in[1][k]->buffer(), in[1][k]->size()));
+            }
+            sends.push_back(sendF(*a, out[0][k]->buffer(), out[0][k]->size()));
+            sends.push_back(sendF(*b, out[1][k]->buffer(), out[1][k]->size()));
+            if (k % 3 != 0) {
+              recvs.push_back(recvF(*b, in[0][k]->buffer(), in[0][k]->size()));
+              recvs.push_back(recvF(*a, in[1][k]->buffer(), in[1][k]->size()));
+            }
+          }
+          for (auto& f : sends) {
+            EXPECT_OK(waitFor(f, "send"));
+          }
+          for (auto& f : recvs) {
+            EXPECT_OK(waitFor(f, "recv"));
+          }
+          for (int k = 0; k < kTensors; ++k) {
+            for (int dir = 0; dir < 2; ++dir) {
+              expectBytes(*in[dir][k], pattern(k, dir), "tensor");
+            }
+          }
+        }
+        ctx->join();
+      }
+      ep.barrier();
+    };
+    cases.push_back({"BothEndsOnOneContext", oneContext, oneContext});
+  }
+
+  // Two channels between the same two contexts at once (two pipes between two
+  // workers, as RPC agents open them), traffic flowing the opposite way on each:
+  // they share each context's loop, poller and staging rings, and one tensor is
+  // larger than a whole ring.
+  {
+    auto sizeOf = [](int k) {
+      static const size_t sizes[] = {70000, (1u << 20) + 3, 333, (20u << 20) + 11, 4096, (2u << 20) + 77};
+      return sizes[k % 6] + static_cast<size_t>(k / 6) * 1031;
+    };
+    auto pattern = [sizeOf](int k, int lane) {
+      std::vector<uint8_t> v(sizeOf(k));
+      for (size_t j = 0; j < v.size(); ++j) {
+        v[j] = static_cast<uint8_t>((j * 19 + static_cast<size_t>(k) * 23 + static_cast<size_t>(lane) * 5 + (j >> 12)) % 247);
+      }
+      return v;
+    };
+    auto side = [sizeOf, pattern](Endpoint& ep) {
+      auto ctx = makeContext();
+      ctx->setId(std::string(roleName(ep.role())) + "_ctx");
+      if (!ctx->isViable()) {
+        throw Fatal("context is not viable");
+      }
+      const auto end = ep.isServer() ? channel::Endpoint::kListen : channel::Endpoint::kConnect;
+      {
+        auto first = ctx->createChannel(ep.openConnections(ctx->numConnectionsNeeded()), end);
+        auto second = ctx->createChannel(ep.openConnections(ctx->numConnectionsNeeded()), end);
+        // the server sends on the first and receives on the second, the client the other way round
+        auto& outCh = ep.isServer() ? *first : *second;
+        auto& inCh = ep.isServer() ? *second : *first;
+        const int outLane = ep.isServer() ? 0 : 1;
+        constexpr int kTensors = 12;
+        std::vector<std::unique_ptr<Data>> out, in;
+        std::vector<std::future<Error>> fs;
+        for (int k = 0; k < kTensors; ++k) {
+          out.push_back(makeData(gGpu, pattern(k, outLane)));
+          in.push_back(makeData(gGpu, sizeOf(k)));
+        }
+        for (int k = 0; k < kTensors; ++k) {
+          fs.push_back(sendF(outCh, out[k]->buffer(), out[k]->size()));
+          fs.push_back(recvF(inCh, in[k]->buffer(), in[k]->size()));
+        }
+        for (auto& f : fs) {
+          EXPECT_OK(waitFor(f, "transfer"));
+        }
+        for (int k = 0; k < kTensors; ++k) {
+          expectBytes(*in[k], pattern(k, 1 - outLane), "tensor");
+        }
+        ep.barrier();
+      }
+      ctx->join();
+    };
+    cases.push_back({"TwoChannelsShareTheContexts", side, side});
+  }
+
   // channel_test.cc:191-259: one send and one recv in flight on each side.
   auto bothWays = [](Endpoint& ep) {
     auto o = open(ep);
