@@ -407,6 +407,7 @@ std::vector<Case> makeCases() {
       return v;
     };
     auto oneContext = [sizeOf, pattern](Endpoint& ep) {
+      const std::string base = ep.freshAddr(); // drawn by both ends: they count addresses in step
       if (ep.isServer()) {
         auto ctx = makeContext();
         ctx->setId("talks_to_itself");
@@ -414,7 +415,7 @@ std::vector<Case> makeCases() {
           throw Fatal("context is not viable");
         }
         const size_t n = ctx->numConnectionsNeeded();
-        const std::string addr = ep.freshAddr() + "_self";
+        const std::string addr = base + "_self";
         auto listener = ep.transport()->listen(addr);
         std::vector<std::shared_ptr<transport::Connection>> connecting(n), accepted(n);
         for (size_t i = 0; i < n; ++i) {
