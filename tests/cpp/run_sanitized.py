@@ -1,9 +1,13 @@
 #!/usr/bin/env python3
 """Builds the host library and the C++ test programs with a sanitizer and runs the CPU suites.
 
-    python tests/cpp/run_sanitized.py thread|address [build_dir]
+    python tests/cpp/run_sanitized.py thread|address [build_dir] [--build-only | --run-only] [--gpu]
 
-Host code only (g++ -fsanitize=...); libtphip.so is used as built. Not collected by pytest: a
+Host code only (g++ -fsanitize=...); libtphip.so is used as built. With --gpu the suites of the
+device channels run instead of the CPU ones (on a machine with a GPU; --build-only on one machine
+and --run-only on another share a build directory; next to the HIP runtime AddressSanitizer needs
+ASAN_OPTIONS=use_sigaltstack=0:protect_shadow_gap=0:detect_leaks=0, and ThreadSanitizer does not
+work at all: the runtime finds no device under its address-space layout). Not collected by pytest: a
 full pass takes several minutes. The shm transport tells ThreadSanitizer about the hand-off
 through its rings (two mappings of one segment inside a process), so a clean run reports
 nothing; any "WARNING: ThreadSanitizer" / "ERROR: AddressSanitizer" line fails the run.
@@ -24,10 +28,28 @@ SUITES = [("channel_tests", "xth", False), ("channel_tests", "basic", False),
           ("pipe_tests", "cpu_same_process", True), ("pipe_tests", "cpu_two_process", True)]
 
 
+GPU_SUITES = [("channel_tests", "hip_xth", False), ("channel_tests", "hip_ipc", False),
+              ("channel_tests", "hip_ipc_outbox", False), ("channel_tests", "hip_basic", False),
+              ("pipe_tests", "same_process", False), ("pipe_tests", "two_process", False),
+              ("pipe_tests", "two_process", True)]
+
+
 def main():
-    san = sys.argv[1] if len(sys.argv) > 1 else "thread"
-    out = sys.argv[2] if len(sys.argv) > 2 else tempfile.mkdtemp(prefix=f"tp_{san}_")
+    words = [a for a in sys.argv[1:] if not a.startswith("--")]
+    options = {a for a in sys.argv[1:] if a.startswith("--")}
+    san = words[0] if words else "thread"
+    out = os.path.abspath(words[1]) if len(words) > 1 else tempfile.mkdtemp(prefix=f"tp_{san}_")
     os.makedirs(out, exist_ok=True)
+    if "--run-only" not in options:
+        build(san, out)
+    if "--build-only" in options:
+        return
+    if "--gpu" in options:
+        sys.exit(1 if run_suites(out, GPU_SUITES) else 0)
+    run_cpu(out)
+
+
+def build(san, out):
     flags = ["-O1", "-g", "-std=c++17", "-fPIC", f"-fsanitize={san}", "-fno-omit-frame-pointer", "-pthread",
              f"-I{tp_build.INCLUDE}", f"-I{tp_build.CSRC}"]
     objs = [os.path.join(out, s.replace("/", "_") + ".o") for s in tp_build.HOST_SOURCES]
@@ -45,8 +67,11 @@ def main():
         subprocess.run(["g++", *flags, os.path.join(ROOT, "tests", "cpp", prog + ".cc"), "-o",
                         os.path.join(out, prog), f"-L{out}", "-ltensorpipe_amd", f"-L{tp_build.LIB}", "-ltphip",
                         f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
+
+
+def run_suites(out, suites):
     bad = 0
-    for prog, suite, stock_wire in SUITES:
+    for prog, suite, stock_wire in suites:
         env = dict(os.environ, TP_STOCK_WIRE="1") if stock_wire else None
         proc = subprocess.run([os.path.join(out, prog), "--suite", suite], stdout=subprocess.PIPE,
                               stderr=subprocess.STDOUT, text=True, timeout=1800, env=env)
@@ -57,6 +82,12 @@ def main():
         for l in failed + reports[:5]:
             print("   ", l[:200])
         bad += len(failed) + len(reports) + (0 if results else 1)
+        sys.stdout.flush()
+    return bad
+
+
+def run_cpu(out):
+    bad = run_suites(out, SUITES)
     # random bytes where a pipe's first packets belong
     for seed in (11, 12, 13):
         proc = subprocess.run([os.path.join(out, "unit_tests"), "garbage", str(seed), "150"],
