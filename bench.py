@@ -463,16 +463,14 @@ def bench_cpu_path(stock_wire_tcp=False):
 def bench_torch_rpc():
     """torch.distributed.rpc round trips (PyTorch's own TensorPipe agent) with GPU tensors on this
     library's channels, next to CPU tensors on the agent's stock channels."""
-    import socket
+    import tempfile
 
     from tensorpipe_amd import torch_rpc as tp_rpc
 
     if not os.path.exists(tp_rpc.library_path()):
         return {"error": "libtensorpipe_amd_torch_rpc.so is not built"}
-    with socket.socket() as s:
-        s.bind(("127.0.0.1", 0))
-        port = s.getsockname()[1]
-    ranks = [subprocess.Popen([sys.executable, "-m", "tensorpipe_amd.bench_rpc_peer", str(r), str(port)],
+    meeting = os.path.join(tempfile.mkdtemp(prefix="tp_rpc_"), "rendezvous")
+    ranks = [subprocess.Popen([sys.executable, "-m", "tensorpipe_amd.bench_rpc_peer", str(r), meeting],
                               stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, cwd=ROOT)
              for r in (1, 0)]
     try:

@@ -1,6 +1,6 @@
 """One rank of the torch.distributed.rpc measurement of bench.py (leg "torch_rpc"):
 
-    python -m tensorpipe_amd.bench_rpc_peer <rank> <port>
+    python -m tensorpipe_amd.bench_rpc_peer <rank> <rendezvous file>
 
 Two processes on the one GPU, PyTorch's own TensorPipe agent, this library's channels registered
 with it (tensorpipe_amd.torch_rpc). Rank 0 times rpc_sync(echo) round trips -- the tensor goes to
@@ -22,11 +22,10 @@ def echo(t):
 
 
 def main():
-    rank, port = int(sys.argv[1]), int(sys.argv[2])
+    rank, rendezvous = int(sys.argv[1]), sys.argv[2]
     tp_rpc.load()
-    os.environ["MASTER_ADDR"] = "127.0.0.1"
-    os.environ["MASTER_PORT"] = str(port)
-    opts = rpc.TensorPipeRpcBackendOptions(num_worker_threads=8, rpc_timeout=120)
+    opts = rpc.TensorPipeRpcBackendOptions(num_worker_threads=8, rpc_timeout=120,
+                                           init_method="file://" + rendezvous)
     opts.set_device_map(f"w{1 - rank}", {0: 0})
     rpc.init_rpc(f"w{rank}", rank=rank, world_size=2, rpc_backend_options=opts)
     out = {}

@@ -2,9 +2,9 @@
 channels report themselves not viable, the agent leaves them out, and CPU tensors travel as
 before. (The GPU cases are in test_torch_rpc_gpu.py.)"""
 import os
-import socket
 import subprocess
 import sys
+import tempfile
 
 import pytest
 
@@ -13,22 +13,19 @@ CASES = os.path.join(ROOT, "tests", "torch_rpc_cases.py")
 PLUGIN = os.path.join(ROOT, "tensorpipe_amd", "lib", "libtensorpipe_amd_torch_rpc.so")
 
 
-def free_port():
-    with socket.socket() as s:
-        s.bind(("127.0.0.1", 0))
-        return s.getsockname()[1]
-
 
 def run_group(mode, timeout=120, rank1_exit=0, world=2):
     if not os.path.exists(PLUGIN):
         pytest.skip("libtensorpipe_amd_torch_rpc.so is not built (no RPC agent headers at build time)")
-    port = free_port()
-    print(f"running torch_rpc_cases.py, mode {mode}, port {port}", flush=True)
+    meeting = tempfile.NamedTemporaryFile(prefix="tp_rpc_", suffix=".rendezvous", delete=False)
+    meeting.close()
+    os.unlink(meeting.name)  # the first rank creates it
+    print(f"running torch_rpc_cases.py, mode {mode}, rendezvous {meeting.name}", flush=True)
     # The ranks keep a short timeline of what the channels did last and print it when they end;
     # a rank that stalls ends itself (torch_rpc_cases.py) well inside this function's time limit.
     env = dict(os.environ, TP_TIMELINE=os.environ.get("TP_TIMELINE", "400"))
     ranks = [
-        subprocess.Popen([sys.executable, "-u", CASES, str(rank), str(port), mode],
+        subprocess.Popen([sys.executable, "-u", CASES, str(rank), meeting.name, mode],
                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env)
         for rank in range(world)
     ]
@@ -39,6 +36,8 @@ def run_group(mode, timeout=120, rank1_exit=0, world=2):
         except subprocess.TimeoutExpired:
             p.kill()
             outs.append(p.communicate())
+    if os.path.exists(meeting.name):
+        os.unlink(meeting.name)
     text = outs[0][0]
     results = [line for line in text.splitlines() if line.startswith("RESULT ")]
     tail = "\n".join(f"--- rank {i}\n{o[-2500:]}\n{e[-12000:]}" for i, (o, e) in enumerate(outs))

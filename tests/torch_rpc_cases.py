@@ -1,7 +1,7 @@
 """One rank of a two-process torch.distributed.rpc group whose GPU tensors travel on this
 library's channels (tensorpipe_amd.torch_rpc). Started by tests/test_torch_rpc*.py, once per rank:
 
-    python tests/torch_rpc_cases.py <rank> <port> <mode>
+    python tests/torch_rpc_cases.py <rank> <rendezvous file> <mode>
 
 mode: "cpu"    no device map, CPU tensors only (the module loaded must not disturb the agent)
       "gpu"    device maps 0 -> 0 both ways and to oneself; all three channels registered
@@ -74,7 +74,7 @@ def checksum(t):
 
 
 def main():
-    rank, port, mode = int(sys.argv[1]), int(sys.argv[2]), sys.argv[3]
+    rank, rendezvous, mode = int(sys.argv[1]), sys.argv[2], sys.argv[3]
     # A rank that is still here after this long says where every thread stands and ends, so that
     # the test reports what was reached instead of running into the runner's own time limit.
     limit = int(os.environ.get("TP_RPC_CASES_LIMIT_S", "90"))
@@ -94,9 +94,8 @@ def main():
     gpu = mode in ("gpu", "staged", "peer_dies", "gpu3")
     world = 3 if mode == "gpu3" else 2
     tp_rpc.load()
-    os.environ["MASTER_ADDR"] = "127.0.0.1"
-    os.environ["MASTER_PORT"] = str(port)
-    kwargs = {}
+    # the ranks meet through a file: no port that somebody else might take in between
+    kwargs = {"init_method": "file://" + rendezvous}
     if mode == "staged":
         kwargs["_channels"] = ["hip_basic", "basic"]
     opts = rpc.TensorPipeRpcBackendOptions(num_worker_threads=8, rpc_timeout=90, **kwargs)
