@@ -7,7 +7,6 @@ with it (tensorpipe_amd.torch_rpc). Rank 0 times rpc_sync(echo) round trips -- t
 the other process and comes back -- for GPU tensors, and for CPU tensors of the same sizes on the
 agent's stock channels, and prints one JSON line."""
 import json
-import os
 import sys
 import time
 
