@@ -1,6 +1,6 @@
 """torch.distributed.rpc with this library's module loaded, on a machine without a GPU: the hip_*
 channels report themselves not viable, the agent leaves them out, and CPU tensors travel as
-before. (The GPU cases are in test_torch_rpc_gpu.py.)"""
+before. (The GPU cases are in test_zy_torch_rpc_gpu.py.)"""
 import os
 import subprocess
 import sys
