@@ -1,5 +1,5 @@
 """One rank of a two-process torch.distributed.rpc group whose GPU tensors travel on this
-library's channels (tensorpipe_amd.torch_rpc). Started by tests/test_torch_rpc*.py, once per rank:
+library's channels (tensorpipe_amd.torch_rpc). Started by tests/test_torch_rpc.py and tests/test_zy_torch_rpc_gpu.py, once per rank:
 
     python tests/torch_rpc_cases.py <rank> <rendezvous file> <mode>
 
