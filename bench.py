@@ -474,8 +474,8 @@ def bench_torch_rpc():
                               stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, cwd=ROOT)
              for r in (1, 0)]
     try:
-        out, _ = ranks[1].communicate(timeout=240)
-        ranks[0].communicate(timeout=60)
+        out, _ = ranks[1].communicate(timeout=120)
+        ranks[0].communicate(timeout=30)
     finally:
         for p in ranks:
             if p.poll() is None:
