@@ -272,8 +272,8 @@ static int sameProcess() {
 
 static int twoProcess(const std::string& channel) {
   const std::string addr = "shm://tpamd_conf2_" + channel + "_" + std::to_string(::getpid());
-  int go[2];
-  if (::pipe(go) != 0) {
+  int go[2], over[2];
+  if (::pipe(go) != 0 || ::pipe(over) != 0) {
     return 3;
   }
   pid_t pid = ::fork(); // before anything has touched the GPU
@@ -287,6 +287,12 @@ static int twoProcess(const std::string& channel) {
     std::string problem = recvMessage(*pipe, 1);
     if (problem.empty()) {
       problem = sendMessage(*pipe, 2);
+    }
+    // A write is over when its bytes have been handed on, which on a route through the host's
+    // transport is before the other end has read them: the pipe stays open until the parent has
+    // the message (the reference's tests end their peers behind a barrier for the same reason).
+    if (::read(over[0], &byte, 1) != 1) {
+      problem = problem.empty() ? "the parent left early" : problem;
     }
     if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() != 6) {
       problem = "the GPU tensors did not all travel on this library's channel";
@@ -308,6 +314,9 @@ static int twoProcess(const std::string& channel) {
   std::string problem = pipe ? sendMessage(*pipe, 1) : std::string("accept failed");
   if (problem.empty()) {
     problem = recvMessage(*pipe, 2);
+  }
+  if (::write(over[1], &byte, 1) != 1) {
+    problem = problem.empty() ? "cannot tell the peer that the exchange is over" : problem;
   }
   int status = 0;
   ::waitpid(pid, &status, 0);

@@ -18,11 +18,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PROGRAM = os.path.join(ROOT, "tests", "cpp", "bin", "stock_conformance")
 
 
-def _run(args):
+def _run(args, env=None):
     if not os.path.exists(PROGRAM):
         pytest.skip("tests/cpp/bin/stock_conformance is not built (no stock TensorPipe headers at build time)")
-    print("running stock_conformance", *args, flush=True)
-    proc = subprocess.run([PROGRAM, *args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    print("running stock_conformance", *args, env or "", flush=True)
+    proc = subprocess.run([PROGRAM, *args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120,
+                          env=dict(os.environ, **(env or {})))
     results = [line for line in proc.stdout.splitlines() if line.startswith("RESULT ")]
     assert results, f"no result line; exit code {proc.returncode}\n{proc.stdout[-2000:]}\n{proc.stderr[-2000:]}"
     bad = [line for line in results if line.split()[2] != "OK"]
@@ -36,6 +37,12 @@ def test_hip_xth_in_a_stock_context_same_process():
 @pytest.mark.parametrize("channel", ["hip_ipc", "hip_basic"])
 def test_channel_in_stock_contexts_of_two_processes(channel):
     _run(["two_process", channel])
+
+
+def test_hip_basic_inner_route_over_the_hosts_connections():
+    """hip_basic without the shared ring: every chunk travels through the CPU channel it wraps, which
+    here runs over the stock pipe's own connections (the route between machines, and to oneself)."""
+    _run(["two_process", "hip_basic"], env={"TP_HIP_BASIC_NO_SHARED_RING": "1"})
 
 
 def test_endpoint_with_hip_channels_talks_to_an_unmodified_peer():
