@@ -15,8 +15,9 @@
 // share the next launch (launchReady below): a caller that moves a message
 // tensor by tensor still gets few launches.
 //
-// Same wire protocol as tensorpipe/channel/cuda_xth/channel_impl.cc:30-36,
-// 96-315 (descriptor one way, empty completion back). Differences, all for
+// The wire protocol of tensorpipe/channel/cuda_xth/channel_impl.cc:30-36,
+// 96-315 (descriptor one way, completion back), with a completion that counts
+// the receives it stands for instead of being empty. Differences, all for
 // latency: a whole message travels in one descriptor and one kernel launch
 // instead of one cudaMemcpyAsync per tensor; there are no start/stop events
 // and no stream waits on the common path (a stream wait costs 12-19 us of host
@@ -202,12 +203,35 @@ class ChannelImpl final : public ChannelImplBase {
     TP_VLOG(6) << "Channel " << id_ << " is writing descriptor (#" << seq << ")";
     writeMessage(*descriptorConnection_, std::move(w.bytes()));
     TP_MARK("xth: descriptor written");
-    TP_VLOG(6) << "Channel " << id_ << " is reading completion (#" << seq << ")";
-    completionConnection_->read(nullptr, 0, onRead([this, op] {
-      TP_VLOG(6) << "Channel " << id_ << " done reading completion (#" << op->seq << ")";
+    armCompletionRead();
+  }
+
+  // One read is kept posted while sends are out. A completion message names
+  // how many of them, oldest first, the receiver has copied: receives that
+  // shared a launch are reported together.
+  void armCompletionRead() {
+    if (completionReadArmed_ || sendOps_.empty() || error_) {
+      return;
+    }
+    completionReadArmed_ = true;
+    TP_VLOG(6) << "Channel " << id_ << " is reading a completion";
+    completionConnection_->read(&completedSends_, sizeof(completedSends_), onRead([this] {
+      completionReadArmed_ = false;
+      if (error_) {
+        return;
+      }
       TP_MARK("xth: completion arrived (send callback)");
-      removeSend(op);
-      finishSend(op);
+      if (completedSends_ == 0 || completedSends_ > sendOps_.size()) {
+        setError(TP_CREATE_ERROR(ShortReadError, static_cast<ssize_t>(sendOps_.size()), completedSends_));
+        return;
+      }
+      for (uint32_t k = 0; k < completedSends_ && !sendOps_.empty(); ++k) {
+        auto op = sendOps_.front();
+        sendOps_.pop_front();
+        TP_VLOG(6) << "Channel " << id_ << " done reading completion (#" << op->seq << ")";
+        finishSend(op);
+      }
+      armCompletionRead();
     }));
   }
 
@@ -417,6 +441,7 @@ class ChannelImpl final : public ChannelImplBase {
   // Completions go out in the order the descriptors came in (the sender pairs
   // them by position), each once its copies have finished.
   void flushRecvs() {
+    uint32_t finished = 0;
     while (!recvOps_.empty() && recvOps_.front()->copied && !error_) {
       auto op = recvOps_.front();
       recvOps_.pop_front();
@@ -427,17 +452,13 @@ class ChannelImpl final : public ChannelImplBase {
       // wants to be (the other order saves the sender a microsecond and costs
       // such a caller ten: its next write starts on a foreign thread).
       finishRecv(op);
-      TP_VLOG(6) << "Channel " << id_ << " is writing completion (#" << op->seq << ")";
-      completionConnection_->write(nullptr, 0, onWritten([] {}));
+      ++finished;
     }
-  }
-
-  void removeSend(const std::shared_ptr<SendOp>& op) {
-    for (auto it = sendOps_.begin(); it != sendOps_.end(); ++it) {
-      if (*it == op) {
-        sendOps_.erase(it);
-        return;
-      }
+    if (finished > 0 && !error_) {
+      TP_VLOG(6) << "Channel " << id_ << " is writing the completion of " << finished << " receive(s)";
+      WireWriter w;
+      w.u32(finished);
+      writeMessage(*completionConnection_, std::move(w.bytes()));
     }
   }
 
@@ -468,6 +489,8 @@ class ChannelImpl final : public ChannelImplBase {
   std::vector<std::shared_ptr<RecvOp>> toLaunch_;
   uint64_t toLaunchBytes_{0};
   size_t launchesInFlight_{0};
+  bool completionReadArmed_{false};
+  uint32_t completedSends_{0}; // the posted completion read lands here
   size_t decodedInQueue_{0}; // members of recvOps_ whose descriptor has come in (they sit at its front)
   static constexpr uint64_t kGatherBytes = 8u << 20;
   static constexpr size_t kGatherOps = 256;
