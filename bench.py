@@ -289,6 +289,62 @@ def bench_rpc_message(messages=500, warmup=20):
     }
 
 
+def bench_rpc_message_in_flight(depth=3, messages=1200):
+    """configs[4]'s message with several in flight on the same pipes: `depth` chains of write/read
+    side by side (one caller thread each, receive buffers and stream of their own)."""
+    import threading
+
+    import torch
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    sizes = [int(s) for s in datagen.loguniform_sizes(datagen.SEED_BASE + 5, 256, 4 * MIB, 256)]
+    total = sum(sizes)
+    arena_src = torch.zeros(total + 16 * len(sizes), dtype=torch.uint8, device="cuda")
+    arena_src.random_(0, 256)
+    dsts = [torch.zeros_like(arena_src) for _ in range(depth)]
+    send_stream = torch.cuda.Stream()
+    recv_streams = [torch.cuda.Stream() for _ in range(depth)]
+    st, rts, off = [], [[] for _ in range(depth)], 0
+    for n in sizes:
+        st.append(tp.make_tensor(arena_src.data_ptr() + off, nbytes=n, device=tp.HIP, stream=send_stream,
+                                 target=(tp.HIP, 0)))
+        for k in range(depth):
+            rts[k].append(tp.make_tensor(dsts[k].data_ptr() + off, nbytes=n, device=tp.HIP,
+                                         stream=recv_streams[k]))
+        off += (n + 15) // 16 * 16
+    objs = make_pair("basic:0,hip_xth:10")
+    torch.cuda.synchronize()
+    for k in range(depth):  # every chain's buffers and stream have been used once before the clock starts
+        tp.bench_transfer(objs[0], objs[1], st, rts[k], warmup=0, iters=10)
+    per_chain = messages // depth
+    lined_up = threading.Barrier(depth + 1)
+
+    def chain(k):
+        lined_up.wait()
+        tp.bench_transfer(objs[0], objs[1], st, rts[k], warmup=0, iters=per_chain)
+
+    threads = [threading.Thread(target=chain, args=(k,)) for k in range(depth)]
+    for t in threads:
+        t.start()
+    lined_up.wait()
+    t0 = time.perf_counter()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    done = per_chain * depth
+    ok, o = True, 0
+    for n in sizes:  # the padding between tensors is not part of any message
+        ok = ok and all(bool(torch.equal(arena_src[o:o + n], d[o:o + n])) for d in dsts)
+        o += (n + 15) // 16 * 16
+    destroy(objs)
+    return {"in_flight": depth, "messages": done, "tensors": len(sizes), "total_bytes": total,
+            "us_per_message": dt / done * 1e6, "payload_GBps": total * done / dt / 1e9,
+            "hbm_frac": 2.0 * total * done / dt / 1e9 / HBM_PEAK_GBPS, "byte_exact": ok}
+
+
 class PeerRun:
     """A bench_peer child process connected through one pipe."""
 
@@ -655,6 +711,7 @@ def cpu_baseline():
 # runtime does on later launches, which shifts small-transfer latencies by microseconds).
 LEGS = {
     "rpc_message": bench_rpc_message,
+    "rpc_message_in_flight": bench_rpc_message_in_flight,
     "d2d_in_flight": bench_d2d_in_flight,
     "ipc": bench_ipc,
     "staged": bench_staged,
@@ -741,6 +798,7 @@ def main():
     if not args.skip_extras:
         log("[bench] many-tensor message (256 tensors, one launch per message)")
         extra["rpc_message"] = extra_leg("rpc_message")
+        extra["rpc_message_in_flight"] = extra_leg("rpc_message_in_flight")
         log("[bench] cross-process IPC sweep")
         extra["ipc"] = extra_leg("ipc")
         log("[bench] host-staged 256 MiB")
