@@ -434,18 +434,30 @@ int tpc_op_wait(tpc_op* op, int timeoutMs) {
 // (tensorpipe/benchmark/benchmark_pipe.cc:463-468,571-577): the write of step
 // k+1 is issued from whichever callback of step k (write done, read done) fires
 // last, on the library's threads. The caller only waits for the end.
+// One message after the other from `sender` to `receiver`. Each end carries on
+// from its own callback -- the sender writes message k+1 when its write of
+// message k has completed, the receiver asks for descriptor k+1 when its read
+// of message k has completed -- so that each end's work stays on the threads
+// that serve that end, as it would between two programs (issuing both from
+// whichever callback came last puts the sender's work on the receiver's thread
+// half of the time). A round is over when both of its halves are.
 struct TransferChain : std::enable_shared_from_this<TransferChain> {
   using Clock = std::chrono::steady_clock;
   std::shared_ptr<Pipe> sender, receiver;
   std::vector<tpc_payload> payloads;
   std::vector<void*> recvPayloadPtrs;
   std::vector<tpc_tensor> sendTensors, recvTensors;
-  uint32_t warmup{0}, iters{0}, round{0};
+  uint32_t warmup{0}, iters{0};
   double* perIterUs{nullptr};
-  Clock::time_point begin, end, t0;
-  std::atomic<int> pending{0};
+  Clock::time_point begin, end;
+  std::vector<Clock::time_point> issued;
+  std::unique_ptr<std::atomic<int>[]> halves; // per round: completed halves
   Completion finished;
   std::atomic<bool> failed{false};
+
+  uint32_t total() const {
+    return warmup + iters;
+  }
 
   void fail(const Error& e) {
     if (!failed.exchange(true)) {
@@ -453,48 +465,63 @@ struct TransferChain : std::enable_shared_from_this<TransferChain> {
     }
   }
 
-  void halfDone(const Error& e) {
-    if (e) {
-      fail(e);
-      return;
+  void start() {
+    issued.resize(total());
+    halves.reset(new std::atomic<int>[total() > 0 ? total() : 1]);
+    for (uint32_t r = 0; r < total(); ++r) {
+      halves[r].store(0, std::memory_order_relaxed);
     }
-    if (pending.fetch_sub(1, std::memory_order_acq_rel) != 1) {
-      return;
-    }
-    try {
-      StageScope syncTimer(Stage::kHarnessSync);
-      syncRecvStreams(recvTensors.data(), static_cast<uint32_t>(recvTensors.size()));
-    } catch (const std::exception&) {
-      fail(TP_CREATE_ERROR(HipError, "stream sync", TPHIP_ERR_INVALID_ARG));
-      return;
-    }
-    if (round >= warmup && perIterUs != nullptr) {
-      perIterUs[round - warmup] = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
-    }
-    TP_MARK("harness: step over");
-    ++round;
-    step();
-  }
-
-  void step() {
-    if (round == warmup + iters) {
-      end = Clock::now();
+    if (total() == 0) {
+      begin = end = Clock::now();
       finished.set(Error::kSuccess);
       return;
     }
-    if (round == warmup) {
-      begin = Clock::now();
+    armRead(0);
+    issueWrite(0);
+  }
+
+  void halfDone(uint32_t round) {
+    if (halves[round].fetch_add(1, std::memory_order_acq_rel) != 1) {
+      return;
     }
+    const auto now = Clock::now();
+    if (round >= warmup && perIterUs != nullptr) {
+      perIterUs[round - warmup] = std::chrono::duration<double, std::micro>(now - issued[round]).count();
+    }
+    TP_MARK("harness: step over");
+    if (round + 1 == total()) {
+      end = now;
+      finished.set(Error::kSuccess);
+    }
+  }
+
+  void issueWrite(uint32_t round) {
     auto self = shared_from_this();
-    t0 = Clock::now();
-    pending.store(2, std::memory_order_release);
+    issued[round] = Clock::now();
+    if (round == warmup) {
+      begin = issued[round];
+    }
     optional<StageScope> makeTimer;
     makeTimer.emplace(Stage::kHarnessMakeMessage);
     Message message = makeMessage(
         "", payloads.data(), static_cast<uint32_t>(payloads.size()), sendTensors.data(),
         static_cast<uint32_t>(sendTensors.size()));
     makeTimer.reset();
-    receiver->readDescriptor([self](const Error& e, Descriptor) {
+    sender->write(std::move(message), [self, round](const Error& e) {
+      if (e) {
+        self->fail(e);
+        return;
+      }
+      self->halfDone(round);
+      if (round + 1 < self->total() && !self->failed.load()) {
+        self->issueWrite(round + 1);
+      }
+    });
+  }
+
+  void armRead(uint32_t round) {
+    auto self = shared_from_this();
+    receiver->readDescriptor([self, round](const Error& e, Descriptor) {
       if (e) {
         self->fail(e);
         return;
@@ -503,9 +530,25 @@ struct TransferChain : std::enable_shared_from_this<TransferChain> {
           makeAllocation(
               self->recvPayloadPtrs.data(), static_cast<uint32_t>(self->recvPayloadPtrs.size()),
               self->recvTensors.data(), static_cast<uint32_t>(self->recvTensors.size())),
-          [self](const Error& e2) { self->halfDone(e2); });
+          [self, round](const Error& e2) {
+            if (e2) {
+              self->fail(e2);
+              return;
+            }
+            try {
+              // the bytes are where a reader of these buffers would look before the round counts
+              StageScope syncTimer(Stage::kHarnessSync);
+              syncRecvStreams(self->recvTensors.data(), static_cast<uint32_t>(self->recvTensors.size()));
+            } catch (const std::exception&) {
+              self->fail(TP_CREATE_ERROR(HipError, "stream sync", TPHIP_ERR_INVALID_ARG));
+              return;
+            }
+            self->halfDone(round);
+            if (round + 1 < self->total() && !self->failed.load()) {
+              self->armRead(round + 1);
+            }
+          });
     });
-    sender->write(std::move(message), [self](const Error& e) { self->halfDone(e); });
   }
 };
 
@@ -533,7 +576,7 @@ int tpc_bench_transfer(
   chain->warmup = warmup;
   chain->iters = iters;
   chain->perIterUs = perIterUs;
-  chain->step();
+  chain->start();
   int rc = chain->finished.wait(600000);
   if (rc != 0) {
     return rc;
