@@ -35,7 +35,7 @@ def main():
             legs = {}
             for nbytes, iters in ((4096, 300), (1 << 20, 200), (64 << 20, 30)):
                 x = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g).to(device)
-                for _ in range(5):
+                for _ in range(30):
                     y = rpc.rpc_sync("w1", echo, args=(x,))
                 times = []
                 for _ in range(iters):
