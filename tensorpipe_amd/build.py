@@ -102,6 +102,18 @@ def build_cpp_tests():
              "-Wl,-rpath,$ORIGIN/../../../tensorpipe_amd/lib"])
 
 
+def build_fake_tphip(extra_flags=()):
+    """tests/cpp/bin/fake/libtphip.so: the C ABI of include/tphip.h without a GPU behind it
+    (tests/cpp/fake_tphip.cc). The C++ test programs load it instead of the real library when
+    LD_LIBRARY_PATH names its directory, so the channels' host logic runs on the CPU."""
+    out_dir = os.path.join(ROOT, "tests", "cpp", "bin", "fake")
+    os.makedirs(out_dir, exist_ok=True)
+    run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-Wno-unused-parameter",
+         "-pthread", *extra_flags, f"-I{INCLUDE}", os.path.join(ROOT, "tests", "cpp", "fake_tphip.cc"),
+         "-o", os.path.join(out_dir, "libtphip.so")])
+    return out_dir
+
+
 def stock_tensorpipe():
     """(include dir, lib dir) of the TensorPipe that PyTorch ships prebuilt, or None."""
     try:
@@ -178,6 +190,7 @@ def build_all():
     build_datagen()
     build_host()
     build_cpp_tests()
+    build_fake_tphip()
     build_stock_conformance()
     build_torch_rpc_plugin()
 

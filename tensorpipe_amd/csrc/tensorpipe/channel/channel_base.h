@@ -8,6 +8,7 @@
 
 #include <atomic>
 #include <cstring>
+#include <future>
 #include <memory>
 #include <string>
 #include <unordered_set>
@@ -60,9 +61,20 @@ class ContextCore : public std::enable_shared_from_this<ContextCore> {
   // Subclasses with threads or device resources stop/release them here;
   // called once, after close, from join().
   virtual void joinImpl() {}
+  // close() only queues the closing on the loop, and a queued task may be run
+  // later by another thread: the closing must have happened before joinImpl()
+  // stops the threads that in-flight operations still need, so a second task
+  // is queued behind it and awaited, as
+  // tensorpipe/channel/context_impl_boilerplate.h:242-264 does.
   void join() {
     close();
     if (!joined_.exchange(true)) {
+      if (!inLoop()) {
+        auto closed = std::make_shared<std::promise<void>>();
+        auto done = closed->get_future();
+        defer([closed] { closed->set_value(); });
+        done.wait();
+      }
       joinImpl();
     }
   }

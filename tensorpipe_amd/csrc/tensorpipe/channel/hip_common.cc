@@ -44,20 +44,50 @@ HipEventPoller::~HipEventPoller() {
 
 void HipEventPoller::watch(std::unique_ptr<HipEvent> event, HipEventPool* pool, TCallback fn) {
   {
-    std::lock_guard<std::mutex> lock(mutex_);
-    incoming_.push_back(Item{std::move(event), nullptr, pool, std::move(fn)});
-    incomingPending_.store(true, std::memory_order_release);
+    std::unique_lock<std::mutex> lock(mutex_);
+    if (!stopping_) {
+      incoming_.push_back(Item{std::move(event), nullptr, pool, std::move(fn)});
+      incomingPending_.store(true, std::memory_order_release);
+      lock.unlock();
+      cv_.notify_one();
+      return;
+    }
   }
-  cv_.notify_one();
+  // The thread is on its way out and may never look again: the caller waits
+  // for the GPU itself. Every callback still runs exactly once.
+  int rc = 0;
+  for (int done = 0; rc == 0 && done == 0;) {
+    rc = tphip_event_query(event->device(), event->raw(), &done);
+    if (rc == 0 && done == 0) {
+      std::this_thread::yield();
+    }
+  }
+  fn(rc != 0 ? TP_CREATE_ERROR(HipError, "tphip_event_query", rc) : Error::kSuccess);
+  if (pool != nullptr) {
+    pool->put(std::move(event));
+  }
 }
 
 void HipEventPoller::watchCondition(TCheck check, TCallback fn) {
   {
-    std::lock_guard<std::mutex> lock(mutex_);
-    incoming_.push_back(Item{nullptr, std::move(check), nullptr, std::move(fn)});
-    incomingPending_.store(true, std::memory_order_release);
+    std::unique_lock<std::mutex> lock(mutex_);
+    if (!stopping_) {
+      incoming_.push_back(Item{nullptr, std::move(check), nullptr, std::move(fn)});
+      incomingPending_.store(true, std::memory_order_release);
+      lock.unlock();
+      cv_.notify_one();
+      return;
+    }
   }
-  cv_.notify_one();
+  // Nobody is left to keep looking, and what is awaited may depend on a peer:
+  // one look, then the operation fails.
+  bool happened = false;
+  const int rc = check(&happened);
+  if (rc == 0 && happened) {
+    fn(Error::kSuccess);
+  } else {
+    fn(TP_CREATE_ERROR(HipError, "completion check after the context was joined", rc != 0 ? rc : TPHIP_ERR_BUSY));
+  }
 }
 
 void HipEventPoller::join() {

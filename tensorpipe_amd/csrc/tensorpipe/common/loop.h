@@ -9,19 +9,32 @@
 //                 condition variable.
 //
 // Whose tasks a draining thread runs depends on whose thread it is. A thread
-// the library created (transport reactor, event poller, ThreadLoop) runs
-// whatever is queued, also what other threads add meanwhile. A thread of the
-// application that entered through send/recv/write/read runs only what it
-// queued itself: a completion that a library thread queues at that moment
-// would otherwise run the application's callback on the application's own
-// stack, inside the very call that started the operation -- and a caller that
-// holds a lock its callback also takes would deadlock (the reference checks
-// for exactly that: tensorpipe/test/channel/channel_test_cpu.cc:44-109). The
-// library thread instead waits the few microseconds until the application's
-// thread has left the loop and drains the queue itself.
+// the library created (transport reactor, event poller, ThreadLoop, helper)
+// runs whatever is queued, also what other threads add meanwhile. A thread of
+// the application that entered through send/recv/write/read runs only what it
+// queued itself: a completion that another thread queues at that moment would
+// otherwise run the application's callback on the application's own stack,
+// inside the very call that started the operation -- and a caller that holds a
+// lock its callback also takes would deadlock (the reference checks for
+// exactly that: tensorpipe/test/channel/channel_test_cpu.cc:44-109).
+//
+// Who then runs such a task:
+//  * a library thread that is not inside a task of any loop waits a few
+//    microseconds (bounded) for the application's thread to leave and drains
+//    the queue itself: the common case, a reactor or poller thread delivering
+//    a completion while the application is still inside its call;
+//  * every other thread returns from defer() at once, as the reference's
+//    executor always does (tensorpipe/common/deferred_executor.h:101-124): a
+//    thread inside a task of another loop may be exactly what the draining
+//    thread's task is waiting for (two threads, each in a task of one loop and
+//    deferring to the other's, would wait for each other for good), and an
+//    application thread may hold a lock the draining task wants. The draining
+//    thread, when it leaves with other threads' tasks still queued and nobody
+//    waiting to take over, hands the loop to a helper thread of the library.
 #pragma once
 
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <cstdlib>
 #include <deque>
@@ -29,7 +42,9 @@
 #include <mutex>
 #include <thread>
 
+#include <pthread.h>
 #include <sched.h>
+#include <unistd.h>
 
 #include <tensorpipe/common/defs.h>
 
@@ -42,6 +57,22 @@ inline bool& thisIsLibraryThread() {
   static thread_local bool flag = false;
   return flag;
 }
+
+// How many tasks of this library's loops (any of them) are on the calling
+// thread's stack.
+inline int& loopTaskDepth() {
+  static thread_local int depth = 0;
+  return depth;
+}
+
+struct LoopTaskScope {
+  LoopTaskScope() {
+    ++loopTaskDepth();
+  }
+  ~LoopTaskScope() {
+    --loopTaskDepth();
+  }
+};
 
 // Whether this process has fewer CPUs to run on (affinity mask, pinned
 // containers) than a pipe keeps busy at full tilt: the caller, the context's
@@ -62,11 +93,95 @@ inline bool runsOnFewCpus() {
   return few;
 }
 
+// Library threads that drain on-demand loops whose application-thread drainer
+// left other threads' tasks behind. Started on first need; one more is started
+// whenever work comes in and none is idle (a user's callback may block the one
+// that runs it), up to a small limit; an idle one leaves after a second. Never
+// destroyed: threads of it may still run when static destructors do.
+class LoopHelpers {
+ public:
+  static LoopHelpers& get() {
+    static LoopHelpers* const instance = [] {
+      auto* h = new LoopHelpers();
+      // A forked child has none of the parent's threads.
+      ::pthread_atfork(nullptr, nullptr, [] { new (&LoopHelpers::get()) LoopHelpers(); });
+      return h;
+    }();
+    return *instance;
+  }
+
+  void post(TTask work) {
+    bool spawn = false;
+    {
+      std::unique_lock<std::mutex> lock(mutex_);
+      queue_.push_back(std::move(work));
+      if (idle_ == 0 && threads_ < kMaxThreads) {
+        ++threads_;
+        spawn = true;
+      }
+    }
+    if (spawn) {
+      std::thread([this] { run(); }).detach();
+    } else {
+      cv_.notify_one();
+    }
+  }
+
+ private:
+  static constexpr unsigned kMaxThreads = 8;
+
+  void run() {
+    thisIsLibraryThread() = true;
+    ::pthread_setname_np(::pthread_self(), "tp_loop_helper");
+    std::unique_lock<std::mutex> lock(mutex_);
+    for (;;) {
+      while (!queue_.empty()) {
+        TTask work = std::move(queue_.front());
+        queue_.pop_front();
+        lock.unlock();
+        work();
+        work = nullptr;
+        lock.lock();
+      }
+      ++idle_;
+      const bool more = cv_.wait_for(lock, std::chrono::seconds(1), [this] { return !queue_.empty(); });
+      --idle_;
+      if (!more) {
+        --threads_;
+        return;
+      }
+    }
+  }
+
+  std::mutex mutex_;
+  std::condition_variable cv_;
+  std::deque<TTask> queue_;
+  unsigned threads_{0};
+  unsigned idle_{0};
+};
+
 class OnDemandLoop {
  public:
+  OnDemandLoop() = default;
+  OnDemandLoop(const OnDemandLoop&) = delete;
+  OnDemandLoop& operator=(const OnDemandLoop&) = delete;
+
+  // Waits for a helper that still has this loop on its list. Like the queue
+  // itself, not to be destroyed from inside one of its own tasks.
+  ~OnDemandLoop() {
+    for (;;) {
+      {
+        std::unique_lock<std::mutex> lock(mutex_);
+        if (helperRefs_ == 0) {
+          return;
+        }
+      }
+      std::this_thread::yield();
+    }
+  }
+
   void defer(TTask fn) {
     const std::thread::id me = std::this_thread::get_id();
-    bool wait = false;
     {
       std::unique_lock<std::mutex> lock(mutex_);
       queue_.push_back(Item{std::move(fn), me});
@@ -75,57 +190,46 @@ class OnDemandLoop {
           return; // the draining thread will get to it
         }
         // An application thread is draining: it leaves our task alone.
+        if (!thisIsLibraryThread() || loopTaskDepth() > 0) {
+          return; // may not wait (see the top of this file); a helper will run it
+        }
         ++waiters_;
-        wait = true;
       } else {
-        draining_ = true;
-        drainer_ = me;
-        guestDrainer_ = !thisIsLibraryThread();
+        takeOver(me);
+        lock.unlock();
+        drain(me);
+        return;
       }
     }
-    if (wait) {
-      for (unsigned spins = 0;; ++spins) {
-        {
-          std::unique_lock<std::mutex> lock(mutex_);
-          if (!draining_) {
-            --waiters_;
-            draining_ = true;
-            drainer_ = me;
-            guestDrainer_ = !thisIsLibraryThread();
-            break;
-          }
-          if (!guestDrainer_) {
-            --waiters_;
-            return; // a library thread took over and will run it
-          }
-        }
-        if (spins < 2000) {
-#if defined(__x86_64__)
-          __builtin_ia32_pause();
-#endif
-        } else {
-          std::this_thread::yield();
-        }
-      }
-    }
-    owner_.store(me, std::memory_order_relaxed);
-    for (;;) {
-      TTask task;
+    // A library thread with no task of any loop on its stack: wait, briefly,
+    // for the application's thread to leave.
+    const auto giveUpAt = std::chrono::steady_clock::now() + std::chrono::microseconds(kMaxWaitUs);
+    for (unsigned spins = 0;; ++spins) {
       {
         std::unique_lock<std::mutex> lock(mutex_);
-        // A guest stops at the first task that is not its own when that task's
-        // owner is waiting to take over; with nobody waiting it carries on, so
-        // that no task is left behind.
-        if (queue_.empty() || (guestDrainer_ && queue_.front().from != me && waiters_ > 0)) {
-          owner_.store(std::thread::id(), std::memory_order_relaxed);
-          draining_ = false;
-          return;
+        if (!draining_) {
+          --waiters_;
+          takeOver(me);
+          break;
         }
-        task = std::move(queue_.front().fn);
-        queue_.pop_front();
+        if (!guestDrainer_) {
+          --waiters_;
+          return; // a library thread took over and will run it
+        }
+        if ((spins & 63) == 63 && std::chrono::steady_clock::now() > giveUpAt) {
+          --waiters_;
+          return; // the drainer finds nobody waiting when it leaves and calls a helper
+        }
       }
-      task();
+      if (spins < 2000) {
+#if defined(__x86_64__)
+        __builtin_ia32_pause();
+#endif
+      } else {
+        std::this_thread::yield();
+      }
     }
+    drain(me);
   }
 
   bool inLoop() const {
@@ -133,16 +237,78 @@ class OnDemandLoop {
   }
 
  private:
+  static constexpr int kMaxWaitUs = 100;
+
   struct Item {
     TTask fn;
     std::thread::id from;
   };
+
+  // mutex_ held.
+  void takeOver(std::thread::id me) {
+    draining_ = true;
+    drainer_ = me;
+    guestDrainer_ = !thisIsLibraryThread();
+  }
+
+  void drain(std::thread::id me) {
+    owner_.store(me, std::memory_order_relaxed);
+    for (;;) {
+      TTask task;
+      {
+        std::unique_lock<std::mutex> lock(mutex_);
+        if (queue_.empty()) {
+          owner_.store(std::thread::id(), std::memory_order_relaxed);
+          draining_ = false;
+          return;
+        }
+        if (guestDrainer_ && queue_.front().from != me) {
+          // Not this application thread's task. Whoever waits takes over; with
+          // nobody waiting a helper is called.
+          owner_.store(std::thread::id(), std::memory_order_relaxed);
+          draining_ = false;
+          if (waiters_ == 0 && !helperCalled_) {
+            helperCalled_ = true;
+            ++helperRefs_;
+            lock.unlock();
+            LoopHelpers::get().post([this] { drainAsHelper(); });
+          }
+          return;
+        }
+        task = std::move(queue_.front().fn);
+        queue_.pop_front();
+      }
+      LoopTaskScope scope;
+      task();
+    }
+  }
+
+  void drainAsHelper() {
+    const std::thread::id me = std::this_thread::get_id();
+    {
+      std::unique_lock<std::mutex> lock(mutex_);
+      helperCalled_ = false;
+      // Somebody drains already: a library thread runs everything, an
+      // application thread calls again when it leaves.
+      if (draining_ || queue_.empty()) {
+        --helperRefs_;
+        return;
+      }
+      takeOver(me);
+    }
+    drain(me);
+    std::unique_lock<std::mutex> lock(mutex_);
+    --helperRefs_;
+  }
+
   std::mutex mutex_;
   std::deque<Item> queue_;
   bool draining_{false};
   bool guestDrainer_{false}; // the draining thread belongs to the application
+  bool helperCalled_{false}; // a helper is on its way and has not looked yet
   std::thread::id drainer_;
-  unsigned waiters_{0}; // threads waiting for a guest drainer to leave
+  unsigned waiters_{0}; // library threads waiting for a guest drainer to leave
+  unsigned helperRefs_{0}; // helpers that will still touch this object
   std::atomic<std::thread::id> owner_{std::thread::id()};
 };
 
@@ -193,7 +359,11 @@ class ThreadLoop {
         TTask task = std::move(queue_.front());
         queue_.pop_front();
         lock.unlock();
-        task();
+        {
+          LoopTaskScope scope;
+          task();
+        }
+        task = nullptr;
         lock.lock();
       }
       if (stopping_) {

@@ -33,6 +33,7 @@
 #include <vector>
 
 #include <tensorpipe/common/defs.h>
+#include <tensorpipe/common/loop.h>
 #include <tensorpipe/transport/connection.h>
 #include <tensorpipe/transport/error.h>
 #include <tensorpipe/transport/listener.h>
@@ -210,6 +211,7 @@ class Reactor final : public std::enable_shared_from_this<Reactor> {
 
  private:
   void run() {
+    thisIsLibraryThread() = true;
     std::vector<epoll_event> events(64);
     // After an event the loop keeps asking without sleeping for a short while:
     // in a ping-pong the next message is a few microseconds away, and a wake-up
@@ -505,7 +507,7 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
     while (!reads_.empty() && !error_) {
       ReadOp& op = reads_.front();
       if (headerDone_ < kHeader) {
-        const ssize_t r = ::recv(fd_, header_ + headerDone_, kHeader - headerDone_, 0);
+        const ssize_t r = recvRetrying(header_ + headerDone_, kHeader - headerDone_);
         if (!absorb(r)) {
           return;
         }
@@ -543,7 +545,7 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
           }
         }
         uint8_t* dst = op.exact ? op.ptr : scratch_.data();
-        const ssize_t r = ::recv(fd_, dst + payloadDone_, static_cast<size_t>(room), 0);
+        const ssize_t r = recvRetrying(dst + payloadDone_, static_cast<size_t>(room));
         if (!absorb(r)) {
           return;
         }
@@ -557,6 +559,17 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
     }
   }
 
+  // recv() that starts over when a signal cut it short: after the hang-up has
+  // taken the socket out of the epoll set nothing else would ask again.
+  ssize_t recvRetrying(uint8_t* dst, size_t room) {
+    for (;;) {
+      const ssize_t r = ::recv(fd_, dst, room, 0);
+      if (r >= 0 || errno != EINTR) {
+        return r;
+      }
+    }
+  }
+
   // Whether recv's result is bytes to use; EOF and errors fail the connection,
   // "nothing yet" just returns false.
   bool absorb(ssize_t r) {
@@ -567,8 +580,8 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       fail(TP_CREATE_ERROR(EOFError));
       return false;
     }
-    if (errno == EAGAIN || errno == EWOULDBLOCK || errno == EINTR) {
-      if (peerClosed_ && errno != EINTR) {
+    if (errno == EAGAIN || errno == EWOULDBLOCK) {
+      if (peerClosed_) {
         // the hang-up was seen and the socket is drained
         fail(TP_CREATE_ERROR(EOFError));
       }

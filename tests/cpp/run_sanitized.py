@@ -1,13 +1,18 @@
 #!/usr/bin/env python3
 """Builds the host library and the C++ test programs with a sanitizer and runs the CPU suites.
 
-    python tests/cpp/run_sanitized.py thread|address [build_dir] [--build-only | --run-only] [--gpu]
+    python tests/cpp/run_sanitized.py thread|address [build_dir] [--build-only | --run-only] [--gpu | --stand-in]
 
 Host code only (g++ -fsanitize=...); libtphip.so is used as built. With --gpu the suites of the
 device channels run instead of the CPU ones (on a machine with a GPU; --build-only on one machine
 and --run-only on another share a build directory; next to the HIP runtime AddressSanitizer needs
 ASAN_OPTIONS=use_sigaltstack=0:protect_shadow_gap=0:detect_leaks=0, and ThreadSanitizer does not
-work at all: the runtime finds no device under its address-space layout). Not collected by pytest: a
+work at all: the runtime finds no device under its address-space layout). With --stand-in the same
+device-channel suites run on the CPU against tests/cpp/fake_tphip.cc, the host-only stand-in for
+libtphip.so built with the same sanitizer (streams are threads, copies are memcpy, events and signal
+words are real synchronisation): the channels' host logic, which ThreadSanitizer cannot see next to
+the HIP runtime, is checked there, a missing wait between a copy and its consumer included; the
+executor cases (unit_tests loops) run in every mode. Not collected by pytest: a
 full pass takes several minutes. The shm transport tells ThreadSanitizer about the hand-off
 through its rings (two mappings of one segment inside a process), so a clean run reports
 nothing; any "WARNING: ThreadSanitizer" / "ERROR: AddressSanitizer" line fails the run.
@@ -34,6 +39,9 @@ GPU_SUITES = [("channel_tests", "hip_xth", False), ("channel_tests", "hip_ipc", 
               ("pipe_tests", "two_process", True)]
 
 
+STAND_IN_SUITES = GPU_SUITES + [("channel_tests", "hip_ipc_gated", False), ("channel_tests", "hip_ipc_messages", False)]
+
+
 def main():
     words = [a for a in sys.argv[1:] if not a.startswith("--")]
     options = {a for a in sys.argv[1:] if a.startswith("--")}
@@ -46,6 +54,11 @@ def main():
         return
     if "--gpu" in options:
         sys.exit(1 if run_suites(out, GPU_SUITES) else 0)
+    if "--stand-in" in options:
+        env = dict(os.environ, LD_LIBRARY_PATH=os.path.join(out, "fake"))
+        bad = run_suites(out, STAND_IN_SUITES, env)
+        bad += run_unit(out, ["loops"], env)
+        sys.exit(1 if bad else 0)
     run_cpu(out)
 
 
@@ -60,6 +73,10 @@ def build(san, out):
 
     with ThreadPoolExecutor(max_workers=8) as pool:
         list(pool.map(compile_one, zip(tp_build.HOST_SOURCES, objs)))
+    # the stand-in for libtphip.so, sanitized like the rest (chosen at run time by LD_LIBRARY_PATH)
+    os.makedirs(os.path.join(out, "fake"), exist_ok=True)
+    subprocess.run(["g++", *flags, "-shared", os.path.join(ROOT, "tests", "cpp", "fake_tphip.cc"), "-o",
+                    os.path.join(out, "fake", "libtphip.so")], check=True)
     lib = os.path.join(out, "libtensorpipe_amd.so")
     subprocess.run(["g++", "-shared", f"-fsanitize={san}", "-pthread", "-o", lib, *objs, f"-L{tp_build.LIB}",
                     "-ltphip", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
@@ -69,10 +86,23 @@ def build(san, out):
                         f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
 
 
-def run_suites(out, suites):
+def run_unit(out, args, env=None):
+    proc = subprocess.run([os.path.join(out, "unit_tests"), *args],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900, env=env)
+    reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+    lines = proc.stdout.strip().splitlines()
+    ok = proc.returncode == 0 and bool(lines) and lines[-1].startswith("OK")
+    print(f"unit_tests {args[0]}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
+    for l in reports[:5] + ([] if ok else lines[-5:]):
+        print("   ", l[:200])
+    sys.stdout.flush()
+    return (0 if ok else 1) + len(reports)
+
+
+def run_suites(out, suites, base_env=None):
     bad = 0
     for prog, suite, stock_wire in suites:
-        env = dict(os.environ, TP_STOCK_WIRE="1") if stock_wire else None
+        env = dict(base_env or os.environ, TP_STOCK_WIRE="1") if stock_wire else base_env
         proc = subprocess.run([os.path.join(out, prog), "--suite", suite], stdout=subprocess.PIPE,
                               stderr=subprocess.STDOUT, text=True, timeout=1800, env=env)
         results = [l for l in proc.stdout.splitlines() if l.startswith("RESULT")]
@@ -88,6 +118,7 @@ def run_suites(out, suites):
 
 def run_cpu(out):
     bad = run_suites(out, SUITES)
+    bad += run_unit(out, ["loops"])
     # random bytes where a pipe's first packets belong
     for seed in (11, 12, 13):
         proc = subprocess.run([os.path.join(out, "unit_tests"), "garbage", str(seed), "150"],

@@ -9,6 +9,12 @@
 //
 //   stock_conformance same_process   hip_xth between two contexts of this process
 //   stock_conformance two_process    hip_ipc and hip_basic between this process and a child
+//   stock_conformance to_self <channel> <rounds>
+//       ONE context with a pipe to itself, as an RPC agent has for calls to its
+//       own rank, messages travelling both ways at the same moment from
+//       threads of the application: with hip_basic every GPU tensor then takes
+//       the route through the wrapped CPU channel, whose loop and the staged
+//       channel's own loop are both driven by whichever thread comes by
 //
 // Prints "RESULT <case> OK" or "RESULT <case> FAIL <why>" per case.
 #include <tensorpipe/tensorpipe.h>
@@ -103,6 +109,19 @@ struct GpuTensor {
   }
 };
 
+// Frees the tensors of a message when the function that made them returns.
+struct GpuTensors : std::vector<GpuTensor> {
+  GpuTensors() = default;
+  GpuTensors(const GpuTensors&) = delete;
+  ~GpuTensors() {
+    for (auto& t : *this) {
+      tphip_stream_sync(0, t.stream);
+      tphip_free(0, t.dev);
+      tphip_stream_destroy(0, t.stream);
+    }
+  }
+};
+
 static GpuTensor makeGpu(size_t bytes) {
   GpuTensor t;
   t.bytes = bytes;
@@ -119,7 +138,7 @@ static const std::string kPayload = "payload #1";
 
 // Sends the test message on `pipe` and waits for the write callback.
 static std::string sendMessage(Pipe& pipe, int salt) {
-  std::vector<GpuTensor> gpus;
+  GpuTensors gpus;
   std::vector<uint8_t> cpu(kCpuBytes);
   for (size_t i = 0; i < cpu.size(); ++i) {
     cpu[i] = pattern(i, salt + 50);
@@ -155,7 +174,7 @@ static std::string sendMessage(Pipe& pipe, int salt) {
 
 static std::string recvMessage(Pipe& pipe, int salt) {
   std::promise<std::string> done;
-  std::vector<GpuTensor> gpus;
+  GpuTensors gpus;
   std::vector<uint8_t> cpu;
   std::string payload;
   pipe.readDescriptor([&](const Error& e, Descriptor d) {
@@ -267,6 +286,42 @@ static int sameProcess() {
   listener.reset();
   client->join();
   server->join();
+  return problem.empty() ? 0 : 1;
+}
+
+
+// One context talking to itself, both directions busy at once, `rounds` times.
+// Every thread here is the application's: the host's transport threads and the
+// four below are all strangers to this library's loops.
+static int toSelf(const std::string& channel, int rounds) {
+  const std::string addr = "shm://tpamd_conf_self_" + std::to_string(::getpid());
+  auto ctx = makeContext("self", {channel});
+  auto listener = ctx->listen({addr});
+  auto cpipe = ctx->connect(listener->url("shm"));
+  auto spipe = acceptOne(*listener);
+  std::string problem = spipe ? std::string() : std::string("accept failed");
+  for (int round = 0; round < rounds && problem.empty(); ++round) {
+    auto w1 = std::async(std::launch::async, [&] { return sendMessage(*cpipe, 10 * round); });
+    auto w2 = std::async(std::launch::async, [&] { return sendMessage(*spipe, 10 * round + 5); });
+    auto r1 = std::async(std::launch::async, [&] { return recvMessage(*spipe, 10 * round); });
+    auto r2 = std::async(std::launch::async, [&] { return recvMessage(*cpipe, 10 * round + 5); });
+    for (auto* f : {&w1, &w2, &r1, &r2}) {
+      const std::string p = f->get();
+      if (problem.empty()) {
+        problem = p;
+      }
+    }
+  }
+  const size_t expected = static_cast<size_t>(rounds) * 2 * kGpuSizes.size() * 2;
+  if (problem.empty() && tensorpipe_amd_bridge::gpuOperationsServed() != expected) {
+    problem = "the GPU tensors did not all travel on this library's channel: " +
+        std::to_string(tensorpipe_amd_bridge::gpuOperationsServed()) + " operations served";
+  }
+  report(channel + "_to_self_in_stock_context", problem);
+  cpipe.reset();
+  spipe.reset();
+  listener.reset();
+  ctx->join();
   return problem.empty() ? 0 : 1;
 }
 
@@ -722,6 +777,9 @@ int main(int argc, char** argv) {
   if (argc == 3 && std::strcmp(argv[1], "two_process") == 0) {
     return twoProcess(argv[2]);
   }
+  if (argc == 4 && std::strcmp(argv[1], "to_self") == 0) {
+    return toSelf(argv[2], std::atoi(argv[3]));
+  }
   if (argc == 2 && std::strcmp(argv[1], "unmodified_peer") == 0) {
     return unmodifiedPeer();
   }
@@ -737,6 +795,6 @@ int main(int argc, char** argv) {
     }
     return timeSameProcess(bytes, std::atoi(argv[3]), pieces);
   }
-  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic | time_same_process <bytes> <messages> [tensors per message]\n", argv[0]);
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | to_self <channel> <rounds> | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic | time_same_process <bytes> <messages> [tensors per message]\n", argv[0]);
   return 2;
 }

@@ -21,12 +21,25 @@
 //       flipped, a frame must be refused without reading out of bounds.
 //   unit_tests compat_pipe
 //       two ends of the stock-protocol endpoint talk to each other over TCP.
+//   unit_tests loops
+//       the on-demand executor: two application threads, each inside a task of
+//       one loop, defer to the other's loop at the same moment and both return
+//       (no thread ever waits for a loop while it sits in a task of another);
+//       a caller holding a lock that the draining thread's task wants returns
+//       from defer() as well; a task queued by another thread while an
+//       application thread drains is never run by that application thread and
+//       still runs; tasks run exactly once, in the order they were queued; a
+//       loop goes away cleanly while a helper still has it on its list.
 //   unit_tests tcp
 //       the TCP transport: messages of every size class both ways (empty, small,
 //       many MiB: partial reads and writes), exact-length reads, a peer that
 //       wrote and left, a frame written by hand with the reference's framing,
 //       and a pipe with payloads and CPU tensors over it.
+#include <atomic>
 #include <chrono>
+#include <condition_variable>
+#include <functional>
+#include <memory>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -49,6 +62,7 @@
 #include <tensorpipe/common/device.h>
 #include <tensorpipe/common/error.h>
 #include <tensorpipe/common/hip_buffer.h>
+#include <tensorpipe/common/loop.h>
 #include <tensorpipe/common/slot_allocator.h>
 #include <tensorpipe/common/wire.h>
 #include <tensorpipe/channel/error.h>
@@ -934,6 +948,248 @@ static int runTcp() {
   return failed == 0 ? 0 : 1;
 }
 
+
+// ---- on-demand loops ---------------------------------------------------------
+
+namespace {
+
+// Two threads meet here; returns false when the other one has not arrived
+// within the time limit (the case then fails instead of hanging).
+class Rendezvous {
+ public:
+  bool arrive(std::chrono::milliseconds limit = std::chrono::milliseconds(2000)) {
+    std::unique_lock<std::mutex> lock(m_);
+    const unsigned turn = turn_;
+    if (++count_ == 2) {
+      count_ = 0;
+      ++turn_;
+      cv_.notify_all();
+      return true;
+    }
+    return cv_.wait_for(lock, limit, [&] { return turn_ != turn; });
+  }
+
+ private:
+  std::mutex m_;
+  std::condition_variable cv_;
+  unsigned count_{0};
+  unsigned turn_{0};
+};
+
+// Ends the process when a case is stuck, naming it: a hung unit test tells
+// nothing, a line and an exit code do.
+class Watchdog {
+ public:
+  Watchdog(const char* what, int seconds) : what_(what) {
+    thread_ = std::thread([this, seconds] {
+      std::unique_lock<std::mutex> lock(m_);
+      if (!cv_.wait_for(lock, std::chrono::seconds(seconds), [this] { return done_; })) {
+        std::printf("TIMEOUT %s\n", what_);
+        std::fflush(stdout);
+        _exit(3);
+      }
+    });
+  }
+  ~Watchdog() {
+    {
+      std::unique_lock<std::mutex> lock(m_);
+      done_ = true;
+    }
+    cv_.notify_all();
+    thread_.join();
+  }
+
+ private:
+  const char* what_;
+  std::mutex m_;
+  std::condition_variable cv_;
+  bool done_{false};
+  std::thread thread_;
+};
+
+bool waitFor(const std::function<bool()>& cond, int ms = 2000) {
+  const auto until = std::chrono::steady_clock::now() + std::chrono::milliseconds(ms);
+  while (!cond()) {
+    if (std::chrono::steady_clock::now() > until) {
+      return false;
+    }
+    std::this_thread::sleep_for(std::chrono::microseconds(50));
+  }
+  return true;
+}
+
+} // namespace
+
+static int runLoops() {
+  int failed = 0;
+  // 1. Thread A sits in a task of loop one and defers to loop two while thread
+  // B sits in a task of loop two and defers to loop one. Neither is a thread
+  // of the library. Both defer() calls must return, and both tasks must run.
+  {
+    Watchdog dog("crossed defers of two application threads", 5);
+    OnDemandLoop one, two;
+    Rendezvous inside, leaving;
+    std::atomic<int> ran{0};
+    bool metA = false, metB = false;
+    std::thread a([&] {
+      one.defer([&] {
+        metA = inside.arrive();
+        two.defer([&] { ++ran; });
+        leaving.arrive();
+      });
+    });
+    std::thread b([&] {
+      two.defer([&] {
+        metB = inside.arrive();
+        one.defer([&] { ++ran; });
+        leaving.arrive();
+      });
+    });
+    a.join();
+    b.join();
+    CHECK(metA && metB);
+    CHECK(waitFor([&] { return ran.load() == 2; }));
+  }
+  // 2. A caller that holds a lock while it calls defer() gets out again although
+  // the thread that drains the loop is blocked, inside its own task, on that lock.
+  {
+    Watchdog dog("defer() with a lock held that the draining task wants", 5);
+    OnDemandLoop loop;
+    std::mutex userLock;
+    Rendezvous drainerInside;
+    std::atomic<int> ran{0};
+    std::thread drainer([&] {
+      loop.defer([&] {
+        drainerInside.arrive();
+        std::this_thread::sleep_for(std::chrono::milliseconds(20));
+        std::lock_guard<std::mutex> g(userLock); // what a user's callback may do
+        ++ran;
+      });
+    });
+    std::thread caller([&] {
+      std::lock_guard<std::mutex> g(userLock);
+      drainerInside.arrive();
+      loop.defer([&] { ++ran; }); // must come back while the drainer wants userLock
+    });
+    caller.join();
+    drainer.join();
+    CHECK(waitFor([&] { return ran.load() == 2; }));
+  }
+  // 3. What another thread queues while an application thread drains the loop is
+  // not run on the application thread's stack (its own call is still on it),
+  // and is run all the same -- whether the other thread is the library's or not,
+  // inside a task of another loop or not.
+  for (int variant = 0; variant < 3; ++variant) {
+    Watchdog dog("a task queued beside a draining application thread", 5);
+    OnDemandLoop loop, other;
+    Rendezvous inside, queued;
+    std::atomic<int> ran{0};
+    std::thread::id ranOn;
+    std::thread::id appId;
+    std::thread app([&] {
+      appId = std::this_thread::get_id();
+      loop.defer([&] {
+        inside.arrive();
+        queued.arrive(std::chrono::milliseconds(300)); // a waiting library thread never gets here: fine
+        std::this_thread::sleep_for(std::chrono::milliseconds(2));
+      });
+    });
+    std::thread foreign([&] {
+      thisIsLibraryThread() = (variant == 1);
+      auto post = [&] {
+        loop.defer([&] {
+          ranOn = std::this_thread::get_id();
+          ++ran;
+        });
+        queued.arrive(std::chrono::milliseconds(300));
+      };
+      inside.arrive();
+      if (variant == 2) {
+        other.defer(post);
+      } else {
+        post();
+      }
+    });
+    app.join();
+    foreign.join();
+    CHECK(waitFor([&] { return ran.load() == 1; }));
+    CHECK(ranOn != appId);
+  }
+  // 4. Many threads, two loops, tasks that hop between them: each runs once, and
+  // the tasks one thread queued on one loop run in the order it queued them.
+  {
+    Watchdog dog("tasks from many threads over two loops", 30);
+    OnDemandLoop loops[2];
+    constexpr int kThreads = 6, kPerThread = 3000;
+    std::atomic<int> ran{0};
+    std::atomic<int> concurrent[2] = {{0}, {0}};
+    std::atomic<bool> overlapped{false}, disorder{false};
+    std::vector<std::vector<int>> seen(kThreads * 2);
+    std::vector<std::thread> threads;
+    for (int t = 0; t < kThreads; ++t) {
+      threads.emplace_back([&, t] {
+        thisIsLibraryThread() = (t % 3 == 0);
+        for (int i = 0; i < kPerThread; ++i) {
+          const int first = (t + i) & 1;
+          loops[first].defer([&, t, i, first] {
+            if (concurrent[first].fetch_add(1) != 0) {
+              overlapped = true;
+            }
+            seen[t * 2 + first].push_back(i);
+            concurrent[first].fetch_sub(1);
+            loops[1 - first].defer([&, first] {
+              if (concurrent[1 - first].fetch_add(1) != 0) {
+                overlapped = true;
+              }
+              ++ran;
+              concurrent[1 - first].fetch_sub(1);
+            });
+          });
+        }
+      });
+    }
+    for (auto& th : threads) {
+      th.join();
+    }
+    CHECK(waitFor([&] { return ran.load() == kThreads * kPerThread; }, 20000));
+    CHECK(!overlapped.load());
+    for (auto& v : seen) {
+      for (size_t k = 1; k < v.size(); ++k) {
+        if (v[k] <= v[k - 1]) {
+          disorder = true;
+        }
+      }
+    }
+    CHECK(!disorder.load());
+  }
+  // 5. A loop is destroyed right after an application thread left it with
+  // another thread's task still queued.
+  for (int round = 0; round < 200; ++round) {
+    Watchdog dog("a loop destroyed with a helper on its way", 10);
+    auto loop = std::make_unique<OnDemandLoop>();
+    Rendezvous inside;
+    std::atomic<int> ran{0};
+    std::thread app([&] {
+      loop->defer([&] {
+        inside.arrive();
+        std::this_thread::sleep_for(std::chrono::microseconds(100));
+      });
+    });
+    std::thread foreign([&] {
+      inside.arrive();
+      loop->defer([&] { ++ran; });
+    });
+    app.join();
+    foreign.join();
+    CHECK(waitFor([&] { return ran.load() == 1; }));
+    loop.reset();
+  }
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
 static void onFatalSignal(int sig) {
   void* frames[48];
   const int n = backtrace(frames, 48);
@@ -971,6 +1227,9 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "tcp") == 0) {
     return runTcp();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp\n", argv[0]);
+  if (argc == 2 && std::strcmp(argv[1], "loops") == 0) {
+    return runLoops();
+  }
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | loops\n", argv[0]);
   return 2;
 }

@@ -21,6 +21,9 @@ GPU_SUITES = [("channel_tests", "hip_xth"), ("channel_tests", "hip_ipc"), ("chan
               ("channel_tests", "hip_basic"),
               ("pipe_tests", "same_process"), ("pipe_tests", "two_process")]
 
+# tests/cpp/fake_tphip.cc: the C ABI of include/tphip.h with threads and memcpy behind it
+STAND_IN = os.path.join(BIN, "fake")
+
 _results = {}
 
 
@@ -39,12 +42,16 @@ def list_cases(program, suite):
     return out.stdout.split()
 
 
-def run_suite(program, suite, stock_wire=False):
+def run_suite(program, suite, stock_wire=False, stand_in=False):
     """One run per suite and session; returns {case: [(role, ok, detail), ...]}."""
-    key = (program, suite, stock_wire)
+    key = (program, suite, stock_wire, stand_in)
     if key not in _results:
         print(f"running {program} --suite {suite}" + (" in stock wire format" if stock_wire else ""), flush=True)
         env = dict(os.environ, TP_STOCK_WIRE="1") if stock_wire else None
+        if stand_in:
+            if not os.path.exists(os.path.join(STAND_IN, "libtphip.so")):
+                pytest.fail(f"{STAND_IN}/libtphip.so is not built (run __graft_entry__.build())")
+            env = dict(env or os.environ, LD_LIBRARY_PATH=STAND_IN)
         proc = subprocess.run([_binary(program), "--suite", suite], stdout=subprocess.PIPE,
                               stderr=subprocess.PIPE, text=True, timeout=600, env=env)
         per_case = {}
@@ -57,8 +64,8 @@ def run_suite(program, suite, stock_wire=False):
     return _results[key]
 
 
-def check_case(program, suite, case, stock_wire=False):
-    rc, per_case, out, err = run_suite(program, suite, stock_wire)
+def check_case(program, suite, case, stock_wire=False, stand_in=False):
+    rc, per_case, out, err = run_suite(program, suite, stock_wire, stand_in)
     assert case in per_case, f"no result for {case}; exit code {rc}\n{out}\n{err}"
     bad = [line for _, ok, line in per_case[case] if not ok]
     assert not bad, "\n".join(bad) + "\n" + err
@@ -80,6 +87,15 @@ def test_cpu_suite(program, suite, case):
 @pytest.mark.parametrize("program,suite,case", _params(GPU_SUITES))
 def test_gpu_suite(program, suite, case):
     check_case(program, suite, case)
+
+
+# The suites of the device channels once more without a GPU: libtphip.so replaced by the host-only
+# stand-in (streams are threads, copies memcpy), which leaves the channels' own host logic -- state
+# machines, control messages, slot rings, signal words, error paths -- to be checked on the CPU.
+# Parity of the kernels is NOT what these show; the -m gpu runs of the same suites are.
+@pytest.mark.parametrize("program,suite,case", _params(GPU_SUITES))
+def test_device_channel_host_logic_on_the_stand_in_runtime(program, suite, case):
+    check_case(program, suite, case, stand_in=True)
 
 
 # The pipe suites once more with the reference's encodings on the wire (TP_STOCK_WIRE=1: its

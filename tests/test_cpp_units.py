@@ -60,6 +60,15 @@ def test_basics():
     assert rc == 0 and out.strip() == "OK", out
 
 
+def test_on_demand_loops_never_wait_inside_a_task():
+    """Two application threads, each in a task of one loop, defer to the other's loop at once (the
+    previous executor waited there for good); a caller holding a lock the drainer's task wants; a
+    task queued beside a draining application thread runs, and not on that thread; order and
+    exactly-once under load; destruction with a helper on its way."""
+    rc, out = run("loops")
+    assert rc == 0 and out.strip() == "OK", out
+
+
 def test_messages_of_a_departed_peer_are_delivered():
     # the writer exits before the reader posts its reads: the stream hands over what arrived,
     # then reports the end
