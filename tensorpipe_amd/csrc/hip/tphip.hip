@@ -6,11 +6,13 @@
 #include <hip/hip_ext.h>
 
 #include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <thread>
 #include <tuple>
 #include <vector>
 
@@ -684,33 +686,38 @@ constexpr size_t kNoAllocScratchBytes = (kNoAllocPlanBytes + 255) / 256 * 256;
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
 struct NoAllocDevice {
-  std::once_flag once;
-  int initError{0};
+  std::mutex mutex;
+  std::atomic<bool> ready{false};
   int numCus{0};
   char* scratchPtr{nullptr}; // this device's copy of `scratch`
 };
 NoAllocDevice gNoAlloc[kMaxDevices];
 
-// Call with `dev` current.
+// Call with `dev` current. A failed set-up is not remembered: the next call
+// tries again (a query refused once, say on a stream that is being captured,
+// must not disable the entry point for the rest of the process).
 int getNoAllocDevice(int dev, NoAllocDevice** out) {
   NoAllocDevice& st = gNoAlloc[dev];
-  std::call_once(st.once, [&] {
-    hipError_t e = hipDeviceGetAttribute(&st.numCus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e == hipSuccess) {
+  if (!st.ready.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(st.mutex);
+    if (!st.ready.load(std::memory_order_relaxed)) {
+      int cus = 0;
       void* p = nullptr;
-      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e == hipSuccess) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      }
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+      }
+      if (p == nullptr || cus <= 0) {
+        return TPHIP_ERR_INVALID_ARG;
+      }
+      st.numCus = cus;
       st.scratchPtr = static_cast<char*>(p);
+      st.ready.store(true, std::memory_order_release);
     }
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-    }
-    st.initError = static_cast<int>(e);
-  });
-  if (st.initError != 0) {
-    return st.initError;
-  }
-  if (st.scratchPtr == nullptr) {
-    return TPHIP_ERR_INVALID_ARG;
   }
   *out = &st;
   return 0;
@@ -827,8 +834,8 @@ constexpr uint32_t kGateStates = 256;
 static __device__ __align__(256) uint64_t gateStates[kGateStates];
 
 struct GateDevice {
-  std::once_flag once;
-  int initError{0};
+  std::mutex mutex;
+  std::atomic<bool> ready{false};
   int wallClockKhz{0};
   uint64_t* states{nullptr};
   std::atomic<uint64_t> next{0};
@@ -1317,12 +1324,28 @@ int tphip_agent_destroy(void* agent) {
   if (a == nullptr) {
     return TPHIP_ERR_INVALID_ARG;
   }
+  int unserved = 0;
   {
-    std::lock_guard<std::mutex> lock(a->mutex);
-    a->stopped = true;
+    std::unique_lock<std::mutex> lock(a->mutex);
+    a->stopped = true; // nothing is posted from here on
+    // Everything posted so far is served first: the stop command needs a free
+    // line of the ring (with the ring full it would land on the oldest
+    // unserved command), and an agent that left just before the last command
+    // was posted has to be started once more for it.
+    DeviceScope scope(a->dev);
+    const auto giveUpAt = std::chrono::steady_clock::now() + std::chrono::seconds(5);
+    while (loadWord(&a->ctl->done) < a->nextTicket - 1) {
+      if (agentEnsureRunning(*a) != 0 || std::chrono::steady_clock::now() > giveUpAt) {
+        unserved = 1; // the GPU does not run the agent any more; say so below
+        break;
+      }
+      lock.unlock();
+      std::this_thread::yield();
+      lock.lock();
+    }
     const uint64_t epoch = a->epoch.load(std::memory_order_relaxed);
-    if (epoch != 0 && loadWord(&a->ctl->exited) != epoch) {
-      // A running agent leaves at this command (after everything posted before it).
+    if (unserved == 0 && epoch != 0 && loadWord(&a->ctl->exited) != epoch) {
+      // A running agent leaves at this command.
       const uint64_t t = a->nextTicket++;
       const uint64_t tag = (t & 0xffffu) << 48;
       AgentCommand& c = a->ring[t & (kAgentRing - 1)];
@@ -1350,7 +1373,7 @@ int tphip_agent_destroy(void* agent) {
     }
   }
   delete a;
-  return rc;
+  return rc != 0 ? rc : (unserved != 0 ? TPHIP_ERR_BUSY : 0);
 }
 
 int tphip_batched_copy_gated(int dev, const tphip_copy_desc* table, uint32_t n, void* stream,
@@ -1362,20 +1385,27 @@ int tphip_batched_copy_gated(int dev, const tphip_copy_desc* table, uint32_t n, 
   }
   TPHIP_ON_DEVICE(dev);
   GateDevice& gd = gGateDevices[dev];
-  std::call_once(gd.once, [&] {
-    hipError_t e = hipDeviceGetAttribute(&gd.wallClockKhz, hipDeviceAttributeWallClockRate, dev);
-    if (e == hipSuccess) {
+  if (!gd.ready.load(std::memory_order_acquire)) {
+    // A failed set-up is not remembered: the next call tries again.
+    std::lock_guard<std::mutex> lock(gd.mutex);
+    if (!gd.ready.load(std::memory_order_relaxed)) {
+      int khz = 0;
       void* p = nullptr;
-      e = hipGetSymbolAddress(&p, HIP_SYMBOL(gateStates));
+      hipError_t e = hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev);
+      if (e == hipSuccess) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(gateStates));
+      }
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+      }
+      if (p == nullptr) {
+        return TPHIP_ERR_INVALID_ARG;
+      }
+      gd.wallClockKhz = khz;
       gd.states = static_cast<uint64_t*>(p);
+      gd.ready.store(true, std::memory_order_release);
     }
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-    }
-    gd.initError = static_cast<int>(e);
-  });
-  if (gd.initError != 0) {
-    return gd.initError;
   }
   const int khz = gd.wallClockKhz > 0 ? gd.wallClockKhz : 100000;
   uint64_t* state = gd.states + gd.next.fetch_add(1, std::memory_order_relaxed) % kGateStates;

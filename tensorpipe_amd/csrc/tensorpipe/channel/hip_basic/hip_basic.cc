@@ -555,7 +555,7 @@ class ChannelImpl final : public ChannelImplBase {
           ++it;
         }
       }
-      auto ev = bctx_->events.get(device);
+      auto ev = bctx_->events.get(device, stream);
       if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/true, *ev)) {
         return;
       }
@@ -794,7 +794,7 @@ class ChannelImpl final : public ChannelImplBase {
         setError(TP_CREATE_ERROR(HipError, "tphip_stream_create", TPHIP_ERR_INVALID_ARG));
         return;
       }
-      auto ev = bctx_->events.get(0);
+      auto ev = bctx_->events.get(0, stream);
       if (!launchHostLinkCopy(
               0,
               stream,
@@ -833,7 +833,7 @@ class ChannelImpl final : public ChannelImplBase {
           ++it;
         }
       }
-      auto ev = bctx_->events.get(device);
+      auto ev = bctx_->events.get(device, stream);
       if (!launchHostLinkCopy(device, stream, table, /*towardsHost=*/false, *ev)) {
         return;
       }
@@ -929,7 +929,7 @@ class ChannelImpl final : public ChannelImplBase {
     const HipBuffer hb = chunk->op->buffer.unwrap<HipBuffer>();
     PinnedRing& rring = bctx_->recvRing();
     const int device = hipDeviceForPointer(hb.ptr);
-    auto ev = bctx_->events.get(device);
+    auto ev = bctx_->events.get(device, hb.stream);
     if (!launchHostLinkCopy(
             device,
             hb.stream,

@@ -250,7 +250,7 @@ class StreamMarkers {
  private:
   static void record(int device, void* stream, HipEventPool& pool) {
     try {
-      auto marker = pool.get(device);
+      auto marker = pool.get(device, stream);
       marker->record(stream);
       pool.put(std::move(marker)); // nobody waits for it
     } catch (const std::exception&) {

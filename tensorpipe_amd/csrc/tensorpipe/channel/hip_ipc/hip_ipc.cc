@@ -830,7 +830,7 @@ class ChannelImpl final : public ChannelImplBase {
               &ictx_->signals->devWords(wordsIndex_)->ready[gateSlot],
               gateValue));
           // a marker, so that the runtime knows when the stream has drained
-          auto marker = ictx_->events.get(busy[0].device);
+          auto marker = ictx_->events.get(busy[0].device, busy[0].stream);
           marker->record(busy[0].stream);
           ictx_->events.put(std::move(marker));
           unit->bytes[gateAt] = 1;
@@ -844,7 +844,7 @@ class ChannelImpl final : public ChannelImplBase {
         }
         auto remaining = std::make_shared<size_t>(busy.size());
         for (auto& s : busy) {
-          auto ev = ictx_->events.get(s.device);
+          auto ev = ictx_->events.get(s.device, s.stream);
           ev->record(s.stream);
           watch(std::move(ev), [this, unit, remaining] {
             if (--*remaining == 0) {
@@ -903,7 +903,7 @@ class ChannelImpl final : public ChannelImplBase {
       std::unique_ptr<HipEvent> ev;
       bool onKernel = false;
       try {
-        ev = ictx_->events.get(device);
+        ev = ictx_->events.get(device, hb.stream);
         // The chunks of a long tensor queue up on the caller's stream several
         // deep: the kernels' own completion signals then, and no marker between
         // two of them (1 GiB: 1.4 instead of 1.2 TB/s). A short tensor is better
@@ -1343,7 +1343,7 @@ class ChannelImpl final : public ChannelImplBase {
         }
         if (!viaAgent && !gatedLaunched) {
           for (auto& g : groups) {
-            auto ev = ictx_->events.get(g.dst.device);
+            auto ev = ictx_->events.get(g.dst.device, g.dst.stream);
             hipBatchedCopy(g.dst.device, g.dst.stream, g.table, *ev, /*signalOnKernel=*/false);
             launched.push_back(std::move(ev));
             launchedOn.push_back(g.dst);
@@ -1416,7 +1416,7 @@ class ChannelImpl final : public ChannelImplBase {
           failProtocol();
           return;
         }
-        auto ev = ictx_->events.get(device);
+        auto ev = ictx_->events.get(device, hb.stream);
         chunkOnKernel = hipBatchedCopy(
             device,
             hb.stream,
@@ -1543,7 +1543,7 @@ class ChannelImpl final : public ChannelImplBase {
     g.expiredSlot = static_cast<uint32_t>(nextExpired_++ % kWordSlots);
     ChannelWords* mine = ictx_->signals->hostWords(wordsIndex_);
     __atomic_store_n(&mine->expired[g.expiredSlot], uint64_t(0), __ATOMIC_RELEASE);
-    auto ev = ictx_->events.get(g.dst.device);
+    auto ev = ictx_->events.get(g.dst.device, g.dst.stream);
     TP_HIP_CHECK(tphip_batched_copy_gated(
         g.dst.device,
         g.table.data(),

@@ -371,7 +371,7 @@ class ChannelImpl final : public ChannelImplBase {
         // enqueued before recv() on that buffer's stream is done.
         for (auto& d : g.dstStreams) {
           if (!xctx_->idleProbe.idle(d.device, d.stream)) {
-            auto ev = xctx_->events.get(d.device);
+            auto ev = xctx_->events.get(d.device, d.stream);
             ev->record(d.stream);
             ev->wait(g.src.stream, g.src.device);
             xctx_->events.put(std::move(ev)); // the wait captured the record
@@ -380,7 +380,7 @@ class ChannelImpl final : public ChannelImplBase {
         TP_VLOG(6) << "Channel " << id_ << " is copying payload (#" << g.ops.front()->seq << " to #"
                    << g.ops.back()->seq << ")";
         TP_MARK("xth: destination streams checked");
-        auto done = xctx_->events.get(g.src.device);
+        auto done = xctx_->events.get(g.src.device, g.src.stream);
         const bool onKernel =
             hipBatchedCopy(g.src.device, g.src.stream, g.table, *done, /*signalOnKernel=*/true);
         TP_MARK("xth: kernel launch call returned");

@@ -5,6 +5,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -65,38 +66,58 @@ class HipEvent {
   int device() const {
     return device_;
   }
+  // The one stream this event is used on (see HipEventPool).
+  void* home() const {
+    return home_;
+  }
+  void setHome(void* stream) {
+    home_ = stream;
+  }
 
  private:
   int device_;
   void* ev_{nullptr};
+  void* home_{nullptr};
 };
 
-// Recycles events per device so the per-message path creates none.
+// Recycles events so that the per-message path creates none. An event is only
+// ever reused on the stream it was first used on. A caller may destroy its
+// stream as soon as the callbacks of its operations have fired, and an event
+// that had been recorded on such a stream and was later handed out for another
+// one has been seen to fail its query there ("operation not permitted on an
+// event last recorded in a capturing stream", with no capture anywhere): what
+// the runtime remembers inside an event about the stream of its last record
+// is not ours to rely on once that stream is gone. Events that touched a
+// stream stay with it; they go away with the pool.
 class HipEventPool {
  public:
-  std::unique_ptr<HipEvent> get(int device) {
+  std::unique_ptr<HipEvent> get(int device, void* stream) {
     {
       std::lock_guard<std::mutex> lock(mutex_);
-      if (device < static_cast<int>(free_.size()) && !free_[device].empty()) {
-        auto ev = std::move(free_[device].back());
-        free_[device].pop_back();
+      auto it = free_.find(Key{device, stream});
+      if (it != free_.end() && !it->second.empty()) {
+        auto ev = std::move(it->second.back());
+        it->second.pop_back();
         return ev;
       }
     }
-    return std::make_unique<HipEvent>(device);
+    auto ev = std::make_unique<HipEvent>(device);
+    ev->setHome(stream);
+    return ev;
   }
   void put(std::unique_ptr<HipEvent> ev) {
     std::lock_guard<std::mutex> lock(mutex_);
-    const int device = ev->device();
-    if (device >= static_cast<int>(free_.size())) {
-      free_.resize(device + 1);
+    auto& list = free_[Key{ev->device(), ev->home()}];
+    if (list.size() < kMaxPerStream) {
+      list.push_back(std::move(ev));
     }
-    free_[device].push_back(std::move(ev));
   }
 
  private:
+  static constexpr size_t kMaxPerStream = 64;
+  using Key = std::pair<int, void*>;
   std::mutex mutex_;
-  std::vector<std::vector<std::unique_ptr<HipEvent>>> free_;
+  std::map<Key, std::vector<std::unique_ptr<HipEvent>>> free_;
 };
 
 // Pinned, device-mapped host slab (tensorpipe/common/cuda.h:183-188).

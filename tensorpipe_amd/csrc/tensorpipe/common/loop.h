@@ -144,7 +144,10 @@ class LoopHelpers {
         lock.lock();
       }
       ++idle_;
-      const bool more = cv_.wait_for(lock, std::chrono::seconds(1), [this] { return !queue_.empty(); });
+      // (wall-clock deadline: the sanitizers of this toolchain follow
+      // pthread_cond_timedwait, not the monotonic variant wait_for() uses)
+      const bool more = cv_.wait_until(
+          lock, std::chrono::system_clock::now() + std::chrono::seconds(1), [this] { return !queue_.empty(); });
       --idle_;
       if (!more) {
         --threads_;

@@ -215,13 +215,24 @@ Stream& streamOf(void* handle) {
 
 // ---- events --------------------------------------------------------------------
 
-struct Event {
+struct EventState {
   std::mutex m;
   std::condition_variable cv;
   uint64_t recorded{0};
   uint64_t completed{0};
   Clock::time_point when{};
 };
+
+// An event may be destroyed while a stream still has its marker queued, as
+// with the real runtime: the queued work holds the state alive.
+using EventRef = std::shared_ptr<EventState>;
+struct Event {
+  EventRef state{std::make_shared<EventState>()};
+};
+
+EventRef ref(void* event) {
+  return event != nullptr ? static_cast<Event*>(event)->state : nullptr;
+}
 
 // ---- copies --------------------------------------------------------------------
 
@@ -266,7 +277,7 @@ void runCopies(const std::vector<tphip_copy_desc>& t) {
   }
 }
 
-void completeEvent(Event* ev, uint64_t seq) {
+void completeEvent(const EventRef& ev, uint64_t seq) {
   std::lock_guard<std::mutex> lock(ev->m);
   if (seq > ev->completed) {
     ev->completed = seq;
@@ -275,7 +286,7 @@ void completeEvent(Event* ev, uint64_t seq) {
   ev->cv.notify_all();
 }
 
-uint64_t beginRecord(Event* ev) {
+uint64_t beginRecord(const EventRef& ev) {
   std::lock_guard<std::mutex> lock(ev->m);
   return ++ev->recorded;
 }
@@ -474,14 +485,14 @@ int tphip_event_destroy(int dev, void* event) {
 }
 
 int tphip_event_record(int dev, void* event, void* stream) {
-  auto* ev = static_cast<Event*>(event);
+  auto ev = ref(event);
   const uint64_t seq = beginRecord(ev);
   streamOf(stream).push([ev, seq] { completeEvent(ev, seq); });
   return 0;
 }
 
 int tphip_stream_wait_event(int dev, void* stream, void* event) {
-  auto* ev = static_cast<Event*>(event);
+  auto ev = ref(event);
   uint64_t target;
   {
     std::lock_guard<std::mutex> lock(ev->m);
@@ -498,14 +509,14 @@ int tphip_stream_wait_event(int dev, void* stream, void* event) {
 }
 
 int tphip_event_query(int dev, void* event, int* done) {
-  auto* ev = static_cast<Event*>(event);
+  auto ev = ref(event);
   std::lock_guard<std::mutex> lock(ev->m);
   *done = ev->completed >= ev->recorded ? 1 : 0;
   return 0;
 }
 
 int tphip_event_sync(int dev, void* event) {
-  auto* ev = static_cast<Event*>(event);
+  auto ev = ref(event);
   std::unique_lock<std::mutex> lock(ev->m);
   const uint64_t target = ev->recorded;
   ev->cv.wait(lock, [&] { return ev->completed >= target; });
@@ -513,8 +524,8 @@ int tphip_event_sync(int dev, void* event) {
 }
 
 int tphip_event_elapsed_ms(void* start, void* stop, float* ms) {
-  auto* a = static_cast<Event*>(start);
-  auto* b = static_cast<Event*>(stop);
+  auto a = ref(start);
+  auto b = ref(stop);
   *ms = std::chrono::duration<float, std::milli>(b->when - a->when).count();
   return 0;
 }
@@ -598,7 +609,7 @@ int tphip_batched_copy_signal(int dev, const tphip_copy_desc* table, uint32_t n,
     return TPHIP_ERR_TOO_LARGE;
   }
   auto t = snapshot(table, n);
-  auto* ev = static_cast<Event*>(event);
+  auto ev = ref(event);
   const uint64_t seq = ev != nullptr ? beginRecord(ev) : 0;
   if (t.empty() && ev == nullptr) {
     return 0;
@@ -652,7 +663,7 @@ int tphip_batched_copy_gated(int dev, const tphip_copy_desc* table, uint32_t n, 
     return TPHIP_ERR_INVALID_ARG;
   }
   auto t = snapshot(table, n);
-  auto* ev = static_cast<Event*>(event);
+  auto ev = ref(event);
   const uint64_t seq = ev != nullptr ? beginRecord(ev) : 0;
   streamOf(stream).push([t{std::move(t)}, ev, seq, gate_word, gate_value, max_wait_us, expired_word] {
     const auto until = Clock::now() + std::chrono::microseconds(max_wait_us);

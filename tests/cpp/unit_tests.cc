@@ -966,7 +966,8 @@ class Rendezvous {
       cv_.notify_all();
       return true;
     }
-    return cv_.wait_for(lock, limit, [&] { return turn_ != turn; });
+    // wall-clock deadlines here and below: ThreadSanitizer follows pthread_cond_timedwait only
+    return cv_.wait_until(lock, std::chrono::system_clock::now() + limit, [&] { return turn_ != turn; });
   }
 
  private:
@@ -983,7 +984,7 @@ class Watchdog {
   Watchdog(const char* what, int seconds) : what_(what) {
     thread_ = std::thread([this, seconds] {
       std::unique_lock<std::mutex> lock(m_);
-      if (!cv_.wait_for(lock, std::chrono::seconds(seconds), [this] { return done_; })) {
+      if (!cv_.wait_until(lock, std::chrono::system_clock::now() + std::chrono::seconds(seconds), [this] { return done_; })) {
         std::printf("TIMEOUT %s\n", what_);
         std::fflush(stdout);
         _exit(3);
