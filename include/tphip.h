@@ -234,6 +234,50 @@ int tphip_agent_submit(void* agent, const tphip_copy_desc* table, uint32_t n, vo
  * saw the command. */
 int tphip_agent_done(void* agent, uint64_t ticket, int* done);
 
+/* ---- GPU-driven staging ring ------------------------------------------------ */
+
+/* One end of a staging ring that kernels walk by themselves: `num_slots` slots
+ * of `slot_bytes` in pinned host memory, and two 64-bit counters in pinned
+ * host memory, `produced` (chunks written into the ring) and `consumed`
+ * (chunks read out of it), counted over the life of the ring, zero at the
+ * start. Both ends -- normally two processes -- have slots and counters mapped
+ * on their GPU (an IPC handle for the other side's memory). tphip_ring_push
+ * enqueues ONE kernel that copies `bytes` bytes from `src` into the ring,
+ * chunk by chunk (a chunk is one slot, the last may be shorter), waiting on
+ * the GPU for `consumed` before it reuses a slot and raising `produced` behind
+ * every chunk; tphip_ring_pull is the other half: it waits for `produced`,
+ * copies slot -> `dst`, raises `consumed`. `first_seq` is the ring sequence
+ * number of the call's first chunk (the total of all chunks moved before).
+ * Replaces the per-chunk cudaMemcpyAsync + stream callback + control messages
+ * of tensorpipe/channel/cuda_basic/channel_impl.cc:117-229 (send) and
+ * :380-506 (recv).
+ *
+ * The kernels never wait for good: when nothing has moved for `yield_us`, or
+ * the host has made *abort non-zero, the kernel leaves. Once `event` has
+ * completed, *status (pinned host memory of this process) holds the ring
+ * sequence number up to which this end is complete, with TPHIP_RING_YIELDED set
+ * if the kernel left early; the caller then calls again for the rest
+ * (src/dst and bytes advanced by the chunks done, first_seq = that number).
+ * `scratch` is device memory of this end's own, tphip_ring_scratch_bytes()
+ * long and zero before the first call; one call at a time per end. */
+#define TPHIP_RING_YIELDED (1ull << 63)
+typedef struct tphip_ring_end {
+  void* slots;
+  uint64_t slot_bytes;
+  uint32_t num_slots;
+  void* produced;
+  void* consumed;
+  void* scratch;
+  void* status;
+  const void* abort;
+} tphip_ring_end;
+size_t tphip_ring_scratch_bytes(uint32_t num_slots);
+/* `blocks` workgroups of 256 threads (0 = the library's choice). */
+int tphip_ring_push(int dev, const tphip_ring_end* ring, const void* src, uint64_t bytes,
+                    uint64_t first_seq, uint32_t yield_us, uint32_t blocks, void* stream, void* event);
+int tphip_ring_pull(int dev, const tphip_ring_end* ring, void* dst, uint64_t bytes,
+                    uint64_t first_seq, uint32_t yield_us, uint32_t blocks, void* stream, void* event);
+
 /* Single-copy convenience wrapper over the same kernel (n == 1, descriptor
  * travels in the kernel arguments). */
 int tphip_copy(int dev, void* dst, const void* src, uint64_t bytes, void* stream);

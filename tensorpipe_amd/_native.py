@@ -68,6 +68,14 @@ class CopyDesc(ctypes.Structure):
     _fields_ = [("src", ctypes.c_void_p), ("dst", ctypes.c_void_p), ("bytes", ctypes.c_uint64)]
 
 
+class RingEnd(ctypes.Structure):
+    """Mirror of tphip_ring_end (include/tphip.h)."""
+
+    _fields_ = [("slots", ctypes.c_void_p), ("slot_bytes", ctypes.c_uint64), ("num_slots", ctypes.c_uint32),
+                ("produced", ctypes.c_void_p), ("consumed", ctypes.c_void_p), ("scratch", ctypes.c_void_p),
+                ("status", ctypes.c_void_p), ("abort", ctypes.c_void_p)]
+
+
 _tphip = None
 _datagen = None
 _tpc = None
@@ -125,6 +133,10 @@ def tphip():
         lib.tphip_fill.argtypes = [i32, vp, i32, u64, vp]
         lib.tphip_test_slow_kernel.argtypes = [i32, vp, u64, vp]
         lib.tphip_test_set_table_limit.argtypes = [u64]
+        lib.tphip_ring_scratch_bytes.restype = ctypes.c_size_t
+        lib.tphip_ring_scratch_bytes.argtypes = [u32]
+        lib.tphip_ring_push.argtypes = [i32, P(RingEnd), vp, u64, u64, u32, u32, vp, vp]
+        lib.tphip_ring_pull.argtypes = [i32, P(RingEnd), vp, u64, u64, u32, u32, vp, vp]
         _tphip = lib
     return _tphip
 

@@ -18,9 +18,11 @@
 // (or a wavefront) each. With one workgroup per CU the whole grid sweeps a
 // compact window of memory at a time, which keeps HBM pages open; measured on
 // MI355X this beats "many small slices per wavefront" by 10-15 %.
-// Heads and tails of 64 entries at a time are gathered by one wavefront: a
-// ballot skips the common all-aligned case, an inclusive wave scan of the
-// per-entry byte counts compacts the odd bytes over the 64 lanes.
+// Heads and tails are moved by the waves at the far end of the grid, sixteen
+// lanes per entry (four entries per wavefront): lane k of an entry's sixteen
+// owns byte k of its head and byte k of its tail, loads them ahead of the
+// wave's chunks and stores them behind the first one. No lane needs to know
+// about another entry, so nothing is scanned or searched across lanes.
 //
 // No LDS tiling is needed beyond the prefix array: the kernel is a pure HBM
 // stream (2 bytes of traffic per payload byte), never touches MFMA.
@@ -724,6 +726,217 @@ __global__ __launch_bounds__(kWave) void agent_kernel(
   }
   if (lane == 0) {
     raise_signal(&ctl->exited, epoch);
+  }
+}
+
+
+// ---- GPU-driven staging ring ---------------------------------------------------
+//
+// The host-staged channel moves a tensor through a ring of pinned host slots
+// (tensorpipe/channel/cuda_basic/channel_impl.cc:117-229 send, :380-506 recv:
+// one copy, one stream callback and two control messages per chunk). Here one
+// kernel per tensor and side walks the ring by itself: the pushing kernel
+// copies chunk after chunk from the source into slot (sequence % slots) and
+// raises `produced`, the pulling kernel of the other process waits for
+// `produced`, copies slot -> destination and raises `consumed`, which is what
+// the pusher waits for before it overwrites a slot. Chunks are numbered over
+// the life of the ring, so the two counters only ever grow. The slots and the
+// two counters are pinned host memory that both processes' GPUs have mapped
+// (plain loads and stores only: nothing relies on atomics across the host
+// link, nor on two processes seeing each other's device memory mid-kernel).
+//
+// The workgroups form `groups` teams; team t copies chunks t, t + groups, ...
+// so that while one team sits at a chunk boundary (its stores draining, the
+// counter of the other side being read) the others keep the link busy. Every
+// workgroup of a team copies its share of the team's chunk. A chunk is complete
+// when the whole team has arrived at its slot's counter (device memory of this
+// side); the last one to arrive resets that counter, waits until the chunk
+// before has been published (the last arrivals of two consecutive chunks may
+// be different workgroups, and the shared word must never step back) and
+// raises the shared word.
+//
+// No wait is unbounded, and no kernel relies on another kernel of its own
+// process running at the same time (two streams may share one hardware queue):
+// a workgroup that sees no progress for `yieldTicks` of the 100 MHz wall
+// clock, or finds `*abort` raised by the host, sets the launch's stop flag and
+// everybody leaves at their next wait. The last workgroup to leave tells the
+// host (`status`, pinned memory) how many chunks are complete and whether the
+// kernel gave up (kRingYielded), and leaves the scratch words as the next
+// launch needs them (a chunk may have been half arrived); the host launches
+// again from there, behind whatever else it has queued meanwhile.
+constexpr uint64_t kRingYielded = 1ull << 63;
+
+// This side's own words in device memory, all zero before the first launch.
+struct RingScratch {
+  uint64_t published; // chunks complete on this side (ring sequence)
+  uint32_t stop;      // raised by the workgroup that gave up
+  uint32_t exits;     // workgroups that have left
+  uint32_t arrivals[1]; // numSlots of them
+};
+
+struct RingArgs {
+  char* user;          // source (push) or destination (pull) of this launch's first chunk
+  uint64_t bytes;      // bytes this launch moves (whole chunks but the last)
+  char* slots;         // slot 0 of the ring
+  uint64_t slotBytes;
+  uint32_t numSlots;
+  uint64_t firstSeq;   // ring sequence number of this launch's first chunk
+  uint64_t* produced;  // shared, host memory
+  uint64_t* consumed;  // shared, host memory
+  RingScratch* scratch;
+  uint64_t* status;    // host-visible: chunks complete (ring sequence) | kRingYielded
+  const uint64_t* abort; // host-written; non-zero: leave
+  uint64_t yieldTicks;
+  uint32_t groups;     // teams of workgroups; gridDim.x is a multiple of it
+};
+
+template <bool PUSH, int U>
+__global__ __launch_bounds__(kBlockThreads) void ring_kernel(const RingArgs a) {
+  __shared__ uint32_t sGo;
+  const uint32_t team = blockIdx.x % a.groups;
+  const uint32_t teamBlocks = gridDim.x / a.groups;
+  const uint64_t g = static_cast<uint64_t>(blockIdx.x / a.groups) * kBlockThreads + threadIdx.x;
+  const uint64_t G = static_cast<uint64_t>(teamBlocks) * kBlockThreads;
+  const uint64_t nChunks = (a.bytes + a.slotBytes - 1) / a.slotBytes;
+  RingScratch* sc = a.scratch;
+  if (threadIdx.x == 0) {
+    sGo = 1; // a team without a chunk leaves as "not stopped"
+  }
+  // What thread 0 last read of the other side's counter: the counter only
+  // grows, so a value that is enough needs no second look (a look costs a
+  // round trip that queues behind the copy's own traffic).
+  uint64_t seen = 0;
+  const uint64_t* awaited = PUSH ? a.consumed : a.produced;
+  uint64_t* raised = PUSH ? a.produced : a.consumed;
+
+  for (uint64_t k = team; k < nChunks; k += a.groups) {
+    const uint64_t seq = a.firstSeq + k;
+    const uint32_t slot = static_cast<uint32_t>(seq % a.numSlots);
+    if (threadIdx.x == 0) {
+      // push: the chunk that used this slot last has been read out;
+      // pull: this chunk has been written.
+      const uint64_t need = PUSH ? (seq >= a.numSlots ? seq - a.numSlots + 1 : 0) : seq + 1;
+      uint32_t go = 1;
+      if (seen < need) {
+        const uint64_t t0 = wall_clock64();
+        for (uint32_t spins = 0;; ++spins) {
+          seen = read_signal(awaited);
+          if (seen >= need) {
+            break;
+          }
+          if (__hip_atomic_load(&sc->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+            go = 0;
+            break;
+          }
+          if (wall_clock64() - t0 > a.yieldTicks || ((spins & 63u) == 63u && read_signal(a.abort) != 0)) {
+            __hip_atomic_store(&sc->stop, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            go = 0;
+            break;
+          }
+          // about a microsecond: every look may be a read across the host link
+          __builtin_amdgcn_s_sleep(32);
+        }
+      }
+      sGo = go;
+    }
+    __syncthreads();
+    if (sGo == 0) {
+      break;
+    }
+    // Nothing the other side wrote may be served from this CU's caches.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+
+    const uint64_t off = k * a.slotBytes;
+    const uint64_t len = a.bytes - off < a.slotBytes ? a.bytes - off : a.slotBytes;
+    const char* src = PUSH ? a.user + off : a.slots + static_cast<uint64_t>(slot) * a.slotBytes;
+    char* dst = PUSH ? a.slots + static_cast<uint64_t>(slot) * a.slotBytes : a.user + off;
+    {
+      // The grid-wide single-entry copy: destination-aligned 16-byte vectors,
+      // lane g of G takes vectors g, g+G, ... U at a time; device memory is
+      // streamed past the caches, the host side is uncached anyway.
+      constexpr int NT = 3;
+      const uint32_t head = head_bytes(dst, len);
+      const uint64_t nvec = (len - head) >> 4;
+      const uint32_t tail = static_cast<uint32_t>((len - head) & 15u);
+      if (g < 64) {
+        const uint32_t lane = static_cast<uint32_t>(g);
+        if (lane < head) {
+          dst[lane] = src[lane];
+        } else if (lane >= 16 && lane - 16 < tail) {
+          const uint64_t o = len - tail + (lane - 16);
+          dst[o] = src[o];
+        }
+      }
+      const char* s = src + head;
+      char* d = dst + head;
+      const uint64_t step = G * U;
+      const uint64_t full = nvec / step * step;
+#pragma clang loop unroll(disable)
+      for (uint64_t base = 0; base < full; base += step) {
+        u32x4 v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+          v[j] = load16<NT>(s + (base + j * G + g) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+          store16<NT>(d + (base + j * G + g) * 16, v[j]);
+        }
+      }
+#pragma clang loop unroll(disable)
+      for (uint64_t i = full + g; i < nvec; i += G) {
+        store16<NT>(d + i * 16, load16<NT>(s + i * 16));
+      }
+    }
+    // Before the workgroup arrives: a pushing thread's stores have been taken
+    // by the host's memory (the slots are uncached host memory: a store is
+    // counted done when it is, there is nothing of it in a cache to write
+    // back); a pulling thread's loads have returned, which its stores already
+    // waited for -- what it wrote to the destination is nobody's business
+    // before the kernel ends.
+    if (PUSH) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const uint32_t before =
+          __hip_atomic_fetch_add(&sc->arrivals[slot], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      if (before == teamBlocks - 1) {
+        // (The slot's next chunk cannot arrive before the word below has been
+        // raised and answered by the other side.)
+        __hip_atomic_store(&sc->arrivals[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // In order: the chunk before belongs to another team; its word is
+        // on its way at the latest -- unless its team gave up, in which case
+        // this chunk stays unpublished as well and is copied again later.
+        bool inOrder = true;
+        while (__hip_atomic_load(&sc->published, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < seq) {
+          if (__hip_atomic_load(&sc->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+            inOrder = false;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        if (inOrder) {
+          raise_signal(raised, seq + 1);
+          __hip_atomic_store(&sc->published, seq + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
+  }
+  if (threadIdx.x == 0) {
+    const uint32_t before =
+        __hip_atomic_fetch_add(&sc->exits, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    if (before == gridDim.x - 1) {
+      // Last one out: everybody else has left, the scratch words are ours.
+      const uint32_t yielded = __hip_atomic_load(&sc->stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint64_t done = __hip_atomic_load(&sc->published, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+      for (uint32_t i = 0; i < a.numSlots; ++i) {
+        __hip_atomic_store(&sc->arrivals[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __hip_atomic_store(&sc->stop, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&sc->exits, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      raise_signal(a.status, done | (yielded != 0 ? kRingYielded : 0));
+    }
   }
 }
 

@@ -13,6 +13,18 @@
 //         acknowledges the slot. The bytes cross the host link twice and are
 //         never touched by a CPU; the two directions overlap, which is what
 //         lets the path approach the PCIe rate.
+//  stream (GPU source of more than one chunk, peer on this machine) The ring
+//         route with the GPUs driving the ring themselves: the channel has a
+//         pinned ring of its own, one kernel per tensor on the sender's GPU
+//         pushes chunk after chunk into it and one kernel on the receiver's GPU
+//         pulls them out, the two kept apart by a pair of counters beside the
+//         slots (tphip_ring_push / tphip_ring_pull). Per tensor one route
+//         message goes out and one "pulling" message comes back; no launch, no
+//         polled event and no control message per chunk. The kernels run on
+//         streams of the channel's own, never on the caller's: a kernel that
+//         waits for the peer's progress there would hold the caller's later
+//         work behind it. They give up after a bounded wait and are launched
+//         again, so no kernel relies on another one running at the same time.
 //  inner  (CPU source, or the ring could not be shared) What the reference
 //         does for every chunk (tensorpipe/channel/cuda_basic/channel_impl.cc
 //         :84-229 send, :335-506 recv): GPU -> pinned slot, the wrapped CPU
@@ -30,7 +42,8 @@
 //
 // Callbacks: send fires once the last chunk has left the GPU (source
 // reusable); recv fires once the last host-to-device copy has been enqueued
-// (GPU target) or the last byte has landed (CPU target).
+// (GPU target) or the last byte has landed (CPU target, and every target on
+// the stream route, whose copies are not on the caller's stream).
 
 #include <tensorpipe/channel/hip_basic/factory.h>
 
@@ -71,6 +84,59 @@ bool ringSharingDisabled() {
   const char* e = std::getenv("TP_HIP_BASIC_NO_SHARED_RING");
   return e != nullptr && e[0] == '1';
 }
+
+// TP_HIP_BASIC_GPU_RING=0 keeps every tensor on the host-driven routes.
+bool gpuRingDisabled() {
+  const char* e = std::getenv("TP_HIP_BASIC_GPU_RING");
+  return e != nullptr && e[0] == '0';
+}
+
+// How long a ring kernel watches a counter that does not move before it leaves
+// (and is launched again): long enough for the peer's kernel to be launched
+// and start, short enough that a kernel whose peer cannot run meanwhile (two
+// streams on one hardware queue) does not hold the GPU for long.
+uint32_t ringYieldUs() {
+  static const uint32_t v = [] {
+    const char* e = std::getenv("TP_HIP_BASIC_RING_YIELD_US");
+    const long us = e != nullptr ? std::atol(e) : 500;
+    return static_cast<uint32_t>(us < 1 ? 1 : us);
+  }();
+  return v;
+}
+
+// The kernels of the stream route hand the ring over in pieces smaller than a
+// slot: the pulling kernel can only start on a piece once all of it is there,
+// and each workgroup moves whole pieces by itself, so the ring should hold a
+// few dozen of them. A thirty-second of the ring, between 128 and 512 KiB
+// (measured, 256 MiB through 4 slots, GB/s with 1 MiB / 4 MiB slots: pieces of
+// 64 KiB 34.4 / 22.7, 128 KiB 38.7 / 21.2, 256 KiB 37.9 / 33.1, 512 KiB
+// 35.7 / 45.1, 1 MiB 32.3 / 35.7; the host-driven route: 29.4 / 35.1).
+// TP_HIP_BASIC_RING_PIECE_BYTES overrides the target.
+size_t ringPieceBytes(size_t slotBytes, size_t numSlots) {
+  static const size_t forced = [] {
+    const char* e = std::getenv("TP_HIP_BASIC_RING_PIECE_BYTES");
+    return e != nullptr ? std::strtoull(e, nullptr, 10) : size_t(0);
+  }();
+  size_t wanted = forced;
+  if (wanted == 0) {
+    wanted = slotBytes * numSlots / 32;
+    wanted = std::min<size_t>(std::max<size_t>(wanted, size_t(128) << 10), size_t(512) << 10);
+  }
+  wanted = std::max<size_t>(wanted, 4096);
+  size_t piece = slotBytes;
+  while (piece > wanted && piece % 2 == 0 && (piece / 2) % 16 == 0) {
+    piece /= 2;
+  }
+  return piece;
+}
+
+// Head of a stream ring's slab: the two counters the kernels of both sides
+// share, then words of the owner's own.
+constexpr size_t kRingHeaderBytes = 4096;
+constexpr size_t kRingProducedAt = 0;
+constexpr size_t kRingConsumedAt = 64;
+constexpr size_t kRingStatusAt = 128;
+constexpr size_t kRingAbortAt = 192;
 
 struct PinnedRing {
   PinnedRing(int device, size_t slots, size_t bytes)
@@ -161,9 +227,10 @@ enum MsgKind : uint8_t {
   kRoute = 3,    // start of a tensor: route and length
   kNotify = 4,   // ring route: chunk staged in {slot}
   kAck = 5,      // ring route: slot consumed
+  kPulling = 6,  // stream route: the receiver's kernel for the next tensor has been launched
 };
 
-enum Route : uint8_t { kRouteInner = 0, kRouteRing = 1 };
+enum Route : uint8_t { kRouteInner = 0, kRouteRing = 1, kRouteStream = 2 };
 
 class ChannelImpl final : public ChannelImplBase {
  public:
@@ -182,6 +249,14 @@ class ChannelImpl final : public ChannelImplBase {
   ~ChannelImpl() override {
     if (remoteRing_ != nullptr) {
       HipIpcImports::get().release(0, remoteRingPeer_, remoteRingId_);
+    }
+    if (streamIn_.ring != nullptr) {
+      HipIpcImports::get().release(0, remoteRingPeer_, streamIn_.ringId);
+    }
+    for (void* stream : {streamOut_.stream, streamIn_.stream}) {
+      if (stream != nullptr) {
+        tphip_stream_destroy(0, stream);
+      }
     }
   }
 
@@ -242,6 +317,15 @@ class ChannelImpl final : public ChannelImplBase {
   }
 
   void handleError() override {
+    // Ring kernels that wait for the peer leave at their next look.
+    if (streamOut_.slab) {
+      __atomic_store_n(hostWord(streamOut_.slab->host(), kRingAbortAt), uint64_t(1), __ATOMIC_RELEASE);
+    }
+    if (streamIn_.own) {
+      __atomic_store_n(hostWord(streamIn_.own->host(), kRingAbortAt), uint64_t(1), __ATOMIC_RELEASE);
+    }
+    streamOut_.jobs.clear();
+    streamIn_.jobs.clear();
     controlConnection_->close();
     cpuChannel_->close();
     if (ctx_->closed()) {
@@ -258,7 +342,9 @@ class ChannelImpl final : public ChannelImplBase {
     auto ops = std::move(ops_);
     ops_.clear();
     for (auto& op : ops) {
-      finish(op);
+      if (!op->kernelBusy) {
+        finish(op);
+      }
     }
   }
 
@@ -274,6 +360,9 @@ class ChannelImpl final : public ChannelImplBase {
     uint8_t route{kRouteInner};
     size_t received{0}; // bytes of this tensor already handled (ring route)
     bool done{false};
+    // A ring kernel is reading or writing the buffer: on error the callback,
+    // which hands the buffer back, waits until that kernel has ended.
+    bool kernelBusy{false};
   };
 
   // A chunk waiting for its turn: inner sends / control notifications must go
@@ -285,8 +374,57 @@ class ChannelImpl final : public ChannelImplBase {
     bool ready{false};
     bool ring{false};
     bool isRoute{false}; // not a chunk: the tensor's route message
+    bool stream{false};  // ... of a tensor on the stream route: the push kernel follows it
     std::shared_ptr<Op> op;
   };
+
+  // One tensor on the stream route, either side.
+  struct RingJob {
+    std::shared_ptr<Op> op;
+    uint64_t index{0};    // among the channel's stream-route tensors of this direction
+    uint64_t firstSeq{0}; // ring sequence number of its first chunk
+    uint64_t chunks{0};
+    uint64_t done{0};     // chunks complete
+    bool launchedOnce{false};
+    bool waitsForPeer{false}; // sender: gave up once before the receiver said it was pulling
+  };
+
+  // Sending end of the channel's own ring.
+  struct StreamOut {
+    std::unique_ptr<HipPinnedSlab> slab; // header page, then the slots
+    std::unique_ptr<HipDeviceSlab> scratch;
+    HandleBytes handle{};
+    uint64_t id{0};
+    bool announced{false};
+    void* stream{nullptr};
+    uint64_t pieceBytes{0}; // what the kernels call a slot
+    uint32_t numPieces{0};
+    uint64_t nextSeq{0};
+    uint64_t nextIndex{0};
+    uint64_t pullingSeen{0}; // kPulling messages so far
+    std::deque<std::shared_ptr<RingJob>> jobs;
+    bool running{false};
+  };
+
+  // Receiving end: the peer's ring as mapped here, and a page of this side's own.
+  struct StreamIn {
+    uint8_t* ring{nullptr};
+    uint64_t ringId{0};
+    uint64_t slotBytes{0};
+    uint32_t numSlots{0};
+    std::unique_ptr<HipPinnedSlab> own; // status and abort words
+    std::unique_ptr<HipDeviceSlab> scratch;
+    std::unique_ptr<HipPinnedSlab> bounce; // landing area for CPU targets, one ring's worth
+    void* stream{nullptr};
+    uint64_t nextSeq{0};
+    uint64_t nextIndex{0};
+    std::deque<std::shared_ptr<RingJob>> jobs;
+    bool running{false};
+  };
+
+  static uint64_t* hostWord(uint8_t* base, size_t at) {
+    return reinterpret_cast<uint64_t*>(base + at);
+  }
 
   struct RecvChunk {
     void* hostPtr{nullptr};
@@ -320,6 +458,14 @@ class ChannelImpl final : public ChannelImplBase {
     uint8_t route;
     uint32_t slot;
     uint64_t length;
+    // stream route, first tensor: where the sender's ring is
+    bool announce{false};
+    uint64_t ringId{0};
+    HandleBytes handle{};
+    uint64_t ringBase{0};
+    uint64_t ringSize{0};
+    uint64_t slotBytes{0};
+    uint32_t numSlots{0};
   };
 
   void whenReady(std::function<void()> fn) {
@@ -411,12 +557,26 @@ class ChannelImpl final : public ChannelImplBase {
       in.kind = kind;
       in.route = r.u8();
       in.length = r.u64();
+      if (in.route == kRouteStream) {
+        in.announce = r.u8() != 0;
+        if (in.announce) {
+          in.ringId = r.u64();
+          r.raw(in.handle.data(), in.handle.size());
+          in.ringBase = r.u64();
+          in.ringSize = r.u64();
+          in.slotBytes = r.u64();
+          in.numSlots = r.u32();
+        }
+      }
       if (!r.ok()) {
         failProtocol();
         return;
       }
       inbox_.push_back(in);
       advanceRecvs();
+    } else if (kind == kPulling) {
+      ++streamOut_.pullingSeen;
+      pumpStreamOut();
     } else if (kind == kNotify) {
       const uint32_t count = r.u32();
       for (uint32_t i = 0; i < count; ++i) {
@@ -460,6 +620,10 @@ class ChannelImpl final : public ChannelImplBase {
     }
     const bool cpuSource = isCpu(op->buffer);
     const bool ring = !cpuSource && peerMappedOurRing_;
+    if (ring && op->length > chunkBytes_ && !gpuRingDisabled() && streamOutReady()) {
+      startStreamSend(op);
+      return;
+    }
     {
       // The route message takes its place in the queue: it must reach the peer
       // after the last notification of the previous tensor.
@@ -663,6 +827,11 @@ class ChannelImpl final : public ChannelImplBase {
     while (!sendQueue_.empty() && sendQueue_.front()->ready && !error_) {
       auto chunk = sendQueue_.front();
       sendQueue_.pop_front();
+      if (chunk->isRoute && chunk->stream) {
+        flushNotifies();
+        routeStreamTensor(chunk->op);
+        continue;
+      }
       if (chunk->isRoute) {
         flushNotifies();
         WireWriter w;
@@ -729,7 +898,12 @@ class ChannelImpl final : public ChannelImplBase {
         op->route = in.route;
         const size_t chunks = (op->length + chunkBytes_ - 1) / chunkBytes_;
         op->pending = chunks; // chunks not yet landed (CPU) / enqueued (GPU)
-        if (op->route == kRouteInner) {
+        if (op->route == kRouteStream) {
+          recvOps_.pop_front();
+          if (!startStreamRecv(op, in)) {
+            return;
+          }
+        } else if (op->route == kRouteInner) {
           recvOps_.pop_front();
           startInnerRecv(op);
         } else if (remoteRing_ == nullptr) {
@@ -954,6 +1128,300 @@ class ChannelImpl final : public ChannelImplBase {
     finish(op);
   }
 
+
+  // ---- stream route: the GPUs drive the channel's own ring -------------------------
+
+  // Creates this channel's ring on first use. False: stay on the other routes.
+  bool streamOutReady() {
+    StreamOut& so = streamOut_;
+    if (so.slab) {
+      return true;
+    }
+    if (streamOutFailed_) {
+      return false;
+    }
+    try {
+      auto slab = std::make_unique<HipPinnedSlab>(0, kRingHeaderBytes + bctx_->numSlots * bctx_->slotBytes);
+      std::memset(slab->host(), 0, kRingHeaderBytes);
+      HandleBytes handle{};
+      TP_HIP_CHECK(tphip_ipc_mem_export(0, slab->host(), handle.data()));
+      const uint64_t pieceBytes = ringPieceBytes(bctx_->slotBytes, bctx_->numSlots);
+      const uint32_t numPieces = static_cast<uint32_t>(bctx_->numSlots * (bctx_->slotBytes / pieceBytes));
+      auto scratch = std::make_unique<HipDeviceSlab>(0, tphip_ring_scratch_bytes(numPieces));
+      void* stream = nullptr;
+      TP_HIP_CHECK(tphip_stream_create(0, &stream));
+      TP_HIP_CHECK(tphip_fill(0, scratch->ptr(), 0, scratch->size(), stream));
+      TP_HIP_CHECK(tphip_stream_sync(0, stream));
+      so.slab = std::move(slab);
+      so.scratch = std::move(scratch);
+      so.handle = handle;
+      so.id = nextExportId();
+      so.stream = stream;
+      so.pieceBytes = pieceBytes;
+      so.numPieces = numPieces;
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " cannot set up its own ring: " << ex.what();
+      streamOutFailed_ = true;
+      return false;
+    }
+    return true;
+  }
+
+  // The tensor keeps its place among the channel's sends: its route message
+  // goes out in order, once everything queued on the source's stream has run
+  // (a pull kernel of the peer then never waits for the caller's own work).
+  void startStreamSend(const std::shared_ptr<Op>& op) {
+    auto marker = std::make_shared<SendChunk>();
+    marker->isRoute = true;
+    marker->stream = true;
+    marker->ring = true;
+    marker->length = op->length;
+    marker->op = op;
+    op->pending = 1;
+    sendQueue_.push_back(marker);
+    const HipBuffer hb = op->buffer.unwrap<HipBuffer>();
+    const int device = hipDeviceForPointer(hb.ptr);
+    try {
+      auto ev = bctx_->events.get(device, hb.stream);
+      ev->record(hb.stream);
+      watch(std::move(ev), [this, marker] {
+        marker->ready = true;
+        flushSends();
+      });
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " cannot order a send behind its stream: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "hip_basic stream route", TPHIP_ERR_INVALID_ARG));
+    }
+  }
+
+  // From flushSends(), in the tensor's turn.
+  void routeStreamTensor(const std::shared_ptr<Op>& op) {
+    StreamOut& so = streamOut_;
+    auto job = std::make_shared<RingJob>();
+    job->op = op;
+    job->index = so.nextIndex++;
+    job->firstSeq = so.nextSeq;
+    job->chunks = (op->length + so.pieceBytes - 1) / so.pieceBytes;
+    so.nextSeq += job->chunks;
+    WireWriter w;
+    w.u8(kRoute);
+    w.u8(kRouteStream);
+    w.u64(op->length);
+    w.u8(so.announced ? 0 : 1);
+    if (!so.announced) {
+      so.announced = true;
+      w.u64(so.id);
+      w.raw(so.handle.data(), so.handle.size());
+      w.u64(reinterpret_cast<uint64_t>(so.slab->host()));
+      w.u64(so.slab->size());
+      w.u64(so.pieceBytes);
+      w.u32(so.numPieces);
+    }
+    writeMessage(*controlConnection_, std::move(w.bytes()));
+    TP_MARK("basic: stream route announced");
+    so.jobs.push_back(std::move(job));
+    pumpStreamOut();
+  }
+
+  // One push kernel at a time, for the oldest tensor that still has chunks to push.
+  void pumpStreamOut() {
+    StreamOut& so = streamOut_;
+    if (so.running || so.jobs.empty() || error_) {
+      return;
+    }
+    auto job = so.jobs.front();
+    if (job->waitsForPeer && so.pullingSeen <= job->index) {
+      return; // the ring is full and nobody pulls yet: kPulling launches the next one
+    }
+    const HipBuffer hb = job->op->buffer.unwrap<HipBuffer>();
+    const uint64_t offset = job->done * so.pieceBytes;
+    tphip_ring_end end{};
+    end.slots = so.slab->dev() + kRingHeaderBytes;
+    end.slot_bytes = so.pieceBytes;
+    end.num_slots = so.numPieces;
+    end.produced = so.slab->dev() + kRingProducedAt;
+    end.consumed = so.slab->dev() + kRingConsumedAt;
+    end.scratch = so.scratch->ptr();
+    end.status = so.slab->dev() + kRingStatusAt;
+    end.abort = so.slab->dev() + kRingAbortAt;
+    try {
+      auto ev = bctx_->events.get(0, so.stream);
+      TP_HIP_CHECK(tphip_ring_push(
+          0, &end, static_cast<const uint8_t*>(hb.ptr) + offset, job->op->length - offset,
+          job->firstSeq + job->done, ringYieldUs(), 0, so.stream, ev->raw()));
+      so.running = true;
+      job->launchedOnce = true;
+      job->op->kernelBusy = true;
+      TP_MARK("basic: push kernel launched");
+      watch(std::move(ev), [this, job] { onPushEnded(job); });
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " push kernel failed: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "tphip_ring_push", TPHIP_ERR_INVALID_ARG));
+    }
+  }
+
+  void onPushEnded(const std::shared_ptr<RingJob>& job) {
+    StreamOut& so = streamOut_;
+    so.running = false;
+    job->op->kernelBusy = false;
+    if (error_) {
+      finish(job->op);
+      return;
+    }
+    const uint64_t status = __atomic_load_n(hostWord(so.slab->host(), kRingStatusAt), __ATOMIC_ACQUIRE);
+    const uint64_t seq = status & ~TPHIP_RING_YIELDED;
+    if (seq < job->firstSeq + job->done || seq > job->firstSeq + job->chunks) {
+      failProtocol();
+      return;
+    }
+    job->done = seq - job->firstSeq;
+    TP_MARK("basic: push kernel ended");
+    if (job->done == job->chunks) {
+      so.jobs.pop_front();
+      sourceDone(job->op); // every byte is in the ring: the source is the caller's again
+    } else if (so.pullingSeen <= job->index) {
+      job->waitsForPeer = true;
+    }
+    pumpStreamOut();
+  }
+
+  // The receiving side of a tensor on the stream route. False: the channel failed.
+  bool startStreamRecv(const std::shared_ptr<Op>& op, const Incoming& in) {
+    StreamIn& si = streamIn_;
+    if (in.announce) {
+      // (same conditions as for the context's ring in the hello)
+      void* ptr = nullptr;
+      if (si.ring != nullptr || remoteRing_ == nullptr || in.numSlots == 0 || in.slotBytes == 0 ||
+          in.slotBytes % 16 != 0 || in.ringSize < kRingHeaderBytes ||
+          in.slotBytes > (in.ringSize - kRingHeaderBytes) / in.numSlots ||
+          HipIpcImports::get().acquire(
+              0, remoteRingPeer_, in.ringId, in.handle, in.ringBase, in.ringSize, &ptr) != 0) {
+        failProtocol();
+        return false;
+      }
+      si.ring = static_cast<uint8_t*>(ptr);
+      si.ringId = in.ringId;
+      si.slotBytes = in.slotBytes;
+      si.numSlots = in.numSlots;
+      try {
+        si.own = std::make_unique<HipPinnedSlab>(0, kRingHeaderBytes);
+        std::memset(si.own->host(), 0, kRingHeaderBytes);
+        si.scratch = std::make_unique<HipDeviceSlab>(0, tphip_ring_scratch_bytes(si.numSlots));
+        TP_HIP_CHECK(tphip_stream_create(0, &si.stream));
+        TP_HIP_CHECK(tphip_fill(0, si.scratch->ptr(), 0, si.scratch->size(), si.stream));
+        TP_HIP_CHECK(tphip_stream_sync(0, si.stream));
+      } catch (const std::exception& ex) {
+        TP_LOG_WARNING() << "Channel " << id_ << " cannot set up its end of the peer's ring: " << ex.what();
+        setError(TP_CREATE_ERROR(HipError, "hip_basic stream route", TPHIP_ERR_INVALID_ARG));
+        return false;
+      }
+    } else if (si.ring == nullptr) {
+      failProtocol();
+      return false;
+    }
+    auto job = std::make_shared<RingJob>();
+    job->op = op;
+    job->index = si.nextIndex++;
+    job->firstSeq = si.nextSeq;
+    job->chunks = (op->length + si.slotBytes - 1) / si.slotBytes;
+    si.nextSeq += job->chunks;
+    op->pending = 1;
+    si.jobs.push_back(std::move(job));
+    pumpStreamIn();
+    return !error_;
+  }
+
+  // One pull kernel at a time, for the oldest tensor that still has chunks in the ring.
+  void pumpStreamIn() {
+    StreamIn& si = streamIn_;
+    if (si.running || si.jobs.empty() || error_) {
+      return;
+    }
+    auto job = si.jobs.front();
+    const uint64_t offset = job->done * si.slotBytes;
+    uint64_t bytes = job->op->length - offset;
+    uint8_t* target = nullptr;
+    const bool toCpu = isCpu(job->op->buffer);
+    tphip_ring_end end{};
+    end.slots = si.ring + kRingHeaderBytes;
+    end.slot_bytes = si.slotBytes;
+    end.num_slots = si.numSlots;
+    end.produced = si.ring + kRingProducedAt;
+    end.consumed = si.ring + kRingConsumedAt;
+    try {
+      if (toCpu) {
+        // The GPU cannot write the caller's memory: a ring's worth at a time
+        // lands in pinned memory of the channel's and is copied on from there.
+        if (!si.bounce) {
+          si.bounce = std::make_unique<HipPinnedSlab>(0, si.numSlots * si.slotBytes);
+        }
+        bytes = std::min<uint64_t>(bytes, si.numSlots * si.slotBytes);
+        target = si.bounce->dev();
+      } else {
+        const HipBuffer hb = job->op->buffer.unwrap<HipBuffer>();
+        target = static_cast<uint8_t*>(hb.ptr) + offset;
+        if (!job->launchedOnce) {
+          // The kernel may touch the target once everything the receiver had
+          // queued on the buffer's stream before recv() is done.
+          const int device = hipDeviceForPointer(hb.ptr);
+          auto ready = bctx_->events.get(device, hb.stream);
+          ready->record(hb.stream);
+          ready->wait(si.stream, 0);
+          bctx_->events.put(std::move(ready)); // the wait captured the record
+        }
+      }
+      end.scratch = si.scratch->ptr();
+      end.status = si.own->dev() + kRingStatusAt;
+      end.abort = si.own->dev() + kRingAbortAt;
+      auto ev = bctx_->events.get(0, si.stream);
+      TP_HIP_CHECK(tphip_ring_pull(
+          0, &end, target, bytes, job->firstSeq + job->done, ringYieldUs(), 0, si.stream, ev->raw()));
+      si.running = true;
+      job->op->kernelBusy = true;
+      TP_MARK("basic: pull kernel launched");
+      if (!job->launchedOnce) {
+        job->launchedOnce = true;
+        WireWriter w;
+        w.u8(kPulling);
+        writeMessage(*controlConnection_, std::move(w.bytes()));
+      }
+      watch(std::move(ev), [this, job, toCpu] { onPullEnded(job, toCpu); });
+    } catch (const std::exception& ex) {
+      TP_LOG_WARNING() << "Channel " << id_ << " pull kernel failed: " << ex.what();
+      setError(TP_CREATE_ERROR(HipError, "tphip_ring_pull", TPHIP_ERR_INVALID_ARG));
+    }
+  }
+
+  void onPullEnded(const std::shared_ptr<RingJob>& job, bool toCpu) {
+    StreamIn& si = streamIn_;
+    si.running = false;
+    job->op->kernelBusy = false;
+    if (error_) {
+      finish(job->op);
+      return;
+    }
+    const uint64_t status = __atomic_load_n(hostWord(si.own->host(), kRingStatusAt), __ATOMIC_ACQUIRE);
+    const uint64_t seq = status & ~TPHIP_RING_YIELDED;
+    if (seq < job->firstSeq + job->done || seq > job->firstSeq + job->chunks) {
+      failProtocol();
+      return;
+    }
+    const uint64_t before = job->done;
+    job->done = seq - job->firstSeq;
+    TP_MARK("basic: pull kernel ended");
+    if (toCpu && job->done > before) {
+      const uint64_t from = before * si.slotBytes;
+      const uint64_t to = std::min<uint64_t>(job->done * si.slotBytes, job->op->length);
+      std::memcpy(
+          static_cast<uint8_t*>(job->op->buffer.unwrap<CpuBuffer>().ptr) + from, si.bounce->host(), to - from);
+    }
+    if (job->done == job->chunks) {
+      si.jobs.pop_front();
+      chunkLanded(job->op);
+    }
+    pumpStreamIn();
+  }
+
   // ---- helpers ------------------------------------------------------------------
 
   template <typename F>
@@ -1009,6 +1477,9 @@ class ChannelImpl final : public ChannelImplBase {
   std::vector<StageItem> stagePending_;
   std::vector<RingItem> ringPending_;
   bool launchScheduled_{false};
+  StreamOut streamOut_;
+  StreamIn streamIn_;
+  bool streamOutFailed_{false};
 };
 
 class ContextImpl final : public Context {

@@ -2,7 +2,7 @@
 // plugin surface itself: channel::Context::createChannel over raw transport
 // connections, then Channel::send / recv with Buffer{HipBuffer|CpuBuffer}.
 //
-//   channel_tests --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_ipc_gated|hip_ipc_messages|hip_basic|basic|xth [--case SUBSTRING] [--list]
+//   channel_tests --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_ipc_gated|hip_ipc_messages|hip_basic|hip_basic_host_ring|hip_basic_small_ring|basic|xth [--case SUBSTRING] [--list]
 //
 // hip_xth and xth run both endpoints as two threads of this process; hip_ipc,
 // hip_basic and basic run them as two processes. The CPU channels (basic, xth)
@@ -26,13 +26,13 @@ bool gGpu = true; // whether the suite's tensors live on the GPU
 
 bool knownSuite(const std::string& s) {
   return s == "hip_xth" || s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_ipc_gated" ||
-      s == "hip_ipc_messages" || s == "hip_basic" ||
-      s == "basic" || s == "xth";
+      s == "hip_ipc_messages" || s == "hip_basic" || s == "hip_basic_host_ring" ||
+      s == "hip_basic_small_ring" || s == "basic" || s == "xth";
 }
 
 bool twoProcessSuite(const std::string& s) {
   return s == "hip_ipc" || s == "hip_ipc_outbox" || s == "hip_ipc_gated" || s == "hip_ipc_messages" ||
-      s == "hip_basic" || s == "basic";
+      s == "hip_basic" || s == "hip_basic_host_ring" || s == "hip_basic_small_ring" || s == "basic";
 }
 
 Buffer nullBuffer() {
@@ -50,7 +50,7 @@ std::shared_ptr<channel::Context> makeContext() {
       gSuite == "hip_ipc_messages") {
     return channel::hip_ipc::create();
   }
-  if (gSuite == "hip_basic") {
+  if (gSuite.rfind("hip_basic", 0) == 0) {
     return channel::hip_basic::create(channel::basic::create());
   }
   if (gSuite == "basic") {
@@ -137,7 +137,7 @@ void receiver(Endpoint& ep, bool gpu, const std::vector<uint8_t>& want) {
 
 std::vector<Case> makeCases() {
   std::vector<Case> cases;
-  const bool staged = gSuite == "hip_basic";
+  const bool staged = gSuite.rfind("hip_basic", 0) == 0;
 
   // channel_test.cc:19-43
   auto descriptors = [](Endpoint&) {
@@ -679,6 +679,47 @@ std::vector<Case> makeCases() {
     cases.push_back({"SendFromCpuToCpuSeveralChunks",
                      [](Endpoint& ep) { sender(ep, false, iota(3 * 1024 * 1024 + 5)); },
                      [](Endpoint& ep) { receiver(ep, false, iota(3 * 1024 * 1024 + 5)); }});
+    // A GPU tensor of several chunks landing in CPU memory (on the GPU-driven
+    // route the receiver's GPU cannot write the target itself).
+    cases.push_back({"SendFromGpuToCpuSeveralChunks",
+                     [](Endpoint& ep) { sender(ep, true, iota(5 * 1024 * 1024 + 3)); },
+                     [](Endpoint& ep) { receiver(ep, false, iota(5 * 1024 * 1024 + 3)); }});
+    // Tensors of several chunks in both directions at the same moment, three
+    // in a row each way with a one-chunk tensor in between: every end pushes
+    // into its own ring while it pulls from the peer's.
+    auto chunkedBothWays = [](Endpoint& ep) {
+      auto o = open(ep);
+      const int salt = ep.isServer() ? 3 : 11;
+      const size_t sizes[] = {6 * 1024 * 1024 + 17, 4096, 9 * 1024 * 1024, 3 * 1024 * 1024 + 1};
+      std::vector<std::unique_ptr<Data>> out, in;
+      std::vector<std::future<Error>> fs;
+      for (size_t n : sizes) {
+        std::vector<uint8_t> bytes(n);
+        for (size_t i = 0; i < n; ++i) {
+          bytes[i] = static_cast<uint8_t>((i * 31 + (i >> 11) + salt + n) & 0xff);
+        }
+        out.push_back(makeData(true, bytes));
+        in.push_back(makeData(true, n));
+      }
+      for (size_t k = 0; k < out.size(); ++k) {
+        fs.push_back(recvF(*o->ch, in[k]->buffer(), in[k]->size()));
+        fs.push_back(sendF(*o->ch, out[k]->buffer(), out[k]->size()));
+      }
+      for (auto& f : fs) {
+        EXPECT_OK(waitFor(f, "transfer"));
+      }
+      const int peerSalt = ep.isServer() ? 11 : 3;
+      for (size_t k = 0; k < in.size(); ++k) {
+        const size_t n = in[k]->size();
+        std::vector<uint8_t> want(n);
+        for (size_t i = 0; i < n; ++i) {
+          want[i] = static_cast<uint8_t>((i * 31 + (i >> 11) + peerSalt + n) & 0xff);
+        }
+        expectBytes(*in[k], want, "tensor from the peer");
+      }
+      ep.barrier();
+    };
+    cases.push_back({"ChunkedTensorsBothWaysAtOnce", chunkedBothWays, chunkedBothWays});
     // cuda_basic_test.cc:40-62: a pair of CPU endpoints is left to CPU channels.
     auto cpuToCpu = [](Endpoint&) {
       auto c = makeContext();
@@ -981,7 +1022,7 @@ int main(int argc, char** argv) {
   Args args = parseArgs(argc, argv);
   if (!knownSuite(args.suite)) {
     std::fprintf(
-        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_ipc_gated|hip_ipc_messages|hip_basic|basic|xth [--case S] [--list]\n",
+        stderr, "usage: %s --suite hip_xth|hip_ipc|hip_ipc_outbox|hip_ipc_gated|hip_ipc_messages|hip_basic|hip_basic_host_ring|hip_basic_small_ring|basic|xth [--case S] [--list]\n",
         argv[0]);
     return 2;
   }
@@ -999,6 +1040,17 @@ int main(int argc, char** argv) {
     // GPU waits for their word (short waits, so that the retry path runs too).
     ::setenv("TP_HIP_IPC_GATES", "1", 1);
     ::setenv("TP_HIP_IPC_GATE_WAIT_US", "200", 1);
+  }
+  if (gSuite == "hip_basic_host_ring") {
+    // Every tensor on the host-driven routes (one launch, event and message per chunk).
+    ::setenv("TP_HIP_BASIC_GPU_RING", "0", 1);
+  }
+  if (gSuite == "hip_basic_small_ring") {
+    // Three small slots and an impatient kernel: tensors span many turns of the
+    // ring, and ring kernels give up and are launched again all the time.
+    ::setenv("TP_HIP_BASIC_SLOT_BYTES", "65536", 1);
+    ::setenv("TP_HIP_BASIC_NUM_SLOTS", "3", 1);
+    ::setenv("TP_HIP_BASIC_RING_YIELD_US", "20", 1);
   }
   if (gSuite == "hip_ipc_messages") {
     // No signal words, no copy agent: every unit acknowledged by a message.

@@ -24,6 +24,7 @@
 // which is the closest a CPU run comes to a GPU memory fault.
 #include <tphip.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -748,6 +749,86 @@ int tphip_agent_done(void* agent, uint64_t ticket, int* done) {
   }
   *done = a->done.load(std::memory_order_acquire) >= ticket ? 1 : 0;
   return 0;
+}
+
+size_t tphip_ring_scratch_bytes(uint32_t num_slots) {
+  return 256;
+}
+
+} // extern "C"
+
+namespace {
+
+// The ring kernels of the real library, one chunk after the other on the
+// stream's thread: wait (bounded) for the other side's counter, copy, raise
+// this side's. The scratch holds what this end has completed, as the kernels
+// keep it.
+int ringTransfer(bool push, const tphip_ring_end* ring, const void* user, uint64_t bytes,
+                 uint64_t firstSeq, uint32_t yieldUs, void* stream, void* event) {
+  if (ring == nullptr || ring->slots == nullptr || ring->slot_bytes == 0 || ring->slot_bytes % 16 != 0 ||
+      ring->num_slots == 0 || ring->produced == nullptr || ring->consumed == nullptr ||
+      ring->scratch == nullptr || ring->status == nullptr || ring->abort == nullptr || user == nullptr ||
+      bytes == 0) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  const tphip_ring_end r = *ring;
+  auto ev = ref(event);
+  const uint64_t evSeq = ev != nullptr ? beginRecord(ev) : 0;
+  streamOf(stream).push([=] {
+    auto* published = word(r.scratch);
+    const auto* awaited = word(push ? r.consumed : r.produced);
+    auto* raised = word(push ? r.produced : r.consumed);
+    const uint64_t nChunks = (bytes + r.slot_bytes - 1) / r.slot_bytes;
+    bool yielded = false;
+    for (uint64_t k = 0; k < nChunks && !yielded; ++k) {
+      const uint64_t seq = firstSeq + k;
+      const uint64_t slot = seq % r.num_slots;
+      const uint64_t need = push ? (seq >= r.num_slots ? seq - r.num_slots + 1 : 0) : seq + 1;
+      const auto until = Clock::now() + std::chrono::microseconds(yieldUs);
+      while (awaited->load(std::memory_order_acquire) < need) {
+        if (Clock::now() > until || word(r.abort)->load(std::memory_order_acquire) != 0) {
+          yielded = true;
+          break;
+        }
+        std::this_thread::yield();
+      }
+      if (yielded) {
+        break;
+      }
+      const uint64_t off = k * r.slot_bytes;
+      const uint64_t len = std::min<uint64_t>(bytes - off, r.slot_bytes);
+      char* slotPtr = static_cast<char*>(r.slots) + slot * r.slot_bytes;
+      char* userPtr = static_cast<char*>(const_cast<void*>(user)) + off;
+      runCopies({push ? tphip_copy_desc{userPtr, slotPtr, len} : tphip_copy_desc{slotPtr, userPtr, len}});
+      if (published->load(std::memory_order_relaxed) != seq) {
+        std::fprintf(stderr, "fake tphip: ring call out of sequence (%llu complete, chunk %llu)\n",
+                     static_cast<unsigned long long>(published->load()), static_cast<unsigned long long>(seq));
+        std::abort();
+      }
+      published->store(seq + 1, std::memory_order_relaxed);
+      raised->store(seq + 1, std::memory_order_release);
+    }
+    word(r.status)->store(published->load(std::memory_order_relaxed) | (yielded ? TPHIP_RING_YIELDED : 0),
+                          std::memory_order_release);
+    if (ev != nullptr) {
+      completeEvent(ev, evSeq);
+    }
+  });
+  return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int tphip_ring_push(int dev, const tphip_ring_end* ring, const void* src, uint64_t bytes,
+                    uint64_t first_seq, uint32_t yield_us, uint32_t blocks, void* stream, void* event) {
+  return dev != 0 ? TPHIP_ERR_NO_DEVICE : ringTransfer(true, ring, src, bytes, first_seq, yield_us, stream, event);
+}
+
+int tphip_ring_pull(int dev, const tphip_ring_end* ring, void* dst, uint64_t bytes,
+                    uint64_t first_seq, uint32_t yield_us, uint32_t blocks, void* stream, void* event) {
+  return dev != 0 ? TPHIP_ERR_NO_DEVICE : ringTransfer(false, ring, dst, bytes, first_seq, yield_us, stream, event);
 }
 
 int tphip_profile_start(int dev, uint32_t max_launches) {

@@ -39,7 +39,9 @@ GPU_SUITES = [("channel_tests", "hip_xth", False), ("channel_tests", "hip_ipc", 
               ("pipe_tests", "two_process", True)]
 
 
-STAND_IN_SUITES = GPU_SUITES + [("channel_tests", "hip_ipc_gated", False), ("channel_tests", "hip_ipc_messages", False)]
+STAND_IN_SUITES = GPU_SUITES + [("channel_tests", "hip_ipc_gated", False), ("channel_tests", "hip_ipc_messages", False),
+                                ("channel_tests", "hip_basic_host_ring", False),
+                                ("channel_tests", "hip_basic_small_ring", False)]
 
 
 def main():

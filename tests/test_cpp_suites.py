@@ -18,7 +18,8 @@ CPU_SUITES = [("channel_tests", "basic"), ("channel_tests", "xth"),
               ("pipe_tests", "cpu_same_process"), ("pipe_tests", "cpu_two_process")]
 GPU_SUITES = [("channel_tests", "hip_xth"), ("channel_tests", "hip_ipc"), ("channel_tests", "hip_ipc_outbox"),
               ("channel_tests", "hip_ipc_gated"), ("channel_tests", "hip_ipc_messages"),
-              ("channel_tests", "hip_basic"),
+              ("channel_tests", "hip_basic"), ("channel_tests", "hip_basic_host_ring"),
+              ("channel_tests", "hip_basic_small_ring"),
               ("pipe_tests", "same_process"), ("pipe_tests", "two_process")]
 
 # tests/cpp/fake_tphip.cc: the C ABI of include/tphip.h with threads and memcpy behind it
@@ -70,7 +71,7 @@ def check_case(program, suite, case, stock_wire=False, stand_in=False):
     bad = [line for _, ok, line in per_case[case] if not ok]
     assert not bad, "\n".join(bad) + "\n" + err
     two_process = suite in ("basic", "hip_ipc", "hip_ipc_outbox", "hip_ipc_gated", "hip_ipc_messages", "hip_basic",
-                            "two_process", "cpu_two_process")
+                            "hip_basic_host_ring", "hip_basic_small_ring", "two_process", "cpu_two_process")
     assert len(per_case[case]) == (2 if two_process else 1), per_case[case]
 
 
