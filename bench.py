@@ -382,6 +382,43 @@ class PeerRun:
         return self.tp.bench_pingpong(self.pipe, True, send, recv, payloads=payloads,
                                       recv_payloads=recv_payloads, warmup=warmup, iters=iters)
 
+    def open_more(self, count):
+        """`count` more pipes between the two processes (same contexts, same channels)."""
+        self.pipe.write([], metadata=json.dumps({"op": "connect", "count": count})).wait()
+        more = [self.listener.accept(60000) for _ in range(count)]
+        d = self.pipe.read_descriptor(120000)
+        self.pipe.read([], []).wait()
+        assert d.metadata.decode() == "connected"
+        self.more = getattr(self, "more", []) + more
+        return more
+
+    def pingpong_multi(self, sends, recvs, size, warmup, iters):
+        """One ping-pong chain per pipe, all at once; returns (seconds of the timed rounds of the
+        slowest chain, timed round trips in all)."""
+        import threading
+
+        pipes = [self.pipe] + getattr(self, "more", [])
+        cmd = {"op": "pingpong_multi", "sizes": [size], "warmup": warmup, "iters": iters}
+        self.pipe.write([], metadata=json.dumps(cmd)).wait()
+        d = self.pipe.read_descriptor(120000)
+        self.pipe.read([], []).wait()
+        assert d.metadata.decode() == "ready"
+        lined_up = threading.Barrier(len(pipes) + 1)
+
+        totals = [0.0] * len(pipes)
+
+        def chain(k, q, st, rt):
+            lined_up.wait()
+            _, totals[k] = self.tp.bench_pingpong(q, True, st, rt, warmup=warmup, iters=iters)
+
+        threads = [threading.Thread(target=chain, args=(k,) + a) for k, a in enumerate(zip(pipes, sends, recvs))]
+        for t in threads:
+            t.start()
+        lined_up.wait()
+        for t in threads:
+            t.join()
+        return max(totals), len(pipes) * iters
+
     def close(self):
         try:
             try:
@@ -392,7 +429,7 @@ class PeerRun:
         finally:
             if self.proc.poll() is None:
                 self.proc.kill()
-            destroy([self.pipe, self.listener, self.ctx])
+            destroy(getattr(self, "more", []) + [self.pipe, self.listener, self.ctx])
 
 
 def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30, min_bytes=4096):
@@ -443,6 +480,49 @@ def bench_ipc(iters=100, warmup=5, max_bytes=1 << 30, min_bytes=4096):
             size *= 4
         if "4096" in out["sizes"]:
             out["rtt_4KiB_p50_us"] = out["sizes"]["4096"]["rtt_p50_us"]
+    finally:
+        peer.close()
+    return out
+
+
+def bench_ipc_in_flight(depth=4, sizes=(64 * MIB, 256 * MIB, 1 << 30)):
+    """configs[2]'s large tensors with `depth` transfers in flight between the two processes:
+    `depth` pipes over the same pair of contexts, one ping-pong chain on each, every chain with
+    buffers and a stream of its own on both sides. What the channel moves when it is kept busy,
+    beside the one-at-a-time round trips of the sweep."""
+    import numpy as np
+    import torch
+
+    from tensorpipe_amd import datagen
+    from tensorpipe_amd import pipe as tp
+
+    peer = PeerRun("basic:0,hip_ipc:11")
+    out = {"in_flight": depth, "sizes": {}}
+    try:
+        peer.open_more(depth - 1)
+        for size in sizes:
+            host = datagen.normal_large(datagen.SEED_BASE + 3, size // 4, "f32").view(np.uint8)
+            srcs = [torch.from_numpy(host).cuda() for _ in range(depth)]
+            del host
+            dsts = [torch.zeros(size, dtype=torch.uint8, device="cuda") for _ in range(depth)]
+            streams = [torch.cuda.Stream() for _ in range(depth)]
+            sends = [[tp.make_tensor(s, stream=st, target=(tp.HIP, 0))] for s, st in zip(srcs, streams)]
+            recvs = [[tp.make_tensor(d, stream=st)] for d, st in zip(dsts, streams)]
+            torch.cuda.synchronize()
+            iters = 200 if size <= 64 * MIB else 60 if size <= 256 * MIB else 16
+            warm = 10
+            dt, trips = peer.pingpong_multi(sends, recvs, size, warm, iters)
+            torch.cuda.synchronize()
+            ok = all(bool(torch.equal(s, d)) for s, d in zip(srcs, dsts))
+            # every round trip carries the tensor once in each direction
+            gbps = 2.0 * size * trips / dt / 1e9
+            out["sizes"][str(size)] = {
+                "round_trips": trips, "us_per_transfer": dt / (2 * trips) * 1e6, "payload_GBps": gbps,
+                "hbm_frac": 2.0 * gbps / HBM_PEAK_GBPS, "byte_exact": ok}
+            log(f"  ipc {depth} in flight {size:>11d} B  {dt / (2 * trips) * 1e6:9.1f} us per transfer  "
+                f"payload {gbps:8.1f} GB/s  hbm {2.0 * gbps / HBM_PEAK_GBPS:.3f}  exact={ok}")
+            del srcs, dsts, sends, recvs
+            torch.cuda.empty_cache()
     finally:
         peer.close()
     return out
@@ -714,6 +794,7 @@ LEGS = {
     "rpc_message_in_flight": bench_rpc_message_in_flight,
     "d2d_in_flight": bench_d2d_in_flight,
     "ipc": bench_ipc,
+    "ipc_in_flight": bench_ipc_in_flight,
     "staged": bench_staged,
     "staged_short": lambda: bench_staged(iters=20),
     "host_link": bench_link_ceiling,
@@ -801,6 +882,8 @@ def main():
         extra["rpc_message_in_flight"] = extra_leg("rpc_message_in_flight")
         log("[bench] cross-process IPC sweep")
         extra["ipc"] = extra_leg("ipc")
+        # the large tensors of the sweep with four transfers in flight between the processes
+        extra["ipc_in_flight"] = extra_leg("ipc_in_flight")
         log("[bench] host-staged 256 MiB")
         extra["staged"] = extra_leg("staged")
         # the same transfers with the runtime's hipMemcpyAsync instead of the copy kernel

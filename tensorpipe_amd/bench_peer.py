@@ -5,7 +5,9 @@
 Connects to URL, then serves commands that arrive as the metadata (JSON) of
 tensor-less messages: {"op": "pingpong", "sizes": [...], "device": "gpu"|"cpu",
 "warmup": W, "iters": K} allocates buffers, answers "ready" and runs the native
-echo loop; {"op": "quit"} ends the process."""
+echo loop; {"op": "connect", "count": N} opens N more pipes to the same URL;
+{"op": "pingpong_multi", ...} runs one echo loop per pipe side by side, each
+with buffers and a stream of its own; {"op": "quit"} ends the process."""
 import json
 import sys
 
@@ -33,12 +35,35 @@ def main(url, channels):
     # the transport is the one the URL names ("uv" is this library's TCP transport)
     ctx = tp.Context("bench_peer", transports=url.split("://", 1)[0] + ":0", channels=channels)
     p = ctx.connect(url)
+    extra = []
     while True:
         d = p.read_descriptor(timeout_ms=600000)
         p.read([], []).wait()
         cmd = json.loads(d.metadata.decode())
         if cmd["op"] == "quit":
             break
+        if cmd["op"] == "connect":
+            extra += [ctx.connect(url) for _ in range(cmd["count"])]
+            p.write([], metadata="connected").wait()
+            continue
+        if cmd["op"] == "pingpong_multi":
+            import threading
+
+            pipes = [p] + extra
+            n = cmd["sizes"][0]
+            bufs = [torch.zeros(n, dtype=torch.uint8, device="cuda") for _ in pipes]
+            streams = [torch.cuda.Stream() for _ in pipes]
+            tensors = [[tp.make_tensor(b, nbytes=n, stream=s, target=(tp.HIP, 0))] for b, s in zip(bufs, streams)]
+            torch.cuda.synchronize()
+            p.write([], metadata="ready").wait()
+            threads = [threading.Thread(target=tp.bench_pingpong, args=(q, False, t, t),
+                                        kwargs={"warmup": cmd["warmup"], "iters": cmd["iters"]})
+                       for q, t in zip(pipes, tensors)]
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join()
+            continue
         if cmd["op"] == "pingpong":
             bufs, tensors = [], []
             for n in cmd["sizes"]:
@@ -56,6 +81,8 @@ def main(url, channels):
             p.write([], metadata="ready").wait()
             tp.bench_pingpong(p, False, tensors, tensors, payloads=payloads,
                               recv_payloads=payloads, warmup=cmd["warmup"], iters=cmd["iters"])
+    for q in extra:
+        q.destroy()
     p.destroy()
     ctx.destroy()
 
