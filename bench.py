@@ -368,7 +368,7 @@ class PeerRun:
         child_env.update(env or {})
         child_env["PYTHONPATH"] = ROOT + os.pathsep + child_env.get("PYTHONPATH", "")
         self.proc = subprocess.Popen(
-            [sys.executable, "-m", "tensorpipe_amd.bench_peer", self.listener.url(self.transport), channels],
+            [sys.executable, os.path.join(ROOT, "bench_peer.py"), self.listener.url(self.transport), channels],
             env=child_env, cwd=ROOT)
         self.pipe = self.listener.accept(180000)
 
@@ -606,7 +606,7 @@ def bench_torch_rpc():
     if not os.path.exists(tp_rpc.library_path()):
         return {"error": "libtensorpipe_amd_torch_rpc.so is not built"}
     meeting = os.path.join(tempfile.mkdtemp(prefix="tp_rpc_"), "rendezvous")
-    ranks = [subprocess.Popen([sys.executable, "-m", "tensorpipe_amd.bench_rpc_peer", str(r), meeting],
+    ranks = [subprocess.Popen([sys.executable, os.path.join(ROOT, "bench_rpc_peer.py"), str(r), meeting],
                               stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, cwd=ROOT)
              for r in (1, 0)]
     try:
@@ -651,11 +651,85 @@ def bench_cold_copy():
         gbps = 2.0 * nbytes / (cold_us * 1e-6) / 1e9
         out[name] = {"kernel_avg_us": cold_us, "hbm_GBps": gbps, "hbm_frac": gbps / HBM_PEAK_GBPS,
                      "working_set_bytes": 2 * npairs * nbytes, "byte_exact": ok}
+        # The same with loads and stores both streaming past the caches, whatever the size:
+        # what a caller gets who knows that neither side will be touched again soon. (The
+        # channels keep cached stores up to 64 MiB: what arrives is what the receiver reads next.)
+        tables = [hip.make_table([(a, b, nbytes)])[0] for a, b in pairs]
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def rotate_streaming():
+            for _ in range(rounds):
+                for t in tables:
+                    hip.batched_copy_table(t, 1, stream=stream, unroll=4, blocks=0, nontemporal=3)
+            torch.cuda.synchronize()
+
+        rotate_streaming()
+        _, s_n, s_ms, _ = profiled(rotate_streaming, 64)
+        s_us = s_ms / max(s_n, 1) * 1e3
+        out[name]["streaming_kernel_avg_us"] = s_us
+        out[name]["streaming_hbm_frac"] = 2.0 * nbytes / (s_us * 1e-6) / 1e9 / HBM_PEAK_GBPS
         del pairs
         torch.cuda.empty_cache()
     # the figures of the 64 MiB case at the top level, where they have always been
     out.update(out["64MiB"])
     return out
+
+
+def bench_hbm_streams(nbytes=256 * MIB, nbuffers=8, rounds=4):
+    """What bounds a copy whose bytes all come from and go to HBM: a kernel that only reads and
+    one that only writes, with the copy kernels' access pattern, over rotating 256 MiB buffers
+    (2 GiB working set: nothing comes from the 256 MiB Infinity Cache), and the copy kernel over
+    the same buffers. A copy reads a byte for every byte it writes, so it cannot beat the mix of
+    the two one-directional rates, 2RW/(R+W)."""
+    import ctypes
+
+    import torch
+
+    from tensorpipe_amd import _native, hip
+
+    lib = _native.tphip()
+    bufs = [torch.empty(nbytes // 8, dtype=torch.int64, device="cuda").random_().view(torch.uint8)
+            for _ in range(nbuffers)]
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+
+    def measure(fn):
+        fn()
+        _, n, ms, _ = profiled(fn, nbuffers * rounds + 8)
+        return ms / max(n, 1) * 1e3
+
+    def reads():
+        for _ in range(rounds):
+            for b in bufs:
+                _native.check(lib.tphip_bench_stream(0, 0, b.data_ptr(), nbytes, stream))
+        torch.cuda.synchronize()
+
+    def writes():
+        for _ in range(rounds):
+            for b in bufs:
+                _native.check(lib.tphip_bench_stream(0, 1, b.data_ptr(), nbytes, stream))
+        torch.cuda.synchronize()
+
+    def copies():
+        for _ in range(rounds):
+            for k in range(0, nbuffers, 2):
+                hip.copy(bufs[k + 1], bufs[k], nbytes)
+                hip.copy(bufs[k], bufs[k + 1], nbytes)
+        torch.cuda.synchronize()
+
+    read_us = measure(reads)
+    copy_us = measure(copies)
+    write_us = measure(writes)  # last: it overwrites the buffers
+    r = nbytes / (read_us * 1e-6) / 1e9
+    w = nbytes / (write_us * 1e-6) / 1e9
+    c = 2.0 * nbytes / (copy_us * 1e-6) / 1e9
+    mix = 2.0 * r * w / (r + w)
+    return {"bytes": nbytes, "working_set_bytes": nbuffers * nbytes,
+            "read_only_us": read_us, "read_only_GBps": r, "read_only_frac": r / HBM_PEAK_GBPS,
+            "write_only_us": write_us, "write_only_GBps": w, "write_only_frac": w / HBM_PEAK_GBPS,
+            "mix_bound_GBps": mix, "mix_bound_frac": mix / HBM_PEAK_GBPS,
+            "copy_us": copy_us, "copy_hbm_GBps": c, "copy_frac": c / HBM_PEAK_GBPS,
+            "copy_frac_of_mix_bound": c / mix}
 
 
 def bench_link_duplex(nbytes=256 * MIB):
@@ -799,6 +873,7 @@ LEGS = {
     "staged_short": lambda: bench_staged(iters=20),
     "host_link": bench_link_ceiling,
     "host_link_duplex": bench_link_duplex,
+    "hbm_streams": bench_hbm_streams,
     "ipc_rtt": lambda: bench_ipc(iters=300, warmup=30, max_bytes=4096),
     "ipc_large": lambda: bench_ipc(iters=40, warmup=3, min_bytes=256 * MIB),
     "cpu_path": bench_cpu_path,
@@ -888,6 +963,9 @@ def main():
         extra["staged"] = extra_leg("staged")
         # the same transfers with the runtime's hipMemcpyAsync instead of the copy kernel
         extra["staged_hipMemcpyAsync"] = extra_leg("staged_short", env={"TP_HIP_BASIC_ENGINE": "sdma"})
+        # ... and with the copy kernel launched per chunk by the host (one launch, one polled
+        # event and two control messages per chunk) instead of the two kernels that walk the ring
+        extra["staged_host_driven"] = extra_leg("staged_short", env={"TP_HIP_BASIC_GPU_RING": "0"})
         extra["host_link"] = extra_leg("host_link")
         # both directions of the one host link at once: what bounds a staged transfer on one GPU
         duplex = extra_leg("host_link_duplex")
@@ -915,6 +993,8 @@ def main():
         # the headline's tensor with four transfers in flight instead of one
         extra["d2d_in_flight"] = extra_leg("d2d_in_flight")
         extra["d2d_cold_source"] = extra_leg("cold_copy")
+        # what HBM gives a kernel that only reads or only writes: the bound of any copy
+        extra["hbm_streams"] = extra_leg("hbm_streams")
         log("[bench] this library's CPU path (shm + basic)")
         extra["cpu_path"] = extra_leg("cpu_path")
         log("[bench] the same over TCP in the reference's wire format")

@@ -1,6 +1,6 @@
 """Echo side of the two-process benchmark configurations.
 
-    python -m tensorpipe_amd.bench_peer URL CHANNELS
+    python bench_peer.py URL CHANNELS
 
 Connects to URL, then serves commands that arrive as the metadata (JSON) of
 tensor-less messages: {"op": "pingpong", "sizes": [...], "device": "gpu"|"cpu",

@@ -1,6 +1,6 @@
 """One rank of the torch.distributed.rpc measurement of bench.py (leg "torch_rpc"):
 
-    python -m tensorpipe_amd.bench_rpc_peer <rank> <rendezvous file>
+    python bench_rpc_peer.py <rank> <rendezvous file>
 
 Two processes on the one GPU, PyTorch's own TensorPipe agent, this library's channels registered
 with it (tensorpipe_amd.torch_rpc). Rank 0 times rpc_sync(echo) round trips -- the tensor goes to

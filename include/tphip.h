@@ -301,6 +301,13 @@ int tphip_batched_copy_tuned(int dev, const tphip_copy_desc* table, uint32_t n, 
 int tphip_profile_start(int dev, uint32_t max_launches);
 int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* total_bytes);
 
+/* Measurement only: a kernel that only reads (`write` == 0) or only writes
+ * `bytes` bytes at `ptr` (device memory, 16-byte aligned) with the copy
+ * kernels' access pattern and launch shape, eight vectors in flight per lane.
+ * The two rates bound what a copy, which does both, can reach. The reference has
+ * no counterpart. */
+int tphip_bench_stream(int dev, int write, void* ptr, uint64_t bytes, void* stream);
+
 /* Runtime copy engine path (hipMemcpyAsync), kept only as the A/B comparison
  * for the kernel-driven copies; the channels use it only when asked to
  * (TP_HIP_BASIC_ENGINE=sdma|mixed), never by default. */

@@ -133,6 +133,7 @@ def tphip():
         lib.tphip_fill.argtypes = [i32, vp, i32, u64, vp]
         lib.tphip_test_slow_kernel.argtypes = [i32, vp, u64, vp]
         lib.tphip_test_set_table_limit.argtypes = [u64]
+        lib.tphip_bench_stream.argtypes = [i32, i32, vp, u64, vp]
         lib.tphip_ring_scratch_bytes.restype = ctypes.c_size_t
         lib.tphip_ring_scratch_bytes.argtypes = [u32]
         lib.tphip_ring_push.argtypes = [i32, P(RingEnd), vp, u64, u64, u32, u32, vp, vp]

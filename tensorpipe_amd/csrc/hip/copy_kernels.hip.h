@@ -940,6 +940,60 @@ __global__ __launch_bounds__(kBlockThreads) void ring_kernel(const RingArgs a) {
   }
 }
 
+// One-directional streams, for measurement only: what HBM gives a kernel that
+// only reads, or only writes, with the access pattern of the copy kernels
+// (lane g of G touches vectors g, g+G, ... U at a time, nontemporal). A copy
+// moves one byte each way, so its rate is bounded by the mix of the two.
+template <int U>
+__global__ __launch_bounds__(kBlockThreads) void read_stream_kernel(
+    const char* __restrict__ src, uint64_t bytes, u32x4* __restrict__ sink) {
+  const uint64_t g = static_cast<uint64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+  const uint64_t G = static_cast<uint64_t>(gridDim.x) * kBlockThreads;
+  const uint64_t nvec = bytes >> 4;
+  const uint64_t step = G * U;
+  const uint64_t full = nvec / step * step;
+  u32x4 acc = {0, 0, 0, 0};
+#pragma clang loop unroll(disable)
+  for (uint64_t base = 0; base < full; base += step) {
+    u32x4 v[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      v[j] = load16<1>(src + (base + j * G + g) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      acc ^= v[j];
+    }
+  }
+  for (uint64_t i = full + g; i < nvec; i += G) {
+    acc ^= load16<1>(src + i * 16);
+  }
+  // Keeps the loads alive; random data never produces this value in every lane.
+  if (acc.x == 0x9e3779b9u && acc.y == 0x7f4a7c15u && acc.z == 0xf39cc060u && acc.w == 0x5cedc834u) {
+    sink[0] = acc;
+  }
+}
+
+template <int U>
+__global__ __launch_bounds__(kBlockThreads) void write_stream_kernel(char* __restrict__ dst, uint64_t bytes, uint32_t seed) {
+  const uint64_t g = static_cast<uint64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+  const uint64_t G = static_cast<uint64_t>(gridDim.x) * kBlockThreads;
+  const uint64_t nvec = bytes >> 4;
+  const uint64_t step = G * U;
+  const uint64_t full = nvec / step * step;
+  const u32x4 v = {seed, static_cast<uint32_t>(g), seed ^ 0xa5a5a5a5u, static_cast<uint32_t>(g >> 32)};
+#pragma clang loop unroll(disable)
+  for (uint64_t base = 0; base < full; base += step) {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      store16<2>(dst + (base + j * G + g) * 16, v);
+    }
+  }
+  for (uint64_t i = full + g; i < nvec; i += G) {
+    store16<2>(dst + i * 16, v);
+  }
+}
+
 // A piece of a plan carried in the kernel arguments, written to device memory
 // at `byteOffset` of `dst` by one workgroup. Lets a caller that may not touch
 // pinned host memory or the copy engines put a plan of any size into device

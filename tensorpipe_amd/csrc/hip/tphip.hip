@@ -1592,6 +1592,27 @@ int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* 
   return count > 0 ? 0 : err;
 }
 
+int tphip_bench_stream(int dev, int write, void* ptr, uint64_t bytes, void* stream) {
+  if (ptr == nullptr || (reinterpret_cast<uintptr_t>(ptr) & 15u) != 0 || bytes < 16) {
+    return TPHIP_ERR_INVALID_ARG;
+  }
+  TPHIP_ON_DEVICE(dev);
+  DeviceState* st = nullptr;
+  int rc = getDevice(dev, &st);
+  if (rc != 0) {
+    return rc;
+  }
+  const dim3 grid(static_cast<uint32_t>(st->numCus > 0 ? st->numCus : 256));
+  ProfileScope prof(*st, static_cast<hipStream_t>(stream), bytes);
+  if (write != 0) {
+    return launchKernel(write_stream_kernel<8>, grid, dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream),
+                        static_cast<char*>(ptr), bytes, 0x5bd1e995u);
+  }
+  // the sink is never written (see the kernel): the buffer itself will do
+  return launchKernel(read_stream_kernel<8>, grid, dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream),
+                      static_cast<const char*>(ptr), bytes, static_cast<u32x4*>(ptr));
+}
+
 int tphip_memcpy_async(int dev, void* dst, const void* src, uint64_t bytes, void* stream) {
   TPHIP_ON_DEVICE(dev);
   TPHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, static_cast<hipStream_t>(stream)));

@@ -620,7 +620,9 @@ class ChannelImpl final : public ChannelImplBase {
     }
     const bool cpuSource = isCpu(op->buffer);
     const bool ring = !cpuSource && peerMappedOurRing_;
-    if (ring && op->length > chunkBytes_ && !gpuRingDisabled() && streamOutReady()) {
+    // (a ring that the runtime's copy engine is asked to fill cannot be driven by kernels)
+    if (ring && op->length > chunkBytes_ && !gpuRingDisabled() && engine() == Engine::kKernel &&
+        streamOutReady()) {
       startStreamSend(op);
       return;
     }

@@ -30,6 +30,9 @@
 
 #include <deque>
 
+#include <mutex>
+#include <unordered_map>
+
 #include <tensorpipe/channel/channel_base.h>
 #include <tensorpipe/channel/hip_common.h>
 #include <tensorpipe/common/hip_buffer.h>
@@ -59,6 +62,51 @@ struct StreamRef {
   bool operator==(const StreamRef& o) const {
     return stream == o.stream && device == o.device;
   }
+};
+
+// Where the tensors of one send come from. Both ends of this channel live in
+// one process, so the sender does not spell the list out on the connection: it
+// parks it here and sends its ticket, the receiver takes it out (for the 256
+// tensors of a many-tensor message that is 16 bytes on the wire instead of
+// 7 KiB, and no encoding or decoding on either side). A ticket that is not
+// here any more -- the sender failed and took its list back -- is an error, not
+// a dangling pointer.
+struct SourceList {
+  struct Item {
+    StreamRef src;
+    const void* ptr;
+    uint64_t length;
+  };
+  std::vector<Item> items;
+};
+
+class SourceLists {
+ public:
+  static SourceLists& get() {
+    static SourceLists* lists = new SourceLists();
+    return *lists;
+  }
+  uint64_t park(std::unique_ptr<SourceList> list) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    const uint64_t ticket = next_++;
+    parked_[ticket] = std::move(list);
+    return ticket;
+  }
+  std::unique_ptr<SourceList> take(uint64_t ticket) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    auto it = parked_.find(ticket);
+    if (it == parked_.end()) {
+      return nullptr;
+    }
+    auto list = std::move(it->second);
+    parked_.erase(it);
+    return list;
+  }
+
+ private:
+  std::mutex mutex_;
+  uint64_t next_{1};
+  std::unordered_map<uint64_t, std::unique_ptr<SourceList>> parked_;
 };
 
 class ChannelImpl final : public ChannelImplBase {
@@ -120,6 +168,7 @@ class ChannelImpl final : public ChannelImplBase {
     auto sends = std::move(sendOps_);
     sendOps_.clear();
     for (auto& op : sends) {
+      SourceLists::get().take(op->ticket); // if the receiver has not come for it, nobody will
       finishSend(op);
     }
     toLaunch_.clear();
@@ -138,6 +187,7 @@ class ChannelImpl final : public ChannelImplBase {
   struct SendOp {
     uint64_t seq;
     TSendCallback cb;
+    uint64_t ticket{0}; // of the source list parked for the receiver
     bool done{false};
   };
 
@@ -177,20 +227,16 @@ class ChannelImpl final : public ChannelImplBase {
     op->cb = std::move(cb);
     TP_VLOG(9) << "Channel " << id_ << " is encoding descriptor (#" << seq << ")";
 
-    // Wire format: n, then per tensor {src stream, src device, src pointer, length}.
+    // On the wire: how many tensors, and the ticket of their list.
     StageScope timer(Stage::kXthEncode);
-    WireWriter w;
-    w.reserve(8 + 28 * live.size());
-    w.u32(static_cast<uint32_t>(live.size()));
+    auto list = std::make_unique<SourceList>();
+    list->items.reserve(live.size());
     try {
       for (auto& e : live) {
         const HipBuffer& hb = e.buffer.unwrap<HipBuffer>();
         const int device = hipDeviceForPointer(hb.ptr);
         TP_THROW_ASSERT_IF(device < 0);
-        w.u64(reinterpret_cast<uint64_t>(hb.stream));
-        w.u32(static_cast<uint32_t>(device));
-        w.u64(reinterpret_cast<uint64_t>(hb.ptr));
-        w.u64(e.length);
+        list->items.push_back(SourceList::Item{StreamRef{hb.stream, device}, hb.ptr, e.length});
       }
     } catch (const std::exception& ex) {
       TP_LOG_WARNING() << "Channel " << id_ << " send failed: " << ex.what();
@@ -198,6 +244,10 @@ class ChannelImpl final : public ChannelImplBase {
       setError(TP_CREATE_ERROR(HipError, "hip_xth send", TPHIP_ERR_INVALID_ARG));
       return;
     }
+    WireWriter w;
+    w.u32(static_cast<uint32_t>(live.size()));
+    op->ticket = SourceLists::get().park(std::move(list));
+    w.u64(op->ticket);
 
     sendOps_.push_back(op);
     TP_VLOG(6) << "Channel " << id_ << " is writing descriptor (#" << seq << ")";
@@ -265,30 +315,33 @@ class ChannelImpl final : public ChannelImplBase {
   void copyFromDescriptor(const std::shared_ptr<RecvOp>& op, const std::vector<uint8_t>& bytes) {
     WireReader r(bytes.data(), bytes.size());
     const uint32_t n = r.u32();
+    const uint64_t ticket = r.u64();
     if (!r.ok() || n != op->entries.size()) {
       setError(TP_CREATE_ERROR(ShortReadError, static_cast<ssize_t>(op->entries.size()), n));
       return;
     }
     {
       StageScope decodeTimer(Stage::kXthDecode);
+      auto list = SourceLists::get().take(ticket);
+      if (!list || list->items.size() != n) {
+        // the sender is gone, or this is not a descriptor of this library's
+        setError(TP_CREATE_ERROR(ShortReadError, static_cast<ssize_t>(n), list ? static_cast<ssize_t>(list->items.size()) : -1));
+        return;
+      }
       try {
         op->pieces.reserve(n);
         for (uint32_t i = 0; i < n; ++i) {
-          StreamRef srcRef;
-          srcRef.stream = reinterpret_cast<void*>(r.u64());
-          srcRef.device = static_cast<int>(r.u32());
-          const void* src = reinterpret_cast<const void*>(r.u64());
-          const uint64_t len = r.u64();
-          if (!r.ok() || len != op->entries[i].length) {
+          const SourceList::Item& item = list->items[i];
+          if (item.length != op->entries[i].length) {
             setError(TP_CREATE_ERROR(
-                ShortReadError, static_cast<ssize_t>(op->entries[i].length), static_cast<ssize_t>(len)));
+                ShortReadError, static_cast<ssize_t>(op->entries[i].length), static_cast<ssize_t>(item.length)));
             return;
           }
           const HipBuffer& hb = op->entries[i].buffer.unwrap<HipBuffer>();
           StreamRef dstRef{hb.stream, hipDeviceForPointer(hb.ptr)};
           TP_THROW_ASSERT_IF(dstRef.device < 0);
-          op->pieces.push_back(RecvOp::Piece{srcRef, dstRef, tphip_copy_desc{src, hb.ptr, len}});
-          op->bytes += len;
+          op->pieces.push_back(RecvOp::Piece{item.src, dstRef, tphip_copy_desc{item.ptr, hb.ptr, item.length}});
+          op->bytes += item.length;
         }
       } catch (const std::exception& ex) {
         TP_LOG_WARNING() << "Channel " << id_ << " copy failed: " << ex.what();

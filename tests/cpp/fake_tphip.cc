@@ -848,6 +848,13 @@ int tphip_profile_stop(int dev, uint32_t* launches, double* total_ms, uint64_t* 
   return 0;
 }
 
+int tphip_bench_stream(int dev, int write, void* ptr, uint64_t bytes, void* stream) {
+  if (write != 0) {
+    return tphip_fill(dev, ptr, 0x5b, bytes, stream);
+  }
+  return 0;
+}
+
 int tphip_fill(int dev, void* ptr, int value, uint64_t bytes, void* stream) {
   streamOf(stream).push([ptr, value, bytes] {
     checkRange("fill target", ptr, bytes);

@@ -342,6 +342,28 @@ def test_ipc_direct_sizes(oracle, ipc_peer):
                [256, 4096, 16384, 65536, 1 << 20, (8 << 20) + 4, 64 << 20, 1, 17, 0])
 
 
+def test_ipc_sweep_points_between_the_others(oracle, ipc_peer):
+    # the sizes of the benchmark's sweep (4 KiB * 4^k) that the case above leaves out
+    _ipc_cases(oracle, ipc_peer, 8 << 20, [256 << 10, 4 << 20, 16 << 20])
+
+
+def test_ipc_at_the_boundary_between_copy_agent_and_launched_copy(oracle, ipc_peer):
+    """A unit of at most 128 KiB and 16 tensors is copied by the receiver's resident agent and
+    acknowledged by a signal word, anything larger by a launched kernel and a message: both sides
+    of both limits, every tensor against the oracle's per-tensor transfer."""
+    limit = 128 << 10
+    _ipc_cases(oracle, ipc_peer, 8 << 20, [limit - 1, limit, limit + 1, limit + 16])
+    for count in (16, 17):
+        for each in (limit // count, limit // count + 1):  # in all just inside / just outside the byte limit
+            hosts = [datagen.uniform_u8(900 + 31 * count + i, each) for i in range(count)]
+            srcs = [_gpu(h) for h in hosts]
+            outs, _ = ipc_peer.echo([tp.make_tensor(s, nbytes=each, target=(tp.HIP, 0)) for s in srcs], "gpu")
+            for o, h in zip(outs, hosts):
+                ref = np.full(each, FILL, np.uint8)
+                oracle.ipc_tensor(h, ref, each, slot=8 << 20, num_slots=4, in_flight=4)
+                _check_echo(o, ref, each)
+
+
 def test_ipc_direct_many_tensors_and_offsets(oracle, ipc_peer):
     import torch
 
