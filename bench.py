@@ -393,31 +393,40 @@ class PeerRun:
         return more
 
     def pingpong_multi(self, sends, recvs, size, warmup, iters):
-        """One ping-pong chain per pipe, all at once; returns (seconds of the timed rounds of the
-        slowest chain, timed round trips in all)."""
+        """One ping-pong chain per pipe, all at once; returns (seconds from the first chain's start
+        to the last chain's end, round trips in that time). The warm-up rounds are a run of their
+        own before it: first use maps the peer's buffers."""
         import threading
 
         pipes = [self.pipe] + getattr(self, "more", [])
-        cmd = {"op": "pingpong_multi", "sizes": [size], "warmup": warmup, "iters": iters}
-        self.pipe.write([], metadata=json.dumps(cmd)).wait()
-        d = self.pipe.read_descriptor(120000)
-        self.pipe.read([], []).wait()
-        assert d.metadata.decode() == "ready"
-        lined_up = threading.Barrier(len(pipes) + 1)
 
-        totals = [0.0] * len(pipes)
+        def run(rounds):
+            cmd = {"op": "pingpong_multi", "sizes": [size], "warmup": 0, "iters": rounds}
+            self.pipe.write([], metadata=json.dumps(cmd)).wait()
+            d = self.pipe.read_descriptor(120000)
+            self.pipe.read([], []).wait()
+            assert d.metadata.decode() == "ready"
+            lined_up = threading.Barrier(len(pipes) + 1)
+            began, ended = [0.0] * len(pipes), [0.0] * len(pipes)
 
-        def chain(k, q, st, rt):
+            def chain(k, q, st, rt):
+                lined_up.wait()
+                began[k] = time.perf_counter()
+                # 2: each chain waits for its receive stream on a thread of its own, not on the context's
+                self.tp.bench_pingpong(q, 2, st, rt, warmup=0, iters=rounds)
+                ended[k] = time.perf_counter()
+
+            threads = [threading.Thread(target=chain, args=(k,) + a)
+                       for k, a in enumerate(zip(pipes, sends, recvs))]
+            for t in threads:
+                t.start()
             lined_up.wait()
-            _, totals[k] = self.tp.bench_pingpong(q, True, st, rt, warmup=warmup, iters=iters)
+            for t in threads:
+                t.join()
+            return max(ended) - min(began)
 
-        threads = [threading.Thread(target=chain, args=(k,) + a) for k, a in enumerate(zip(pipes, sends, recvs))]
-        for t in threads:
-            t.start()
-        lined_up.wait()
-        for t in threads:
-            t.join()
-        return max(totals), len(pipes) * iters
+        run(warmup)
+        return run(iters), len(pipes) * iters
 
     def close(self):
         try:

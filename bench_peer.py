@@ -36,6 +36,7 @@ def main(url, channels):
     ctx = tp.Context("bench_peer", transports=url.split("://", 1)[0] + ":0", channels=channels)
     p = ctx.connect(url)
     extra = []
+    multi_bufs = multi_streams = bufs = tensors = None  # kept from one pingpong_multi to the next of the same size
     while True:
         d = p.read_descriptor(timeout_ms=600000)
         p.read([], []).wait()
@@ -51,8 +52,11 @@ def main(url, channels):
 
             pipes = [p] + extra
             n = cmd["sizes"][0]
-            bufs = [torch.zeros(n, dtype=torch.uint8, device="cuda") for _ in pipes]
-            streams = [torch.cuda.Stream() for _ in pipes]
+            if multi_bufs is None or multi_bufs[0].numel() != n or len(multi_bufs) != len(pipes):
+                multi_bufs = bufs = tensors = None  # the previous size's buffers go before the next size's come
+                multi_bufs = [torch.zeros(n, dtype=torch.uint8, device="cuda") for _ in pipes]
+                multi_streams = [torch.cuda.Stream() for _ in pipes]
+            bufs, streams = multi_bufs, multi_streams
             tensors = [[tp.make_tensor(b, nbytes=n, stream=s, target=(tp.HIP, 0))] for b, s in zip(bufs, streams)]
             torch.cuda.synchronize()
             p.write([], metadata="ready").wait()

@@ -126,7 +126,11 @@ int tpc_bench_transfer(tpc_pipe* sender, tpc_pipe* receiver, const tpc_payload* 
  * the initiator writes the message and waits to read it back; the echo side
  * reads and writes back. Both sides pass their own buffers. The initiator's
  * per_iter_us receives round-trip times including the final stream
- * synchronisation (tensorpipe/benchmark/benchmark_pipe.cc:463-468,571-577). */
+ * synchronisation (tensorpipe/benchmark/benchmark_pipe.cc:463-468,571-577).
+ * initiator: 0 = echo side, 1 = initiator, 2 = initiator that waits for its
+ * receive streams on a thread of the chain's own instead of the context's
+ * (for several chains side by side on one context: a wait on the context's
+ * thread would hold up every other chain's messages for a kernel's length). */
 int tpc_bench_pingpong(tpc_pipe* p, int initiator, const tpc_payload* payloads,
                        uint32_t num_payloads, void* const* recv_payload_ptrs,
                        const tpc_tensor* send_tensors, const tpc_tensor* recv_tensors,

@@ -11,6 +11,7 @@
 #include <mutex>
 #include <sstream>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include <tensorpipe/common/stage_timer.h>
@@ -604,11 +605,64 @@ struct PingPong : std::enable_shared_from_this<PingPong> {
   Clock::time_point begin, end, t0;
   Completion finished;
   std::atomic<bool> failed{false};
+  // With several chains side by side on one context the initiator's wait for
+  // its receive stream may not sit on the context's thread (every chain's
+  // messages pass through it): a thread of the chain's own waits instead.
+  bool syncOffLoop{false};
+  std::thread syncThread;
+  std::mutex syncMutex;
+  std::condition_variable syncCv;
+  bool syncPending{false}, syncQuit{false};
 
   void fail(const Error& e) {
     if (!failed.exchange(true)) {
       finished.set(e);
     }
+  }
+
+  // The initiator's end of a round: the bytes are in place, the round counts,
+  // the next one starts.
+  void roundTripOver() {
+    try {
+      syncRecvStreams(recvTensors.data(), static_cast<uint32_t>(recvTensors.size()));
+    } catch (const std::exception&) {
+      fail(TP_CREATE_ERROR(HipError, "stream sync", TPHIP_ERR_INVALID_ARG));
+      return;
+    }
+    if (round >= warmup && perIterUs != nullptr) {
+      perIterUs[round - warmup] = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+    }
+    ++round;
+    step();
+  }
+
+  void startSyncThread() {
+    syncOffLoop = true;
+    syncThread = std::thread([this] {
+      std::unique_lock<std::mutex> lock(syncMutex);
+      for (;;) {
+        syncCv.wait(lock, [this] { return syncPending || syncQuit; });
+        if (syncQuit) {
+          return;
+        }
+        syncPending = false;
+        lock.unlock();
+        roundTripOver();
+        lock.lock();
+      }
+    });
+  }
+
+  void stopSyncThread() {
+    if (!syncThread.joinable()) {
+      return;
+    }
+    {
+      std::lock_guard<std::mutex> lock(syncMutex);
+      syncQuit = true;
+    }
+    syncCv.notify_one();
+    syncThread.join();
   }
 
   void doWrite(std::function<void()> next) {
@@ -661,18 +715,15 @@ struct PingPong : std::enable_shared_from_this<PingPong> {
       t0 = Clock::now();
       doWrite(nullptr);
       doRead([self] {
-        try {
-          syncRecvStreams(self->recvTensors.data(), static_cast<uint32_t>(self->recvTensors.size()));
-        } catch (const std::exception&) {
-          self->fail(TP_CREATE_ERROR(HipError, "stream sync", TPHIP_ERR_INVALID_ARG));
+        if (!self->syncOffLoop) {
+          self->roundTripOver();
           return;
         }
-        if (self->round >= self->warmup && self->perIterUs != nullptr) {
-          self->perIterUs[self->round - self->warmup] =
-              std::chrono::duration<double, std::micro>(Clock::now() - self->t0).count();
+        {
+          std::lock_guard<std::mutex> lock(self->syncMutex);
+          self->syncPending = true;
         }
-        ++self->round;
-        self->step();
+        self->syncCv.notify_one();
       });
     } else {
       // The echo leaves from the buffers the message arrived in; a channel
@@ -705,6 +756,9 @@ int tpc_bench_pingpong(
   auto pp = std::make_shared<PingPong>();
   pp->pipe = p->pipe;
   pp->initiator = initiator != 0;
+  if (initiator == 2) {
+    pp->startSyncThread();
+  }
   pp->payloads.assign(payloads, payloads + numPayloads);
   pp->recvPayloadPtrs.assign(recvPayloadPtrs, recvPayloadPtrs + numPayloads);
   pp->sendTensors.assign(sendTensors, sendTensors + numTensors);
@@ -714,6 +768,7 @@ int tpc_bench_pingpong(
   pp->perIterUs = perIterUs;
   pp->step();
   int rc = pp->finished.wait(600000);
+  pp->stopSyncThread();
   if (rc != 0) {
     return rc;
   }

@@ -280,6 +280,8 @@ def bench_transfer(sender, receiver, send_tensors, recv_tensors, payloads=(), re
 
 def bench_pingpong(pipe, initiator, send_tensors, recv_tensors, payloads=(), recv_payloads=(),
                    warmup=5, iters=50):
+    """initiator: False/0 echo side, True/1 initiator, 2 initiator whose wait for the receive
+    streams runs on a thread of the chain's own (several chains side by side on one context)."""
     st, rt = _tensor_array(list(send_tensors)), _tensor_array(list(recv_tensors))
     parr, keep = _payload_array(list(payloads))
     pptrs = (ctypes.c_void_p * max(len(recv_payloads), 1))()
@@ -288,7 +290,7 @@ def bench_pingpong(pipe, initiator, send_tensors, recv_tensors, payloads=(), rec
     per = (ctypes.c_double * iters)()
     total = ctypes.c_double()
     rc = lib().tpc_bench_pingpong(
-        pipe._h, 1 if initiator else 0, parr, len(payloads), pptrs, st, rt, len(send_tensors),
+        pipe._h, int(initiator), parr, len(payloads), pptrs, st, rt, len(send_tensors),
         warmup, iters, per, ctypes.byref(total))
     if rc != 0:
         _fail("bench_pingpong")

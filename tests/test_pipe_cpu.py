@@ -137,6 +137,56 @@ def test_many_messages_in_order(pair):
         w.wait()
 
 
+@pytest.mark.parametrize("initiator", [1, 2])
+def test_ping_pong_chains_side_by_side(initiator):
+    """The benchmark harness's echo loop (tensorpipe/benchmark/benchmark_pipe.cc:463-468,571-577),
+    three chains at once over one pair of contexts, the initiator finishing its rounds on the
+    pipe's thread (1) or on a thread of the chain's own (2): every chain's last echo is its
+    own source, byte for byte."""
+    import threading
+
+    server = tp.Context("server", channels="basic:0")
+    client = tp.Context("client", channels="basic:0")
+    listener = server.listen()
+    pipes = []
+    for _ in range(3):
+        c = client.connect(listener.url())
+        pipes.append((c, listener.accept()))
+    rng = np.random.default_rng(7)
+    srcs = [rng.integers(0, 256, 70000 + 13 * k, dtype=np.uint8) for k in range(3)]
+    backs = [np.zeros_like(s) for s in srcs]
+    echo_bufs = [np.zeros_like(s) for s in srcs]
+    errors = []
+
+    def side(fn, *args, **kwargs):
+        try:
+            fn(*args, **kwargs)
+        except Exception as e:  # noqa: BLE001 - reported by the assertion below
+            errors.append(e)
+
+    threads = []
+    for (c, s), src, back, buf in zip(pipes, srcs, backs, echo_bufs):
+        t = [tp.make_tensor(buf)]
+        threads.append(threading.Thread(target=side, args=(tp.bench_pingpong, s, 0, t, t),
+                                        kwargs={"warmup": 2, "iters": 20}))
+        threads.append(threading.Thread(target=side, args=(tp.bench_pingpong, c, initiator,
+                                                           [tp.make_tensor(src)], [tp.make_tensor(back)]),
+                                        kwargs={"warmup": 2, "iters": 20}))
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(60)
+    assert not errors and not any(t.is_alive() for t in threads), errors
+    for src, back in zip(srcs, backs):
+        assert (src == back).all()
+    for c, s in pipes:
+        c.destroy()
+        s.destroy()
+    listener.destroy()
+    client.destroy()
+    server.destroy()
+
+
 def test_close_fails_pending_and_future_ops(pair):
     cpipe, spipe = pair()
     # make sure the pipe is established first
