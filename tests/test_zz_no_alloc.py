@@ -89,3 +89,39 @@ def test_limits_and_empty_tables():
 def test_full_size_table(oracle):
     sizes = [int(s) for s in datagen.loguniform_sizes(73, 16, 1 << 14, 1024)]
     _both_ways(oracle, sizes, seed=7005)
+
+
+def test_captured_in_a_graph_and_replayed(oracle):
+    """The callers this entry point is for include code under stream capture: a captured call
+    (plan pieces and table kernel, nothing else) copies on every replay what the sources hold
+    then, with eager calls that overwrite the shared plan array in between."""
+    import torch
+
+    lib = _native.tphip()
+    sizes = [int(s) for s in datagen.loguniform_sizes(74, 1, 1 << 18, 300)] + [0, 1, 15, 16, 17, 1 << 21]
+    layout, src_size, dst_size = _layout(sizes, 7006)
+    src = torch.zeros(src_size, dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(dst_size, dtype=torch.uint8, device="cuda")
+    table, n = hip.make_table([(src.data_ptr() + s, dst.data_ptr() + d, b) for s, d, b in layout])
+    # the device's array is looked up on the first call: that one stays outside the capture
+    _native.check(lib.tphip_batched_copy_noalloc(0, table, n, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = torch.cuda.current_stream().cuda_stream
+        _native.check(lib.tphip_batched_copy_noalloc(0, table, n, stream), "tphip_batched_copy_noalloc (capturing)")
+
+    for replay in range(3):
+        host_src = datagen.uniform_u8(7100 + replay, src_size)
+        src.copy_(torch.from_numpy(host_src))
+        dst.fill_(FILL)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = np.full(dst_size, FILL, dtype=np.uint8)
+        oracle.xth_message([(host_src[s:], ref[d:], b) for s, d, b in layout])
+        bad = np.nonzero(dst.cpu().numpy() != ref)[0]
+        assert bad.size == 0, f"replay {replay}: {bad.size} bytes differ from the oracle, first at {bad[0]}"
+        # an eager call with another table leaves its own plan in the array before the next replay
+        _both_ways(oracle, [333 + replay, 70000, 5], seed=7200 + replay)
