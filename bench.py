@@ -614,21 +614,29 @@ def bench_torch_rpc():
 
     if not os.path.exists(tp_rpc.library_path()):
         return {"error": "libtensorpipe_amd_torch_rpc.so is not built"}
-    meeting = os.path.join(tempfile.mkdtemp(prefix="tp_rpc_"), "rendezvous")
-    ranks = [subprocess.Popen([sys.executable, os.path.join(ROOT, "bench_rpc_peer.py"), str(r), meeting],
-                              stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, cwd=ROOT)
-             for r in (1, 0)]
-    try:
-        out, _ = ranks[1].communicate(timeout=120)
-        ranks[0].communicate(timeout=30)
-    finally:
-        for p in ranks:
-            if p.poll() is None:
-                p.kill()
-                p.wait()
-    if ranks[1].returncode != 0:
-        raise RuntimeError(f"rank 0 of the RPC group ended with {ranks[1].returncode}")
-    return json.loads(out.decode().strip().splitlines()[-1])
+    def run(mode):
+        meeting = os.path.join(tempfile.mkdtemp(prefix="tp_rpc_"), "rendezvous")
+        ranks = [subprocess.Popen([sys.executable, os.path.join(ROOT, "bench_rpc_peer.py"), str(r), meeting, mode],
+                                  stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, cwd=ROOT)
+                 for r in (1, 0)]
+        try:
+            out, _ = ranks[1].communicate(timeout=180)
+            ranks[0].communicate(timeout=30)
+        finally:
+            for p in ranks:
+                if p.poll() is None:
+                    p.kill()
+                    p.wait()
+        if ranks[1].returncode != 0:
+            raise RuntimeError(f"rank 0 of the RPC group ({mode}) ended with {ranks[1].returncode}")
+        return json.loads(out.decode().strip().splitlines()[-1])
+
+    out = run("all")
+    staged = run("staged")
+    out["gpu_tensors_hip_basic"] = staged["gpu_tensors_hip_basic"]
+    for k, v in staged["gpu_buffers_by_channel"].items():
+        out["gpu_buffers_by_channel"][k] = out["gpu_buffers_by_channel"].get(k, 0) + v
+    return out
 
 
 def bench_cold_copy():
