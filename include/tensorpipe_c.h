@@ -87,6 +87,7 @@ void tpc_context_destroy(tpc_context* ctx); /* join + free */
 /* 1 if the named channel was viable and got registered. */
 int tpc_context_has_channel(tpc_context* ctx, const char* name);
 
+/* url: one URL, or several separated by commas (one listener per transport). */
 tpc_listener* tpc_listen(tpc_context* ctx, const char* url);
 int tpc_listener_url(tpc_listener* l, const char* transport, char* out, size_t out_len);
 tpc_pipe* tpc_accept(tpc_listener* l, int timeout_ms);
@@ -96,6 +97,10 @@ tpc_pipe* tpc_connect(tpc_context* ctx, const char* url);
 void tpc_pipe_close(tpc_pipe* p);
 void tpc_pipe_destroy(tpc_pipe* p);
 int tpc_pipe_remote_name(tpc_pipe* p, char* out, size_t out_len);
+/* The transport the pipe's own connections run on after the handshake ("" before): the server
+ * moves a pipe to the best transport both ends have (tensorpipe/core/pipe_impl.cc:987-1042,
+ * 1108-1125). Not from a callback of the pipe. */
+int tpc_pipe_transport(tpc_pipe* p, char* out, size_t out_len);
 
 /* Pipe::write; returns an operation to wait on. Payload and tensor memory must
  * stay valid until the operation completed. */

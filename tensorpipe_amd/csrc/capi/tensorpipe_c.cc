@@ -276,7 +276,14 @@ int tpc_context_has_channel(tpc_context* ctx, const char* name) {
 tpc_listener* tpc_listen(tpc_context* ctx, const char* url) {
   TPC_GUARD_BEGIN
   auto out = std::make_unique<tpc_listener>();
-  out->listener = ctx->ctx->listen({std::string(url)});
+  // one URL, or several separated by commas (one per transport)
+  std::vector<std::string> urls;
+  std::string rest(url);
+  for (size_t at; (at = rest.find(',')) != std::string::npos; rest = rest.substr(at + 1)) {
+    urls.push_back(rest.substr(0, at));
+  }
+  urls.push_back(rest);
+  out->listener = ctx->ctx->listen(urls);
   return out.release();
   TPC_GUARD_END(nullptr)
 }
@@ -339,6 +346,17 @@ int tpc_pipe_remote_name(tpc_pipe* p, char* out, size_t outLen) {
   }
   std::memcpy(out, n.c_str(), n.size() + 1);
   return 0;
+}
+
+int tpc_pipe_transport(tpc_pipe* p, char* out, size_t outLen) {
+  TPC_GUARD_BEGIN
+  const std::string n = p->pipe->transportInUse();
+  if (n.size() + 1 > outLen) {
+    return TPC_ERR_FAILED;
+  }
+  std::memcpy(out, n.c_str(), n.size() + 1);
+  return 0;
+  TPC_GUARD_END(TPC_ERR_FAILED)
 }
 
 tpc_op* tpc_write_async(

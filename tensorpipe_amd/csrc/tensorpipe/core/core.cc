@@ -4,7 +4,9 @@
 // readDescriptor / read exactly the way user code drives the reference.
 //
 // Differences from the reference that a user can observe:
-//  * the pipe stays on the transport it was opened on (no transport upgrade);
+//  * the pipe moves to the best transport both ends have, as the reference's
+//    does (tensorpipe/core/pipe_impl.cc:987-1042,1108-1125): the server names
+//    it in its answer, the client opens the pipe's connections there;
 //  * by default control messages use common/wire.h instead of libnop, and
 //    all tensors of a message that map to one channel are handed to that
 //    channel as ONE batch when it implements channel::BatchedChannel, so a
@@ -21,8 +23,10 @@
 #include <tensorpipe/core/listener.h>
 #include <tensorpipe/core/pipe.h>
 
+#include <algorithm>
 #include <atomic>
 #include <deque>
+#include <future>
 #include <mutex>
 
 #include <unistd.h>
@@ -256,6 +260,22 @@ class ContextImpl final : public std::enable_shared_from_this<ContextImpl> {
       }
     }
     return nullptr;
+  }
+
+  // Names of the registered transports, the preferred (highest priority) one
+  // first (tensorpipe/core/context_impl.cc: transports are kept by priority).
+  std::vector<std::string> transportsByPriority() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    std::vector<std::pair<int64_t, std::string>> order;
+    for (auto& t : transports_) {
+      order.emplace_back(-t.second.first, t.first);
+    }
+    std::sort(order.begin(), order.end());
+    std::vector<std::string> names;
+    for (auto& o : order) {
+      names.push_back(std::move(o.second));
+    }
+    return names;
   }
 
   std::unordered_map<std::string, std::string> transportDescriptors() {
@@ -584,6 +604,16 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     return remoteName_;
   }
 
+  std::string transportInUse() {
+    auto self = shared_from_this();
+    auto answer = std::make_shared<std::promise<std::string>>();
+    auto ready = answer->get_future();
+    ctx_->defer([self, answer] {
+      answer->set_value(self->established_ ? self->transport_ : std::string());
+    });
+    return ready.get();
+  }
+
   void close() {
     auto self = shared_from_this();
     ctx_->defer([self] { self->setError(TP_CREATE_ERROR(PipeClosedError)); });
@@ -711,26 +741,26 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       return;
     }
     const uint64_t* replyToken = nullptr;
+    const uint64_t* descriptorToken = nullptr;
     for (auto& kv : answer.transportRegistrationIds) {
       if (kv.first == 1) {
         replyToken = &kv.second;
+      } else if (kv.first == 0) {
+        descriptorToken = &kv.second;
       }
     }
-    if (answer.transport != transport_ || replyToken == nullptr) {
-      // A peer that wants another transport for the pipe's own connections
-      // would have to be followed there; this library has one per pipe.
-      setError(TP_CREATE_ERROR(LogicError, "the peer chose transport " + answer.transport));
+    if (replyToken == nullptr || (answer.transport != transport_ && descriptorToken == nullptr)) {
+      setError(TP_CREATE_ERROR(LogicError, "brochure answer without the tokens it needs"));
       return;
     }
-    addr_ = answer.address; // where requested connections go
-    auto tctx = ctx_->transport(transport_);
-    replyConnection_ = tctx->connect(addr_);
-    replyConnection_->setId(id_ + ".r.tr_" + transport_);
-    introduce(*replyConnection_, *replyToken);
+    stockReplyToken_ = *replyToken;
     // From here on as with this library's own answer.
     WireWriter w;
     w.u8(kBrochureAnswer);
     w.str(remoteName_);
+    w.str(answer.transport);
+    w.str(answer.address);
+    w.u64(answer.transport != transport_ ? *descriptorToken : 0);
     w.u32(static_cast<uint32_t>(answer.channelRegistrationIds.size()));
     for (auto& c : answer.channelRegistrationIds) {
       w.str(c.first);
@@ -762,7 +792,40 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     } else {
       (void)r.str();
     }
-    auto tctx = ctx_->transport(transport_);
+    // tensorpipe/core/pipe_impl.cc:1108-1125: the server names the transport
+    // the pipe runs on from here. If that is not the one the pipe was opened
+    // on, its connection is opened again there, introduced by the token the
+    // server holds for it, and the first one is dropped.
+    const std::string chosen = r.str();
+    const std::string address = r.str();
+    const uint64_t descriptorToken = r.u64();
+    if (!r.ok()) {
+      setError(TP_CREATE_ERROR(LogicError, "malformed brochure answer"));
+      return;
+    }
+    auto tctx = ctx_->transport(chosen);
+    if (tctx == nullptr) {
+      setError(TP_CREATE_ERROR(LogicError, "the peer chose transport " + chosen + ", which this context lacks"));
+      return;
+    }
+    if (chosen != transport_) {
+      TP_VLOG(3) << "Pipe " << id_ << " moves from transport " << transport_ << " to " << chosen;
+      auto replacement = tctx->connect(address);
+      replacement->setId(id_ + ".tr_" + chosen);
+      introduce(*replacement, descriptorToken);
+      auto first = std::move(connection_);
+      connection_ = std::move(replacement);
+      first->close();
+      transport_ = chosen;
+      addr_ = address; // where requested connections go
+    } else if (stock_) {
+      addr_ = address; // tensorpipe/core/pipe_impl.cc:1091: the reference always goes by the answer
+    }
+    if (stock_) {
+      replyConnection_ = tctx->connect(addr_);
+      replyConnection_->setId(id_ + ".r.tr_" + transport_);
+      introduce(*replyConnection_, stockReplyToken_);
+    }
     const uint32_t nChannels = r.u32();
     for (uint32_t i = 0; i < nChannels && r.ok(); ++i) {
       std::string name = r.str();
@@ -853,15 +916,61 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       }
     }
 
+    // tensorpipe/core/pipe_impl.cc:987-1042: the preferred transport that both
+    // ends have, that reaches the peer, and that this listener listens on; the
+    // one the connection came in on if there is no better.
+    std::string chosen = transport_;
+    for (auto& name : ctx_->transportsByPriority()) {
+      auto remote = remoteTransports.find(name);
+      auto tctx = ctx_->transport(name);
+      auto addr = listener_->addresses().find(name);
+      if (remote == remoteTransports.end() || tctx == nullptr || addr == listener_->addresses().end() ||
+          !tctx->canCommunicateWithRemote(remote->second)) {
+        continue;
+      }
+      chosen = name;
+      break;
+    }
+    uint64_t descriptorToken = 0;
+    auto self = shared_from_this();
+    if (chosen != transport_) {
+      TP_VLOG(3) << "Pipe " << id_ << " moves from transport " << transport_ << " to " << chosen;
+      ++connectionsAwaited_;
+      replacingConnection_ = true;
+      descriptorToken = listener_->registerConnectionRequest(
+          [self, chosen](const Error& error, std::shared_ptr<transport::Connection> conn) {
+            if (self->error_) {
+              return;
+            }
+            if (error) {
+              self->setError(error);
+              return;
+            }
+            conn->setId(self->id_ + ".tr_" + chosen);
+            auto first = std::move(self->connection_);
+            self->connection_ = std::move(conn);
+            first->close();
+            self->transport_ = chosen;
+            self->replacingConnection_ = false;
+            if (--self->connectionsAwaited_ == 0) {
+              self->createServerChannels();
+            }
+          });
+      tokens_.push_back(descriptorToken);
+    }
+    auto chosenAddr = listener_->addresses().find(chosen);
+    const std::string address = chosenAddr != listener_->addresses().end() ? chosenAddr->second : std::string();
     if (stock_) {
-      writeStockBrochureAnswer(selected);
+      writeStockBrochureAnswer(selected, chosen, address, descriptorToken);
       return;
     }
     WireWriter w;
     w.u8(kBrochureAnswer);
     w.str(ctx_->name());
+    w.str(chosen);
+    w.str(address);
+    w.u64(descriptorToken);
     w.u32(static_cast<uint32_t>(selected.size()));
-    auto self = shared_from_this();
     for (auto& name : selected) {
       auto cctx = ctx_->channel(name);
       const size_t n = cctx->numConnectionsNeeded();
@@ -893,22 +1002,31 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     // While the client opens the channel connections nothing else would be
     // reading the primary connection, and a client that goes away now would
     // never be noticed: keep a read posted. Whatever it delivers before the
-    // pipe is established waits in earlyPacket_.
-    awaitingChannelConnections_ = true;
-    pumpPackets();
+    // pipe is established waits in earlyPacket_. (Not on a connection that
+    // the client is about to drop for its replacement on another transport.)
+    if (!replacingConnection_) {
+      awaitingChannelConnections_ = true;
+      pumpPackets();
+    }
   }
 
-  // tensorpipe/core/pipe_impl.cc:987-1042. The pipe's own connection keeps its
-  // transport, so only the descriptor reply connection is asked for besides
-  // those of the channels.
-  void writeStockBrochureAnswer(const std::vector<std::string>& selected) {
+  // tensorpipe/core/pipe_impl.cc:987-1042: the transport and where to reach
+  // it, a token for the descriptor connection when it moves there, one for the
+  // descriptor reply connection, and those of the channels.
+  void writeStockBrochureAnswer(
+      const std::vector<std::string>& selected,
+      const std::string& chosen,
+      const std::string& address,
+      uint64_t descriptorToken) {
     auto self = shared_from_this();
     tpnop::BrochureAnswer answer;
-    answer.transport = transport_;
-    auto addrIt = listener_->addresses().find(transport_);
-    answer.address = addrIt != listener_->addresses().end() ? addrIt->second : std::string();
-    auto tctx = ctx_->transport(transport_);
+    answer.transport = chosen;
+    answer.address = address;
+    auto tctx = ctx_->transport(chosen);
     answer.transportDomainDescriptor = tctx ? tctx->domainDescriptor() : std::string();
+    if (chosen != transport_) {
+      answer.transportRegistrationIds.emplace_back(0, descriptorToken);
+    }
     ++connectionsAwaited_;
     const uint64_t replyToken = listener_->registerConnectionRequest(
         [self](const Error& error, std::shared_ptr<transport::Connection> conn) {
@@ -919,7 +1037,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
             self->setError(error);
             return;
           }
-          conn->setId(self->id_ + ".r.tr_" + self->transport_);
+          conn->setId(self->id_ + ".r.tr");
           self->replyConnection_ = std::move(conn);
           if (--self->connectionsAwaited_ == 0) {
             self->createServerChannels();
@@ -953,8 +1071,10 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       answer.channelForDevicePair.emplace_back(std::make_pair(toNop(p.first.first), toNop(p.first.second)), p.second);
     }
     writeControl(tpnop::encode(answer));
-    awaitingChannelConnections_ = true;
-    pumpPackets();
+    if (!replacingConnection_) {
+      awaitingChannelConnections_ = true;
+      pumpPackets();
+    }
   }
 
   void onRequestedConnection(
@@ -1737,6 +1857,8 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   bool established_{false};
   // Server side, between the brochure answer and the last channel connection.
   bool awaitingChannelConnections_{false};
+  bool replacingConnection_{false}; // server: the client opens the pipe's connection again on another transport
+  uint64_t stockReplyToken_{0};
   bool haveEarlyPacket_{false};
   std::vector<uint8_t> earlyPacket_;
 
@@ -1937,6 +2059,10 @@ void Pipe::write(Message message, write_callback_fn fn) {
 
 const std::string& Pipe::getRemoteName() {
   return impl_->remoteName();
+}
+
+std::string Pipe::transportInUse() {
+  return impl_->transportInUse();
 }
 
 void Pipe::close() {

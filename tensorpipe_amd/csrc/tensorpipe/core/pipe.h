@@ -31,6 +31,12 @@ class Pipe final {
 
   const std::string& getRemoteName();
 
+  // Not in the reference: the name of the transport the pipe's own connections
+  // run on once the handshake is over (it may differ from the one the pipe was
+  // opened on, tensorpipe/core/pipe_impl.cc:1108-1125); empty until then. Waits
+  // for the pipe's loop: not to be called from one of its callbacks.
+  std::string transportInUse();
+
   void close();
 
   ~Pipe();

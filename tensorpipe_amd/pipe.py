@@ -78,6 +78,7 @@ def lib():
         l.tpc_pipe_close.argtypes = [vp]
         l.tpc_pipe_destroy.argtypes = [vp]
         l.tpc_pipe_remote_name.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
+        l.tpc_pipe_transport.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
         l.tpc_write_async.restype = vp
         l.tpc_write_async.argtypes = [vp, ctypes.c_char_p, P(Payload), u32, P(Tensor), u32]
         l.tpc_read_descriptor.argtypes = [vp, P(Descriptor), i32]
@@ -200,6 +201,12 @@ class Pipe:
         lib().tpc_pipe_remote_name(self._h, buf, 256)
         return buf.value.decode()
 
+    def transport(self):
+        """The transport the pipe runs on once the handshake is over ("" before)."""
+        buf = ctypes.create_string_buffer(64)
+        lib().tpc_pipe_transport(self._h, buf, 64)
+        return buf.value.decode()
+
     def close(self):
         lib().tpc_pipe_close(self._h)
 
@@ -246,6 +253,8 @@ class Context:
         return bool(lib().tpc_context_has_channel(self._h, name.encode()))
 
     def listen(self, url="shm://"):
+        """One URL, or several separated by commas: one listener per transport (a pipe opened on
+        one of them moves to the best transport both ends have)."""
         return Listener(lib().tpc_listen(self._h, url.encode()))
 
     def connect(self, url):

@@ -869,6 +869,48 @@ std::vector<Case> makeCases() {
   };
   cases.push_back({"WriteFromBothThenRead", writeThenRead, writeThenRead});
 
+  // tensorpipe/core/pipe_impl.cc:987-1042,1108-1125: a pipe opened over TCP
+  // between two contexts that both hold shm, preferred, moves there during the
+  // handshake; messages then flow both ways (CPU tensors: the case is about
+  // the pipe's own connections).
+  auto movesToShm = [](Endpoint& ep) {
+    auto e = std::make_unique<PipeEnd>();
+    e->ctx = std::make_shared<Context>(ContextOptions().name(ep.isServer() ? "server" : "client"));
+    e->ctx->registerTransport(1, "uv", transport::tcp::create());
+    e->ctx->registerTransport(2, "shm", transport::shm::create());
+    e->ctx->registerChannel(100, "basic", channel::basic::create());
+    const std::string shmUrl = "shm://" + ep.freshAddr();
+    InlineMessage im;
+    im.metadata = "after the move";
+    im.payloads = {{"payload #1", "payload metadata #1"}};
+    im.tensors = {{std::string(300000, 'x'), "tensor metadata #1", kCpu, nullopt},
+                  {"tensor #2", "", kCpu, kCpu}};
+    if (ep.isServer()) {
+      e->listener = e->ctx->listen({"uv://127.0.0.1:0", shmUrl});
+      const std::string url = e->listener->url("uv");
+      ep.sendNumber(static_cast<uint16_t>(std::stoi(url.substr(url.rfind(':') + 1))));
+      auto p = std::make_shared<std::promise<std::pair<Error, std::shared_ptr<Pipe>>>>();
+      auto f = p->get_future();
+      e->listener->accept([p](const Error& err, std::shared_ptr<Pipe> pipe) {
+        p->set_value({err, std::move(pipe)});
+      });
+      auto r = waitFor(f, "accept");
+      if (r.first) {
+        throw Fatal("accept failed: " + r.first.what());
+      }
+      e->pipe = std::move(r.second);
+      writeMessage(*e->pipe, im);
+      readAndCheck(*e->pipe, im, {kCpu, kCpu});
+    } else {
+      e->pipe = e->ctx->connect("uv://127.0.0.1:" + std::to_string(ep.recvNumber()));
+      readAndCheck(*e->pipe, im, {kCpu, kCpu});
+      writeMessage(*e->pipe, im);
+    }
+    EXPECT_EQ(e->pipe->transportInUse(), std::string("shm"));
+    ep.barrier();
+  };
+  cases.push_back({"PipeOpenedOverTcpMovesToShm", movesToShm, movesToShm});
+
   // listener_test.cc:21-60 (ClosingAbortsOperations): an accept that is pending
   // when the listener closes fails, once.
   auto listenerClose = [](Endpoint& ep) {

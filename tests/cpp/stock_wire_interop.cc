@@ -19,6 +19,7 @@
 #include <tensorpipe/tensorpipe.h> // the stock headers: listed first on the include path
 
 #include <cstdio>
+#include <unistd.h>
 #include <cstring>
 #include <future>
 #include <map>
@@ -32,9 +33,15 @@ using namespace tensorpipe;
 
 namespace {
 
-std::shared_ptr<Context> stockContext(const char* name) {
+// withShm: the stock end also holds its shm transport and prefers it. The native
+// end's transport of that name does not speak the stock one's protocol and says
+// so in its domain descriptor, so a pipe between the two must stay on "uv".
+std::shared_ptr<Context> stockContext(const char* name, bool withShm = false) {
   auto ctx = std::make_shared<Context>(ContextOptions().name(name));
   ctx->registerTransport(0, "uv", transport::uv::create());
+  if (withShm) {
+    ctx->registerTransport(1, "shm", transport::shm::create());
+  }
   ctx->registerChannel(0, "basic", channel::basic::create());
   return ctx;
 }
@@ -406,12 +413,21 @@ std::string nativeExchange(tpc_pipe* native, Pipe& stock, int salt) {
   return "";
 }
 
-int nativeConnectsToStock() {
-  auto ctx = stockContext("stock_server");
-  auto listener = ctx->listen({"uv://127.0.0.1"});
+std::string stayedOnUv(tpc_pipe* pipe) {
+  char transport[64] = {0};
+  if (tpc_pipe_transport(pipe, transport, sizeof(transport)) != 0 || std::string(transport) != "uv") {
+    return std::string("the native end runs on transport \"") + transport + "\"";
+  }
+  return "";
+}
+
+int nativeConnectsToStock(bool withShm) {
+  auto ctx = stockContext("stock_server", withShm);
+  auto listener = withShm ? ctx->listen({"uv://127.0.0.1", "shm://stock_wire_interop_" + std::to_string(::getpid())})
+                          : ctx->listen({"uv://127.0.0.1"});
   auto accepted = std::make_shared<std::promise<std::shared_ptr<Pipe>>>();
   listener->accept([accepted](const Error& e, std::shared_ptr<Pipe> p) { accepted->set_value(e ? nullptr : p); });
-  tpc_context* native = tpc_context_create_ex("native_client", "uv:0", "basic:0", 1);
+  tpc_context* native = tpc_context_create_ex("native_client", withShm ? "uv:0,shm:1" : "uv:0", "basic:0", 1);
   tpc_pipe* pipe = native != nullptr ? tpc_connect(native, listener->url("uv").c_str()) : nullptr;
   std::string problem;
   std::shared_ptr<Pipe> stock;
@@ -429,7 +445,10 @@ int nativeConnectsToStock() {
   if (problem.empty()) {
     problem = nativeExchange(pipe, *stock, 200);
   }
-  report("native_client_with_stock_server", problem);
+  if (problem.empty()) {
+    problem = stayedOnUv(pipe);
+  }
+  report(withShm ? "native_client_with_stock_server_both_hold_shm" : "native_client_with_stock_server", problem);
   stock.reset();
   if (pipe != nullptr) {
     tpc_pipe_destroy(pipe);
@@ -442,17 +461,19 @@ int nativeConnectsToStock() {
   return problem.empty() ? 0 : 1;
 }
 
-int stockConnectsToNative() {
-  tpc_context* native = tpc_context_create_ex("native_server", "uv:0", "basic:0", 1);
-  tpc_listener* listener = native != nullptr ? tpc_listen(native, "uv://127.0.0.1") : nullptr;
+int stockConnectsToNative(bool withShm) {
+  const char* caseName = withShm ? "stock_client_with_native_server_both_hold_shm" : "stock_client_with_native_server";
+  tpc_context* native = tpc_context_create_ex("native_server", withShm ? "uv:0,shm:1" : "uv:0", "basic:0", 1);
+  tpc_listener* listener =
+      native != nullptr ? tpc_listen(native, withShm ? "uv://127.0.0.1,shm://" : "uv://127.0.0.1") : nullptr;
   char url[256] = {0};
   std::string problem;
   if (listener == nullptr || tpc_listener_url(listener, "uv", url, sizeof(url)) != 0) {
     problem = std::string("native listen: ") + tpc_last_error();
-    report("stock_client_with_native_server", problem);
+    report(caseName, problem);
     return 1;
   }
-  auto ctx = stockContext("stock_client");
+  auto ctx = stockContext("stock_client", withShm);
   auto stock = ctx->connect(url);
   tpc_pipe* pipe = tpc_accept(listener, 30000);
   char name[256] = {0};
@@ -464,7 +485,10 @@ int stockConnectsToNative() {
   if (problem.empty()) {
     problem = nativeExchange(pipe, *stock, 300);
   }
-  report("stock_client_with_native_server", problem);
+  if (problem.empty()) {
+    problem = stayedOnUv(pipe);
+  }
+  report(caseName, problem);
   stock.reset();
   if (pipe != nullptr) {
     tpc_pipe_destroy(pipe);
@@ -485,8 +509,10 @@ int main(int argc, char** argv) {
   }
   int rc = compatConnectsToStock();
   rc |= stockConnectsToCompat();
-  rc |= nativeConnectsToStock();
-  rc |= stockConnectsToNative();
+  rc |= nativeConnectsToStock(false);
+  rc |= stockConnectsToNative(false);
+  rc |= nativeConnectsToStock(true);
+  rc |= stockConnectsToNative(true);
   if (std::strcmp(argv[1], "capture") == 0 && rc == 0) {
     FILE* f = std::fopen(argv[2], "w");
     if (f == nullptr) {

@@ -347,6 +347,17 @@ class Endpoint {
     }
   }
 
+  // A small number from one endpoint to the other (a port that the listening
+  // side only learns once it is bound).
+  void sendNumber(uint16_t v) {
+    writeByte(*control_, static_cast<uint8_t>(v >> 8));
+    writeByte(*control_, static_cast<uint8_t>(v & 0xff));
+  }
+  uint16_t recvNumber() {
+    const uint16_t hi = readByte(*control_);
+    return static_cast<uint16_t>(hi << 8 | readByte(*control_));
+  }
+
   // `n` connections whose i-th ends pair up on both sides.
   std::vector<std::shared_ptr<transport::Connection>> openConnections(size_t n) {
     const std::string addr = freshAddr();

@@ -187,6 +187,39 @@ def test_ping_pong_chains_side_by_side(initiator):
     server.destroy()
 
 
+@pytest.mark.parametrize("stock_wire", [False, True])
+@pytest.mark.parametrize("client_transports,server_transports,opened_on,ends_on", [
+    ("uv:1,shm:2", "uv:1,shm:2", "uv", "shm"),   # both prefer shm: the pipe moves there
+    ("uv:2,shm:1", "uv:1,shm:2", "uv", "shm"),   # the server's order decides
+    ("uv:1,shm:2", "uv:2,shm:1", "uv", "uv"),    # the server prefers what the pipe is on
+    ("uv:1", "uv:1,shm:2", "uv", "uv"),          # the client lacks the better one
+    ("uv:1,shm:2", "uv:1,shm:2", "shm", "shm"),  # already on the best
+])
+def test_pipe_moves_to_the_best_common_transport(stock_wire, client_transports, server_transports,
+                                                 opened_on, ends_on):
+    """tensorpipe/core/pipe_impl.cc:987-1042 (the server picks the transport, by its own
+    priorities, among those both ends have and it listens on) and :1108-1125 (the client opens
+    the pipe's connection again there): messages flow both ways afterwards, on the transport
+    the rule names."""
+    server = tp.Context("server", transports=server_transports, channels="basic:0", stock_wire=stock_wire)
+    client = tp.Context("client", transports=client_transports, channels="basic:0", stock_wire=stock_wire)
+    listener = server.listen("uv://127.0.0.1:0,shm://")
+    cpipe = client.connect(listener.url(opened_on))
+    spipe = listener.accept()
+    try:
+        rng = np.random.default_rng(11)
+        for sender, receiver in ((cpipe, spipe), (spipe, cpipe), (cpipe, spipe)):
+            data = rng.integers(0, 256, 3 * 1024 * 1024 + 5, dtype=np.uint8)
+            outs, pouts = _roundtrip(sender, receiver, [data, data[:77].copy()], payloads=[b"payload"])
+            assert (outs[0] == data).all() and (outs[1] == data[:77]).all()
+            assert bytes(pouts[0]) == b"payload"
+        assert cpipe.transport() == ends_on and spipe.transport() == ends_on
+        assert spipe.remote_name() == "client"
+    finally:
+        for o in (cpipe, spipe, listener, client, server):
+            o.destroy()
+
+
 def test_close_fails_pending_and_future_ops(pair):
     cpipe, spipe = pair()
     # make sure the pipe is established first

@@ -21,7 +21,10 @@ def test_compat_endpoint_and_stock_endpoint_understand_each_other():
     results = [line for line in proc.stdout.splitlines() if line.startswith("RESULT ")]
     assert [r.split()[1] for r in results] == [
         "compat_client_with_stock_server", "stock_client_with_compat_server",
-        "native_client_with_stock_server", "stock_client_with_native_server"], (
+        "native_client_with_stock_server", "stock_client_with_native_server",
+        # both ends also hold a transport called "shm" that the other's does not understand:
+        # the pipe stays on uv (tensorpipe/core/pipe_impl.cc:996-1012 goes by the domain descriptors)
+        "native_client_with_stock_server_both_hold_shm", "stock_client_with_native_server_both_hold_shm"], (
         proc.stdout[-2000:] + proc.stderr[-2000:])
     bad = [r for r in results if r.split()[2] != "OK"]
     assert not bad and proc.returncode == 0, "\n".join(bad) + proc.stderr[-2000:]
