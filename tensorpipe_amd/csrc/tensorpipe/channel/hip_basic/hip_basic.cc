@@ -228,6 +228,7 @@ enum MsgKind : uint8_t {
   kNotify = 4,   // ring route: chunk staged in {slot}
   kAck = 5,      // ring route: slot consumed
   kPulling = 6,  // stream route: the receiver's kernel for the next tensor has been launched
+  kStaged = 7,   // inner route: {count} more chunks are on their way through the inner channel
 };
 
 enum Route : uint8_t { kRouteInner = 0, kRouteRing = 1, kRouteStream = 2 };
@@ -334,6 +335,7 @@ class ChannelImpl final : public ChannelImplBase {
     deferred_.clear();
     sendQueue_.clear();
     recvPostQueue_.clear();
+    innerAwaited_.clear();
     recvOps_.clear();
     inbox_.clear();
     slotsInFlight_.clear();
@@ -577,6 +579,14 @@ class ChannelImpl final : public ChannelImplBase {
     } else if (kind == kPulling) {
       ++streamOut_.pullingSeen;
       pumpStreamOut();
+    } else if (kind == kStaged) {
+      const uint32_t count = r.u32();
+      if (!r.ok() || count == 0) {
+        failProtocol();
+        return;
+      }
+      innerChunksOnTheirWay_ += count;
+      admitInnerChunks();
     } else if (kind == kNotify) {
       const uint32_t count = r.u32();
       for (uint32_t i = 0; i < count; ++i) {
@@ -861,6 +871,7 @@ class ChannelImpl final : public ChannelImplBase {
       if (staged) {
         sourceDone(chunk->op); // the bytes now live in the pinned slot
       }
+      ++stagedToAnnounce_;
       cpuChannel_->send(
           CpuBuffer{chunk->hostPtr}, chunk->length, [this, self, chunk, staged](const Error& error) {
             ctx_->defer([this, self, chunk, staged, error] {
@@ -873,6 +884,20 @@ class ChannelImpl final : public ChannelImplBase {
           });
     }
     flushNotifies();
+    if (stagedToAnnounce_ > 0 && !error_) {
+      // The receiver takes a landing slot for a chunk only once the chunk is on
+      // its way (tensorpipe/channel/cuda_basic/channel_impl.cc:152-166,413-441:
+      // ready-to-send first, the receive buffer after it). A receiver that took
+      // its slots when the recv was posted would hold them while waiting for
+      // sends that may themselves be waiting, for send slots held by another
+      // channel of this context whose receiver finds no landing slot: with two
+      // channels sharing the contexts' rings that is a deadlock.
+      WireWriter w;
+      w.u8(kStaged);
+      w.u32(stagedToAnnounce_);
+      stagedToAnnounce_ = 0;
+      writeMessage(*controlConnection_, std::move(w.bytes()));
+    }
   }
 
   void sourceDone(const std::shared_ptr<Op>& op) {
@@ -1053,9 +1078,21 @@ class ChannelImpl final : public ChannelImplBase {
       chunk->length = len;
       chunk->offset = offset;
       chunk->op = op;
+      innerAwaited_.push_back(std::move(chunk));
+    }
+    admitInnerChunks();
+  }
+
+  // A chunk gets its landing area, and its inner recv, once the sender has said
+  // that it is on its way (kStaged), in chunk order.
+  void admitInnerChunks() {
+    while (innerChunksOnTheirWay_ > 0 && !innerAwaited_.empty() && !error_) {
+      --innerChunksOnTheirWay_;
+      auto chunk = innerAwaited_.front();
+      innerAwaited_.pop_front();
       recvPostQueue_.push_back(chunk);
-      if (isCpu(op->buffer)) {
-        chunk->hostPtr = static_cast<uint8_t*>(op->buffer.unwrap<CpuBuffer>().ptr) + offset;
+      if (isCpu(chunk->op->buffer)) {
+        chunk->hostPtr = static_cast<uint8_t*>(chunk->op->buffer.unwrap<CpuBuffer>().ptr) + chunk->offset;
         chunk->ready = true;
         continue;
       }
@@ -1475,6 +1512,9 @@ class ChannelImpl final : public ChannelImplBase {
   std::deque<Incoming> inbox_;
   std::deque<std::shared_ptr<SendChunk>> sendQueue_;
   std::deque<std::shared_ptr<RecvChunk>> recvPostQueue_;
+  std::deque<std::shared_ptr<RecvChunk>> innerAwaited_; // inner-route chunks the sender has not announced yet
+  uint32_t innerChunksOnTheirWay_{0}; // announced by the sender (kStaged), not yet matched with a chunk
+  uint32_t stagedToAnnounce_{0}; // inner sends started since the last kStaged message
   std::map<uint32_t, SlotAllocator::TSlot> slotsInFlight_;
   std::vector<StageItem> stagePending_;
   std::vector<RingItem> ringPending_;

@@ -472,6 +472,76 @@ std::vector<Case> makeCases() {
     cases.push_back({"BothEndsOnOneContext", oneContext, oneContext});
   }
 
+  // Two channels of one context carrying tensors the SAME way, receives and
+  // sends posted crosswise: the first channel's receive is posted before
+  // anything is sent on it, the second channel's send (far more than the
+  // connection buffers and the staging slots hold) before its receive. A
+  // receiver that took its landing slots when the receive was posted would hold
+  // them all for the first channel while the second one's sends hold every send
+  // slot: the reference takes a receive buffer only for a chunk that is on its
+  // way (tensorpipe/channel/cuda_basic/channel_impl.cc:413-441).
+  if (gSuite != "hip_ipc" && gSuite.rfind("hip_ipc_", 0) != 0) {
+    auto crosswise = [](Endpoint& ep) {
+      const std::string base = ep.freshAddr();
+      if (ep.isServer()) {
+        auto ctx = makeContext();
+        ctx->setId("two_flows_one_way");
+        if (!ctx->isViable()) {
+          throw Fatal("context is not viable");
+        }
+        const size_t n = ctx->numConnectionsNeeded();
+        const std::string addr = base + "_flows";
+        auto listener = ep.transport()->listen(addr);
+        std::shared_ptr<channel::Channel> from[2], to[2];
+        for (int flow = 0; flow < 2; ++flow) {
+          std::vector<std::shared_ptr<transport::Connection>> connecting(n), accepted(n);
+          for (size_t i = 0; i < n; ++i) {
+            connecting[i] = ep.transport()->connect(addr);
+            accepted[i] = acceptOne(*listener);
+            writeByte(*connecting[i], static_cast<uint8_t>(i));
+            if (readByte(*accepted[i]) != i) {
+              throw Fatal("connections paired out of order");
+            }
+          }
+          from[flow] = ctx->createChannel(std::move(accepted), channel::Endpoint::kListen);
+          to[flow] = ctx->createChannel(std::move(connecting), channel::Endpoint::kConnect);
+        }
+        listener->close();
+        {
+          auto fill = [](size_t bytes, int salt) {
+            std::vector<uint8_t> v(bytes);
+            for (size_t j = 0; j < v.size(); ++j) {
+              v[j] = static_cast<uint8_t>((j * 23 + static_cast<size_t>(salt) * 31 + (j >> 13)) % 241);
+            }
+            return v;
+          };
+          const size_t small = 6 * 65536 + 17, large = (5u << 20) + 3;
+          auto out0 = makeData(gGpu, fill(small, 1)), out1 = makeData(gGpu, fill(large, 2));
+          auto in0 = makeData(gGpu, small), in1 = makeData(gGpu, large);
+          std::vector<std::future<Error>> fs;
+          fs.push_back(recvF(*to[0], in0->buffer(), small));
+          fs.push_back(sendF(*from[1], out1->buffer(), large));
+          std::this_thread::sleep_for(std::chrono::milliseconds(100)); // the second flow fills what it can
+          fs.push_back(sendF(*from[0], out0->buffer(), small));
+          std::this_thread::sleep_for(std::chrono::milliseconds(100)); // the first flow's receiver has heard of it
+          fs.push_back(recvF(*to[1], in1->buffer(), large));
+          for (auto& f : fs) {
+            EXPECT_OK(waitFor(f, "transfer"));
+          }
+          expectBytes(*in0, fill(small, 1), "first flow");
+          expectBytes(*in1, fill(large, 2), "second flow");
+        }
+        for (int flow = 0; flow < 2; ++flow) {
+          from[flow].reset();
+          to[flow].reset();
+        }
+        ctx->join();
+      }
+      ep.barrier();
+    };
+    cases.push_back({"TwoFlowsOneWayPostedCrosswise", crosswise, crosswise});
+  }
+
   // Two channels between the same two contexts at once (two pipes between two
   // workers, as RPC agents open them), traffic flowing the opposite way on each:
   // they share each context's loop, poller and staging rings, and one tensor is
