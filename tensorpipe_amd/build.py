@@ -61,6 +61,7 @@ HOST_SOURCES = [
     "capi/tensorpipe_c.cc",
     "bridge/bridge_amd.cc",
     "tensorpipe/transport/tcp/tcp.cc",
+    "tensorpipe/transport/shm_stock/shm_stock.cc",
     "nopwire/nop_wire.cc",
     "nopwire/compat_pipe.cc",
 ]

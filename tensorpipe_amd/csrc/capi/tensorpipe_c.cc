@@ -221,6 +221,9 @@ tpc_context* tpc_context_create_ex(const char* name, const char* transports, con
       out->ctx->registerTransport(t.second, "shm", transport::shm::create());
     } else if (t.first == "uv") {
       out->ctx->registerTransport(t.second, "uv", transport::tcp::create());
+    } else if (t.first == "shm_stock") {
+      // the reference's shm protocol, under the name its contexts know it by
+      out->ctx->registerTransport(t.second, "shm", transport::shm_stock::create());
     } else {
       setLastError("unknown transport " + t.first);
       return nullptr;

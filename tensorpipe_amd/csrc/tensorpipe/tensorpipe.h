@@ -18,6 +18,7 @@
 #include <tensorpipe/transport/error.h>
 #include <tensorpipe/transport/shm/factory.h>
 #include <tensorpipe/transport/tcp/factory.h>
+#include <tensorpipe/transport/shm_stock/factory.h>
 
 #include <tensorpipe/channel/context.h>
 #include <tensorpipe/channel/error.h>

@@ -413,21 +413,35 @@ std::string nativeExchange(tpc_pipe* native, Pipe& stock, int salt) {
   return "";
 }
 
-std::string stayedOnUv(tpc_pipe* pipe) {
+std::string runsOn(tpc_pipe* pipe, const std::string& expected) {
   char transport[64] = {0};
-  if (tpc_pipe_transport(pipe, transport, sizeof(transport)) != 0 || std::string(transport) != "uv") {
-    return std::string("the native end runs on transport \"") + transport + "\"";
+  if (tpc_pipe_transport(pipe, transport, sizeof(transport)) != 0 || std::string(transport) != expected) {
+    return std::string("the native end runs on transport \"") + transport + "\", not on " + expected;
   }
   return "";
 }
 
-int nativeConnectsToStock(bool withShm) {
+// What the native end holds beside uv: nothing, this library's own shm transport
+// (another protocol under the same name: the pipe must stay on uv), or the
+// transport that speaks the stock shm protocol (the pipe must move there, in
+// both roles: tensorpipe/core/pipe_impl.cc:987-1042,1108-1125).
+enum class NativeShm { kNone, kOwnProtocol, kStockProtocol };
+
+const char* nativeTransports(NativeShm shm) {
+  return shm == NativeShm::kNone ? "uv:0" : shm == NativeShm::kOwnProtocol ? "uv:0,shm:1" : "uv:0,shm_stock:1";
+}
+std::string caseSuffix(NativeShm shm) {
+  return shm == NativeShm::kNone ? "" : shm == NativeShm::kOwnProtocol ? "_both_hold_shm" : "_moves_to_shm";
+}
+
+int nativeConnectsToStock(NativeShm shm) {
+  const bool withShm = shm != NativeShm::kNone;
   auto ctx = stockContext("stock_server", withShm);
   auto listener = withShm ? ctx->listen({"uv://127.0.0.1", "shm://stock_wire_interop_" + std::to_string(::getpid())})
                           : ctx->listen({"uv://127.0.0.1"});
   auto accepted = std::make_shared<std::promise<std::shared_ptr<Pipe>>>();
   listener->accept([accepted](const Error& e, std::shared_ptr<Pipe> p) { accepted->set_value(e ? nullptr : p); });
-  tpc_context* native = tpc_context_create_ex("native_client", withShm ? "uv:0,shm:1" : "uv:0", "basic:0", 1);
+  tpc_context* native = tpc_context_create_ex("native_client", nativeTransports(shm), "basic:0", 1);
   tpc_pipe* pipe = native != nullptr ? tpc_connect(native, listener->url("uv").c_str()) : nullptr;
   std::string problem;
   std::shared_ptr<Pipe> stock;
@@ -446,9 +460,9 @@ int nativeConnectsToStock(bool withShm) {
     problem = nativeExchange(pipe, *stock, 200);
   }
   if (problem.empty()) {
-    problem = stayedOnUv(pipe);
+    problem = runsOn(pipe, shm == NativeShm::kStockProtocol ? "shm" : "uv");
   }
-  report(withShm ? "native_client_with_stock_server_both_hold_shm" : "native_client_with_stock_server", problem);
+  report("native_client_with_stock_server" + caseSuffix(shm), problem);
   stock.reset();
   if (pipe != nullptr) {
     tpc_pipe_destroy(pipe);
@@ -461,9 +475,10 @@ int nativeConnectsToStock(bool withShm) {
   return problem.empty() ? 0 : 1;
 }
 
-int stockConnectsToNative(bool withShm) {
-  const char* caseName = withShm ? "stock_client_with_native_server_both_hold_shm" : "stock_client_with_native_server";
-  tpc_context* native = tpc_context_create_ex("native_server", withShm ? "uv:0,shm:1" : "uv:0", "basic:0", 1);
+int stockConnectsToNative(NativeShm shm) {
+  const bool withShm = shm != NativeShm::kNone;
+  const std::string caseName = "stock_client_with_native_server" + caseSuffix(shm);
+  tpc_context* native = tpc_context_create_ex("native_server", nativeTransports(shm), "basic:0", 1);
   tpc_listener* listener =
       native != nullptr ? tpc_listen(native, withShm ? "uv://127.0.0.1,shm://" : "uv://127.0.0.1") : nullptr;
   char url[256] = {0};
@@ -486,7 +501,7 @@ int stockConnectsToNative(bool withShm) {
     problem = nativeExchange(pipe, *stock, 300);
   }
   if (problem.empty()) {
-    problem = stayedOnUv(pipe);
+    problem = runsOn(pipe, shm == NativeShm::kStockProtocol ? "shm" : "uv");
   }
   report(caseName, problem);
   stock.reset();
@@ -509,10 +524,12 @@ int main(int argc, char** argv) {
   }
   int rc = compatConnectsToStock();
   rc |= stockConnectsToCompat();
-  rc |= nativeConnectsToStock(false);
-  rc |= stockConnectsToNative(false);
-  rc |= nativeConnectsToStock(true);
-  rc |= stockConnectsToNative(true);
+  rc |= nativeConnectsToStock(NativeShm::kNone);
+  rc |= stockConnectsToNative(NativeShm::kNone);
+  rc |= nativeConnectsToStock(NativeShm::kOwnProtocol);
+  rc |= stockConnectsToNative(NativeShm::kOwnProtocol);
+  rc |= nativeConnectsToStock(NativeShm::kStockProtocol);
+  rc |= stockConnectsToNative(NativeShm::kStockProtocol);
   if (std::strcmp(argv[1], "capture") == 0 && rc == 0) {
     FILE* f = std::fopen(argv[2], "w");
     if (f == nullptr) {

@@ -646,6 +646,179 @@ static int runCompatPipe() {
   return failures == 0 ? 0 : 1;
 }
 
+// Messages of every size class both ways over one connection of any transport, reads
+// posted before and after the writes, unsized and exact-length reads alternating; then
+// an exact-length read that meets a message of another length. Returns the failures.
+static int exerciseConnections(
+    transport::Context& serverSide,
+    transport::Context& clientSide,
+    transport::Listener& listener,
+    const std::string& addr) {
+  int failed = 0;
+  std::promise<std::shared_ptr<transport::Connection>> acceptedP;
+  listener.accept([&](const Error& e, std::shared_ptr<transport::Connection> c) {
+    acceptedP.set_value(e ? nullptr : std::move(c));
+  });
+  auto conn = clientSide.connect(addr);
+  auto acceptedF = acceptedP.get_future();
+  CHECK(acceptedF.wait_for(std::chrono::seconds(30)) == std::future_status::ready);
+  auto accepted = acceptedF.get();
+  CHECK(accepted != nullptr);
+  if (!accepted) {
+    return failed + 1;
+  }
+  (void)serverSide;
+  const std::vector<size_t> sizes = {0, 1, 3, 4, 5, 4096, 65537, 1 << 20, (2u << 20) - 4, 2u << 20, (24u << 20) + 3};
+  for (int direction = 0; direction < 2; ++direction) {
+    auto& from = direction == 0 ? conn : accepted;
+    auto& to = direction == 0 ? accepted : conn;
+    std::vector<std::vector<uint8_t>> sent;
+    for (size_t k = 0; k < sizes.size(); ++k) {
+      std::vector<uint8_t> m(sizes[k]);
+      for (size_t i = 0; i < m.size(); ++i) {
+        m[i] = static_cast<uint8_t>((i * 13 + k * 7 + direction) % 251);
+      }
+      sent.push_back(std::move(m));
+    }
+    std::vector<std::future<bool>> results;
+    auto postRead = [&](size_t k) {
+      auto p = std::make_shared<std::promise<bool>>();
+      results.push_back(p->get_future());
+      const std::vector<uint8_t>* want = &sent[k];
+      if (k % 2 == 0) {
+        to->read([p, want](const Error& e, const void* ptr, size_t len) {
+          p->set_value(!e && len == want->size() && (len == 0 || std::memcmp(ptr, want->data(), len) == 0));
+        });
+      } else {
+        auto buf = std::make_shared<std::vector<uint8_t>>(want->size());
+        to->read(buf->data(), buf->size(), [p, want, buf](const Error& e, const void*, size_t len) {
+          p->set_value(!e && len == want->size() && *buf == *want);
+        });
+      }
+    };
+    for (size_t k = 0; k < sizes.size() / 2; ++k) {
+      postRead(k); // these wait for their bytes
+    }
+    auto wroteAll = std::make_shared<std::promise<bool>>();
+    auto allFine = std::make_shared<std::atomic<bool>>(true);
+    for (size_t k = 0; k < sizes.size(); ++k) {
+      const bool last = k + 1 == sizes.size();
+      from->write(sent[k].data(), sent[k].size(), [wroteAll, allFine, last](const Error& e) {
+        if (e) {
+          allFine->store(false);
+        }
+        if (last) {
+          wroteAll->set_value(allFine->load());
+        }
+      });
+    }
+    for (size_t k = sizes.size() / 2; k < sizes.size(); ++k) {
+      postRead(k); // these find their bytes already there, or on their way
+    }
+    for (auto& r : results) {
+      CHECK(r.wait_for(std::chrono::seconds(30)) == std::future_status::ready && r.get());
+    }
+    auto wroteF = wroteAll->get_future();
+    CHECK(wroteF.wait_for(std::chrono::seconds(30)) == std::future_status::ready && wroteF.get());
+  }
+  // An exact-length read that meets a message of another length fails the connection.
+  {
+    auto other = clientSide.connect(addr);
+    std::promise<std::shared_ptr<transport::Connection>> p2;
+    listener.accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p2.set_value(e ? nullptr : std::move(c)); });
+    auto acc2 = p2.get_future().get();
+    CHECK(acc2 != nullptr);
+    const std::string msg = "five!";
+    other->write(msg.data(), msg.size(), [](const Error&) {});
+    char buf[4];
+    std::promise<bool> failedRead;
+    acc2->read(buf, sizeof(buf), [&](const Error& e, const void*, size_t) { failedRead.set_value(static_cast<bool>(e)); });
+    CHECK(failedRead.get_future().get());
+  }
+  // A peer that writes and leaves before anybody reads: the messages, then the end; a write
+  // to it fails.
+  {
+    auto other = clientSide.connect(addr);
+    std::promise<std::shared_ptr<transport::Connection>> p3;
+    listener.accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p3.set_value(e ? nullptr : std::move(c)); });
+    auto acc3 = p3.get_future().get();
+    CHECK(acc3 != nullptr);
+    const std::string one = "first", two(70000, 'z');
+    std::promise<void> wrote;
+    other->write(one.data(), one.size(), [](const Error&) {});
+    other->write(two.data(), two.size(), [&](const Error&) { wrote.set_value(); });
+    wrote.get_future().get();
+    other->close();
+    other.reset();
+    std::this_thread::sleep_for(std::chrono::milliseconds(100));
+    for (int i = 0; i < 3; ++i) {
+      std::promise<std::pair<bool, std::string>> gotP;
+      acc3->read([&](const Error& e, const void* ptr, size_t len) {
+        gotP.set_value({static_cast<bool>(e), e ? e.what() : std::string(static_cast<const char*>(ptr), len)});
+      });
+      auto g = gotP.get_future().get();
+      if (i == 0) {
+        CHECK(!g.first && g.second == one);
+      } else if (i == 1) {
+        CHECK(!g.first && g.second == two);
+      } else {
+        CHECK(g.first && g.second.find("eof") != std::string::npos);
+      }
+    }
+    std::promise<bool> lateWrite;
+    acc3->write(one.data(), one.size(), [&](const Error& e) { lateWrite.set_value(static_cast<bool>(e)); });
+    CHECK(lateWrite.get_future().get());
+  }
+  // Closing a listener fails its pending accept; closing a connection fails its pending read.
+  {
+    auto other = clientSide.connect(addr);
+    std::promise<std::shared_ptr<transport::Connection>> p4;
+    listener.accept([&](const Error& e, std::shared_ptr<transport::Connection> c) { p4.set_value(e ? nullptr : std::move(c)); });
+    auto acc4 = p4.get_future().get();
+    CHECK(acc4 != nullptr);
+    std::promise<bool> pendingRead;
+    acc4->read([&](const Error& e, const void*, size_t) { pendingRead.set_value(static_cast<bool>(e)); });
+    acc4->close();
+    CHECK(pendingRead.get_future().get());
+    std::promise<bool> peersRead;
+    other->read([&](const Error& e, const void*, size_t) { peersRead.set_value(static_cast<bool>(e)); });
+    CHECK(peersRead.get_future().get());
+  }
+  return failed;
+}
+
+// The transport that speaks the reference's shm protocol, both ends this library's.
+static int runShmStock() {
+  int failed = 0;
+  auto serverSide = transport::shm_stock::create();
+  auto clientSide = transport::shm_stock::create();
+  CHECK(serverSide->isViable());
+  // tensorpipe/transport/shm/context_impl.cc:29-47: shm:<boot id>_<device>_<inode of the network namespace>
+  const std::string d = serverSide->domainDescriptor();
+  CHECK(d.rfind("shm:", 0) == 0 && std::count(d.begin(), d.end(), '_') == 2 && d == clientSide->domainDescriptor());
+  CHECK(serverSide->canCommunicateWithRemote(d) && !serverSide->canCommunicateWithRemote(d + "x"));
+  // a name the kernel picks, and one the caller picks
+  auto anonymous = serverSide->listen("");
+  CHECK(!anonymous->addr().empty());
+  const std::string name = "tp_amd_unit_" + std::to_string(::getpid());
+  auto listener = serverSide->listen(name);
+  CHECK(listener->addr() == name);
+  failed += exerciseConnections(*serverSide, *clientSide, *listener, name);
+  failed += exerciseConnections(*serverSide, *serverSide, *anonymous, anonymous->addr()); // both ends on one thread
+  std::promise<bool> closedAccept;
+  listener->accept([&](const Error& e, std::shared_ptr<transport::Connection>) { closedAccept.set_value(static_cast<bool>(e)); });
+  listener->close();
+  CHECK(closedAccept.get_future().get());
+  anonymous.reset();
+  listener.reset();
+  clientSide->join();
+  serverSide->join();
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
 static int runTcp() {
   int failed = 0;
   auto serverSide = transport::tcp::create();
@@ -1225,12 +1398,15 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "compat_pipe") == 0) {
     return runCompatPipe();
   }
+  if (argc == 2 && std::strcmp(argv[1], "shm_stock") == 0) {
+    return runShmStock();
+  }
   if (argc == 2 && std::strcmp(argv[1], "tcp") == 0) {
     return runTcp();
   }
   if (argc == 2 && std::strcmp(argv[1], "loops") == 0) {
     return runLoops();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | loops\n", argv[0]);
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | shm_stock | loops\n", argv[0]);
   return 2;
 }

@@ -129,6 +129,15 @@ def test_compat_pipe_talks_to_itself():
     assert rc == 0 and out.strip() == "OK", out
 
 
+def test_shm_transport_in_the_reference_protocol():
+    """transport/shm_stock, both ends this library's: messages of every size class both ways
+    (below, at and far above the 2 MiB ring), exact-length reads, a peer that wrote and left,
+    closes, listeners by chosen and by kernel-picked name. (Against the unmodified build:
+    tests/test_stock_wire_interop.py.)"""
+    rc, out = run("shm_stock")
+    assert rc == 0 and out.strip() == "OK", out
+
+
 def test_tcp_transport():
     """Messages of every size class both ways, exact-length reads, the reference's stream framing
     written and read by hand, a peer that wrote and left, and a pipe over it."""
