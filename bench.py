@@ -363,9 +363,11 @@ class PeerRun:
                 else:
                     os.environ[k] = v
         self.listener = self.ctx.listen("uv://127.0.0.1" if transport == "uv" else "shm://")
-        self.transport = transport
+        # "shm_stock" (the reference's shm protocol) registers under the name "shm"
+        self.transport = "shm" if transport == "shm_stock" else transport
         child_env = dict(os.environ)
         child_env.update(env or {})
+        child_env["TP_BENCH_PEER_TRANSPORT"] = transport
         child_env["PYTHONPATH"] = ROOT + os.pathsep + child_env.get("PYTHONPATH", "")
         self.proc = subprocess.Popen(
             [sys.executable, os.path.join(ROOT, "bench_peer.py"), self.listener.url(self.transport), channels],
@@ -575,18 +577,22 @@ def bench_staged(iters=50, warmup=3, nbytes=256 * MIB):
     return out
 
 
-def bench_cpu_path(stock_wire_tcp=False):
+def bench_cpu_path(stock_wire_tcp=False, stock_wire_shm=False):
     """configs[0] on this library's own CPU side (Pipe + shm transport + basic channel, two
     processes): the control plane the device channels ride on, next to the reference's. With
-    `stock_wire_tcp` the same over the TCP transport with the reference's encodings on the wire:
-    what the route to unmodified peers costs."""
+    `stock_wire_tcp` the same over the TCP transport with the reference's encodings on the wire,
+    with `stock_wire_shm` over the transport that speaks the reference's shm protocol: what the
+    two routes to unmodified peers cost (both ends here are this library's)."""
     import numpy as np
 
     from tensorpipe_amd import datagen
     from tensorpipe_amd import pipe as tp
 
     out = {}
-    peer = PeerRun("basic:0", env={"TP_STOCK_WIRE": "1"}, transport="uv") if stock_wire_tcp else PeerRun("basic:0")
+    if stock_wire_tcp or stock_wire_shm:
+        peer = PeerRun("basic:0", env={"TP_STOCK_WIRE": "1"}, transport="uv" if stock_wire_tcp else "shm_stock")
+    else:
+        peer = PeerRun("basic:0")
     try:
         for name, n, iters in (("4KiB", 4096, 2000), ("1MiB", MIB, 1000), ("64MiB", 64 * MIB, 40)):
             src = datagen.uniform_u8(datagen.SEED_BASE + 1, n)
@@ -895,6 +901,7 @@ LEGS = {
     "ipc_large": lambda: bench_ipc(iters=40, warmup=3, min_bytes=256 * MIB),
     "cpu_path": bench_cpu_path,
     "cpu_path_stock_wire_tcp": lambda: bench_cpu_path(stock_wire_tcp=True),
+    "cpu_path_stock_wire_shm": lambda: bench_cpu_path(stock_wire_shm=True),
     "cold_copy": bench_cold_copy,
     "torch_rpc": bench_torch_rpc,
 }
@@ -1016,6 +1023,7 @@ def main():
         extra["cpu_path"] = extra_leg("cpu_path")
         log("[bench] the same over TCP in the reference's wire format")
         extra["cpu_path_stock_wire_tcp"] = extra_leg("cpu_path_stock_wire_tcp")
+        extra["cpu_path_stock_wire_shm"] = extra_leg("cpu_path_stock_wire_shm")
         log("[bench] torch.distributed.rpc with GPU tensors on these channels")
         extra["torch_rpc"] = extra_leg("torch_rpc")
     log("[bench] CPU baseline (port of shm + basic)")

@@ -33,7 +33,11 @@ def main(url, channels):
     from tensorpipe_amd import pipe as tp
 
     # the transport is the one the URL names ("uv" is this library's TCP transport)
-    ctx = tp.Context("bench_peer", transports=url.split("://", 1)[0] + ":0", channels=channels)
+    import os
+
+    # (the starter names the transport where the URL's scheme does not: "shm_stock" listens on shm://)
+    transport = os.environ.get("TP_BENCH_PEER_TRANSPORT") or url.split("://", 1)[0]
+    ctx = tp.Context("bench_peer", transports=transport + ":0", channels=channels)
     p = ctx.connect(url)
     extra = []
     multi_bufs = multi_streams = bufs = tensors = None  # kept from one pingpong_multi to the next of the same size
