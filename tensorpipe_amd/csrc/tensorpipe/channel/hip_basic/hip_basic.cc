@@ -289,6 +289,7 @@ class ChannelImpl final : public ChannelImplBase {
   }
 
   void sendFromLoop(uint64_t seq, Buffer buffer, size_t length, TSendCallback cb) override {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this call only
     if (length == 0) {
       cb(error_); // tensorpipe/channel/cuda_basic/channel_impl.cc:78-81
       return;
@@ -303,6 +304,7 @@ class ChannelImpl final : public ChannelImplBase {
   }
 
   void recvFromLoop(uint64_t seq, Buffer buffer, size_t length, TRecvCallback cb) override {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this call only
     if (length == 0) {
       cb(error_);
       return;

@@ -705,6 +705,7 @@ class ChannelImpl final : public ChannelImplBase {
   // ---- send -----------------------------------------------------------------
 
   void sendEntries(uint64_t seq, std::vector<BatchEntry> entries, TSendCallback cb) {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this call only
     std::vector<BatchEntry> live;
     for (auto& e : entries) {
       if (e.length > 0) {
@@ -1070,6 +1071,7 @@ class ChannelImpl final : public ChannelImplBase {
   // ---- recv -----------------------------------------------------------------
 
   void recvEntries(uint64_t seq, std::vector<BatchEntry> entries, TRecvCallback cb) {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this call only
     TP_MARK("ipc: recv");
     reapAcks();
     auto op = std::make_shared<RecvOp>();

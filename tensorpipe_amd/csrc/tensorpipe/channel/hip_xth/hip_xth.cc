@@ -209,6 +209,7 @@ class ChannelImpl final : public ChannelImplBase {
   };
 
   void sendEntries(uint64_t seq, std::vector<BatchEntry> entries, TSendCallback cb) {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this call only
     // Zero-length tensors complete at once and put nothing on the wire
     // (tensorpipe/channel/cuda_xth/channel_impl.cc:122-126).
     std::vector<BatchEntry> live;
@@ -286,6 +287,7 @@ class ChannelImpl final : public ChannelImplBase {
   }
 
   void recvEntries(uint64_t seq, std::vector<BatchEntry> entries, TRecvCallback cb) {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this call only
     TP_MARK("xth: recv");
     auto op = std::make_shared<RecvOp>();
     op->seq = seq;

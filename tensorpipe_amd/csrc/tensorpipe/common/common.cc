@@ -66,11 +66,19 @@ namespace {
 // "which device owns this pointer" costs a map lookup instead of driver calls
 // (the reference asks the driver every time,
 // tensorpipe/common/cuda.h:141-166). A range is entered after the runtime has
-// named its device and its extent; a pointer outside every known range goes
-// to the runtime, and one the runtime does not know (plain host memory) is
-// reported as such. A range stays until the table is cleared for size, so an
-// address freed and handed out again by the runtime keeps its answer: on one
-// device that answer is still right.
+// named its device, its extent and the id of its allocation; a pointer outside
+// every known range goes to the runtime, and one the runtime does not know
+// (plain host memory) is reported as such.
+//
+// An address may be freed and handed out again, to the runtime or to somebody
+// else (a plain mmap). So a remembered range is believed only for a while: the
+// callers mark the start of every message they handle (hipPointerCheckpoint),
+// and the first hit on a range after such a mark asks the runtime whether the
+// allocation there is still the one remembered (one query per range and
+// message, not per tensor). If it is not, the range is forgotten and the
+// pointer is looked up from scratch.
+thread_local uint64_t tlsPointerEpoch = 1;
+
 class PointerRanges {
  public:
   int lookup(const void* ptr) {
@@ -78,22 +86,45 @@ class PointerRanges {
     struct Last {
       uintptr_t begin{0}, end{0};
       int device{-1};
+      uint64_t bufferId{0};
       uint64_t generation{0};
+      uint64_t checkedAt{0};
     };
     thread_local Last last;
     const uint64_t gen = generation_.load(std::memory_order_acquire);
     if (last.generation == gen && p >= last.begin && p < last.end) {
-      return last.device;
-    }
-    {
-      std::lock_guard<std::mutex> lock(mutex_);
-      auto it = ranges_.upper_bound(p);
-      if (it != ranges_.begin()) {
-        --it;
-        if (p < it->second.end) {
-          last = Last{it->first, it->second.end, it->second.device, gen};
-          return it->second.device;
+      if (last.checkedAt == tlsPointerEpoch) {
+        return last.device;
+      }
+      if (stillThere(ptr, last.bufferId)) {
+        last.checkedAt = tlsPointerEpoch;
+        return last.device;
+      }
+      forget(last.begin);
+      last = Last{};
+    } else {
+      Range found{};
+      uintptr_t begin = 0;
+      bool hit = false;
+      {
+        std::lock_guard<std::mutex> lock(mutex_);
+        auto it = ranges_.upper_bound(p);
+        if (it != ranges_.begin()) {
+          --it;
+          if (p < it->second.end) {
+            begin = it->first;
+            found = it->second;
+            hit = true;
+          }
         }
+      }
+      if (hit) {
+        if (stillThere(ptr, found.bufferId)) {
+          last = Last{begin, found.end, found.device, found.bufferId, generation_.load(std::memory_order_acquire),
+                      tlsPointerEpoch};
+          return found.device;
+        }
+        forget(begin);
       }
     }
     int dev = -1;
@@ -104,8 +135,10 @@ class PointerRanges {
     }
     void* base = nullptr;
     size_t size = 0;
-    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr || size == 0) {
-      return dev; // known to the runtime, extent unknown: answer, do not remember
+    uint64_t id = 0;
+    if (tphip_mem_base(ptr, &base, &size) != 0 || base == nullptr || size == 0 ||
+        tphip_mem_buffer_id(ptr, &id) != 0 || id == 0) {
+      return dev; // known to the runtime, extent or identity unknown: answer, do not remember
     }
     const uintptr_t b = reinterpret_cast<uintptr_t>(base);
     std::lock_guard<std::mutex> lock(mutex_);
@@ -122,7 +155,7 @@ class PointerRanges {
       it = ranges_.erase(it);
       generation_.fetch_add(1, std::memory_order_acq_rel);
     }
-    ranges_[b] = Range{b + size, dev};
+    ranges_[b] = Range{b + size, dev, id};
     return dev;
   }
 
@@ -130,7 +163,22 @@ class PointerRanges {
   struct Range {
     uintptr_t end;
     int device;
+    uint64_t bufferId;
   };
+
+  // Is the allocation at ptr still the one that was remembered?
+  static bool stillThere(const void* ptr, uint64_t bufferId) {
+    uint64_t id = 0;
+    return tphip_mem_buffer_id(ptr, &id) == 0 && id != 0 && id == bufferId;
+  }
+
+  void forget(uintptr_t begin) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (ranges_.erase(begin) != 0) {
+      generation_.fetch_add(1, std::memory_order_acq_rel);
+    }
+  }
+
   std::mutex mutex_;
   std::map<uintptr_t, Range> ranges_;
   std::atomic<uint64_t> generation_{1};
@@ -141,6 +189,10 @@ class PointerRanges {
 int hipDeviceForPointer(const void* ptr) {
   static PointerRanges* ranges = new PointerRanges();
   return ranges->lookup(ptr);
+}
+
+void hipPointerCheckpoint() {
+  ++tlsPointerEpoch;
 }
 
 Device HipBuffer::getDevice() const {

@@ -33,8 +33,16 @@ int hipDeviceCountNoThrow();
 // pinned host memory yield their device, memory the runtime does not know
 // (plain host memory, null) yields -1, which callers turn into an exception as
 // the reference's driver check does. Answers are remembered per allocation, so
-// the runtime is asked once per allocation and not once per tensor.
+// the runtime is asked once per allocation and not once per tensor -- and once
+// more per allocation after every hipPointerCheckpoint() of the calling thread,
+// whether the allocation is still the one remembered.
 int hipDeviceForPointer(const void* ptr);
+
+// Marks the start of a unit of work on this thread (a message, a send, a
+// recv): remembered answers of hipDeviceForPointer are checked against the
+// runtime once before they are used again, so that an address which has been
+// freed and handed out anew since is not taken for what it used to be.
+void hipPointerCheckpoint();
 
 class HipEvent {
  public:

@@ -18,4 +18,8 @@ struct HipBuffer {
   Device getDevice() const;
 };
 
+// Start of a unit of work on the calling thread (see common/hip_api.h): what
+// getDevice() remembers about address ranges is checked once before its next use.
+void hipPointerCheckpoint();
+
 TP_AMD_NAMESPACE_END

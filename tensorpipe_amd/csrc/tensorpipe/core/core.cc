@@ -36,6 +36,7 @@
 #include <unordered_set>
 
 #include <tensorpipe/channel/channel.h>
+#include <tensorpipe/common/hip_buffer.h>
 #include <tensorpipe/common/loop.h>
 #include <tensorpipe/common/stage_timer.h>
 #include <tensorpipe/common/wire.h>
@@ -1388,6 +1389,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       fn(error_);
       return;
     }
+    hipPointerCheckpoint(); // the caller's buffers: believed for this message only
     TP_VLOG(9) << "Pipe " << id_ << " received a read request";
     TP_MARK("pipe: read()");
     StageScope timer(Stage::kPipeReadRequest);
@@ -1551,6 +1553,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   // ---- write side ---------------------------------------------------------
 
   void writeFromLoop(Message message, Pipe::write_callback_fn fn) {
+    hipPointerCheckpoint(); // the caller's buffers: believed for this message only
     if (error_) {
       fn(error_);
       return;

@@ -66,6 +66,8 @@
 #include <tensorpipe/common/slot_allocator.h>
 #include <tensorpipe/common/wire.h>
 #include <tensorpipe/channel/error.h>
+#include <sys/mman.h>
+
 #include <tensorpipe/tensorpipe.h>
 #include <tensorpipe/tensorpipe_hip.h>
 #include <tensorpipe/transport/connection.h>
@@ -385,7 +387,9 @@ static int runGarbage(int argc, char** argv) {
 // device; plain host memory is refused with std::runtime_error, as the
 // reference's driver query does (tensorpipe/common/cuda.h:141-166,
 // tensorpipe/common/cuda_buffer.cc:16-28). Needs a GPU.
-static int runPointers() {
+// mapOver: the runtime in use leaves freed ranges mapped and unreadable (the host-only stand-in
+// does), so the plain memory of the last case is mapped over the freed range.
+static int runPointers(bool mapOver) {
   int failed = 0;
   void* dev = nullptr;
   CHECK(tphip_malloc(0, 1 << 20, &dev) == 0);
@@ -415,6 +419,41 @@ static int runPointers() {
   CHECK((HipBuffer{again, nullptr}.getDevice().index == 0));
   CHECK(tphip_free(0, again) == 0);
   CHECK(tphip_host_free(pinned) == 0);
+  // ... and none once memory lives there that the runtime knows nothing about: the remembered
+  // answer is checked again at the start of the next unit of work
+  void* gone = nullptr;
+  CHECK(tphip_malloc(0, 1 << 20, &gone) == 0);
+  CHECK((HipBuffer{gone, nullptr}.getDevice().index == 0));
+  CHECK((HipBuffer{static_cast<uint8_t*>(gone) + 4096, nullptr}.getDevice().index == 0)); // remembered
+  CHECK(tphip_free(0, gone) == 0);
+#ifdef MAP_FIXED_NOREPLACE
+  void* plain = ::mmap(gone, 1 << 20, PROT_READ | PROT_WRITE,
+                       MAP_PRIVATE | MAP_ANONYMOUS | (mapOver ? MAP_FIXED : MAP_FIXED_NOREPLACE), -1, 0);
+  if (plain == gone) {
+    hipPointerCheckpoint();
+    bool threw = false;
+    try {
+      (void)(HipBuffer{static_cast<uint8_t*>(gone) + 4096, nullptr}.getDevice());
+    } catch (const std::runtime_error&) {
+      threw = true;
+    }
+    CHECK(threw);
+    ::munmap(plain, 1 << 20);
+  } else {
+    if (plain != MAP_FAILED) {
+      ::munmap(plain, 1 << 20);
+    }
+    std::printf("note: the freed range could not be mapped again; the stale-answer case did not run\n");
+  }
+#endif
+  // a range that is still what it was costs one look per unit of work and keeps its answer
+  void* kept = nullptr;
+  CHECK(tphip_malloc(0, 1 << 16, &kept) == 0);
+  for (int round = 0; round < 3; ++round) {
+    hipPointerCheckpoint();
+    CHECK((HipBuffer{kept, nullptr}.getDevice().index == 0));
+  }
+  CHECK(tphip_free(0, kept) == 0);
   if (failed == 0) {
     std::printf("OK\n");
   }
@@ -1389,8 +1428,8 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "departed_peer") == 0) {
     return runDepartedPeer();
   }
-  if (argc == 2 && std::strcmp(argv[1], "pointers") == 0) {
-    return runPointers();
+  if (argc >= 2 && std::strcmp(argv[1], "pointers") == 0) {
+    return runPointers(argc == 3 && std::strcmp(argv[2], "map_over") == 0);
   }
   if (argc == 3 && std::strcmp(argv[1], "nop_wire") == 0) {
     return runNopWire(argv[2]);

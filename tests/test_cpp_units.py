@@ -79,7 +79,18 @@ def test_messages_of_a_departed_peer_are_delivered():
 @pytest.mark.gpu
 def test_host_pointer_in_a_hip_buffer_is_refused():
     rc, out = run("pointers")
-    assert rc == 0 and out.strip() == "OK", out
+    assert rc == 0 and out.strip().splitlines()[-1] == "OK", out
+
+
+def test_remembered_pointer_answers_are_checked_again_per_message():
+    """The same on the host-only stand-in runtime, where a freed device range can be mapped again
+    as plain memory: after the next checkpoint the address is no longer taken for device memory."""
+    fake = os.path.join(os.path.dirname(BIN), "fake")
+    proc = subprocess.run([BIN, "pointers", "map_over"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120,
+                          env=dict(os.environ, LD_LIBRARY_PATH=fake))
+    lines = proc.stdout.strip().splitlines()
+    assert proc.returncode == 0 and lines and lines[-1] == "OK", proc.stdout
+    assert not any(l.startswith("note:") for l in lines), proc.stdout
 
 
 @pytest.mark.parametrize("seed", [4, 5])
