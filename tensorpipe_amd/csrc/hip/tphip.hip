@@ -133,6 +133,17 @@ int defaultBlocksPerCu(bool table) {
   return table ? multi : single;
 }
 
+// Copies of two pieces and more leave as launches of this many bytes each
+// (TPHIP_COPY_SPLIT_BYTES, 0 = never split).
+uint64_t splitPieceBytes() {
+  static const uint64_t v = [] {
+    const char* e = getenv("TPHIP_COPY_SPLIT_BYTES");
+    uint64_t b = e != nullptr ? strtoull(e, nullptr, 10) : (256ull << 20);
+    return b / 4096 * 4096; // pieces keep the alignment of the whole
+  }();
+  return v;
+}
+
 // Cache policy mask (bit 0 = nontemporal loads, bit 1 = nontemporal stores),
 // by the bytes of the launch. Up to 64 MiB everything may stay in the caches
 // (256 MiB Infinity Cache): the bytes were usually just produced and will be
@@ -260,7 +271,7 @@ int launchKernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, h
   size_t i = 0;
   std::apply([&](auto&... v) { ((argv[i++] = static_cast<void*>(&v)), ...); }, values);
   hipError_t e;
-  if (tlsProfStart != nullptr) {
+  if (tlsProfStart != nullptr || tlsProfStop != nullptr) {
     e = hipExtLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream,
                            tlsProfStart, tlsProfStop, 0);
     tlsProfStart = nullptr;
@@ -364,22 +375,71 @@ int copySingle(DeviceState& st, const tphip_copy_desc& d, hipStream_t stream, in
   if (nt < 0) {
     nt = defaultNontemporal(d.bytes, false);
   }
-  const uint64_t nvec = d.bytes >> 4;
-  const uint64_t perBlock = uint64_t(kBlockThreads) * unroll;
-  const uint32_t grid = pickBlocks(st.numCus, (nvec + perBlock - 1) / perBlock, 1, blocks, false);
   const char* src = static_cast<const char*>(d.src);
   char* dst = static_cast<char*>(d.dst);
   ProfileScope prof(st, stream, d.bytes);
-  switch (nt & 3) {
-    case 0:
-      return launchSingle<0>(unroll, grid, stream, src, dst, d.bytes);
-    case 1:
-      return launchSingle<1>(unroll, grid, stream, src, dst, d.bytes);
-    case 2:
-      return launchSingle<2>(unroll, grid, stream, src, dst, d.bytes);
-    default:
-      return launchSingle<3>(unroll, grid, stream, src, dst, d.bytes);
+  auto launchOne = [&](const char* s, char* t, uint64_t bytes) {
+    const uint64_t nvec = bytes >> 4;
+    const uint64_t perBlock = uint64_t(kBlockThreads) * unroll;
+    const uint32_t grid = pickBlocks(st.numCus, (nvec + perBlock - 1) / perBlock, 1, blocks, false);
+    switch (nt & 3) {
+      case 0:
+        return launchSingle<0>(unroll, grid, stream, s, t, bytes);
+      case 1:
+        return launchSingle<1>(unroll, grid, stream, s, t, bytes);
+      case 2:
+        return launchSingle<2>(unroll, grid, stream, s, t, bytes);
+      default:
+        return launchSingle<3>(unroll, grid, stream, s, t, bytes);
+    }
+  };
+  // A very large copy goes out as several launches in a row. The workgroups of
+  // one launch sweep memory as one compact window only while they keep pace;
+  // over hundreds of iterations they drift apart and the window widens (1 GiB
+  // in one launch: 357 us; as four of 256 MiB: 337 us, the three gaps between
+  // kernels included; as eight: 342 us; 256 MiB itself loses when split).
+  const uint64_t piece = splitPieceBytes();
+  if (piece == 0 || d.bytes < 2 * piece) {
+    return launchOne(src, dst, d.bytes);
   }
+  const uint64_t pieces = d.bytes / piece; // the last one takes the remainder
+  // What rides on "the" launch is spread over the row: a gate holds the first
+  // piece back (the others follow in stream order), the completion signal and
+  // the profiling stop belong to the last one, the profiling start to the first.
+  const hipEvent_t signal = tlsSignal;
+  const hipEvent_t profStart = tlsProfStart;
+  const hipEvent_t profStop = tlsProfStop;
+  const Gate gate = tlsGate;
+  struct Restore {
+    Gate gate;
+    ~Restore() {
+      tlsGate = gate;
+    }
+  } restore{gate};
+  tlsSignal = nullptr;
+  tlsProfStart = nullptr;
+  tlsProfStop = nullptr;
+  for (uint64_t k = 0; k < pieces; ++k) {
+    const bool first = k == 0;
+    const bool last = k + 1 == pieces;
+    const uint64_t offset = k * piece;
+    const uint64_t bytes = last ? d.bytes - offset : piece;
+    tlsGate = first ? gate : Gate{nullptr};
+    tlsProfStart = first ? profStart : nullptr;
+    tlsProfStop = last ? profStop : nullptr;
+    if (last && profStart == nullptr && profStop == nullptr) {
+      tlsSignal = signal;
+    }
+    const int rc = launchOne(src + offset, dst + offset, bytes);
+    if (rc != 0) {
+      tlsSignal = signal; // not attached: for the caller to see
+      return rc;
+    }
+  }
+  if (profStart != nullptr || profStop != nullptr) {
+    tlsSignal = signal; // the profiling events took the last launch's slots: the caller records it
+  }
+  return 0;
 }
 
 // A table of at most N entries, plan in the kernel arguments.

@@ -384,6 +384,51 @@ def test_full_size_roundtrip_property():
     assert torch.equal(a, c) and torch.equal(a, b)
 
 
+def test_copies_that_leave_as_several_launches():
+    # From twice 256 MiB on a single copy goes out as launches of 256 MiB, the last one with the
+    # remainder: odd lengths, both ends misaligned, guard bytes on either side untouched, the
+    # completion event behind the last piece, and a captured copy of that size replayed.
+    import torch
+
+    lib = _native.tphip()
+    for nbytes, so, do in (((512 << 20) + 4099, 3, 5), ((768 << 20) - 1, 0, 13), (512 << 20, 16, 0)):
+        src = torch.empty((nbytes + 64 + 7) // 8, dtype=torch.int64, device="cuda").random_().view(torch.uint8)
+        dst = torch.full((nbytes + 64,), FILL, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        stream, event = ctypes.c_void_p(), ctypes.c_void_p()
+        _native.check(lib.tphip_stream_create(0, ctypes.byref(stream)))
+        _native.check(lib.tphip_event_create(0, 0, ctypes.byref(event)))
+        table, n = hip.make_table([(src.data_ptr() + so, dst.data_ptr() + do, nbytes)])
+        _native.check(lib.tphip_batched_copy_signal(0, table, n, stream, event, 0, 0, -1))
+        done = ctypes.c_int(0)
+        for _ in range(2000000):
+            _native.check(lib.tphip_event_query(0, event, ctypes.byref(done)))
+            if done.value:
+                break
+        assert done.value, "the completion event behind the last piece never completed"
+        # the event says the bytes are there: no further synchronisation with that stream
+        assert torch.equal(dst[do:do + nbytes], src[so:so + nbytes])
+        assert bool((dst[:do] == FILL).all()) and bool((dst[do + nbytes:] == FILL).all())
+        _native.check(lib.tphip_event_destroy(0, event))
+        _native.check(lib.tphip_stream_destroy(0, stream))
+        del src, dst
+        torch.cuda.empty_cache()
+    nbytes = (512 << 20) + 16
+    src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hip.copy(dst, src, nbytes)
+    for replay in range(2):
+        src.random_(0, 256)
+        dst.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst), f"replay {replay} of a captured multi-launch copy differs"
+
+
 def test_pinned_host_endpoints(oracle):
     # device -> mapped pinned host -> device, the staged channel's two hops
     import torch
