@@ -5,6 +5,7 @@
 #pragma once
 
 #include <cstddef>
+#include <cstdint>
 #include <new>
 #include <stdexcept>
 #include <type_traits>
@@ -15,10 +16,23 @@
 
 TP_AMD_NAMESPACE_BEGIN
 
+namespace buffer_detail {
+// T::getDeviceKey() where a buffer type has one, 0 ("ask getDevice()") otherwise.
+template <typename T>
+auto deviceKeyOf(const T& v, int) -> decltype(v.getDeviceKey()) {
+  return v.getDeviceKey();
+}
+template <typename T>
+uint32_t deviceKeyOf(const T&, long) {
+  return 0;
+}
+} // namespace buffer_detail
+
 class Buffer {
   struct Concept {
     virtual Device device() const = 0;
     virtual void cloneInto(void* where) const = 0;
+    virtual uint32_t deviceKey() const = 0;
     virtual ~Concept() = default;
   };
 
@@ -32,6 +46,9 @@ class Buffer {
     }
     void cloneInto(void* where) const override {
       new (where) Model(*this);
+    }
+    uint32_t deviceKey() const override {
+      return buffer_detail::deviceKeyOf(value, 0);
     }
   };
 
@@ -83,6 +100,15 @@ class Buffer {
 
   Device device() const {
     return self()->device();
+  }
+
+  // Not in the reference: a small number that is equal for two buffers exactly
+  // when their devices are equal, or 0 where the buffer's type cannot say
+  // without building the Device. Lets a loop over the tensors of a message
+  // build and compare a Device (a string and an index) once per run of equal
+  // devices instead of once per tensor.
+  uint32_t deviceKey() const {
+    return self()->deviceKey();
   }
 
  private:

@@ -201,6 +201,12 @@ Device HipBuffer::getDevice() const {
   return Device{kHipDeviceType, dev};
 }
 
+uint32_t HipBuffer::getDeviceKey() const {
+  int dev = hipDeviceForPointer(ptr);
+  TP_THROW_ASSERT_IF(dev < 0);
+  return (2u << 16) | static_cast<uint32_t>(dev & 0xffff);
+}
+
 TP_AMD_NAMESPACE_END
 
 #include <tensorpipe/common/stage_timer.h>

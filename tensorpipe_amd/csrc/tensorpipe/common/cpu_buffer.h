@@ -1,5 +1,7 @@
 #pragma once
 
+#include <cstdint>
+
 #include <tensorpipe/common/device.h>
 
 TP_AMD_NAMESPACE_BEGIN
@@ -10,6 +12,10 @@ struct CpuBuffer {
 
   Device getDevice() const {
     return Device{kCpuDeviceType, 0};
+  }
+  // See Buffer::deviceKey().
+  uint32_t getDeviceKey() const {
+    return 1u << 16;
   }
 };
 

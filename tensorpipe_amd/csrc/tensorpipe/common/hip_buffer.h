@@ -1,5 +1,7 @@
 #pragma once
 
+#include <cstdint>
+
 #include <tensorpipe/common/device.h>
 
 TP_AMD_NAMESPACE_BEGIN
@@ -16,6 +18,8 @@ struct HipBuffer {
 
   // Device that owns `ptr` (tensorpipe/common/cuda_buffer.cc:16-28).
   Device getDevice() const;
+  // See Buffer::deviceKey(); throws like getDevice() for memory no GPU owns.
+  uint32_t getDeviceKey() const;
 };
 
 // Start of a unit of work on the calling thread (see common/hip_api.h): what

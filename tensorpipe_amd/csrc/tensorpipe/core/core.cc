@@ -1413,12 +1413,38 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     TP_THROW_ASSERT_IF(op->allocation.tensors.size() != shapes.size());
     const size_t nT = shapes.size();
     bool needsReply = false;
-    std::vector<Device> targets;
-    targets.reserve(nT);
+    // Where every tensor lands, as an index into the few distinct devices of
+    // the allocation (a Device is a string and an index: built and compared
+    // once per run of equal devices, which the buffers' keys tell apart).
+    std::vector<Device> targetDevices;
+    std::vector<uint16_t> targetOf(nT);
+    uint32_t prevKey = 0;
+    uint16_t prevIdx = 0;
+    uint16_t checkedIdx = kNoDevice, checkedAgainst = kNoDevice;
     for (size_t i = 0; i < nT; ++i) {
-      targets.push_back(op->allocation.tensors[i].buffer.device());
+      const uint32_t key = op->allocation.tensors[i].buffer.deviceKey();
+      uint16_t idx = prevIdx;
+      if (i == 0 || key == 0 || key != prevKey) {
+        Device dev = op->allocation.tensors[i].buffer.device();
+        size_t k = 0;
+        while (k < targetDevices.size() && !(targetDevices[k] == dev)) {
+          ++k;
+        }
+        if (k == targetDevices.size()) {
+          TP_THROW_ASSERT_IF(k >= kNoDevice);
+          targetDevices.push_back(std::move(dev));
+        }
+        idx = static_cast<uint16_t>(k);
+      }
+      prevKey = key;
+      prevIdx = idx;
+      targetOf[i] = idx;
       if (shapes[i].target != kNoDevice) {
-        TP_THROW_ASSERT_IF(shapes[i].length > 0 && !(targets[i] == op->devices[shapes[i].target]));
+        if (shapes[i].length > 0 && !(idx == checkedIdx && shapes[i].target == checkedAgainst)) {
+          TP_THROW_ASSERT_IF(!(targetDevices[idx] == op->devices[shapes[i].target]));
+          checkedIdx = idx;
+          checkedAgainst = shapes[i].target;
+        }
       } else {
         needsReply = true;
       }
@@ -1454,7 +1480,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       tpnop::DescriptorReply reply;
       for (size_t i = 0; i < nT; ++i) {
         if (shapes[i].target == kNoDevice) {
-          reply.targetDevices.push_back(toNop(targets[i]));
+          reply.targetDevices.push_back(toNop(targetDevices[targetOf[i]]));
         }
       }
       auto holder = std::make_shared<std::vector<uint8_t>>(tpnop::encode(reply));
@@ -1468,9 +1494,9 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     } else if (needsReply) {
       WireWriter w;
       w.u8(kDescriptorReply);
-      w.u32(static_cast<uint32_t>(targets.size()));
-      for (auto& dev : targets) {
-        putDevice(w, dev);
+      w.u32(static_cast<uint32_t>(nT));
+      for (size_t i = 0; i < nT; ++i) {
+        putDevice(w, targetDevices[targetOf[i]]);
       }
       writeControl(std::move(w.bytes()));
     }
@@ -1478,14 +1504,22 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     // Tensors, grouped per channel in message order.
     std::vector<ChannelGroup> groups;
     ChannelLookup lookup(channelForDevicePair_);
+    const std::string* prevName = nullptr;
+    uint16_t prevTarget = kNoDevice, prevSource = kNoDevice;
     for (size_t i = 0; i < nT; ++i) {
-      const Device& source = op->devices[shapes[i].source];
-      const std::string* name = lookup.find(targets[i], source);
-      if (name == nullptr) {
-        setError(TP_CREATE_ERROR(
-            LogicError,
-            "no channel between " + targets[i].toString() + " and " + source.toString()));
-        return;
+      const std::string* name = prevName;
+      if (prevName == nullptr || targetOf[i] != prevTarget || shapes[i].source != prevSource) {
+        const Device& target = targetDevices[targetOf[i]];
+        const Device& source = op->devices[shapes[i].source];
+        name = lookup.find(target, source);
+        if (name == nullptr) {
+          setError(TP_CREATE_ERROR(
+              LogicError, "no channel between " + target.toString() + " and " + source.toString()));
+          return;
+        }
+        prevName = name;
+        prevTarget = targetOf[i];
+        prevSource = shapes[i].source;
       }
       addToGroup(groups, name, i, nT);
     }
@@ -1621,12 +1655,21 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     // previous tensor's only.
     w.u32(static_cast<uint32_t>(m.tensors.size()));
     Device prevSource;
+    uint32_t prevSourceKey = 0;
     const Device* prevTarget = nullptr;
     for (size_t i = 0; i < m.tensors.size(); ++i) {
       const Message::Tensor& t = m.tensors[i];
-      Device source = t.buffer.device();
+      // (a Device is a string and an index: built and compared once per run of
+      // equal devices, which the buffers' keys tell apart)
+      const uint32_t sourceKey = t.buffer.deviceKey();
+      bool sameSource = i > 0 && sourceKey != 0 && sourceKey == prevSourceKey;
+      Device source;
+      if (!sameSource) {
+        source = t.buffer.device();
+        sameSource = i > 0 && source == prevSource;
+      }
+      prevSourceKey = sourceKey;
       uint8_t flags = 0;
-      const bool sameSource = i > 0 && source == prevSource;
       const bool hasTarget = t.targetDevice.has_value();
       const bool sameTarget = hasTarget && prevTarget != nullptr && *t.targetDevice == *prevTarget;
       flags |= hasTarget ? kTensorHasTarget : 0;
@@ -1700,16 +1743,28 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
     const size_t nT = m.tensors.size();
     std::vector<ChannelGroup> groups;
     ChannelLookup lookup(channelForDevicePair_);
+    uint32_t prevKey = 0;
+    const std::string* prevName = nullptr;
+    const Device* prevDst = nullptr;
     for (size_t i = 0; i < nT; ++i) {
-      const Device src = m.tensors[i].buffer.device();
       const Device& dst =
           m.tensors[i].targetDevice.has_value() ? *m.tensors[i].targetDevice : op->targetDevices[i];
-      const std::string* name = lookup.find(src, dst);
-      if (name == nullptr) {
-        setError(TP_CREATE_ERROR(
-            LogicError, "no channel between " + src.toString() + " and " + dst.toString()));
-        return;
+      const uint32_t key = m.tensors[i].buffer.deviceKey();
+      const std::string* name = nullptr;
+      if (prevName != nullptr && key != 0 && key == prevKey && dst == *prevDst) {
+        name = prevName; // same pair of devices as the tensor before
+      } else {
+        const Device src = m.tensors[i].buffer.device();
+        name = lookup.find(src, dst);
+        if (name == nullptr) {
+          setError(TP_CREATE_ERROR(
+              LogicError, "no channel between " + src.toString() + " and " + dst.toString()));
+          return;
+        }
       }
+      prevKey = key;
+      prevName = name;
+      prevDst = &dst;
       addToGroup(groups, name, i, nT);
     }
     auto self = shared_from_this();
