@@ -77,32 +77,52 @@ namespace {
 // allocation there is still the one remembered (one query per range and
 // message, not per tensor). If it is not, the range is forgotten and the
 // pointer is looked up from scratch.
-thread_local uint64_t tlsPointerEpoch = 1;
+// What a thread remembers: the mark of its current unit of work and the ranges
+// it has used last (a message's tensors come from a handful of allocations, and
+// a thread may alternate between two of them), each with the mark up to which
+// it has been checked. One object, so that a lookup finds the thread's block once.
+struct RecentRange {
+  uintptr_t begin{0}, end{0};
+  int device{-1};
+  uint64_t bufferId{0};
+  uint64_t generation{0};
+  uint64_t checkedAt{0};
+};
+constexpr int kRecentRanges = 4;
+struct PointerMemo {
+  uint64_t epoch{1};
+  int hot{0};
+  int nextVictim{0};
+  RecentRange recent[kRecentRanges];
+};
+thread_local PointerMemo tlsPointerMemo;
 
 class PointerRanges {
  public:
   int lookup(const void* ptr) {
     const uintptr_t p = reinterpret_cast<uintptr_t>(ptr);
-    struct Last {
-      uintptr_t begin{0}, end{0};
-      int device{-1};
-      uint64_t bufferId{0};
-      uint64_t generation{0};
-      uint64_t checkedAt{0};
-    };
-    thread_local Last last;
+    PointerMemo& memo = tlsPointerMemo;
     const uint64_t gen = generation_.load(std::memory_order_acquire);
-    if (last.generation == gen && p >= last.begin && p < last.end) {
-      if (last.checkedAt == tlsPointerEpoch) {
-        return last.device;
+    for (int n = 0; n < kRecentRanges; ++n) {
+      const int k = (memo.hot + n) % kRecentRanges; // the one that answered last goes first
+      RecentRange& r = memo.recent[k];
+      if (r.generation != gen || p < r.begin || p >= r.end) {
+        continue;
       }
-      if (stillThere(ptr, last.bufferId)) {
-        last.checkedAt = tlsPointerEpoch;
-        return last.device;
+      if (r.checkedAt == memo.epoch) {
+        memo.hot = k;
+        return r.device;
       }
-      forget(last.begin);
-      last = Last{};
-    } else {
+      if (stillThere(ptr, r.bufferId)) {
+        r.checkedAt = memo.epoch;
+        memo.hot = k;
+        return r.device;
+      }
+      forget(r.begin);
+      r = RecentRange{};
+      break;
+    }
+    {
       Range found{};
       uintptr_t begin = 0;
       bool hit = false;
@@ -120,8 +140,10 @@ class PointerRanges {
       }
       if (hit) {
         if (stillThere(ptr, found.bufferId)) {
-          last = Last{begin, found.end, found.device, found.bufferId, generation_.load(std::memory_order_acquire),
-                      tlsPointerEpoch};
+          memo.recent[memo.nextVictim] = RecentRange{begin, found.end, found.device, found.bufferId,
+                                                     generation_.load(std::memory_order_acquire), memo.epoch};
+          memo.hot = memo.nextVictim;
+          memo.nextVictim = (memo.nextVictim + 1) % kRecentRanges;
           return found.device;
         }
         forget(begin);
@@ -192,7 +214,7 @@ int hipDeviceForPointer(const void* ptr) {
 }
 
 void hipPointerCheckpoint() {
-  ++tlsPointerEpoch;
+  ++tlsPointerMemo.epoch;
 }
 
 Device HipBuffer::getDevice() const {
