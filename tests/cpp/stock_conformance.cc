@@ -48,10 +48,13 @@ using tensorpipe_amd_bridge::HipBuffer;
     }                                                                          \
   } while (0)
 
-static std::shared_ptr<Context> makeContext(const char* name, const std::vector<std::string>& channels, bool withUv = false) {
+static std::shared_ptr<Context> makeContext(const char* name, const std::vector<std::string>& channels, bool withUv = false, bool alsoShm = false) {
   auto ctx = std::make_shared<Context>(ContextOptions().name(name));
   if (withUv) {
     ctx->registerTransport(0, "uv", transport::uv::create());
+    if (alsoShm) {
+      ctx->registerTransport(1, "shm", transport::shm::create()); // preferred where the peer speaks it
+    }
   } else {
     ctx->registerTransport(0, "shm", transport::shm::create());
   }
@@ -705,7 +708,10 @@ static int nativePeerSameProcess() {
 }
 
 // hip_ipc / hip_basic: the native end in a child process, the stock end here.
-static int nativePeerTwoProcess(const std::string& channel) {
+// overShm: both ends also hold the reference's shm transport (the native end
+// through transport/shm_stock), preferred; the stock end connects over uv and
+// the pipe moves to shm before the first message.
+static int nativePeerTwoProcess(const std::string& channel, bool overShm) {
   int toChild[2], toParent[2];
   if (::pipe(toChild) != 0 || ::pipe(toParent) != 0) {
     return 3;
@@ -713,8 +719,9 @@ static int nativePeerTwoProcess(const std::string& channel) {
   pid_t pid = ::fork(); // before anything has touched the GPU
   if (pid == 0) {
     const std::string channels = "basic:0," + channel + ":10";
-    tpc_context* native = tpc_context_create_ex("native_peer", "uv:0", channels.c_str(), 1);
-    tpc_listener* listener = native != nullptr ? tpc_listen(native, "uv://127.0.0.1") : nullptr;
+    tpc_context* native = tpc_context_create_ex("native_peer", overShm ? "uv:0,shm_stock:1" : "uv:0", channels.c_str(), 1);
+    tpc_listener* listener =
+        native != nullptr ? tpc_listen(native, overShm ? "uv://127.0.0.1,shm://" : "uv://127.0.0.1") : nullptr;
     char url[256] = {0};
     if (listener == nullptr || tpc_listener_url(listener, "uv", url, sizeof(url)) != 0) {
       std::fprintf(stderr, "[native] listen: %s\n", tpc_last_error());
@@ -730,6 +737,13 @@ static int nativePeerTwoProcess(const std::string& channel) {
     }
     if (problem.empty()) {
       problem = nativeSend(pipe, 2);
+    }
+    if (problem.empty()) {
+      char transport[64] = {0};
+      const std::string expected = overShm ? "shm" : "uv";
+      if (tpc_pipe_transport(pipe, transport, sizeof(transport)) != 0 || expected != transport) {
+        problem = std::string("the pipe runs on transport \"") + transport + "\", not on " + expected;
+      }
     }
     if (!problem.empty()) {
       std::fprintf(stderr, "[native] %s\n", problem.c_str());
@@ -748,7 +762,7 @@ static int nativePeerTwoProcess(const std::string& channel) {
     report("native_" + channel + "_with_stock_peer", "the native process did not come up");
     return 1;
   }
-  auto ctx = makeContext("stock_main", {channel}, /*withUv=*/true);
+  auto ctx = makeContext("stock_main", {channel}, /*withUv=*/true, /*alsoShm=*/overShm);
   auto pipe = ctx->connect(url);
   std::string problem = sendMessage(*pipe, 1);
   if (problem.empty()) {
@@ -783,8 +797,9 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "unmodified_peer") == 0) {
     return unmodifiedPeer();
   }
-  if (argc == 3 && std::strcmp(argv[1], "native_peer") == 0) {
-    return std::strcmp(argv[2], "hip_xth") == 0 ? nativePeerSameProcess() : nativePeerTwoProcess(argv[2]);
+  if ((argc == 3 || argc == 4) && std::strcmp(argv[1], "native_peer") == 0) {
+    const bool overShm = argc == 4 && std::strcmp(argv[3], "shm") == 0;
+    return std::strcmp(argv[2], "hip_xth") == 0 ? nativePeerSameProcess() : nativePeerTwoProcess(argv[2], overShm);
   }
   if ((argc == 4 || argc == 5) && std::strcmp(argv[1], "time_same_process") == 0) {
     const size_t pieces = argc == 5 ? std::strtoull(argv[4], nullptr, 10) : 1;
@@ -795,6 +810,6 @@ int main(int argc, char** argv) {
     }
     return timeSameProcess(bytes, std::atoi(argv[3]), pieces);
   }
-  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | to_self <channel> <rounds> | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic | time_same_process <bytes> <messages> [tensors per message]\n", argv[0]);
+  std::fprintf(stderr, "usage: %s same_process | two_process hip_ipc|hip_basic | to_self <channel> <rounds> | unmodified_peer | native_peer hip_xth|hip_ipc|hip_basic [shm] | time_same_process <bytes> <messages> [tensors per message]\n", argv[0]);
   return 2;
 }

@@ -82,3 +82,12 @@ def test_native_pipe_in_stock_wire_format_with_a_stock_peer(channel, runtime):
     TCP transport registered as "uv", the channel natively), the other the stock TensorPipe with the
     same channel through the bridge: payload, GPU tensors and a CPU tensor both ways, byte for byte."""
     _run(["native_peer", channel], runtime=runtime)
+
+
+@runtimes
+@pytest.mark.parametrize("channel", ["hip_ipc", "hip_basic"])
+def test_native_pipe_with_a_stock_peer_moves_to_the_reference_shm_transport(channel, runtime):
+    """The same two processes when both ends also hold the reference's shm transport (this
+    library's end through transport/shm_stock), preferred: the stock end connects over uv, the
+    pipe moves to shm during the handshake, and payload, GPU tensors and a CPU tensor flow there."""
+    _run(["native_peer", channel, "shm"], runtime=runtime)
