@@ -1,9 +1,13 @@
 #include <atomic>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <iterator>
 #include <map>
 #include <mutex>
 #include <sstream>
+
+#include <unistd.h>
 
 #include <tensorpipe/common/error.h>
 #include <tensorpipe/common/hip_api.h>
@@ -79,8 +83,30 @@ namespace {
 // pointer is looked up from scratch.
 // What a thread remembers: the mark of its current unit of work and the ranges
 // it has used last (a message's tensors come from a handful of allocations, and
-// a thread may alternate between two of them), each with the mark up to which
-// it has been checked. One object, so that a lookup finds the thread's block once.
+// a peer's may come from dozens of the caching allocator's segments), sorted by
+// address, each with the mark up to which it has been checked. One object, so that a lookup finds the thread's block once.
+// TP_POINTER_STATS=1: how often the runtime was asked, printed when the process ends.
+struct PointerStats {
+  std::atomic<uint64_t> checks{0}, stale{0}, fromScratch{0}, sharedHits{0};
+  bool print{false};
+  PointerStats() {
+    const char* e = std::getenv("TP_POINTER_STATS");
+    print = e != nullptr && e[0] == '1';
+  }
+  ~PointerStats() {
+    if (print) {
+      std::fprintf(stderr, "[pointers %d] rechecks %llu (stale %llu), looked up from scratch %llu, found in the shared table %llu\n",
+                   static_cast<int>(::getpid()), static_cast<unsigned long long>(checks.load()),
+                   static_cast<unsigned long long>(stale.load()), static_cast<unsigned long long>(fromScratch.load()),
+                   static_cast<unsigned long long>(sharedHits.load()));
+    }
+  }
+};
+PointerStats& pointerStats() {
+  static PointerStats s;
+  return s;
+}
+
 struct RecentRange {
   uintptr_t begin{0}, end{0};
   int device{-1};
@@ -88,12 +114,13 @@ struct RecentRange {
   uint64_t generation{0};
   uint64_t checkedAt{0};
 };
-constexpr int kRecentRanges = 4;
+constexpr int kRecentRanges = 32;
 struct PointerMemo {
   uint64_t epoch{1};
-  int hot{0};
-  int nextVictim{0};
-  RecentRange recent[kRecentRanges];
+  int scopes{0}; // open HipPointerScopes on this thread
+  int hot{-1}; // the entry that answered last
+  int used{0};
+  RecentRange recent[kRecentRanges]; // sorted by begin
 };
 thread_local PointerMemo tlsPointerMemo;
 
@@ -103,24 +130,41 @@ class PointerRanges {
     const uintptr_t p = reinterpret_cast<uintptr_t>(ptr);
     PointerMemo& memo = tlsPointerMemo;
     const uint64_t gen = generation_.load(std::memory_order_acquire);
-    for (int n = 0; n < kRecentRanges; ++n) {
-      const int k = (memo.hot + n) % kRecentRanges; // the one that answered last goes first
-      RecentRange& r = memo.recent[k];
-      if (r.generation != gen || p < r.begin || p >= r.end) {
-        continue;
+    int k = -1;
+    if (memo.hot >= 0 && p >= memo.recent[memo.hot].begin && p < memo.recent[memo.hot].end) {
+      k = memo.hot;
+    } else {
+      // the last entry that begins at or below p
+      int lo = 0, hi = memo.used;
+      while (lo < hi) {
+        const int mid = (lo + hi) / 2;
+        if (memo.recent[mid].begin <= p) {
+          lo = mid + 1;
+        } else {
+          hi = mid;
+        }
       }
-      if (r.checkedAt == memo.epoch) {
+      if (lo > 0 && p < memo.recent[lo - 1].end) {
+        k = lo - 1;
+      }
+    }
+    if (k >= 0) {
+      RecentRange& r = memo.recent[k];
+      if (r.generation != gen) {
+        memo.used = 0; // the shared table has changed under what this thread remembers
+        memo.hot = -1;
+      } else if (r.checkedAt == memo.epoch) {
         memo.hot = k;
         return r.device;
-      }
-      if (stillThere(ptr, r.bufferId)) {
+      } else if (stillThere(ptr, r.bufferId)) {
         r.checkedAt = memo.epoch;
         memo.hot = k;
         return r.device;
+      } else {
+        forget(r.begin);
+        memo.used = 0;
+        memo.hot = -1;
       }
-      forget(r.begin);
-      r = RecentRange{};
-      break;
     }
     {
       Range found{};
@@ -139,16 +183,26 @@ class PointerRanges {
         }
       }
       if (hit) {
+        pointerStats().sharedHits.fetch_add(1, std::memory_order_relaxed);
         if (stillThere(ptr, found.bufferId)) {
-          memo.recent[memo.nextVictim] = RecentRange{begin, found.end, found.device, found.bufferId,
-                                                     generation_.load(std::memory_order_acquire), memo.epoch};
-          memo.hot = memo.nextVictim;
-          memo.nextVictim = (memo.nextVictim + 1) % kRecentRanges;
+          const uint64_t now = generation_.load(std::memory_order_acquire);
+          if (memo.used == kRecentRanges || (memo.used > 0 && memo.recent[0].generation != now)) {
+            memo.used = 0;
+          }
+          int at = memo.used;
+          while (at > 0 && memo.recent[at - 1].begin > begin) {
+            memo.recent[at] = memo.recent[at - 1];
+            --at;
+          }
+          memo.recent[at] = RecentRange{begin, found.end, found.device, found.bufferId, now, memo.epoch};
+          ++memo.used;
+          memo.hot = at;
           return found.device;
         }
         forget(begin);
       }
     }
+    pointerStats().fromScratch.fetch_add(1, std::memory_order_relaxed);
     int dev = -1;
     int isHost = 0;
     TP_HIP_CHECK(tphip_device_for_ptr(ptr, &dev, &isHost));
@@ -190,8 +244,22 @@ class PointerRanges {
 
   // Is the allocation at ptr still the one that was remembered?
   static bool stillThere(const void* ptr, uint64_t bufferId) {
+    // TP_POINTER_RECHECK=0: believe remembered ranges for good (for measuring what the check costs)
+    static const bool recheck = [] {
+      const char* e = std::getenv("TP_POINTER_RECHECK");
+      return e == nullptr || e[0] != '0';
+    }();
+    if (!recheck) {
+      return true;
+    }
     uint64_t id = 0;
-    return tphip_mem_buffer_id(ptr, &id) == 0 && id != 0 && id == bufferId;
+    const bool same = tphip_mem_buffer_id(ptr, &id) == 0 && id != 0 && id == bufferId;
+    PointerStats& stats = pointerStats();
+    stats.checks.fetch_add(1, std::memory_order_relaxed);
+    if (!same) {
+      stats.stale.fetch_add(1, std::memory_order_relaxed);
+    }
+    return same;
   }
 
   void forget(uintptr_t begin) {
@@ -214,7 +282,21 @@ int hipDeviceForPointer(const void* ptr) {
 }
 
 void hipPointerCheckpoint() {
-  ++tlsPointerMemo.epoch;
+  PointerMemo& memo = tlsPointerMemo;
+  if (memo.scopes == 0) {
+    ++memo.epoch;
+  }
+}
+
+HipPointerScope::HipPointerScope() {
+  PointerMemo& memo = tlsPointerMemo;
+  if (memo.scopes++ == 0) {
+    ++memo.epoch;
+  }
+}
+
+HipPointerScope::~HipPointerScope() {
+  --tlsPointerMemo.scopes;
 }
 
 Device HipBuffer::getDevice() const {

@@ -26,4 +26,16 @@ struct HipBuffer {
 // getDevice() remembers about address ranges is checked once before its next use.
 void hipPointerCheckpoint();
 
+// The same for a stretch of code: one mark when the outermost scope of the thread
+// opens, and none from hipPointerCheckpoint() calls further down the stack while it
+// is open (a pipe that handles a message opens one; the channels it calls into
+// from there do not mark again).
+class HipPointerScope {
+ public:
+  HipPointerScope();
+  ~HipPointerScope();
+  HipPointerScope(const HipPointerScope&) = delete;
+  HipPointerScope& operator=(const HipPointerScope&) = delete;
+};
+
 TP_AMD_NAMESPACE_END

@@ -1389,7 +1389,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
       fn(error_);
       return;
     }
-    hipPointerCheckpoint(); // the caller's buffers: believed for this message only
+    HipPointerScope pointersOfThisMessage; // the caller's buffers: believed for this message only
     TP_VLOG(9) << "Pipe " << id_ << " received a read request";
     TP_MARK("pipe: read()");
     StageScope timer(Stage::kPipeReadRequest);
@@ -1587,7 +1587,7 @@ class PipeImpl final : public std::enable_shared_from_this<PipeImpl> {
   // ---- write side ---------------------------------------------------------
 
   void writeFromLoop(Message message, Pipe::write_callback_fn fn) {
-    hipPointerCheckpoint(); // the caller's buffers: believed for this message only
+    HipPointerScope pointersOfThisMessage; // the caller's buffers: believed for this message only
     if (error_) {
       fn(error_);
       return;
