@@ -39,6 +39,7 @@
 #include <cstdlib>
 #include <deque>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <thread>
 
@@ -165,42 +166,41 @@ class LoopHelpers {
 
 class OnDemandLoop {
  public:
-  OnDemandLoop() = default;
+  OnDemandLoop() : state_(std::make_shared<State>()) {}
   OnDemandLoop(const OnDemandLoop&) = delete;
   OnDemandLoop& operator=(const OnDemandLoop&) = delete;
 
-  // Waits for a helper that still has this loop on its list. Like the queue
-  // itself, not to be destroyed from inside one of its own tasks.
-  ~OnDemandLoop() {
-    for (;;) {
-      {
-        std::unique_lock<std::mutex> lock(mutex_);
-        if (helperRefs_ == 0) {
-          return;
-        }
-      }
-      std::this_thread::yield();
-    }
-  }
+  // Nothing to wait for: the queue and its bookkeeping live in an object of
+  // their own that a draining thread (the caller of defer(), a helper) keeps
+  // alive for as long as it drains. The last reference to a loop's owner is
+  // often dropped by a task of that very loop (a callback that held the last
+  // pointer to a listener that held the last pointer to its context), so the
+  // loop may be destroyed from inside one of its own tasks; what is still
+  // queued then runs all the same.
+  ~OnDemandLoop() = default;
 
   void defer(TTask fn) {
+    State& s = *state_;
     const std::thread::id me = std::this_thread::get_id();
+    std::shared_ptr<State> keep;
     {
-      std::unique_lock<std::mutex> lock(mutex_);
-      queue_.push_back(Item{std::move(fn), me});
-      if (draining_) {
-        if (drainer_ == me || !guestDrainer_) {
+      std::unique_lock<std::mutex> lock(s.mutex_);
+      s.queue_.push_back(Item{std::move(fn), me});
+      if (s.draining_) {
+        if (s.drainer_ == me || !s.guestDrainer_) {
           return; // the draining thread will get to it
         }
         // An application thread is draining: it leaves our task alone.
         if (!thisIsLibraryThread() || loopTaskDepth() > 0) {
           return; // may not wait (see the top of this file); a helper will run it
         }
-        ++waiters_;
+        ++s.waiters_;
+        keep = state_;
       } else {
-        takeOver(me);
+        s.takeOver(me);
+        keep = state_;
         lock.unlock();
-        drain(me);
+        s.drain(keep, me);
         return;
       }
     }
@@ -209,18 +209,18 @@ class OnDemandLoop {
     const auto giveUpAt = std::chrono::steady_clock::now() + std::chrono::microseconds(kMaxWaitUs);
     for (unsigned spins = 0;; ++spins) {
       {
-        std::unique_lock<std::mutex> lock(mutex_);
-        if (!draining_) {
-          --waiters_;
-          takeOver(me);
+        std::unique_lock<std::mutex> lock(s.mutex_);
+        if (!s.draining_) {
+          --s.waiters_;
+          s.takeOver(me);
           break;
         }
-        if (!guestDrainer_) {
-          --waiters_;
+        if (!s.guestDrainer_) {
+          --s.waiters_;
           return; // a library thread took over and will run it
         }
         if ((spins & 63) == 63 && std::chrono::steady_clock::now() > giveUpAt) {
-          --waiters_;
+          --s.waiters_;
           return; // the drainer finds nobody waiting when it leaves and calls a helper
         }
       }
@@ -232,11 +232,11 @@ class OnDemandLoop {
         std::this_thread::yield();
       }
     }
-    drain(me);
+    s.drain(keep, me);
   }
 
   bool inLoop() const {
-    return owner_.load(std::memory_order_relaxed) == std::this_thread::get_id();
+    return state_->owner_.load(std::memory_order_relaxed) == std::this_thread::get_id();
   }
 
  private:
@@ -247,72 +247,72 @@ class OnDemandLoop {
     std::thread::id from;
   };
 
-  // mutex_ held.
-  void takeOver(std::thread::id me) {
-    draining_ = true;
-    drainer_ = me;
-    guestDrainer_ = !thisIsLibraryThread();
-  }
+  struct State {
+    // mutex_ held.
+    void takeOver(std::thread::id me) {
+      draining_ = true;
+      drainer_ = me;
+      guestDrainer_ = !thisIsLibraryThread();
+    }
 
-  void drain(std::thread::id me) {
-    owner_.store(me, std::memory_order_relaxed);
-    for (;;) {
-      TTask task;
+    // `self` is what keeps this object alive while a task destroys the loop.
+    void drain(const std::shared_ptr<State>& self, std::thread::id me) {
+      owner_.store(me, std::memory_order_relaxed);
+      for (;;) {
+        TTask task;
+        {
+          std::unique_lock<std::mutex> lock(mutex_);
+          if (queue_.empty()) {
+            owner_.store(std::thread::id(), std::memory_order_relaxed);
+            draining_ = false;
+            return;
+          }
+          if (guestDrainer_ && queue_.front().from != me) {
+            // Not this application thread's task. Whoever waits takes over; with
+            // nobody waiting a helper is called.
+            owner_.store(std::thread::id(), std::memory_order_relaxed);
+            draining_ = false;
+            if (waiters_ == 0 && !helperCalled_) {
+              helperCalled_ = true;
+              lock.unlock();
+              LoopHelpers::get().post([self] { self->drainAsHelper(self); });
+            }
+            return;
+          }
+          task = std::move(queue_.front().fn);
+          queue_.pop_front();
+        }
+        LoopTaskScope scope;
+        task();
+      }
+    }
+
+    void drainAsHelper(const std::shared_ptr<State>& self) {
+      const std::thread::id me = std::this_thread::get_id();
       {
         std::unique_lock<std::mutex> lock(mutex_);
-        if (queue_.empty()) {
-          owner_.store(std::thread::id(), std::memory_order_relaxed);
-          draining_ = false;
+        helperCalled_ = false;
+        // Somebody drains already: a library thread runs everything, an
+        // application thread calls again when it leaves.
+        if (draining_ || queue_.empty()) {
           return;
         }
-        if (guestDrainer_ && queue_.front().from != me) {
-          // Not this application thread's task. Whoever waits takes over; with
-          // nobody waiting a helper is called.
-          owner_.store(std::thread::id(), std::memory_order_relaxed);
-          draining_ = false;
-          if (waiters_ == 0 && !helperCalled_) {
-            helperCalled_ = true;
-            ++helperRefs_;
-            lock.unlock();
-            LoopHelpers::get().post([this] { drainAsHelper(); });
-          }
-          return;
-        }
-        task = std::move(queue_.front().fn);
-        queue_.pop_front();
+        takeOver(me);
       }
-      LoopTaskScope scope;
-      task();
+      drain(self, me);
     }
-  }
 
-  void drainAsHelper() {
-    const std::thread::id me = std::this_thread::get_id();
-    {
-      std::unique_lock<std::mutex> lock(mutex_);
-      helperCalled_ = false;
-      // Somebody drains already: a library thread runs everything, an
-      // application thread calls again when it leaves.
-      if (draining_ || queue_.empty()) {
-        --helperRefs_;
-        return;
-      }
-      takeOver(me);
-    }
-    drain(me);
-    std::unique_lock<std::mutex> lock(mutex_);
-    --helperRefs_;
-  }
+    std::mutex mutex_;
+    std::deque<Item> queue_;
+    bool draining_{false};
+    bool guestDrainer_{false}; // the draining thread belongs to the application
+    bool helperCalled_{false}; // a helper is on its way and has not looked yet
+    std::thread::id drainer_;
+    unsigned waiters_{0}; // library threads waiting for a guest drainer to leave
+    std::atomic<std::thread::id> owner_{std::thread::id()};
+  };
 
-  std::mutex mutex_;
-  std::deque<Item> queue_;
-  bool draining_{false};
-  bool guestDrainer_{false}; // the draining thread belongs to the application
-  bool helperCalled_{false}; // a helper is on its way and has not looked yet
-  std::thread::id drainer_;
-  unsigned waiters_{0}; // library threads waiting for a guest drainer to leave
-  unsigned helperRefs_{0}; // helpers that will still touch this object
-  std::atomic<std::thread::id> owner_{std::thread::id()};
+  const std::shared_ptr<State> state_;
 };
 
 class ThreadLoop {

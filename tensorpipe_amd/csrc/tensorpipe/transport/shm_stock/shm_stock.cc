@@ -55,6 +55,7 @@
 #include <deque>
 #include <fstream>
 #include <mutex>
+#include <new>
 #include <set>
 #include <sstream>
 #include <stdexcept>
@@ -192,6 +193,7 @@ class Ring {
       h->inTransaction[r].store(0, std::memory_order_relaxed);
       h->marker[r].store(0, std::memory_order_relaxed);
     }
+    bytes_ = pow2;
     return true;
   }
 
@@ -203,8 +205,18 @@ class Ring {
       return false;
     }
     const RingHeader* h = header();
-    return h->dataBytes >= 2 && (h->dataBytes & (h->dataBytes - 1)) == 0 && h->dataMask == h->dataBytes - 1 &&
-        data_.size() == h->dataBytes;
+    const uint64_t bytes = h->dataBytes;
+    if (bytes < 2 || (bytes & (bytes - 1)) != 0 || h->dataMask != bytes - 1 || data_.size() != bytes) {
+      return false;
+    }
+    bytes_ = bytes; // the header is memory that the peer can write: never read the size from it again
+    return true;
+  }
+
+  // The markers said something that no ring of this size can be in: the peer
+  // (or whoever else maps the header) has scribbled over it.
+  bool corrupt() const {
+    return corrupt_;
   }
 
   RingHeader* header() const {
@@ -239,14 +251,16 @@ class Ring {
     const uint64_t tail = h->marker[0].load(std::memory_order_relaxed);
     const uint64_t avail = h->marker[1].load(std::memory_order_acquire) - tail;
     size_t take = 0;
-    if (avail >= n) {
+    if (avail > bytes_) {
+      corrupt_ = true;
+    } else if (avail >= n) {
       take = n;
     } else if (partial) {
       take = static_cast<size_t>(avail);
     }
     if (take > 0) {
-      const uint64_t start = tail & h->dataMask;
-      const size_t first = static_cast<size_t>(std::min<uint64_t>(take, h->dataBytes - start));
+      const uint64_t start = tail & (bytes_ - 1);
+      const size_t first = static_cast<size_t>(std::min<uint64_t>(take, bytes_ - start));
       std::memcpy(dst, data_.data() + start, first);
       std::memcpy(static_cast<uint8_t*>(dst) + first, data_.data(), take - first);
       TP_TSAN_RING_RELEASE();
@@ -271,16 +285,18 @@ class Ring {
     }
     TP_TSAN_RING_ACQUIRE();
     const uint64_t head = h->marker[1].load(std::memory_order_relaxed);
-    const uint64_t room = h->marker[0].load(std::memory_order_acquire) + h->dataBytes - head;
+    const uint64_t room = h->marker[0].load(std::memory_order_acquire) + bytes_ - head;
     size_t take = 0;
-    if (room >= n) {
+    if (room > bytes_) {
+      corrupt_ = true;
+    } else if (room >= n) {
       take = n;
     } else if (partial) {
       take = static_cast<size_t>(room);
     }
     if (take > 0) {
-      const uint64_t start = head & h->dataMask;
-      const size_t first = static_cast<size_t>(std::min<uint64_t>(take, h->dataBytes - start));
+      const uint64_t start = head & (bytes_ - 1);
+      const size_t first = static_cast<size_t>(std::min<uint64_t>(take, bytes_ - start));
       std::memcpy(data_.data() + start, src, first);
       std::memcpy(data_.data(), static_cast<const uint8_t*>(src) + first, take - first);
       TP_TSAN_RING_RELEASE();
@@ -294,6 +310,8 @@ class Ring {
  private:
   Segment header_;
   Segment data_;
+  uint64_t bytes_{0}; // of the data segment, as checked when the ring was made or opened
+  bool corrupt_{false};
 };
 
 std::string readLine(const char* path) {
@@ -887,6 +905,10 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       if (peerReactor_.produce(&token, sizeof(token), /*partial=*/false, &put) == Ring::Put::kDone) {
         return true;
       }
+      if (peerReactor_.corrupt()) {
+        fail(TP_CREATE_ERROR(SystemError, "the header of the peer's reactor ring makes no sense", EPROTO));
+        return false;
+      }
       // held by another producer for a few instructions, or full of tokens that
       // the peer's thread has not got to yet
       std::this_thread::yield();
@@ -909,7 +931,9 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       if (!lengthKnown_) {
         uint32_t length = 0;
         if (inbox_.consume(&length, kLengthPrefix, /*partial=*/false) != kLengthPrefix) {
-          if (peerGone_) {
+          if (inbox_.corrupt()) {
+            failCorrupt();
+          } else if (peerGone_) {
             fail(TP_CREATE_ERROR(EOFError));
           }
           return;
@@ -925,7 +949,12 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
             return;
           }
         } else {
-          scratch_.resize(messageLength_);
+          try {
+            scratch_.resize(messageLength_);
+          } catch (const std::bad_alloc&) {
+            fail(TP_CREATE_ERROR(SystemError, "no memory for a message of the announced length", ENOMEM));
+            return;
+          }
         }
       }
       uint8_t* dst = op.exact ? op.ptr : scratch_.data();
@@ -934,6 +963,10 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
             inbox_.consume(dst + payloadDone_, messageLength_ - payloadDone_, /*partial=*/true);
         payloadDone_ += got;
         now += got;
+        if (inbox_.corrupt()) {
+          failCorrupt();
+          return;
+        }
       }
       if (now > 0 && !peerGone_) {
         reactor_->touched();
@@ -969,6 +1002,9 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       if (!op.lengthWritten) {
         const uint32_t length = static_cast<uint32_t>(op.length);
         if (outbox_.produce(&length, kLengthPrefix, /*partial=*/false, &put) != Ring::Put::kDone) {
+          if (outbox_.corrupt()) {
+            failCorrupt();
+          }
           return; // no room for the length: the peer's read will run this again
         }
         op.lengthWritten = true;
@@ -978,6 +1014,10 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
         (void)outbox_.produce(op.ptr + op.done, op.length - op.done, /*partial=*/true, &put);
         op.done += put;
         now += put;
+        if (outbox_.corrupt()) {
+          failCorrupt();
+          return;
+        }
       }
       if (now > 0) {
         reactor_->touched();
@@ -992,6 +1032,10 @@ class ConnectionImpl final : public FdHandler, public std::enable_shared_from_th
       writes_.pop_front();
       finished.fn(Error::kSuccess);
     }
+  }
+
+  void failCorrupt() {
+    fail(TP_CREATE_ERROR(SystemError, "the markers of a ring shared with the peer make no sense", EPROTO));
   }
 
   void fail(Error error) {

@@ -142,7 +142,7 @@ def run_cpu(out):
     bad += (0 if ok else 1) + len(reports)
     # the stock-protocol decoder on whole, cut and bent frames, and two of its endpoints talking
     vectors = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "golden", "stock_wire_vectors.txt")
-    for args in (["nop_wire", vectors], ["compat_pipe"], ["tcp"], ["shm_stock"]):
+    for args in (["nop_wire", vectors], ["compat_pipe"], ["tcp"], ["shm_stock"], ["shm_stock_hostile_peer"]):
         proc = subprocess.run([os.path.join(out, "unit_tests"), *args],
                               stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
         reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]

@@ -9,6 +9,10 @@
 // tensorpipe/test/core/pipe_cuda_test.cc (cited at each case).
 #pragma once
 
+#include <dirent.h>
+#include <execinfo.h>
+#include <signal.h>
+#include <sys/syscall.h>
 #include <sys/types.h>
 #include <sys/wait.h>
 #include <unistd.h>
@@ -42,6 +46,46 @@ namespace tptest {
 using namespace tensorpipe;
 
 constexpr int kWaitSeconds = 30;
+
+// ---- where a stuck program's threads are --------------------------------------
+// `kill -USR1 <pid>` (or `timeout -s USR1 ...`) makes every thread write its
+// call stack to stderr as module + offset lines (addr2line names them): what a
+// program that hangs once in a hundred runs is asked when no debugger is at hand.
+
+inline void writeOwnStack(int) {
+  void* frames[64];
+  const int n = ::backtrace(frames, 64);
+  char head[64];
+  const int len = std::snprintf(head, sizeof(head), "--- stack of thread %ld\n", static_cast<long>(::syscall(SYS_gettid)));
+  (void)!::write(2, head, static_cast<size_t>(len));
+  ::backtrace_symbols_fd(frames, n, 2);
+}
+
+inline void askEveryThreadForItsStack(int) {
+  DIR* dir = ::opendir("/proc/self/task");
+  if (dir == nullptr) {
+    return;
+  }
+  while (dirent* entry = ::readdir(dir)) {
+    const long tid = std::atol(entry->d_name);
+    if (tid > 0) {
+      ::syscall(SYS_tgkill, ::getpid(), tid, SIGUSR2);
+      ::usleep(20000); // one stack at a time keeps the lines together
+    }
+  }
+  ::closedir(dir);
+}
+
+inline void installStackDumper() {
+  void* warm[2];
+  (void)::backtrace(warm, 2); // loads what backtrace() needs outside a handler
+  struct sigaction own {};
+  own.sa_handler = writeOwnStack;
+  ::sigaction(SIGUSR2, &own, nullptr);
+  struct sigaction all {};
+  all.sa_handler = askEveryThreadForItsStack;
+  ::sigaction(SIGUSR1, &all, nullptr);
+}
 
 // ---- failure bookkeeping ----------------------------------------------------
 
@@ -579,6 +623,7 @@ struct Args {
 };
 
 inline Args parseArgs(int argc, char** argv) {
+  installStackDumper();
   Args a;
   for (int i = 1; i < argc; ++i) {
     std::string s = argv[i];

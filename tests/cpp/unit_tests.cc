@@ -78,6 +78,8 @@
 #include <arpa/inet.h>
 #include <netinet/in.h>
 #include <sys/socket.h>
+#include <sys/un.h>
+#include <poll.h>
 
 #include <nopwire/compat_pipe.h>
 #include <nopwire/nop_wire.h>
@@ -858,6 +860,243 @@ static int runShmStock() {
   return failed == 0 ? 0 : 1;
 }
 
+// A peer of the shm transport written against the reference's protocol alone
+// (tensorpipe/transport/shm/connection_impl.cc:231-291, common/shm_ringbuffer.h:23-82,
+// common/ringbuffer.h:50-140), so that it can misbehave: ring headers are memory
+// that both ends can write.
+struct RawShmPeer {
+  struct Header { // RingBufferHeader<2> on x86-64
+    uint64_t dataBytes;
+    uint64_t dataMask;
+    uint8_t inTransaction[2];
+    uint8_t pad[6];
+    std::atomic<uint64_t> marker[2]; // 0: consumed, 1: produced
+  };
+  static_assert(sizeof(Header) == 40, "layout of the reference's ring header");
+
+  int sock{-1};
+  int mine[4]{-1, -1, -1, -1}; // reactor header/data, inbox header/data
+  int theirs[4]{-1, -1, -1, -1};
+  Header* theirReactor{nullptr};
+  uint8_t* theirReactorData{nullptr};
+  Header* theirInbox{nullptr};
+  uint8_t* theirInboxData{nullptr};
+  Header* myInbox{nullptr};
+  uint32_t theirTokens[2]{0, 0}; // run when we wrote into their inbox / read from ours
+
+  static int segment(size_t bytes) {
+    const int fd = ::memfd_create("raw_shm_peer", MFD_CLOEXEC);
+    if (fd >= 0 && ::ftruncate(fd, static_cast<off_t>(bytes)) != 0) {
+      ::close(fd);
+      return -1;
+    }
+    return fd;
+  }
+  static void* mapAll(int fd, size_t bytes) {
+    void* p = ::mmap(nullptr, bytes, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    return p == MAP_FAILED ? nullptr : p;
+  }
+  static Header* ring(int* headerFd, int* dataFd, uint64_t saysBytes, size_t reallyBytes) {
+    *headerFd = segment(sizeof(Header));
+    *dataFd = segment(reallyBytes);
+    auto* h = static_cast<Header*>(mapAll(*headerFd, sizeof(Header)));
+    if (h != nullptr) {
+      h->dataBytes = saysBytes;
+      h->dataMask = saysBytes - 1;
+    }
+    return h;
+  }
+
+  // Connects and swaps descriptors. `inboxReallyBytes` lets the data segment
+  // differ from what the header says.
+  bool connect(const std::string& name, size_t inboxReallyBytes = 2u << 20) {
+    sock = ::socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
+    sockaddr_un sun;
+    std::memset(&sun, 0, sizeof(sun));
+    sun.sun_family = AF_UNIX;
+    std::memcpy(&sun.sun_path[1], name.data(), name.size());
+    if (sock < 0 ||
+        ::connect(sock, reinterpret_cast<sockaddr*>(&sun), static_cast<socklen_t>(sizeof(sun.sun_family) + 1 + name.size())) != 0) {
+      return false;
+    }
+    Header* myReactor = ring(&mine[0], &mine[1], 4u << 20, 4u << 20);
+    myInbox = ring(&mine[2], &mine[3], 2u << 20, inboxReallyBytes);
+    if (myReactor == nullptr || myInbox == nullptr) {
+      return false;
+    }
+    uint32_t tokens[2] = {0, 1};
+    iovec iov{tokens, sizeof(tokens)};
+    alignas(cmsghdr) char control[CMSG_SPACE(sizeof(mine))];
+    std::memset(control, 0, sizeof(control));
+    msghdr msg{};
+    msg.msg_iov = &iov;
+    msg.msg_iovlen = 1;
+    msg.msg_control = control;
+    msg.msg_controllen = sizeof(control);
+    cmsghdr* cmsg = CMSG_FIRSTHDR(&msg);
+    cmsg->cmsg_level = SOL_SOCKET;
+    cmsg->cmsg_type = SCM_RIGHTS;
+    cmsg->cmsg_len = CMSG_LEN(sizeof(mine));
+    std::memcpy(CMSG_DATA(cmsg), mine, sizeof(mine));
+    if (::sendmsg(sock, &msg, MSG_NOSIGNAL) != static_cast<ssize_t>(sizeof(tokens))) {
+      return false;
+    }
+    // their turn
+    std::memset(control, 0, sizeof(control));
+    iov = iovec{theirTokens, sizeof(theirTokens)};
+    msg.msg_controllen = sizeof(control);
+    pollfd pfd{sock, POLLIN, 0};
+    if (::poll(&pfd, 1, 10000) != 1 || ::recvmsg(sock, &msg, MSG_CMSG_CLOEXEC) != static_cast<ssize_t>(sizeof(theirTokens))) {
+      return false;
+    }
+    cmsg = CMSG_FIRSTHDR(&msg);
+    if (cmsg == nullptr || cmsg->cmsg_len != CMSG_LEN(sizeof(theirs))) {
+      return false;
+    }
+    std::memcpy(theirs, CMSG_DATA(cmsg), sizeof(theirs));
+    theirReactor = static_cast<Header*>(mapAll(theirs[0], sizeof(Header)));
+    theirInbox = static_cast<Header*>(mapAll(theirs[2], sizeof(Header)));
+    if (theirReactor == nullptr || theirInbox == nullptr) {
+      return false;
+    }
+    theirReactorData = static_cast<uint8_t*>(mapAll(theirs[1], theirReactor->dataBytes));
+    theirInboxData = static_cast<uint8_t*>(mapAll(theirs[3], theirInbox->dataBytes));
+    return theirReactorData != nullptr && theirInboxData != nullptr;
+  }
+
+  // Appends bytes to a ring the way a well-behaved producer does.
+  static void produce(Header* h, uint8_t* data, const void* src, size_t n) {
+    const uint64_t head = h->marker[1].load();
+    for (size_t i = 0; i < n; ++i) {
+      data[(head + i) & h->dataMask] = static_cast<const uint8_t*>(src)[i];
+    }
+    h->marker[1].store(head + n);
+  }
+  void poke(uint32_t token) {
+    produce(theirReactor, theirReactorData, &token, sizeof(token));
+  }
+  void hangUp() {
+    if (sock >= 0) {
+      ::close(sock);
+      sock = -1;
+    }
+  }
+  ~RawShmPeer() {
+    hangUp();
+    for (int fd : mine) {
+      if (fd >= 0) {
+        ::close(fd);
+      }
+    }
+    for (int fd : theirs) {
+      if (fd >= 0) {
+        ::close(fd);
+      }
+    }
+  }
+};
+
+// What a connection does when the other end breaks the protocol: it reports an
+// error; it neither reads outside the rings nor waits for ever.
+static int runShmStockHostilePeer() {
+  int failed = 0;
+  auto serverSide = transport::shm_stock::create();
+  const std::string name = "tp_amd_unit_hostile_" + std::to_string(::getpid());
+  auto listener = serverSide->listen(name);
+  auto acceptOne = [&]() {
+    auto p = std::make_shared<std::promise<std::shared_ptr<transport::Connection>>>();
+    listener->accept([p](const Error& e, std::shared_ptr<transport::Connection> c) { p->set_value(e ? nullptr : std::move(c)); });
+    return p->get_future();
+  };
+  auto readOutcome = [](transport::Connection& c) {
+    auto p = std::make_shared<std::promise<std::string>>();
+    c.read([p](const Error& e, const void* ptr, size_t len) {
+      p->set_value(e ? "error: " + e.what() : std::string(static_cast<const char*>(ptr), len));
+    });
+    return p->get_future();
+  };
+  const auto patience = std::chrono::seconds(20);
+
+  { // a well-behaved raw peer first: the helper itself speaks the protocol
+    auto acceptedF = acceptOne();
+    RawShmPeer peer;
+    CHECK(peer.connect(name));
+    auto accepted = acceptedF.get();
+    CHECK(accepted != nullptr);
+    auto got = readOutcome(*accepted);
+    const char text[] = "hello";
+    const uint32_t length = 5;
+    RawShmPeer::produce(peer.theirInbox, peer.theirInboxData, &length, 4);
+    RawShmPeer::produce(peer.theirInbox, peer.theirInboxData, text, 5);
+    peer.poke(peer.theirTokens[0]);
+    CHECK(got.wait_for(patience) == std::future_status::ready && got.get() == "hello");
+  }
+  { // a data segment smaller than its header says
+    auto acceptedF = acceptOne();
+    RawShmPeer peer;
+    (void)peer.connect(name, 4096);
+    auto accepted = acceptedF.get();
+    CHECK(accepted != nullptr);
+    auto got = readOutcome(*accepted);
+    CHECK(got.wait_for(patience) == std::future_status::ready && got.get().rfind("error: ", 0) == 0);
+  }
+  { // more bytes announced as produced than the inbox can hold
+    auto acceptedF = acceptOne();
+    RawShmPeer peer;
+    CHECK(peer.connect(name));
+    auto accepted = acceptedF.get();
+    auto got = readOutcome(*accepted);
+    peer.theirInbox->marker[1].store(peer.theirInbox->marker[0].load() + (1ull << 40));
+    peer.poke(peer.theirTokens[0]);
+    CHECK(got.wait_for(patience) == std::future_status::ready && got.get().rfind("error: ", 0) == 0);
+  }
+  { // the ring's size rewritten after set-up: the size checked at set-up is what counts
+    auto acceptedF = acceptOne();
+    RawShmPeer peer;
+    CHECK(peer.connect(name));
+    auto accepted = acceptedF.get();
+    auto got = readOutcome(*accepted);
+    const uint32_t length = 3;
+    RawShmPeer::produce(peer.theirInbox, peer.theirInboxData, &length, 4);
+    RawShmPeer::produce(peer.theirInbox, peer.theirInboxData, "abc", 3);
+    peer.theirInbox->dataBytes = 1ull << 40;
+    peer.theirInbox->dataMask = (1ull << 40) - 1;
+    peer.poke(peer.theirTokens[0]);
+    CHECK(got.wait_for(patience) == std::future_status::ready && got.get() == "abc");
+  }
+  { // our outbox (the peer's inbox) says that more was consumed than was ever produced
+    auto acceptedF = acceptOne();
+    RawShmPeer peer;
+    CHECK(peer.connect(name));
+    auto accepted = acceptedF.get();
+    peer.myInbox->marker[0].store(1ull << 40);
+    auto p = std::make_shared<std::promise<bool>>();
+    static const char payload[64] = {1};
+    accepted->write(payload, sizeof(payload), [p](const Error& e) { p->set_value(static_cast<bool>(e)); });
+    auto f = p->get_future();
+    CHECK(f.wait_for(patience) == std::future_status::ready && f.get());
+  }
+  { // a long message announced, a few bytes of it written, then gone
+    auto acceptedF = acceptOne();
+    RawShmPeer peer;
+    CHECK(peer.connect(name));
+    auto accepted = acceptedF.get();
+    auto got = readOutcome(*accepted);
+    const uint32_t length = 1u << 20;
+    RawShmPeer::produce(peer.theirInbox, peer.theirInboxData, &length, 4);
+    RawShmPeer::produce(peer.theirInbox, peer.theirInboxData, "abc", 3);
+    peer.poke(peer.theirTokens[0]);
+    peer.hangUp();
+    CHECK(got.wait_for(patience) == std::future_status::ready && got.get().rfind("error: ", 0) == 0);
+  }
+  listener.reset();
+  serverSide->join();
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
 static int runTcp() {
   int failed = 0;
   auto serverSide = transport::tcp::create();
@@ -1397,6 +1636,37 @@ static int runLoops() {
     CHECK(waitFor([&] { return ran.load() == 1; }));
     loop.reset();
   }
+  // 6. The last pointer to a loop's owner is held by a task of that loop, and a
+  // helper runs it: the owner, loop included, is destroyed from inside the
+  // loop's own task (a context whose last holder is a callback of one of its
+  // listeners). The helper must come out of it, and the loop's bookkeeping
+  // must outlive the owner for as long as the helper is in it.
+  for (int round = 0; round < 50; ++round) {
+    Watchdog dog("a loop destroyed by one of its own tasks on a helper", 10);
+    struct Owner {
+      OnDemandLoop loop;
+      std::atomic<int>* gone;
+      ~Owner() {
+        ++*gone;
+      }
+    };
+    std::atomic<int> gone{0}, ran{0};
+    auto owner = std::make_shared<Owner>();
+    owner->gone = &gone;
+    Owner* raw = owner.get();
+    Rendezvous inside, queued;
+    std::thread foreign([&, last = std::move(owner)]() mutable {
+      inside.arrive();
+      raw->loop.defer([&ran, last = std::move(last)] { ++ran; }); // an application thread drains: comes back at once
+      queued.arrive();
+    });
+    raw->loop.defer([&] {
+      inside.arrive();
+      queued.arrive();
+    });
+    foreign.join();
+    CHECK(waitFor([&] { return ran.load() == 1 && gone.load() == 1; }));
+  }
   if (failed == 0) {
     std::printf("OK\n");
   }
@@ -1440,12 +1710,15 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "shm_stock") == 0) {
     return runShmStock();
   }
+  if (argc == 2 && std::strcmp(argv[1], "shm_stock_hostile_peer") == 0) {
+    return runShmStockHostilePeer();
+  }
   if (argc == 2 && std::strcmp(argv[1], "tcp") == 0) {
     return runTcp();
   }
   if (argc == 2 && std::strcmp(argv[1], "loops") == 0) {
     return runLoops();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | shm_stock | loops\n", argv[0]);
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | shm_stock | shm_stock_hostile_peer | loops\n", argv[0]);
   return 2;
 }

@@ -149,6 +149,16 @@ def test_shm_transport_in_the_reference_protocol():
     assert rc == 0 and out.strip() == "OK", out
 
 
+def test_shm_transport_with_a_peer_that_breaks_the_protocol():
+    """A peer written in the test against the reference's protocol alone (socket, descriptors by
+    SCM_RIGHTS, ring headers) first behaves, then misbehaves: a data segment smaller than its
+    header says, markers that claim more bytes than a ring holds (inbox and outbox), the ring's
+    size rewritten after set-up, a long message announced and abandoned. Every case ends in an
+    error or in the bytes that were really sent; none reads outside a ring or waits for ever."""
+    rc, out = run("shm_stock_hostile_peer")
+    assert rc == 0 and out.strip() == "OK", out
+
+
 def test_tcp_transport():
     """Messages of every size class both ways, exact-length reads, the reference's stream framing
     written and read by hand, a peer that wrote and left, and a pipe over it."""
