@@ -142,12 +142,13 @@ def run_cpu(out):
     bad += (0 if ok else 1) + len(reports)
     # the stock-protocol decoder on whole, cut and bent frames, and two of its endpoints talking
     vectors = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "golden", "stock_wire_vectors.txt")
-    for args in (["nop_wire", vectors], ["compat_pipe"], ["tcp"], ["shm_stock"], ["shm_stock_hostile_peer"]):
+    for args in (["nop_wire", vectors], ["compat_pipe"], ["tcp"], ["shm_stock"], ["shm_stock_hostile_peer"],
+                 ["transport_suite", "shm"], ["transport_suite", "shm_stock"], ["transport_suite", "tcp"]):
         proc = subprocess.run([os.path.join(out, "unit_tests"), *args],
                               stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
         reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
         ok = proc.returncode == 0 and proc.stdout.strip().splitlines()[-1].startswith("OK")
-        print(f"unit_tests {args[0]}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
+        print(f"unit_tests {' '.join(a for a in args if not os.path.isabs(a))}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
         for l in reports[:5]:
             print("   ", l[:200])
         bad += (0 if ok else 1) + len(reports)

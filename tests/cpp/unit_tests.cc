@@ -1472,6 +1472,400 @@ bool waitFor(const std::function<bool()>& cond, int ms = 2000) {
 
 } // namespace
 
+// The reference's transport suite (tensorpipe/test/transport/listener_test.cc,
+// connection_test.cc, context_test.cc and shm/connection_test.cc), case by
+// case, for a transport of this library: shm (own protocol), shm_stock (the
+// reference's protocol) or tcp. One context per case, both ends in it, as the
+// reference's ThreadPeerGroup does (tensorpipe/test/transport/transport_test.h:34-36).
+namespace transport_suite {
+
+struct Flavour {
+  std::function<std::shared_ptr<transport::Context>()> make;
+  std::string defaultAddr;
+  size_t ringBytes; // what a connection buffers before a write has to wait (0: no such ring)
+};
+
+// A small object with libnop's face (tensorpipe/test/transport/connection_test.cc:86-93):
+// four bytes of length and the characters.
+struct TextHolder final : AbstractNopHolder {
+  std::string text;
+  size_t getSize() const override {
+    return 4 + text.size();
+  }
+  void serialize(uint8_t* out, size_t size) const override {
+    const uint32_t n = static_cast<uint32_t>(text.size());
+    std::memcpy(out, &n, 4);
+    std::memcpy(out + 4, text.data(), std::min(size - 4, text.size()));
+  }
+  bool deserialize(const uint8_t* in, size_t size) override {
+    uint32_t n = 0;
+    if (size < 4) {
+      return false;
+    }
+    std::memcpy(&n, in, 4);
+    if (size != 4 + static_cast<size_t>(n)) {
+      return false;
+    }
+    text.assign(reinterpret_cast<const char*>(in + 4), n);
+    return true;
+  }
+};
+
+template <typename T>
+bool ready(std::future<T>& f, int seconds = 30) {
+  return f.wait_for(std::chrono::seconds(seconds)) == std::future_status::ready;
+}
+
+struct Pair {
+  std::shared_ptr<transport::Connection> server, client;
+};
+
+static Pair connectPair(transport::Context& ctx, transport::Listener& listener) {
+  auto p = std::make_shared<std::promise<std::shared_ptr<transport::Connection>>>();
+  listener.accept([p](const Error& e, std::shared_ptr<transport::Connection> c) { p->set_value(e ? nullptr : std::move(c)); });
+  Pair pair;
+  pair.client = ctx.connect(listener.addr());
+  auto f = p->get_future();
+  if (ready(f)) {
+    pair.server = f.get();
+  }
+  return pair;
+}
+
+static int run(const Flavour& flavour) {
+  int failed = 0;
+  // Context_Basics + Listener_Basics: the accept callback runs for a new connection.
+  {
+    Watchdog dog("Context_Basics", 60);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+    }
+    ctx->join();
+  }
+  // Context_DomainDescriptor
+  {
+    Watchdog dog("Context_DomainDescriptor", 60);
+    auto ctx = flavour.make();
+    CHECK(!ctx->domainDescriptor().empty());
+    ctx->join();
+  }
+  // Listener_AcceptCallbacksAreQueued / Listener_IncomingConnectionsAreQueued:
+  // ten accepts and ten connections, whichever comes first; the callbacks fire
+  // in the order they were given.
+  for (int connectFirst = 0; connectFirst < 2; ++connectFirst) {
+    Watchdog dog("Listener_*AreQueued", 60);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      std::atomic<int> accepts{0};
+      std::atomic<bool> inOrder{true}, anyError{false};
+      std::promise<void> done;
+      std::vector<std::shared_ptr<transport::Connection>> conns, accepted(10);
+      auto connectAll = [&] {
+        for (int i = 0; i < 10; ++i) {
+          conns.push_back(ctx->connect(listener->addr()));
+        }
+      };
+      auto acceptAll = [&] {
+        for (int i = 0; i < 10; ++i) {
+          listener->accept([&, i](const Error& e, std::shared_ptr<transport::Connection> c) {
+            if (e) {
+              anyError = true;
+            }
+            if (accepts.load() != i) {
+              inOrder = false;
+            }
+            accepted[i] = std::move(c);
+            if (++accepts == 10) {
+              done.set_value();
+            }
+          });
+        }
+      };
+      if (connectFirst) {
+        connectAll();
+        acceptAll();
+      } else {
+        acceptAll();
+        connectAll();
+      }
+      auto f = done.get_future();
+      CHECK(ready(f));
+      CHECK(inOrder.load() && !anyError.load());
+    }
+    ctx->join();
+  }
+  // Listener_CreateThenCloseAndThenGetAddress: a closed listener still says
+  // where it was; an accept on it and a write towards it end, with or without
+  // an error, and nothing hangs.
+  {
+    Watchdog dog("Listener_CreateThenCloseAndThenGetAddress", 60);
+    auto ctx = flavour.make();
+    auto listener = ctx->listen(flavour.defaultAddr);
+    listener->close();
+    const std::string addr = listener->addr();
+    CHECK(!addr.empty());
+    std::promise<void> acceptDone, writeDone;
+    listener->accept([&](const Error&, std::shared_ptr<transport::Connection>) { acceptDone.set_value(); });
+    auto conn = ctx->connect(addr);
+    conn->write(nullptr, 0, [&](const Error&) { writeDone.set_value(); });
+    auto fa = acceptDone.get_future();
+    CHECK(ready(fa));
+    conn->close(); // (a write into a ring nobody reads is allowed to wait for ever)
+    auto fw = writeDone.get_future();
+    CHECK(ready(fw));
+    ctx->join();
+  }
+  // Listener_CreateAfterClosingContextAndThenGetAddress: the listener of a
+  // closed context is born closed; everything asked of it ends.
+  {
+    Watchdog dog("Listener_CreateAfterClosingContextAndThenGetAddress", 60);
+    auto ctx = flavour.make();
+    ctx->close();
+    auto listener = ctx->listen(flavour.defaultAddr);
+    const std::string addr = listener->addr();
+    std::promise<bool> acceptDone, writeDone;
+    listener->accept([&](const Error& e, std::shared_ptr<transport::Connection>) { acceptDone.set_value(static_cast<bool>(e)); });
+    auto conn = ctx->connect(addr);
+    conn->write(nullptr, 0, [&](const Error& e) { writeDone.set_value(static_cast<bool>(e)); });
+    auto fa = acceptDone.get_future();
+    CHECK(ready(fa) && fa.get());
+    auto fw = writeDone.get_future();
+    CHECK(ready(fw) && fw.get());
+    ctx->join();
+  }
+  // Connection_Initialization: thirteen bytes written are thirteen bytes read.
+  {
+    Watchdog dog("Connection_Initialization", 60);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+      if (pair.server) {
+        char garbage[13] = {0};
+        std::promise<size_t> got;
+        std::promise<bool> wrote;
+        pair.server->read([&](const Error& e, const void*, size_t len) { got.set_value(e ? size_t(-1) : len); });
+        pair.client->write(garbage, sizeof(garbage), [&](const Error& e) { wrote.set_value(!e); });
+        auto fg = got.get_future();
+        auto fw = wrote.get_future();
+        CHECK(ready(fg) && fg.get() == sizeof(garbage));
+        CHECK(ready(fw) && fw.get());
+      }
+    }
+    ctx->join();
+  }
+  // Connection_InitializationError: the server drops the connection at once;
+  // each of ten reads on the client, one after the other, fails.
+  {
+    Watchdog dog("Connection_InitializationError", 60);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+      pair.server.reset();
+      for (int i = 0; i < 10; ++i) {
+        std::promise<bool> failedRead;
+        pair.client->read([&](const Error& e, const void*, size_t) { failedRead.set_value(static_cast<bool>(e)); });
+        auto f = failedRead.get_future();
+        CHECK(ready(f) && f.get());
+      }
+    }
+    ctx->join();
+  }
+  // Connection_NopWrite: an object written is the object read.
+  {
+    Watchdog dog("Connection_NopWrite", 60);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+      if (pair.server) {
+        auto in = std::make_shared<TextHolder>();
+        auto out = std::make_shared<TextHolder>();
+        out->text = std::string(0x42, 'n');
+        std::promise<bool> got, wrote;
+        pair.server->read(*in, [&, in](const Error& e) { got.set_value(!e && in->text == std::string(0x42, 'n')); });
+        pair.client->write(*out, [&, out](const Error& e) { wrote.set_value(!e); });
+        auto fg = got.get_future();
+        auto fw = wrote.get_future();
+        CHECK(ready(fg) && fg.get());
+        CHECK(ready(fw) && fw.get());
+      }
+    }
+    ctx->join();
+  }
+  // Connection_QueueWritesBeforeReads: ten 16 KiB messages are all written
+  // (their callbacks have fired) before the first read is posted; the reads
+  // then find them in order.
+  {
+    Watchdog dog("Connection_QueueWritesBeforeReads", 60);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+      if (pair.server) {
+        constexpr int kMessages = 10;
+        std::vector<std::string> msg;
+        for (int i = 0; i < kMessages; ++i) {
+          msg.emplace_back(16 * 1024, static_cast<char>(i));
+        }
+        std::promise<bool> wroteAll;
+        std::atomic<bool> writesFine{true};
+        for (int i = 0; i < kMessages; ++i) {
+          pair.server->write(msg[i].data(), msg[i].size(), [&, i](const Error& e) {
+            if (e) {
+              writesFine = false;
+            }
+            if (i == kMessages - 1) {
+              wroteAll.set_value(writesFine.load());
+            }
+          });
+        }
+        auto fw = wroteAll.get_future();
+        CHECK(ready(fw) && fw.get());
+        std::promise<bool> readAll;
+        std::atomic<bool> readsFine{true};
+        for (int i = 0; i < kMessages; ++i) {
+          pair.client->read([&, i](const Error& e, const void* ptr, size_t len) {
+            if (e || len != msg[i].size() || std::memcmp(ptr, msg[i].data(), len) != 0) {
+              readsFine = false;
+            }
+            if (i == kMessages - 1) {
+              readAll.set_value(readsFine.load());
+            }
+          });
+        }
+        auto fr = readAll.get_future();
+        CHECK(ready(fr) && fr.get());
+      }
+    }
+    ctx->join();
+  }
+  // Chunking / ChunkingImplicitRead (shm/connection_test.cc:29-96): a message
+  // five times the ring, into the caller's buffer and into the transport's.
+  // For tcp the same sizes stand for "much more than a socket buffer".
+  for (int implicit = 0; implicit < 2; ++implicit) {
+    Watchdog dog("Chunking", 120);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+      if (pair.server) {
+        const size_t bytes = 5 * (flavour.ringBytes != 0 ? flavour.ringBytes : (2u << 20));
+        std::string src(bytes, 0x42);
+        for (size_t i = 0; i < bytes; i += 4099) {
+          src[i] = static_cast<char>(i / 4099);
+        }
+        std::vector<char> dst(implicit ? 0 : bytes);
+        std::promise<bool> got, wrote;
+        auto check = [&](const Error& e, const void* ptr, size_t len) {
+          got.set_value(!e && len == bytes && (implicit || ptr == dst.data()) && std::memcmp(ptr, src.data(), bytes) == 0);
+        };
+        if (implicit) {
+          pair.server->read(check);
+        } else {
+          pair.server->read(dst.data(), bytes, check);
+        }
+        pair.client->write(src.data(), bytes, [&](const Error& e) { wrote.set_value(!e); });
+        auto fg = got.get_future();
+        auto fw = wrote.get_future();
+        CHECK(ready(fg, 60) && fg.get());
+        CHECK(ready(fw, 60) && fw.get());
+      }
+    }
+    ctx->join();
+  }
+  // QueueWrites (shm/connection_test.cc:98-141): two messages of three
+  // quarters of the ring are queued before anything is read; the second
+  // cannot fit until the first has been taken out.
+  // NopWriteWrapAround (:152-185): the same with objects, whose bytes wrap
+  // around the end of the ring.
+  for (int objects = 0; objects < 2; ++objects) {
+    Watchdog dog("QueueWrites / NopWriteWrapAround", 120);
+    auto ctx = flavour.make();
+    {
+      auto listener = ctx->listen(flavour.defaultAddr);
+      Pair pair = connectPair(*ctx, *listener);
+      CHECK(pair.server != nullptr);
+      if (pair.server) {
+        const size_t bytes = 3 * (flavour.ringBytes != 0 ? flavour.ringBytes : (2u << 20)) / 4;
+        std::vector<std::shared_ptr<TextHolder>> outs, ins;
+        std::vector<std::string> raw;
+        for (int i = 0; i < 2; ++i) {
+          raw.emplace_back(bytes, static_cast<char>('B' + i));
+          outs.push_back(std::make_shared<TextHolder>());
+          outs.back()->text = raw.back();
+          ins.push_back(std::make_shared<TextHolder>());
+        }
+        std::atomic<int> written{0}, readOk{0}, anyError{0};
+        for (int i = 0; i < 2; ++i) {
+          auto done = [&](const Error& e) {
+            if (e) {
+              ++anyError;
+            }
+            ++written;
+          };
+          if (objects) {
+            pair.client->write(*outs[i], done);
+          } else {
+            pair.client->write(raw[i].data(), bytes, done);
+          }
+        }
+        std::this_thread::sleep_for(std::chrono::milliseconds(50)); // the writes are queued, the second one stuck
+        for (int i = 0; i < 2; ++i) {
+          if (objects) {
+            pair.server->read(*ins[i], [&, i](const Error& e) {
+              if (!e && ins[i]->text == raw[i]) {
+                ++readOk;
+              }
+            });
+          } else {
+            pair.server->read([&, i](const Error& e, const void* ptr, size_t len) {
+              if (!e && len == bytes && std::memcmp(ptr, raw[i].data(), bytes) == 0) {
+                ++readOk;
+              }
+            });
+          }
+        }
+        CHECK(waitFor([&] { return readOk.load() == 2 && written.load() == 2; }, 60000));
+        CHECK(anyError.load() == 0);
+      }
+    }
+    ctx->join();
+  }
+  return failed;
+}
+
+} // namespace transport_suite
+
+static int runTransportSuite(const std::string& which) {
+  transport_suite::Flavour flavour;
+  const std::string unique = "tp_amd_suite_" + std::to_string(::getpid());
+  if (which == "shm") {
+    flavour = {[] { return transport::shm::create(); }, "", 0};
+  } else if (which == "shm_stock") {
+    flavour = {[] { return transport::shm_stock::create(); }, "", 2u << 20};
+  } else if (which == "tcp") {
+    flavour = {[] { return transport::tcp::create(); }, "127.0.0.1", 0};
+  } else {
+    return 2;
+  }
+  const int failed = transport_suite::run(flavour);
+  if (failed == 0) {
+    std::printf("OK\n");
+  }
+  return failed == 0 ? 0 : 1;
+}
+
 static int runLoops() {
   int failed = 0;
   // 1. Thread A sits in a task of loop one and defers to loop two while thread
@@ -1713,12 +2107,15 @@ int main(int argc, char** argv) {
   if (argc == 2 && std::strcmp(argv[1], "shm_stock_hostile_peer") == 0) {
     return runShmStockHostilePeer();
   }
+  if (argc == 3 && std::strcmp(argv[1], "transport_suite") == 0) {
+    return runTransportSuite(argv[2]);
+  }
   if (argc == 2 && std::strcmp(argv[1], "tcp") == 0) {
     return runTcp();
   }
   if (argc == 2 && std::strcmp(argv[1], "loops") == 0) {
     return runLoops();
   }
-  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | shm_stock | shm_stock_hostile_peer | loops\n", argv[0]);
+  std::fprintf(stderr, "usage: %s allocator <slots> <events...> | basics | departed_peer | pointers | garbage <seed> <n> | nop_wire <vectors> | compat_pipe | tcp | shm_stock | shm_stock_hostile_peer | transport_suite shm|shm_stock|tcp | loops\n", argv[0]);
   return 2;
 }

@@ -159,6 +159,18 @@ def test_shm_transport_with_a_peer_that_breaks_the_protocol():
     assert rc == 0 and out.strip() == "OK", out
 
 
+@pytest.mark.parametrize("transport", ["shm", "shm_stock", "tcp"])
+def test_transport_suite_after_the_reference(transport):
+    """The reference's transport tests (tensorpipe/test/transport/listener_test.cc,
+    connection_test.cc, context_test.cc, shm/connection_test.cc), case by case, on each of this
+    library's transports: accepts and incoming connections are queued and served in order, a
+    closed listener and the listener of a closed context, a peer that drops the connection at
+    once, objects and raw bytes, writes that complete before any read, messages five times the
+    ring, two messages that do not fit the ring together (raw and as objects)."""
+    rc, out = run("transport_suite", transport)
+    assert rc == 0 and out.strip() == "OK", out
+
+
 def test_tcp_transport():
     """Messages of every size class both ways, exact-length reads, the reference's stream framing
     written and read by hand, a peer that wrote and left, and a pipe over it."""
