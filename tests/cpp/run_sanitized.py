@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Builds the host library and the C++ test programs with a sanitizer and runs the CPU suites.
 
-    python tests/cpp/run_sanitized.py thread|address [build_dir] [--build-only | --run-only] [--gpu | --stand-in]
+    python tests/cpp/run_sanitized.py thread|address [build_dir] [--build-only | --run-only] [--gpu | --stand-in] [--repeat=N]
 
 Host code only (g++ -fsanitize=...); libtphip.so is used as built. With --gpu the suites of the
 device channels run instead of the CPU ones (on a machine with a GPU; --build-only on one machine
@@ -16,11 +16,17 @@ executor cases (unit_tests loops) run in every mode. Not collected by pytest: a
 full pass takes several minutes. The shm transport tells ThreadSanitizer about the hand-off
 through its rings (two mappings of one segment inside a process), so a clean run reports
 nothing; any "WARNING: ThreadSanitizer" / "ERROR: AddressSanitizer" line fails the run.
+With --repeat=N every suite runs up to N times and stops at its first bad turn; a turn that is
+still running after three minutes is asked for the call stacks of all its threads and ended (a
+hang that shows once in a hundred runs is found this way: the sanitizers' slower, differently
+skewed timing brings out orders of events that a plain build almost never takes).
 """
 import os
+import signal
 import subprocess
 import sys
 import tempfile
+import time
 from concurrent.futures import ThreadPoolExecutor
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
@@ -44,9 +50,16 @@ STAND_IN_SUITES = GPU_SUITES + [("channel_tests", "hip_ipc_gated", False), ("cha
                                 ("channel_tests", "hip_basic_small_ring", False)]
 
 
+REPEAT = 1
+
+
 def main():
+    global REPEAT
     words = [a for a in sys.argv[1:] if not a.startswith("--")]
     options = {a for a in sys.argv[1:] if a.startswith("--")}
+    for a in options:
+        if a.startswith("--repeat="):
+            REPEAT = max(1, int(a.split("=", 1)[1]))
     san = words[0] if words else "thread"
     out = os.path.abspath(words[1]) if len(words) > 1 else tempfile.mkdtemp(prefix=f"tp_{san}_")
     os.makedirs(out, exist_ok=True)
@@ -101,19 +114,41 @@ def run_unit(out, args, env=None):
     return (0 if ok else 1) + len(reports)
 
 
+def run_once(cmd, env, limit):
+    """Output of `cmd`, and whether it had to be ended. A program that is still running after
+    `limit` seconds is asked for its threads' stacks (SIGUSR1, tests/cpp/support.h) and killed."""
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+    try:
+        text, _ = proc.communicate(timeout=limit)
+        return text, False
+    except subprocess.TimeoutExpired:
+        proc.send_signal(signal.SIGUSR1)
+        time.sleep(5)
+        proc.kill()
+        text, _ = proc.communicate()
+        return text, True
+
+
 def run_suites(out, suites, base_env=None):
     bad = 0
     for prog, suite, stock_wire in suites:
         env = dict(base_env or os.environ, TP_STOCK_WIRE="1") if stock_wire else base_env
-        proc = subprocess.run([os.path.join(out, prog), "--suite", suite], stdout=subprocess.PIPE,
-                              stderr=subprocess.STDOUT, text=True, timeout=1800, env=env)
-        results = [l for l in proc.stdout.splitlines() if l.startswith("RESULT")]
-        failed = [l for l in results if " OK" not in l]
-        reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
-        print(f"{prog} --suite {suite}{' (stock wire format)' if stock_wire else ''}: {len(results)} results, {len(failed)} failed, {len(reports)} sanitizer reports")
+        label = f"{prog} --suite {suite}{' (stock wire format)' if stock_wire else ''}"
+        for turn in range(REPEAT):
+            text, stuck = run_once([os.path.join(out, prog), "--suite", suite], env, 1800 if REPEAT == 1 else 180)
+            results = [l for l in text.splitlines() if l.startswith("RESULT")]
+            failed = [l for l in results if " OK" not in l]
+            reports = [l for l in text.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+            if stuck or failed or reports or not results:
+                break
+        where = f" (turn {turn + 1} of {REPEAT})" if REPEAT > 1 else ""
+        print(f"{label}{where}: {len(results)} results, {len(failed)} failed, {len(reports)} sanitizer reports"
+              f"{', STUCK: stacks below' if stuck else ''}")
         for l in failed + reports[:5]:
             print("   ", l[:200])
-        bad += len(failed) + len(reports) + (0 if results else 1)
+        if stuck:
+            print(text[-6000:])
+        bad += len(failed) + len(reports) + (0 if results else 1) + (1 if stuck else 0)
         sys.stdout.flush()
     return bad
 
@@ -149,7 +184,7 @@ def run_cpu(out):
         reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
         ok = proc.returncode == 0 and proc.stdout.strip().splitlines()[-1].startswith("OK")
         print(f"unit_tests {' '.join(a for a in args if not os.path.isabs(a))}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
-        for l in reports[:5]:
+        for l in reports[:5] + ([] if ok else proc.stdout.strip().splitlines()[-8:]):
             print("   ", l[:200])
         bad += (0 if ok else 1) + len(reports)
     sys.exit(1 if bad else 0)

@@ -770,11 +770,13 @@ static int exerciseConnections(
     auto acc2 = p2.get_future().get();
     CHECK(acc2 != nullptr);
     const std::string msg = "five!";
-    other->write(msg.data(), msg.size(), [](const Error&) {});
+    std::promise<void> wroteMsg; // the bytes stay the caller's until then: the length may travel ahead of them
+    other->write(msg.data(), msg.size(), [&](const Error&) { wroteMsg.set_value(); });
     char buf[4];
     std::promise<bool> failedRead;
     acc2->read(buf, sizeof(buf), [&](const Error& e, const void*, size_t) { failedRead.set_value(static_cast<bool>(e)); });
     CHECK(failedRead.get_future().get());
+    wroteMsg.get_future().get();
   }
   // A peer that writes and leaves before anybody reads: the messages, then the end; a write
   // to it fails.
@@ -1175,11 +1177,13 @@ static int runTcp() {
     auto acc2 = p2.get_future().get();
     CHECK(acc2 != nullptr);
     const std::string msg = "five!";
-    other->write(msg.data(), msg.size(), [](const Error&) {});
+    std::promise<void> wroteMsg; // the bytes stay the caller's until then: the length may travel ahead of them
+    other->write(msg.data(), msg.size(), [&](const Error&) { wroteMsg.set_value(); });
     char buf[4];
     std::promise<bool> failedRead;
     acc2->read(buf, sizeof(buf), [&](const Error& e, const void*, size_t) { failedRead.set_value(static_cast<bool>(e)); });
     CHECK(failedRead.get_future().get());
+    wroteMsg.get_future().get();
   }
   // A frame written by hand, the way the reference frames a stream: 8-byte little-endian length, bytes.
   {
