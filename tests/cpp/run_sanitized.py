@@ -73,6 +73,7 @@ def main():
         env = dict(os.environ, LD_LIBRARY_PATH=os.path.join(out, "fake"))
         bad = run_suites(out, STAND_IN_SUITES, env)
         bad += run_unit(out, ["loops"], env)
+        bad += run_conformance(out, env)
         sys.exit(1 if bad else 0)
     run_cpu(out)
 
@@ -99,6 +100,52 @@ def build(san, out):
         subprocess.run(["g++", *flags, os.path.join(ROOT, "tests", "cpp", prog + ".cc"), "-o",
                         os.path.join(out, prog), f"-L{out}", "-ltensorpipe_amd", f"-L{tp_build.LIB}", "-ltphip",
                         f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}"], check=True)
+    build_conformance(san, out, flags)
+
+
+# The conformance program: the channels inside the unmodified TensorPipe of libtorch_cpu.so, where
+# every thread but the event poller's is a stranger to this library. AddressSanitizer only: the
+# stock library is not instrumented, and ThreadSanitizer then reports its internals.
+CONFORMANCE_MODES = [["same_process"], ["two_process", "hip_ipc"], ["two_process", "hip_basic"],
+                     ["to_self", "hip_xth", "300"], ["to_self", "hip_basic", "300"],
+                     ["native_peer", "hip_xth"], ["native_peer", "hip_ipc"], ["native_peer", "hip_basic"],
+                     ["native_peer", "hip_basic", "shm"], ["unmodified_peer"]]
+
+
+def build_conformance(san, out, flags):
+    found = tp_build.stock_tensorpipe()
+    if san != "address" or found is None:
+        return
+    inc, lib = found
+    stock_first = [f for f in flags if not f.startswith("-I")]
+    subprocess.run(["g++", *stock_first, f"-I{inc}", f"-I{tp_build.INCLUDE}", f"-I{tp_build.CSRC}",
+                    os.path.join(tp_build.CSRC, "bridge", "stock_adapter.cc"),
+                    os.path.join(ROOT, "tests", "cpp", "stock_conformance.cc"),
+                    "-o", os.path.join(out, "stock_conformance"), f"-L{out}", "-ltensorpipe_amd",
+                    f"-L{tp_build.LIB}", "-ltphip", f"-L{lib}", "-ltorch_cpu", "-lc10",
+                    f"-Wl,-rpath,{out}", f"-Wl,-rpath,{tp_build.LIB}", f"-Wl,-rpath,{lib}"], check=True)
+
+
+def run_conformance(out, env):
+    prog = os.path.join(out, "stock_conformance")
+    if not os.path.exists(prog):
+        return 0
+    bad = 0
+    env = dict(env, ASAN_OPTIONS=(env.get("ASAN_OPTIONS", "") + ":detect_leaks=0").lstrip(":"))
+    for args in CONFORMANCE_MODES:
+        text, stuck = run_once([prog, *args], env, 600)
+        results = [l for l in text.splitlines() if l.startswith("RESULT")]
+        failed = [l for l in results if " OK" not in l]
+        reports = [l for l in text.splitlines() if "ERROR: AddressSanitizer" in l]
+        print(f"stock_conformance {' '.join(args)}: {len(results)} results, {len(failed)} failed, "
+              f"{len(reports)} sanitizer reports{', STUCK: stacks below' if stuck else ''}")
+        for l in failed + reports[:5]:
+            print("   ", l[:200])
+        if stuck:
+            print(text[-6000:])
+        bad += len(failed) + len(reports) + (0 if results else 1) + (1 if stuck else 0)
+        sys.stdout.flush()
+    return bad
 
 
 def run_unit(out, args, env=None):
