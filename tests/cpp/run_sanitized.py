@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Builds the host library and the C++ test programs with a sanitizer and runs the CPU suites.
 
-    python tests/cpp/run_sanitized.py thread|address [build_dir] [--build-only | --run-only] [--gpu | --stand-in] [--repeat=N]
+    python tests/cpp/run_sanitized.py thread|address|undefined [build_dir] [--build-only | --run-only] [--gpu | --stand-in] [--repeat=N]
 
 Host code only (g++ -fsanitize=...); libtphip.so is used as built. With --gpu the suites of the
 device channels run instead of the CPU ones (on a machine with a GPU; --build-only on one machine
@@ -136,7 +136,7 @@ def run_conformance(out, env):
         text, stuck = run_once([prog, *args], env, 600)
         results = [l for l in text.splitlines() if l.startswith("RESULT")]
         failed = [l for l in results if " OK" not in l]
-        reports = [l for l in text.splitlines() if "ERROR: AddressSanitizer" in l]
+        reports = sanitizer_lines(text)
         print(f"stock_conformance {' '.join(args)}: {len(results)} results, {len(failed)} failed, "
               f"{len(reports)} sanitizer reports{', STUCK: stacks below' if stuck else ''}")
         for l in failed + reports[:5]:
@@ -151,7 +151,7 @@ def run_conformance(out, env):
 def run_unit(out, args, env=None):
     proc = subprocess.run([os.path.join(out, "unit_tests"), *args],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900, env=env)
-    reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+    reports = sanitizer_lines(proc.stdout)
     lines = proc.stdout.strip().splitlines()
     ok = proc.returncode == 0 and bool(lines) and lines[-1].startswith("OK")
     print(f"unit_tests {args[0]}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
@@ -159,6 +159,12 @@ def run_unit(out, args, env=None):
         print("   ", l[:200])
     sys.stdout.flush()
     return (0 if ok else 1) + len(reports)
+
+
+def sanitizer_lines(text):
+    """The lines with which a sanitizer announces a finding (thread, address, undefined behaviour)."""
+    marks = ("WARNING: ThreadSanitizer", "ERROR: AddressSanitizer", "runtime error:")
+    return [l for l in text.splitlines() if any(m in l for m in marks)]
 
 
 def run_once(cmd, env, limit):
@@ -185,7 +191,7 @@ def run_suites(out, suites, base_env=None):
             text, stuck = run_once([os.path.join(out, prog), "--suite", suite], env, 1800 if REPEAT == 1 else 180)
             results = [l for l in text.splitlines() if l.startswith("RESULT")]
             failed = [l for l in results if " OK" not in l]
-            reports = [l for l in text.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+            reports = sanitizer_lines(text)
             if stuck or failed or reports or not results:
                 break
         where = f" (turn {turn + 1} of {REPEAT})" if REPEAT > 1 else ""
@@ -207,7 +213,7 @@ def run_cpu(out):
     for seed in (11, 12, 13):
         proc = subprocess.run([os.path.join(out, "unit_tests"), "garbage", str(seed), "150"],
                               stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
-        reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+        reports = sanitizer_lines(proc.stdout)
         ok = proc.returncode == 0 and proc.stdout.strip().endswith("OK")
         print(f"unit_tests garbage {seed}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
         for l in reports[:5]:
@@ -216,7 +222,7 @@ def run_cpu(out):
     # a peer that wrote and left before the reads were posted
     proc = subprocess.run([os.path.join(out, "unit_tests"), "departed_peer"],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
-    reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+    reports = sanitizer_lines(proc.stdout)
     ok = proc.returncode == 0 and proc.stdout.strip().endswith("OK")
     print(f"unit_tests departed_peer: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
     for l in reports[:5]:
@@ -228,7 +234,7 @@ def run_cpu(out):
                  ["transport_suite", "shm"], ["transport_suite", "shm_stock"], ["transport_suite", "tcp"]):
         proc = subprocess.run([os.path.join(out, "unit_tests"), *args],
                               stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
-        reports = [l for l in proc.stdout.splitlines() if "WARNING: ThreadSanitizer" in l or "ERROR: AddressSanitizer" in l]
+        reports = sanitizer_lines(proc.stdout)
         ok = proc.returncode == 0 and proc.stdout.strip().splitlines()[-1].startswith("OK")
         print(f"unit_tests {' '.join(a for a in args if not os.path.isabs(a))}: {'ok' if ok else 'FAILED'}, {len(reports)} sanitizer reports")
         for l in reports[:5] + ([] if ok else proc.stdout.strip().splitlines()[-8:]):
