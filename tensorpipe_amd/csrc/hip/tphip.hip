@@ -44,8 +44,8 @@ constexpr uint64_t kMaxTableVectors = 0xFFFFFFFFull - 64ull * 8ull;
 std::atomic<uint64_t> gTableLimit{kMaxTableVectors}; // lowered by tests only
 
 struct DeviceState {
-  std::once_flag once;
-  int initError{0};
+  std::atomic<bool> ready{false};
+  std::mutex initMutex;
   int numCus{0};
   // Ring of plan slots: host side (pinned, device-mapped) and device side.
   char* hostPlans{nullptr};
@@ -235,27 +235,58 @@ int getDevice(int dev, DeviceState** out) {
   }
   DeviceState& st = gDevices[dev];
   TPHIP_ON_DEVICE(dev);
-  std::call_once(st.once, [&] {
-    hipError_t e = hipDeviceGetAttribute(&st.numCus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e == hipSuccess) {
-      e = hipHostMalloc(
-          reinterpret_cast<void**>(&st.hostPlans),
-          kPlanSlots * kPlanSlotBytes,
-          hipHostMallocMapped | hipHostMallocPortable);
+  // A failure is reported and forgotten: the next call tries again from the
+  // start (an allocation refused once, say while another thread's stream is
+  // being captured, must not disable the device for the rest of the process).
+  if (!st.ready.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(st.initMutex);
+    if (!st.ready.load(std::memory_order_relaxed)) {
+      int cus = 0;
+      char* hostPlans = nullptr;
+      char* hostPlansDev = nullptr;
+      char* devPlans = nullptr;
+      hipEvent_t slotDone[kPlanSlots]{};
+      hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e == hipSuccess) {
+        e = hipHostMalloc(
+            reinterpret_cast<void**>(&hostPlans),
+            kPlanSlots * kPlanSlotBytes,
+            hipHostMallocMapped | hipHostMallocPortable);
+      }
+      if (e == hipSuccess) {
+        e = hipHostGetDevicePointer(reinterpret_cast<void**>(&hostPlansDev), hostPlans, 0);
+      }
+      if (e == hipSuccess) {
+        e = hipMalloc(reinterpret_cast<void**>(&devPlans), kPlanSlots * kPlanSlotBytes);
+      }
+      for (uint32_t i = 0; e == hipSuccess && i < kPlanSlots; ++i) {
+        e = hipEventCreateWithFlags(&slotDone[i], hipEventDisableTiming);
+      }
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        for (uint32_t i = 0; i < kPlanSlots; ++i) {
+          if (slotDone[i] != nullptr) {
+            (void)hipEventDestroy(slotDone[i]);
+          }
+        }
+        if (devPlans != nullptr) {
+          (void)hipFree(devPlans);
+        }
+        if (hostPlans != nullptr) {
+          (void)hipHostFree(hostPlans);
+        }
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+      }
+      st.numCus = cus;
+      st.hostPlans = hostPlans;
+      st.hostPlansDev = hostPlansDev;
+      st.devPlans = devPlans;
+      for (uint32_t i = 0; i < kPlanSlots; ++i) {
+        st.slotDone[i] = slotDone[i];
+      }
+      st.ready.store(true, std::memory_order_release);
     }
-    if (e == hipSuccess) {
-      e = hipHostGetDevicePointer(reinterpret_cast<void**>(&st.hostPlansDev), st.hostPlans, 0);
-    }
-    if (e == hipSuccess) {
-      e = hipMalloc(reinterpret_cast<void**>(&st.devPlans), kPlanSlots * kPlanSlotBytes);
-    }
-    for (uint32_t i = 0; e == hipSuccess && i < kPlanSlots; ++i) {
-      e = hipEventCreateWithFlags(&st.slotDone[i], hipEventDisableTiming);
-    }
-    st.initError = static_cast<int>(e);
-  });
-  if (st.initError != 0) {
-    return st.initError;
   }
   *out = &st;
   return 0;
