@@ -162,8 +162,8 @@ def run_unit(out, args, env=None):
 
 
 def sanitizer_lines(text):
-    """The lines with which a sanitizer announces a finding (thread, address, undefined behaviour)."""
-    marks = ("WARNING: ThreadSanitizer", "ERROR: AddressSanitizer", "runtime error:")
+    """The lines with which a sanitizer announces a finding (thread, address, leak, undefined behaviour)."""
+    marks = ("WARNING: ThreadSanitizer", "ERROR: AddressSanitizer", "ERROR: LeakSanitizer", "runtime error:")
     return [l for l in text.splitlines() if any(m in l for m in marks)]
 
 
